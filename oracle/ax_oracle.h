@@ -1,0 +1,88 @@
+/* ax_oracle.h — CPU restatement of Axiom's GEMM hot path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This library is the checker the GPU results are compared against (and the timed CPU
+ * leg of the benchmark).  Nothing in the product links, loads or calls it: the shipped
+ * libraries fail with an error when the HIP path is unavailable instead of coming here.
+ *
+ * Each function names the reference source it follows (paths relative to the Axiom tree).
+ * Pinning status (what each function has been checked against):
+ *   rng_*            reference known answers + the compiled reference, bit-exact
+ *   quantize_rows    compiled reference, bit-exact; hand-derived vectors (ties, zero row)
+ *   qgemm_w8a32      compiled reference, bit-exact (same lane order and FMA placement)
+ *   gemm_naive       compiled reference cpu_naive backend, bit-exact
+ *   gemm_opt/_nt     fp64 ground truth bound + compiled reference cpu_opt within 1e-4
+ *                    (bit-exact on the skinny/small route, whose order is fully specified)
+ *   gemm_f64         the mathematics: known answers 58/64/139/154, 19/22/43/50, A*I=A
+ *   qgemm_w8a8_acc   exact integer closed form; brute force; the reference's W8A32
+ *                    routine with unit scales for K <= 1040 (partial sums < 2^24)
+ *   gelu_tanh        closed form in fp64 + the compiled reference's ax_gelu within 2e-6
+ *   w8a8 epilogue    defined by this build (no reference counterpart): checked against
+ *                    an fp64 evaluation of the same formula
+ */
+#ifndef AX_ORACLE_H
+#define AX_ORACLE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- RNG: src/core/rng.c ------------------------------------------------ */
+void     axo_rng_seed(uint64_t seed);                 /* rng.c:33-40 (splitmix64 x4) */
+uint64_t axo_rng_uint64(void);                        /* rng.c:56-71 (xoshiro256**)  */
+float    axo_rng_float(void);                         /* rng.c:73-76 (top 24 bits)   */
+float    axo_rng_uniform(float lo, float hi);         /* rng.c:78-80                 */
+float    axo_rng_normal(void);                        /* rng.c:87-105 (polar, cached spare) */
+uint64_t axo_rng_bounded(uint64_t n);                 /* rng.c:111-121 (rejection)   */
+void     axo_rng_drop_spare(void);                    /* forget the cached normal    */
+void     axo_fill_uniform(float *dst, int64_t n, float lo, float hi);   /* tensor.c:520-531 */
+void     axo_fill_normal(float *dst, int64_t n, float mean, float std); /* rng.c:107-109   */
+void     axo_fill_kaiming_uniform(float *dst, int64_t n, int64_t fan_in); /* init.c:84-94  */
+void     axo_fill_int8(int8_t *dst, int64_t n);       /* (int8)(bounded(255) - 127)  */
+
+/* ---- fp32 GEMM ---------------------------------------------------------- */
+/* ground truth: fp64 accumulation, fp64 result.  transb: B stored [N,K]. */
+void axo_gemm_f64(const float *a, const float *b, double *c, int64_t M, int64_t N, int64_t K,
+                  int transb);
+/* sum_k |a_ik|*|b_kj| in fp64: the scale of the rounding-error bound. */
+void axo_gemm_abs_f64(const float *a, const float *b, double *c, int64_t M, int64_t N,
+                      int64_t K, int transb);
+/* cpu_naive.c:150-187: fp32 running sum, k ascending, separate multiply and add. */
+void axo_gemm_naive(const float *a, const float *b, float *c, int64_t M, int64_t N, int64_t K);
+/* cpu_opt.c:3509: 1 when (m,n,k) takes the serial small/skinny-M AXPY route (MR = 6). */
+int  axo_gemm_takes_small_route(int64_t m, int64_t n, int64_t k);
+/* cpu_opt.c:3446-3956: small route, else packed 6x16 BLIS loops (JC-parallel). */
+void axo_gemm_opt(const float *a, const float *b, float *c, int64_t M, int64_t N, int64_t K);
+/* cpu_opt.c:4842-5258: C = A[M,K] * B[N,K]^T through the same packed kernel. */
+void axo_gemm_opt_nt(const float *a, const float *b, float *c, int64_t M, int64_t N, int64_t K);
+/* cpu_opt.c:7148-7194 with the mathematically intended axis: c[m,n] += bias[n]. */
+void axo_bias_add_cols(float *c, const float *bias, int64_t M, int64_t N);
+/* cpu_opt.c:7401-7440: c = max(c + bias[n], 0); bias may be NULL. */
+void axo_bias_relu(float *c, const float *bias, int64_t M, int64_t N);
+/* activations.c:24-25,267-316 (scalar tail form): 0.5x(1+tanh(0.79788456(x+0.044715x^3))). */
+float axo_gelu_tanh(float x);
+void  axo_gelu(float *x, int64_t n);
+double axo_gelu_f64(double x);
+
+/* ---- int8 --------------------------------------------------------------- */
+/* quantize.c:21-57: per-row absmax/127, zero row -> 1, lrintf, clamp +-127. */
+void axo_quantize_rows(const float *w, int64_t N, int64_t K, int8_t *q, float *scales);
+/* quantize.c:66-76 */
+void axo_dequantize_rows(const int8_t *q, const float *scales, int64_t N, int64_t K, float *out);
+/* quantize.c:100-177, AVX2 build: 4x8 lane partial sums, 8-wide tail, pairwise reduce. */
+void axo_qgemm_w8a32(const float *a, const int8_t *q, const float *scales, float *out,
+                     int64_t M, int64_t N, int64_t K);
+/* exact: acc[m,n] = sum_k (int32)x[m,k]*(int32)w[n,k]  (no reference counterpart). */
+void axo_qgemm_w8a8_acc(const int8_t *x, const int8_t *w, int32_t *acc,
+                        int64_t M, int64_t N, int64_t K);
+/* out = act((float)acc * (x_scale*w_scale[n]) + bias[n]); act: 0 none, 1 relu, 2 gelu.
+   Evaluated as one fp32 product of the scales, one int->float convert, one fused
+   multiply-add (plain multiply when bias is NULL). */
+void axo_w8a8_epilogue(const int32_t *acc, float x_scale, const float *w_scales,
+                       const float *bias, int act, float *out, int64_t M, int64_t N);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,115 @@
+"""Writes tests/golden/golden.npz from the compiled reference (oracle/_ref/libaxref.so).
+
+Run where the reference was built:  python tests/golden/make_golden.py
+Every array is an input/output vector of the reference's public C API; the file holds
+data only.  Inputs that tests can regenerate (seeded fills) are stored as checksums.
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+from fills import property_case, xorshift32_unit  # noqa: E402
+from oracle_bind import RefLib  # noqa: E402
+
+r = RefLib()
+L = r.L
+G = {}
+
+# ---- RNG known answers (src/core/rng.c) -----------------------------------
+for seed in (0, 42):
+    L.ax_rng_seed(seed)
+    G[f"rng_u64_seed{seed}"] = np.array([L.ax_rng_uint64() for _ in range(8)], np.uint64)
+    L.ax_rng_seed(seed)
+    G[f"rng_uniform_seed{seed}"] = np.array([L.ax_rng_uniform(-1.0, 1.0) for _ in range(8)], np.float32)
+    L.ax_rng_seed(seed)
+    G[f"rng_normal_seed{seed}"] = np.array([L.ax_rng_normal() for _ in range(8)], np.float32)
+    L.ax_rng_seed(seed)
+    G[f"rng_bounded255_seed{seed}"] = np.array([L.ax_rng_bounded(255) for _ in range(32)], np.uint64)
+
+
+def ref_uniform(n, lo, hi):
+    return np.array([L.ax_rng_uniform(lo, hi) for _ in range(n)], np.float32)
+
+
+# ---- quantizer (src/core/quantize.c:21-57) --------------------------------
+hand = np.array([[0.5, -1.0, 0.25, 0.1], [0.0, 0.0, 0.0, 0.0]], np.float32)
+G["quant_hand_w"] = hand
+G["quant_hand_q"], G["quant_hand_s"] = r.quantize_rows(hand)
+s = np.float32(1.0) / np.float32(127.0)
+ties = np.array([[127 * s, 0.5 * s, 1.5 * s, 2.5 * s, -0.5 * s, -1.5 * s, -2.5 * s, 3.5 * s]], np.float32)
+G["quant_ties_w"] = ties
+G["quant_ties_q"], G["quant_ties_s"] = r.quantize_rows(ties)
+for (N, K) in ((8, 8), (128, 128), (64, 1024)):          # tests/test_quantize.c:60-69 shapes
+    w = xorshift32_unit(N * K, 42).reshape(N, K)
+    q, sc = r.quantize_rows(w)
+    G[f"quant_{N}x{K}_q"], G[f"quant_{N}x{K}_s"] = q, sc
+
+# ---- W8A32 (src/core/quantize.c:100-177) at tests/test_quantize.c:133-137 shapes
+for (M, N, K) in ((1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 1024), (3, 17, 45)):
+    a = xorshift32_unit(M * K, 7).reshape(M, K)
+    w = xorshift32_unit(N * K, 13).reshape(N, K)
+    q, sc = r.quantize_rows(w)
+    G[f"w8a32_{M}x{N}x{K}_out"] = r.qgemm_w8a32(a, q, sc)
+
+# ---- int8 accumulators through the reference's W8A32 routine with unit scales
+for K in (8, 32, 128, 512, 1024):
+    L.ax_rng_seed(1000 + K)
+    x = np.array([int(L.ax_rng_bounded(255)) - 127 for _ in range(4 * K)], np.int8).reshape(4, K)
+    w = np.array([int(L.ax_rng_bounded(255)) - 127 for _ in range(64 * K)], np.int8).reshape(64, K)
+    G[f"acc_K{K}_x_sum"] = np.array([x.astype(np.int64).sum()])
+    G[f"acc_K{K}_w_sum"] = np.array([w.astype(np.int64).sum()])
+    G[f"acc_K{K}"] = r.qgemm_w8a32(x.astype(np.float32), w, np.ones(64, np.float32))
+xs = np.full((2, 1024), 127, np.int8)
+ws = np.full((3, 1024), -127, np.int8)
+G["acc_extreme"] = r.qgemm_w8a32(xs.astype(np.float32), ws, np.ones(3, np.float32))
+
+# ---- fp32 GEMM ---------------------------------------------------------------
+# known answers held by the reference's tests (test_compute.c:162-199, test_cuda.c:44-58)
+a = np.arange(1, 7, dtype=np.float32).reshape(2, 3)
+b = np.arange(7, 13, dtype=np.float32).reshape(3, 2)
+G["gemm_2x3x2"] = r.gemm(a, b)
+G["gemm_2x2x2"] = r.gemm(np.array([[1, 2], [3, 4]], np.float32), np.array([[5, 6], [7, 8]], np.float32))
+for (M, K, N) in ((37, 73, 19), (64, 128, 32), (32, 2048, 16), (1, 784, 64), (7, 300, 130)):
+    L.ax_rng_seed(M * 1000 + N)
+    a = ref_uniform(M * K, -1.0, 1.0).reshape(M, K)
+    b = ref_uniform(K * N, -1.0, 1.0).reshape(K, N)
+    G[f"gemm_{M}x{K}x{N}_opt"] = r.gemm(a, b, backend=1)
+    G[f"gemm_{M}x{K}x{N}_naive"] = r.gemm(a, b, backend=0)
+    G[f"gemm_nt_{M}x{K}x{N}_opt"] = r.gemm(a, np.ascontiguousarray(b.T), backend=1, nt=True)
+# 1024^3 from ax_set_seed(0): checksums only
+L.ax_set_seed(0)
+A = ref_uniform(1024 * 1024, -1.0, 1.0).reshape(1024, 1024)
+B = ref_uniform(1024 * 1024, -1.0, 1.0).reshape(1024, 1024)
+Cm = r.gemm(A, B)
+G["gemm_1024_probe"] = np.array([A[0, 0], B[0, 0], Cm[0, 0], Cm[-1, -1]], np.float32)
+G["gemm_1024_sums"] = np.array([Cm.astype(np.float64).sum(), np.abs(Cm).astype(np.float64).sum()])
+G["gemm_1024_row0"] = Cm[0].copy()
+G["gemm_1024_diag"] = np.diagonal(Cm).copy()
+# the 60 property cases (tests/test_property.c:176-208)
+shapes, sums = [], []
+for i in range(60):
+    M, N, K, a, b = property_case(i)
+    cn = r.gemm(a, b, backend=0)
+    co = r.gemm(a, b, backend=1)
+    shapes.append((M, N, K))
+    sums.append((cn.astype(np.float64).sum(), co.astype(np.float64).sum(),
+                 np.abs(co).astype(np.float64).sum(), float(co[0, 0]), float(co[-1, -1])))
+G["prop_shapes"] = np.array(shapes, np.int64)
+G["prop_sums"] = np.array(sums, np.float64)
+
+# ---- fused bias + relu (cpu_opt.c:7401-7440) and GELU (activations.c:267-316)
+L.ax_rng_seed(77)
+a = ref_uniform(33 * 100, -1.0, 1.0).reshape(33, 100)
+b = ref_uniform(100 * 40, -1.0, 1.0).reshape(100, 40)
+bias = ref_uniform(40, -0.5, 0.5)
+G["gemm_relu_33x100x40"] = r.gemm_relu(a, b, bias)
+G["gemm_relu_33x100x40_nobias"] = r.gemm_relu(a, b, None)
+xg = np.linspace(-6, 6, 1201, dtype=np.float32)
+G["gelu_x"] = xg
+G["gelu_y"] = r.gelu(xg.reshape(1, -1)).reshape(-1)
+
+np.savez_compressed(os.path.join(HERE, "golden.npz"), **G)
+print("wrote", len(G), "arrays,", os.path.getsize(os.path.join(HERE, "golden.npz")), "bytes")

@@ -1,0 +1,362 @@
+"""ctypes bindings for the two checkers used by the tests.
+
+* ``Oracle``  — oracle/libax_oracle.so, this repository's CPU restatement of the path.
+* ``RefLib``  — oracle/_ref/libaxref.so, the unmodified reference library compiled by
+  oracle/Makefile.  Optional: absent unless it was built where the reference tree exists.
+
+Checker code only: nothing under axiom_amd/ imports this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_SO = os.path.join(ROOT, "oracle", "libax_oracle.so")
+REF_SO = os.path.join(ROOT, "oracle", "_ref", "libaxref.so")
+
+f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+f64p = np.ctypeslib.ndpointer(np.float64, flags="C_CONTIGUOUS")
+i8p = np.ctypeslib.ndpointer(np.int8, flags="C_CONTIGUOUS")
+i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
+i64 = C.c_int64
+
+
+def build_oracle():
+    subprocess.check_call(["make", "-s", "-C", os.path.join(ROOT, "oracle"), "oracle"])
+
+
+class Oracle:
+    def __init__(self):
+        if not os.path.exists(ORACLE_SO):
+            build_oracle()
+        L = self.L = C.CDLL(ORACLE_SO)
+        L.axo_rng_seed.argtypes = [C.c_uint64]
+        L.axo_rng_uint64.restype = C.c_uint64
+        L.axo_rng_float.restype = C.c_float
+        L.axo_rng_uniform.restype = C.c_float
+        L.axo_rng_uniform.argtypes = [C.c_float, C.c_float]
+        L.axo_rng_normal.restype = C.c_float
+        L.axo_rng_bounded.restype = C.c_uint64
+        L.axo_rng_bounded.argtypes = [C.c_uint64]
+        L.axo_fill_uniform.argtypes = [f32p, i64, C.c_float, C.c_float]
+        L.axo_fill_normal.argtypes = [f32p, i64, C.c_float, C.c_float]
+        L.axo_fill_kaiming_uniform.argtypes = [f32p, i64, i64]
+        L.axo_fill_int8.argtypes = [i8p, i64]
+        L.axo_gemm_f64.argtypes = [f32p, f32p, f64p, i64, i64, i64, C.c_int]
+        L.axo_gemm_abs_f64.argtypes = [f32p, f32p, f64p, i64, i64, i64, C.c_int]
+        L.axo_gemm_naive.argtypes = [f32p, f32p, f32p, i64, i64, i64]
+        L.axo_gemm_takes_small_route.argtypes = [i64, i64, i64]
+        L.axo_gemm_opt.argtypes = [f32p, f32p, f32p, i64, i64, i64]
+        L.axo_gemm_opt_nt.argtypes = [f32p, f32p, f32p, i64, i64, i64]
+        L.axo_bias_add_cols.argtypes = [f32p, f32p, i64, i64]
+        L.axo_bias_relu.argtypes = [f32p, C.c_void_p, i64, i64]
+        L.axo_gelu_tanh.restype = C.c_float
+        L.axo_gelu_tanh.argtypes = [C.c_float]
+        L.axo_gelu_f64.restype = C.c_double
+        L.axo_gelu_f64.argtypes = [C.c_double]
+        L.axo_gelu.argtypes = [f32p, i64]
+        L.axo_quantize_rows.argtypes = [f32p, i64, i64, i8p, f32p]
+        L.axo_dequantize_rows.argtypes = [i8p, f32p, i64, i64, f32p]
+        L.axo_qgemm_w8a32.argtypes = [f32p, i8p, f32p, f32p, i64, i64, i64]
+        L.axo_qgemm_w8a8_acc.argtypes = [i8p, i8p, i32p, i64, i64, i64]
+        L.axo_w8a8_epilogue.argtypes = [i32p, C.c_float, f32p, C.c_void_p, C.c_int, f32p, i64, i64]
+
+    # ---- RNG -------------------------------------------------------------
+    def seed(self, s, drop_spare=True):
+        self.L.axo_rng_seed(s)
+        if drop_spare:
+            self.L.axo_rng_drop_spare()
+
+    def uniform(self, shape, lo, hi):
+        out = np.empty(shape, np.float32)
+        self.L.axo_fill_uniform(out.reshape(-1), out.size, lo, hi)
+        return out
+
+    def normal(self, shape, mean=0.0, std=1.0):
+        out = np.empty(shape, np.float32)
+        self.L.axo_fill_normal(out.reshape(-1), out.size, mean, std)
+        return out
+
+    def kaiming(self, shape, fan_in):
+        out = np.empty(shape, np.float32)
+        self.L.axo_fill_kaiming_uniform(out.reshape(-1), out.size, fan_in)
+        return out
+
+    def int8(self, shape):
+        out = np.empty(shape, np.int8)
+        self.L.axo_fill_int8(out.reshape(-1), out.size)
+        return out
+
+    # ---- GEMM ------------------------------------------------------------
+    def gemm_f64(self, a, b, transb=False):
+        M, K = a.shape
+        N = b.shape[0] if transb else b.shape[1]
+        c = np.empty((M, N), np.float64)
+        self.L.axo_gemm_f64(a, b, c, M, N, K, int(transb))
+        return c
+
+    def gemm_abs_f64(self, a, b, transb=False):
+        M, K = a.shape
+        N = b.shape[0] if transb else b.shape[1]
+        c = np.empty((M, N), np.float64)
+        self.L.axo_gemm_abs_f64(a, b, c, M, N, K, int(transb))
+        return c
+
+    def gemm_naive(self, a, b):
+        M, K = a.shape
+        N = b.shape[1]
+        c = np.empty((M, N), np.float32)
+        self.L.axo_gemm_naive(a, b, c, M, N, K)
+        return c
+
+    def gemm_opt(self, a, b):
+        M, K = a.shape
+        N = b.shape[1]
+        c = np.empty((M, N), np.float32)
+        self.L.axo_gemm_opt(a, b, c, M, N, K)
+        return c
+
+    def gemm_opt_nt(self, a, b):
+        M, K = a.shape
+        N = b.shape[0]
+        c = np.empty((M, N), np.float32)
+        self.L.axo_gemm_opt_nt(a, b, c, M, N, K)
+        return c
+
+    def small_route(self, m, n, k):
+        return bool(self.L.axo_gemm_takes_small_route(m, n, k))
+
+    def bias_add(self, c, bias):
+        c = np.ascontiguousarray(c, np.float32).copy()
+        self.L.axo_bias_add_cols(c, bias, c.shape[0], c.shape[1])
+        return c
+
+    def bias_relu(self, c, bias):
+        c = np.ascontiguousarray(c, np.float32).copy()
+        bp = bias.ctypes.data_as(C.c_void_p) if bias is not None else None
+        self.L.axo_bias_relu(c, bp, c.shape[0], c.shape[1])
+        return c
+
+    def gelu(self, x):
+        x = np.ascontiguousarray(x, np.float32).copy()
+        self.L.axo_gelu(x.reshape(-1), x.size)
+        return x
+
+    def dense(self, x, w, bias=None, act=0):
+        """act(x @ w + bias[n]) through the cpu_opt restatement; act 0 none, 1 relu, 2 gelu."""
+        c = self.gemm_opt(x, w)
+        if act == 1:
+            return self.bias_relu(c, bias)
+        if bias is not None:
+            c = self.bias_add(c, bias)
+        if act == 2:
+            c = self.gelu(c)
+        return c
+
+    # ---- int8 ------------------------------------------------------------
+    def quantize_rows(self, w):
+        N, K = w.shape
+        q = np.empty((N, K), np.int8)
+        s = np.empty(N, np.float32)
+        self.L.axo_quantize_rows(w, N, K, q, s)
+        return q, s
+
+    def dequantize_rows(self, q, s):
+        out = np.empty(q.shape, np.float32)
+        self.L.axo_dequantize_rows(q, s, q.shape[0], q.shape[1], out)
+        return out
+
+    def qgemm_w8a32(self, a, q, s):
+        M, K = a.shape
+        N = q.shape[0]
+        out = np.empty((M, N), np.float32)
+        self.L.axo_qgemm_w8a32(a, q, s, out, M, N, K)
+        return out
+
+    def qgemm_w8a8_acc(self, x, w):
+        M, K = x.shape
+        N = w.shape[0]
+        acc = np.empty((M, N), np.int32)
+        self.L.axo_qgemm_w8a8_acc(x, w, acc, M, N, K)
+        return acc
+
+    def w8a8_epilogue(self, acc, x_scale, w_scales, bias=None, act=0):
+        M, N = acc.shape
+        out = np.empty((M, N), np.float32)
+        bp = bias.ctypes.data_as(C.c_void_p) if bias is not None else None
+        self.L.axo_w8a8_epilogue(acc, x_scale, w_scales, bp, act, out, M, N)
+        return out
+
+
+# ---------------------------------------------------------------------------
+# the compiled reference
+# ---------------------------------------------------------------------------
+AX_MAX_DIMS = 8
+
+
+class RefStorage(C.Structure):            # include/axiom/tensor.h:29-43
+    _fields_ = [("data", C.c_void_p), ("size_bytes", C.c_size_t), ("refcount", C.c_int),
+                ("device", C.c_int), ("is_arena_temp", C.c_bool), ("generation", C.c_uint64)]
+
+
+class RefTensor(C.Structure):             # include/axiom/tensor.h:53-70
+    pass
+
+
+RefTensor._fields_ = [("storage", C.POINTER(RefStorage)), ("shape", i64 * AX_MAX_DIMS),
+                      ("strides", i64 * AX_MAX_DIMS), ("ndim", C.c_int), ("dtype", C.c_int),
+                      ("offset", i64), ("requires_grad", C.c_bool),
+                      ("grad", C.POINTER(RefTensor)), ("grad_fn", C.c_void_p),
+                      ("layout", C.c_int)]
+
+
+class RefQWeight(C.Structure):            # include/axiom/quantize.h:50-55
+    _fields_ = [("data", C.POINTER(C.c_int8)), ("scales", C.POINTER(C.c_float)),
+                ("N", i64), ("K", i64)]
+
+
+def ref_available():
+    return os.path.exists(REF_SO)
+
+
+class RefLib:
+    """The reference library itself (CPU backends), driven through its public C API."""
+    CPU_NAIVE, CPU_SIMD = 0, 1
+
+    def __init__(self):
+        # keep the reference from calibrating / writing a cache under $HOME
+        os.environ.setdefault("AX_NO_CALIB_CACHE", "1")
+        os.environ.setdefault("AX_GEMM_CALIBRATE", "0")
+        os.environ.setdefault("AX_NO_AUTOTUNE", "1")
+        L = self.L = C.CDLL(REF_SO, mode=C.RTLD_GLOBAL)
+        TP = C.POINTER(RefTensor)
+        L.ax_rng_seed.argtypes = [C.c_uint64]
+        L.ax_rng_uint64.restype = C.c_uint64
+        L.ax_rng_float.restype = C.c_float
+        L.ax_rng_uniform.restype = C.c_float
+        L.ax_rng_uniform.argtypes = [C.c_float, C.c_float]
+        L.ax_rng_normal.restype = C.c_float
+        L.ax_rng_bounded.restype = C.c_uint64
+        L.ax_rng_bounded.argtypes = [C.c_uint64]
+        L.ax_set_seed.argtypes = [C.c_uint]
+        L.ax_tensor_create.restype = TP
+        L.ax_tensor_create.argtypes = [C.POINTER(i64), C.c_int, C.c_int]
+        L.ax_tensor_zeros.restype = TP
+        L.ax_tensor_zeros.argtypes = [C.POINTER(i64), C.c_int, C.c_int]
+        L.ax_tensor_rand.restype = TP
+        L.ax_tensor_rand.argtypes = [C.POINTER(i64), C.c_int, C.c_float, C.c_float]
+        L.ax_tensor_destroy.argtypes = [TP]
+        L.ax_compute_init.restype = C.c_int
+        L.ax_compute_set_backend.argtypes = [C.c_int]
+        L.ax_compute_set_backend.restype = C.c_int
+        for name in ("ax_compute_gemm", "ax_compute_gemm_nt"):
+            getattr(L, name).argtypes = [TP, TP, TP]
+            getattr(L, name).restype = C.c_int
+        L.ax_compute_gemm_relu.argtypes = [TP, TP, TP, TP]
+        L.ax_compute_gemm_relu.restype = C.c_int
+        L.ax_compute_bias_add.argtypes = [TP, TP, C.c_int, TP]
+        L.ax_compute_bias_add.restype = C.c_int
+        L.ax_gelu.restype = TP
+        L.ax_gelu.argtypes = [TP]
+        L.ax_no_grad.restype = None
+        L.ax_qweight_create_from_fp32.restype = C.POINTER(RefQWeight)
+        L.ax_qweight_create_from_fp32.argtypes = [f32p, i64, i64]
+        L.ax_qweight_destroy.argtypes = [C.POINTER(RefQWeight)]
+        L.ax_qgemm_w8a32.restype = C.c_int
+        L.ax_qgemm_w8a32.argtypes = [f32p, C.POINTER(RefQWeight), f32p, i64]
+        L.ax_init_kaiming_uniform.argtypes = [TP, i64]
+        L.ax_dense_create.restype = C.c_void_p
+        L.ax_dense_create.argtypes = [i64, i64, C.c_bool]
+        L.ax_relu_layer_create.restype = C.c_void_p
+        L.ax_sequential_create.restype = C.c_void_p
+        L.ax_sequential_add.restype = C.c_void_p
+        L.ax_sequential_add.argtypes = [C.c_void_p, C.c_void_p]
+        L.ax_layer_forward.restype = TP
+        L.ax_layer_forward.argtypes = [C.c_void_p, TP]
+        L.ax_layer_destroy.argtypes = [C.c_void_p]
+        L.ax_layer_get_params.restype = C.c_int
+        L.ax_layer_get_params.argtypes = [C.c_void_p, C.POINTER(TP), C.c_int]
+        L.ax_compute_init()
+        L.ax_no_grad()
+
+    # ---- tensors ----------------------------------------------------------
+    def tensor(self, arr):
+        arr = np.ascontiguousarray(arr, np.float32)
+        shape = (i64 * arr.ndim)(*arr.shape)
+        t = self.L.ax_tensor_create(shape, arr.ndim, 0)
+        C.memmove(t.contents.storage.contents.data, arr.ctypes.data, arr.nbytes)
+        return t
+
+    def empty(self, *shape):
+        sh = (i64 * len(shape))(*shape)
+        return self.L.ax_tensor_zeros(sh, len(shape), 0)
+
+    @staticmethod
+    def numpy(t):
+        tt = t.contents
+        shape = [tt.shape[i] for i in range(tt.ndim)]
+        n = int(np.prod(shape))
+        buf = (C.c_float * n).from_address(tt.storage.contents.data + 4 * tt.offset)
+        return np.frombuffer(buf, np.float32).reshape(shape).copy()
+
+    def free(self, *ts):
+        for t in ts:
+            self.L.ax_tensor_destroy(t)
+
+    def backend(self, which):
+        assert self.L.ax_compute_set_backend(which) == 0
+
+    # ---- ops --------------------------------------------------------------
+    def gemm(self, a, b, backend=1, nt=False):
+        self.backend(backend)
+        ta, tb = self.tensor(a), self.tensor(b)
+        N = b.shape[0] if nt else b.shape[1]
+        to = self.empty(a.shape[0], N)
+        fn = self.L.ax_compute_gemm_nt if nt else self.L.ax_compute_gemm
+        st = fn(ta, tb, to)
+        assert st == 0, st
+        out = self.numpy(to)
+        self.free(ta, tb, to)
+        return out
+
+    def gemm_relu(self, a, b, bias):
+        self.backend(self.CPU_SIMD)
+        ta, tb = self.tensor(a), self.tensor(b)
+        tbias = self.tensor(bias) if bias is not None else None
+        to = self.empty(a.shape[0], b.shape[1])
+        st = self.L.ax_compute_gemm_relu(ta, tb, tbias, to)
+        assert st == 0, st
+        out = self.numpy(to)
+        self.free(ta, tb, to)
+        if tbias:
+            self.free(tbias)
+        return out
+
+    def gelu(self, x):
+        t = self.tensor(x)
+        o = self.L.ax_gelu(t)
+        out = self.numpy(o)
+        self.free(t, o)
+        return out
+
+    def quantize_rows(self, w):
+        N, K = w.shape
+        qw = self.L.ax_qweight_create_from_fp32(np.ascontiguousarray(w), N, K)
+        q = np.ctypeslib.as_array(qw.contents.data, (N, K)).copy()
+        s = np.ctypeslib.as_array(qw.contents.scales, (N,)).copy()
+        self.L.ax_qweight_destroy(qw)
+        return q, s
+
+    def qgemm_w8a32(self, a, q, s):
+        """The reference routine on a hand-filled ax_qweight_t (a public struct)."""
+        q = np.ascontiguousarray(q, np.int8)
+        s = np.ascontiguousarray(s, np.float32)
+        qw = RefQWeight(q.ctypes.data_as(C.POINTER(C.c_int8)),
+                        s.ctypes.data_as(C.POINTER(C.c_float)), q.shape[0], q.shape[1])
+        out = np.empty((a.shape[0], q.shape[0]), np.float32)
+        st = self.L.ax_qgemm_w8a32(np.ascontiguousarray(a, np.float32), C.byref(qw), out,
+                                   a.shape[0])
+        assert st == 0
+        return out

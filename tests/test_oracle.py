@@ -1,0 +1,224 @@
+"""Pins the CPU oracle: golden vectors from the reference, the compiled reference itself
+(when built), and what the mathematics fixes.  No GPU."""
+import numpy as np
+import pytest
+
+from fills import property_case, xorshift32_unit
+
+
+# ---------------------------------------------------------------- RNG
+@pytest.mark.parametrize("seed", [0, 42])
+def test_rng_matches_reference_vectors(oracle, golden, seed):
+    L = oracle.L
+    oracle.seed(seed)
+    assert [L.axo_rng_uint64() for _ in range(8)] == list(golden[f"rng_u64_seed{seed}"])
+    oracle.seed(seed)
+    got = np.array([L.axo_rng_uniform(-1.0, 1.0) for _ in range(8)], np.float32)
+    assert np.array_equal(got, golden[f"rng_uniform_seed{seed}"])
+    oracle.seed(seed)
+    got = np.array([L.axo_rng_normal() for _ in range(8)], np.float32)
+    assert np.array_equal(got, golden[f"rng_normal_seed{seed}"])
+    oracle.seed(seed)
+    assert [L.axo_rng_bounded(255) for _ in range(32)] == list(golden[f"rng_bounded255_seed{seed}"])
+
+
+def test_rng_published_known_answers(oracle):
+    # xoshiro256** seeded by splitmix64(0): first outputs are a published test vector
+    oracle.seed(0)
+    assert oracle.L.axo_rng_uint64() == 0x99EC5F36CB75F2B4
+    assert oracle.L.axo_rng_uint64() == 0xBF6E1F784956452A
+
+
+def test_rng_statistics(oracle):
+    oracle.seed(123)
+    u = oracle.uniform((200000,), -1.0, 1.0)
+    assert u.min() >= -1.0 and u.max() < 1.0 and abs(u.mean()) < 0.01
+    n = oracle.normal((200000,), 0.0, 0.02)
+    assert abs(n.mean()) < 2e-4 and abs(n.std() - 0.02) < 2e-4
+    q = oracle.int8((100000,))
+    assert q.min() == -127 and q.max() == 127
+
+
+# ---------------------------------------------------------------- quantizer
+def test_quantizer_hand_vectors(oracle, golden):
+    q, s = oracle.quantize_rows(golden["quant_hand_w"])
+    assert np.array_equal(q, golden["quant_hand_q"]) and np.array_equal(s, golden["quant_hand_s"])
+    assert q[0].tolist() == [64, -127, 32, 13] and s[1] == 1.0 and not q[1].any()
+    q, s = oracle.quantize_rows(golden["quant_ties_w"])
+    assert np.array_equal(q, golden["quant_ties_q"]) and np.array_equal(s, golden["quant_ties_s"])
+    assert q[0, :4].tolist() == [127, 0, 2, 2]          # round-half-to-even
+
+
+@pytest.mark.parametrize("N,K", [(8, 8), (128, 128), (64, 1024)])
+def test_quantizer_reference_shapes(oracle, golden, N, K):
+    w = xorshift32_unit(N * K, 42).reshape(N, K)
+    q, s = oracle.quantize_rows(w)
+    assert np.array_equal(q, golden[f"quant_{N}x{K}_q"])
+    assert np.array_equal(s, golden[f"quant_{N}x{K}_s"])
+    # the reference's own invariant (tests/test_quantize.c:47-57)
+    assert (np.abs(w - oracle.dequantize_rows(q, s)) <= 1.5 * s[:, None]).all()
+
+
+# ---------------------------------------------------------------- W8A32
+@pytest.mark.parametrize("M,N,K", [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512),
+                                   (16, 256, 1024), (3, 17, 45)])
+def test_w8a32_matches_reference_output(oracle, golden, M, N, K):
+    a = xorshift32_unit(M * K, 7).reshape(M, K)
+    w = xorshift32_unit(N * K, 13).reshape(N, K)
+    q, s = oracle.quantize_rows(w)
+    out = oracle.qgemm_w8a32(a, q, s)
+    assert np.array_equal(out, golden[f"w8a32_{M}x{N}x{K}_out"])
+    # and the closed form the reference's test uses (tests/test_quantize.c:94-111)
+    want = a.astype(np.float64) @ oracle.dequantize_rows(q, s).astype(np.float64).T
+    diff = np.abs(out - want)
+    assert not ((diff > 1e-2) & (diff / np.maximum(np.abs(want), 1e-30) > 1e-3)).any()
+
+
+# ---------------------------------------------------------------- int8 accumulators
+@pytest.mark.parametrize("K", [8, 32, 128, 512, 1024])
+def test_int8_acc_equals_reference_w8a32_with_unit_scales(oracle, golden, K):
+    oracle.seed(1000 + K)
+    x = oracle.int8((4, K))
+    w = oracle.int8((64, K))
+    assert x.astype(np.int64).sum() == golden[f"acc_K{K}_x_sum"][0]
+    assert w.astype(np.int64).sum() == golden[f"acc_K{K}_w_sum"][0]
+    acc = oracle.qgemm_w8a8_acc(x, w)
+    assert np.array_equal(acc.astype(np.float64), golden[f"acc_K{K}"].astype(np.float64))
+
+
+def test_int8_acc_brute_force_and_extremes(oracle, golden):
+    oracle.seed(5)
+    x, w = oracle.int8((5, 37)), oracle.int8((7, 37))
+    brute = [[sum(int(x[m, k]) * int(w[n, k]) for k in range(37)) for n in range(7)] for m in range(5)]
+    assert oracle.qgemm_w8a8_acc(x, w).tolist() == brute
+    xs, ws = np.full((2, 1024), 127, np.int8), np.full((3, 1024), -127, np.int8)
+    acc = oracle.qgemm_w8a8_acc(xs, ws)
+    assert (acc == -127 * 127 * 1024).all()
+    assert np.array_equal(acc.astype(np.float64), golden["acc_extreme"].astype(np.float64))
+    big = oracle.qgemm_w8a8_acc(np.full((1, 8192), -127, np.int8), np.full((1, 8192), -127, np.int8))
+    assert big[0, 0] == 127 * 127 * 8192                 # largest magnitude at K = 8192
+
+
+def test_w8a8_epilogue_against_fp64(oracle):
+    oracle.seed(9)
+    x, w = oracle.int8((6, 300)), oracle.int8((10, 300))
+    ws = oracle.uniform((10,), 1e-3, 1e-2)
+    bias = oracle.normal((10,), 0.0, 0.02)
+    acc = oracle.qgemm_w8a8_acc(x, w)
+    xs = np.float32(0.0123)
+    for act in (0, 1, 2):
+        got = oracle.w8a8_epilogue(acc, xs, ws, bias, act)
+        v = acc.astype(np.float64) * (np.float64(xs) * ws.astype(np.float64)) + bias
+        if act == 1:
+            v = np.maximum(v, 0)
+        if act == 2:
+            v = 0.5 * v * (1 + np.tanh(0.7978845608028654 * (v + 0.044715 * v ** 3)))
+        assert np.abs(got - v).max() <= 1e-6 * max(1.0, np.abs(v).max())
+    nob = oracle.w8a8_epilogue(acc, xs, ws, None, 0)
+    assert np.array_equal(nob, acc.astype(np.float32) * (xs * ws)[None, :])
+
+
+# ---------------------------------------------------------------- fp32 GEMM
+def test_gemm_known_answers(oracle, golden):
+    a = np.arange(1, 7, dtype=np.float32).reshape(2, 3)
+    b = np.arange(7, 13, dtype=np.float32).reshape(3, 2)
+    for fn in (oracle.gemm_opt, oracle.gemm_naive, oracle.gemm_f64):
+        assert fn(a, b).reshape(-1).tolist() == [58, 64, 139, 154]
+    assert golden["gemm_2x3x2"].reshape(-1).tolist() == [58, 64, 139, 154]
+    c = oracle.gemm_opt(np.array([[1, 2], [3, 4]], np.float32), np.array([[5, 6], [7, 8]], np.float32))
+    assert c.reshape(-1).tolist() == [19, 22, 43, 50] == golden["gemm_2x2x2"].reshape(-1).tolist()
+    oracle.seed(3)
+    a = oracle.uniform((40, 40), -1, 1)
+    assert np.array_equal(oracle.gemm_opt(a, np.eye(40, dtype=np.float32)), a)
+    assert not oracle.gemm_opt(np.zeros((9, 300), np.float32), oracle.uniform((300, 500), -1, 1)).any()
+    # K = 1 outer product
+    u, v = oracle.uniform((33, 1), -1, 1), oracle.uniform((1, 65), -1, 1)
+    assert np.array_equal(oracle.gemm_opt(u, v), u * v)
+
+
+@pytest.mark.parametrize("M,K,N", [(37, 73, 19), (64, 128, 32), (32, 2048, 16), (1, 784, 64), (7, 300, 130)])
+def test_gemm_matches_reference_outputs(oracle, golden, M, K, N):
+    oracle.seed(M * 1000 + N)
+    a = oracle.uniform((M, K), -1, 1)
+    b = oracle.uniform((K, N), -1, 1)
+    assert np.array_equal(oracle.gemm_naive(a, b), golden[f"gemm_{M}x{K}x{N}_naive"])
+    ref = golden[f"gemm_{M}x{K}x{N}_opt"]
+    got = oracle.gemm_opt(a, b)
+    assert np.abs(got - ref).max() <= 1e-4 * np.abs(ref).max()
+    if oracle.small_route(M, N, K):
+        assert np.array_equal(got, ref)                  # order fully specified on this route
+    nt = oracle.gemm_opt_nt(a, np.ascontiguousarray(b.T))
+    assert np.abs(nt - golden[f"gemm_nt_{M}x{K}x{N}_opt"]).max() <= 1e-4 * np.abs(ref).max()
+    c64, cabs = oracle.gemm_f64(a, b), oracle.gemm_abs_f64(a, b)
+    assert (np.abs(got - c64) <= 1e-5 * cabs + 1e-30).all()
+    assert np.allclose(c64, a.astype(np.float64) @ b.astype(np.float64), rtol=1e-12, atol=1e-12)
+
+
+def test_gemm_1024_cube_against_reference_checksums(oracle, golden):
+    oracle.seed(0)
+    a = oracle.uniform((1024, 1024), -1, 1)
+    b = oracle.uniform((1024, 1024), -1, 1)
+    c = oracle.gemm_opt(a, b)
+    probe = golden["gemm_1024_probe"]
+    assert a[0, 0] == probe[0] and b[0, 0] == probe[1]
+    assert np.abs(c[0] - golden["gemm_1024_row0"]).max() <= 1e-4 * 60
+    assert np.abs(np.diagonal(c) - golden["gemm_1024_diag"]).max() <= 1e-4 * 60
+    s, sabs = golden["gemm_1024_sums"]
+    assert abs(c.astype(np.float64).sum() - s) <= 1e-6 * sabs
+    assert abs(np.abs(c).astype(np.float64).sum() - sabs) <= 1e-6 * sabs
+
+
+def test_gemm_property_cases(oracle, golden):
+    shapes, sums = golden["prop_shapes"], golden["prop_sums"]
+    for i in range(60):
+        M, N, K, a, b = property_case(i)
+        assert (M, N, K) == tuple(shapes[i])
+        cn, co = oracle.gemm_naive(a, b), oracle.gemm_opt(a, b)
+        # the reference's own gate (tests/test_property.c:198): atol 1e-3 + rtol 1e-4
+        assert (np.abs(cn - co) <= 1e-3 + 1e-4 * np.abs(cn)).all()
+        assert abs(cn.astype(np.float64).sum() - sums[i, 0]) <= 1e-9 * max(1.0, sums[i, 2])
+        assert abs(co.astype(np.float64).sum() - sums[i, 1]) <= 1e-5 * max(1.0, sums[i, 2])
+
+
+def test_route_predicate(oracle):
+    # src/compute/backends/cpu_opt.c:3509 with MR = 6
+    assert oracle.small_route(1, 4096, 784)              # 3.2 M, m < 6
+    assert not oracle.small_route(1, 4096, 4096)         # 16.8 M
+    assert oracle.small_route(1, 10, 4096)
+    assert oracle.small_route(46, 46, 47) and not oracle.small_route(47, 47, 47)
+    assert not oracle.small_route(6, 100, 1000) and oracle.small_route(5, 100, 1000)
+
+
+def test_bias_relu_and_gelu(oracle, golden):
+    oracle.seed(77)
+    a, b = oracle.uniform((33, 100), -1, 1), oracle.uniform((100, 40), -1, 1)
+    bias = oracle.uniform((40,), -0.5, 0.5)
+    assert np.array_equal(oracle.dense(a, b, bias, 1), golden["gemm_relu_33x100x40"])
+    assert np.array_equal(oracle.dense(a, b, None, 1), golden["gemm_relu_33x100x40_nobias"])
+    lin = oracle.dense(a, b, bias, 0)
+    assert np.array_equal(lin, oracle.gemm_opt(a, b) + bias[None, :])
+    x = golden["gelu_x"]
+    y = oracle.gelu(x)
+    assert np.abs(y - golden["gelu_y"]).max() <= 2e-6
+    y64 = np.array([oracle.L.axo_gelu_f64(float(v)) for v in x])
+    assert np.abs(y - y64).max() <= 1e-6
+    assert oracle.L.axo_gelu_tanh(0.0) == 0.0 and abs(oracle.L.axo_gelu_tanh(10.0) - 10.0) < 1e-6
+
+
+# ---------------------------------------------------------------- live cross-check
+def test_oracle_equals_compiled_reference(oracle, reflib):
+    oracle.seed(11)
+    for (M, K, N) in [(5, 333, 77), (130, 700, 260), (1, 4096, 512), (256, 512, 384)]:
+        a, b = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1)
+        ref = reflib.gemm(a, b)
+        assert np.abs(oracle.gemm_opt(a, b) - ref).max() <= 1e-4 * np.abs(ref).max()
+        assert np.array_equal(oracle.gemm_naive(a, b), reflib.gemm(a, b, backend=0)) or M * N * K > 2e7
+    w = oracle.normal((96, 333), 0, 0.02)
+    q, s = oracle.quantize_rows(w)
+    q2, s2 = reflib.quantize_rows(w)
+    assert np.array_equal(q, q2) and np.array_equal(s, s2)
+    a = oracle.normal((9, 333))
+    assert np.array_equal(oracle.qgemm_w8a32(a, q, s), reflib.qgemm_w8a32(a, q, s))
+    x, wq = oracle.int8((3, 4096)), oracle.int8((32, 4096))
+    via_ref = reflib.qgemm_w8a32(x.astype(np.float32), wq, np.ones(32, np.float32))
+    assert np.array_equal(oracle.qgemm_w8a8_acc(x, wq).astype(np.float64), via_ref.astype(np.float64))
