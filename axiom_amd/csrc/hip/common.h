@@ -1,0 +1,64 @@
+// Internal helpers shared by the kernel translation units of libaxhip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "axhip.h"
+
+namespace axhip {
+
+// Records a failure message for axhip_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// 0 when the runtime is initialised on a usable GPU, else an AXHIP_ERR_* code (message set).
+int ensure_ready();
+// Remembers which kernel variant a GEMM-type entry point chose.
+void note_kernel(const char *name);
+// Checks the launch that was just issued on the null stream.
+int check_launch(const char *what);
+// A device workspace of at least `bytes`, owned by the runtime (grown on demand), or NULL.
+void *workspace(size_t bytes);
+
+constexpr hipStream_t kStream = nullptr;
+
+typedef int   v4i  __attribute__((ext_vector_type(4)));
+typedef int   v16i __attribute__((ext_vector_type(16)));
+typedef float v4f  __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float gelu_tanh(float x) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    float inner = k0 * (x + k1 * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+__device__ __forceinline__ float apply_act(float v, int act) {
+    if (act == AXHIP_ACT_RELU) return v > 0.0f ? v : 0.0f;
+    if (act == AXHIP_ACT_GELU) return gelu_tanh(v);
+    return v;
+}
+
+// Workgroup id -> output tile.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs,
+// each with its own L2; renumbering so that every XCD walks one contiguous run of tiles, in
+// bands of 4 tile-rows, keeps the operand panels an XCD re-reads inside that XCD's L2.
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int &tm, int &tn) {
+    const int total = tiles_m * tiles_n;
+    int id = bid;
+    if ((total & 7) == 0) id = (bid & 7) * (total >> 3) + (bid >> 3);
+    constexpr int BAND = 4;
+    const int per_band = BAND * tiles_n;
+    const int band = id / per_band;
+    const int first = band * BAND;
+    const int rows = (tiles_m - first) < BAND ? (tiles_m - first) : BAND;
+    const int in_band = id - band * per_band;
+    tm = first + in_band % rows;
+    tn = in_band / rows;
+}
+
+}  // namespace axhip
+
+#define AXHIP_HIP_TRY(expr, what)                                                         \
+    do {                                                                                  \
+        hipError_t e_ = (expr);                                                           \
+        if (e_ != hipSuccess)                                                             \
+            return axhip::fail(AXHIP_ERR_BACKEND, "%s: %s", what, hipGetErrorString(e_)); \
+    } while (0)

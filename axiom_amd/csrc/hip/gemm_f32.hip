@@ -1,0 +1,320 @@
+// fp32 GEMM on the fp32 matrix cores (v_mfma_f32_32x32x2_f32), NN / NT / TN, optionally
+// strided-batched, with alpha/beta, per-column scale, bias and activation fused into the
+// write-back.  True fp32 multiply-accumulate throughout.
+//
+// One workgroup owns a BM x BN tile of C and walks K in slabs of 32.  An operand whose
+// K index is contiguous in memory (A of NN/NT, B of NT) is staged as rows of 32 floats padded
+// to 36, and read back with one ds_read_b128 per 8-wide k-block: lane l takes row (l & 31),
+// floats [4*(l>>5), +4) of the block.  An operand whose M/N index is contiguous (B of NN, A of
+// TN) is staged k-major with the row length padded by 8 floats and read with four
+// ds_read_b32: lane l takes column (l & 31) of k = 4*(l>>5) + j.  Either way MFMA j of a k-block
+// multiplies the k = 4*(l>>5) + j elements of both operands, so A and B always pair up.
+// The pads make the 16 lanes a b128 read serves together, the two lane halves of a b32 read,
+// and the staging writes all fall on distinct banks (64 banks x 4 bytes).
+#include "common.h"
+
+namespace {
+using namespace axhip;
+
+constexpr int BK = 32;
+constexpr int KC_STRIDE = BK + 4;          // floats per staged row of a K-contiguous operand
+
+struct SgemmArgs {
+    const void *A, *B;
+    float *C;
+    int64_t M, N, K, lda, ldb, ldc;
+    int64_t stride_a, stride_b, stride_c;  // elements between batch members
+    float alpha, beta;
+    const float *col_scale;                // multiplies column n after alpha (W8A32), or NULL
+    const float *bias;
+    int act;
+};
+
+// One operand's slab: R rows (M or N extent of the tile) x BK.
+template <int R, bool KCONTIG, int T, bool GUARD, typename SRC>
+struct Operand {
+    static constexpr int STRIDE = KCONTIG ? KC_STRIDE : (R + 8);
+    static constexpr int FLOATS = KCONTIG ? R * KC_STRIDE : BK * (R + 8);
+    static constexpr int CHUNKS = R * BK / 4 / T;          // float4 chunks per thread
+    static_assert(CHUNKS * T * 4 == R * BK, "slab must divide over the workgroup");
+
+    v4f reg[CHUNKS];
+
+    // element (r, k) of the logical [R, K] operand lives at src[r*ld + k] (KCONTIG) or
+    // src[k*ld + r]
+    __device__ __forceinline__ void fetch(const SRC *src, int64_t ld, int64_t r0, int64_t rows,
+                                          int64_t k0, int64_t K, int tid, bool vec_ok) {
+#pragma unroll
+        for (int i = 0; i < CHUNKS; i++) {
+            const int c = tid + i * T;
+            int64_t r, k;
+            if (KCONTIG) { r = r0 + (c >> 3); k = k0 + ((c & 7) << 2); }
+            else         { k = k0 + c / (R / 4); r = r0 + ((c % (R / 4)) << 2); }
+            const SRC *p = KCONTIG ? src + r * ld + k : src + k * ld + r;
+            v4f v = {0.f, 0.f, 0.f, 0.f};
+            if (sizeof(SRC) == 1) {                        // int8 source, K-contiguous only
+                const bool whole = !GUARD || (r < rows && k + 4 <= K && vec_ok);
+                if (whole) {
+                    int w = *reinterpret_cast<const int *>(p);
+                    v.x = (float)(signed char)(w & 0xff);
+                    v.y = (float)(signed char)((w >> 8) & 0xff);
+                    v.z = (float)(signed char)((w >> 16) & 0xff);
+                    v.w = (float)(signed char)((w >> 24) & 0xff);
+                } else if (r < rows) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (k + e < K) v[e] = (float)p[e];
+                }
+            } else if (!GUARD) {
+                v = *reinterpret_cast<const v4f *>(p);
+            } else if (KCONTIG) {
+                if (r < rows) {
+                    if (vec_ok && k + 4 <= K) v = *reinterpret_cast<const v4f *>(p);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (k + e < K) v[e] = (float)p[e];
+                    }
+                }
+            } else {
+                if (k < K) {
+                    if (vec_ok && r + 4 <= rows) v = *reinterpret_cast<const v4f *>(p);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (r + e < rows) v[e] = (float)p[e];
+                    }
+                }
+            }
+            reg[i] = v;
+        }
+    }
+
+    __device__ __forceinline__ void stash(float *s, int tid) const {
+#pragma unroll
+        for (int i = 0; i < CHUNKS; i++) {
+            const int c = tid + i * T;
+            if (KCONTIG) *reinterpret_cast<v4f *>(s + (c >> 3) * KC_STRIDE + ((c & 7) << 2)) = reg[i];
+            else *reinterpret_cast<v4f *>(s + (c / (R / 4)) * STRIDE + ((c % (R / 4)) << 2)) = reg[i];
+        }
+    }
+
+    // the 4 values lane (row r, half h) feeds to MFMAs j = 0..3 of k-block kb
+    __device__ __forceinline__ static v4f frag(const float *s, int r, int h, int kb) {
+        if (KCONTIG) return *reinterpret_cast<const v4f *>(s + r * KC_STRIDE + kb + 4 * h);
+        v4f v;
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = s[(kb + 4 * h + j) * STRIDE + r];
+        return v;
+    }
+};
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool GUARD, typename BSRC>
+__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm(SgemmArgs g) {
+    constexpr int T = WAVES_M * WAVES_N * 64;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(TM * 32 * WAVES_M == BM && TN * 32 * WAVES_N == BN, "wave tiling");
+    using OpA = Operand<BM, A_KC, T, GUARD, float>;
+    using OpB = Operand<BN, B_KC, T, GUARD, BSRC>;
+    constexpr int STAGE = OpA::FLOATS + OpB::FLOATS;
+
+    extern __shared__ __attribute__((aligned(16))) float lds_f[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int tiles_m = (int)((g.M + BM - 1) / BM), tiles_n = (int)((g.N + BN - 1) / BN);
+    int tm, tn;
+    tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t batch = blockIdx.y;
+    const float *A = static_cast<const float *>(g.A) + batch * g.stride_a;
+    const BSRC *B = static_cast<const BSRC *>(g.B) + batch * g.stride_b;
+    float *C = g.C + batch * g.stride_c;
+
+    bool vec_a = true, vec_b = true;
+    if (GUARD) {
+        vec_a = ((((uintptr_t)A >> 2) | (uintptr_t)g.lda | (uintptr_t)g.stride_a) & 3) == 0 &&
+                ((uintptr_t)A & 3) == 0;
+        vec_b = sizeof(BSRC) == 1
+                    ? ((((uintptr_t)B) | (uintptr_t)g.ldb) & 3) == 0
+                    : ((((uintptr_t)B >> 2) | (uintptr_t)g.ldb | (uintptr_t)g.stride_b) & 3) == 0;
+    }
+
+    OpA opa;
+    OpB opb;
+    const int64_t slabs = (g.K + BK - 1) / BK;
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    opa.fetch(A, g.lda, m0, g.M, 0, g.K, tid, vec_a);
+    opb.fetch(B, g.ldb, n0, g.N, 0, g.K, tid, vec_b);
+    opa.stash(lds_f, tid);
+    opb.stash(lds_f + OpA::FLOATS, tid);
+    __syncthreads();
+
+    const int frow = lane & 31, fhalf = lane >> 5;
+    for (int64_t s = 0; s < slabs; s++) {
+        const int cur = (int)(s & 1);
+        if (s + 1 < slabs) {
+            opa.fetch(A, g.lda, m0, g.M, (s + 1) * BK, g.K, tid, vec_a);
+            opb.fetch(B, g.ldb, n0, g.N, (s + 1) * BK, g.K, tid, vec_b);
+        }
+        const float *sa = lds_f + cur * STAGE;
+        const float *sb = sa + OpA::FLOATS;
+#pragma unroll
+        for (int kb = 0; kb < BK; kb += 8) {
+            v4f fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) fa[i] = OpA::frag(sa, wm * WTM + i * 32 + frow, fhalf, kb);
+#pragma unroll
+            for (int j = 0; j < TN; j++) fb[j] = OpB::frag(sb, wn * WTN + j * 32 + frow, fhalf, kb);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][e], fb[j][e],
+                                                                         acc[i][j], 0, 0, 0);
+        }
+        if (s + 1 < slabs) {
+            float *na = lds_f + (cur ^ 1) * STAGE;
+            opa.stash(na, tid);
+            opb.stash(na + OpA::FLOATS, tid);
+        }
+        __syncthreads();
+    }
+
+    // accumulator register v of lane l: row (v&3) + 8*(v>>2) + 4*(l>>5), column (l & 31)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int64_t col = n0 + wn * WTN + j * 32 + frow;
+        const bool col_ok = !GUARD || col < g.N;
+        float cs = 1.0f, bv = 0.0f;
+        if (col_ok) {
+            if (g.col_scale) cs = g.col_scale[col];
+            if (g.bias) bv = g.bias[col];
+        }
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int64_t row = m0 + wm * WTM + i * 32 + (v & 3) + 8 * (v >> 2) + 4 * fhalf;
+                if (GUARD && (row >= g.M || !col_ok)) continue;
+                float r = acc[i][j][v];
+                if (g.alpha != 1.0f) r *= g.alpha;
+                if (g.col_scale) r *= cs;
+                float *cp = C + row * g.ldc + col;
+                if (g.beta != 0.0f) r += g.beta * *cp;
+                if (g.bias) r += bv;
+                *cp = apply_act(r, g.act);
+            }
+        }
+    }
+}
+
+template <int BM, int BN, bool A_KC, bool B_KC, bool GUARD, typename BSRC>
+int launch(const char *name, const SgemmArgs &g, int64_t batch) {
+    auto kern = k_sgemm<BM, BN, 2, 2, A_KC, B_KC, GUARD, BSRC>;
+    using OpA = Operand<BM, A_KC, 256, GUARD, float>;
+    using OpB = Operand<BN, B_KC, 256, GUARD, BSRC>;
+    constexpr int smem = 2 * (OpA::FLOATS + OpB::FLOATS) * (int)sizeof(float);
+    static bool attr_set = false;
+    if (!attr_set) {
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem),
+                      "hipFuncSetAttribute");
+        attr_set = true;
+    }
+    const int64_t tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+    if (tiles > 0x7fffffff || batch > 65535)
+        return fail(AXHIP_ERR_SHAPE, "sgemm: grid too large (tiles=%lld batch=%lld)",
+                    (long long)tiles, (long long)batch);
+    note_kernel(name);
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)batch), dim3(256), smem, kStream, g);
+    return check_launch(name);
+}
+
+template <bool A_KC, bool B_KC, typename BSRC>
+int pick_tile(const char *const names[3], const SgemmArgs &g, int64_t batch) {
+    const int esz_b = (int)sizeof(BSRC);
+    bool aligned = (g.K % BK == 0) && g.K > 0 && ((uintptr_t)g.A % 16 == 0) &&
+                   ((uintptr_t)g.B % (esz_b == 1 ? 4 : 16) == 0) && (g.lda % 4 == 0) &&
+                   (g.ldb % 4 == 0) && (g.stride_a % 4 == 0) && (g.stride_b % 4 == 0);
+    if (aligned && g.M % 128 == 0 && g.N % 128 == 0 && (g.M / 128) * (g.N / 128) * batch >= 192)
+        return launch<128, 128, A_KC, B_KC, false, BSRC>(names[0], g, batch);
+    if (aligned && g.M % 64 == 0 && g.N % 64 == 0)
+        return launch<64, 64, A_KC, B_KC, false, BSRC>(names[1], g, batch);
+    return launch<64, 64, A_KC, B_KC, true, BSRC>(names[2], g, batch);
+}
+
+int validate(const char *who, int transa, int transb, int64_t M, int64_t N, int64_t K,
+             const void *A, int64_t lda, const void *B, int64_t ldb, const void *C, int64_t ldc,
+             int act) {
+    if (!A || !B || !C) return fail(AXHIP_ERR_NULL_ARG, "%s: NULL matrix", who);
+    if (M < 0 || N < 0 || K < 0) return fail(AXHIP_ERR_SHAPE, "%s: negative dimension", who);
+    if ((transa & ~1) || (transb & ~1)) return fail(AXHIP_ERR_SHAPE, "%s: trans flag must be 0/1", who);
+    if (lda < (transa ? M : K) || ldb < (transb ? K : N) || ldc < N)
+        return fail(AXHIP_ERR_SHAPE, "%s: leading dimension smaller than the row length", who);
+    if (act < AXHIP_ACT_NONE || act > AXHIP_ACT_GELU)
+        return fail(AXHIP_ERR_SHAPE, "%s: unknown activation %d", who, act);
+    return AXHIP_OK;
+}
+
+int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
+    static const char *const nn[3] = {"sgemm_nn_128x128", "sgemm_nn_64x64", "sgemm_nn_64x64_guarded"};
+    static const char *const nt[3] = {"sgemm_nt_128x128", "sgemm_nt_64x64", "sgemm_nt_64x64_guarded"};
+    static const char *const tn[3] = {"sgemm_tn_128x128", "sgemm_tn_64x64", "sgemm_tn_64x64_guarded"};
+    if (!transa && !transb) return pick_tile<true, false, float>(nn, g, batch);
+    if (!transa && transb) return pick_tile<true, true, float>(nt, g, batch);
+    if (transa && !transb) return pick_tile<false, false, float>(tn, g, batch);
+    return fail(AXHIP_ERR_NOT_IMPLEMENTED, "sgemm: A^T * B^T is not provided");
+}
+
+}  // namespace
+
+namespace axhip {
+// W8A32 through the matrix cores: B is int8 [N,K], converted to fp32 while it is staged.
+int sgemm_i8w(int64_t M, int64_t N, int64_t K, const float *a, const int8_t *w,
+              const float *w_scales, float *out) {
+    static const char *const names[3] = {"qgemm_w8a32_mfma_128x128", "qgemm_w8a32_mfma_64x64",
+                                         "qgemm_w8a32_mfma_64x64_guarded"};
+    SgemmArgs g{a, w, out, M, N, K, K, K, N, 0, 0, 0, 1.0f, 0.0f, w_scales, nullptr, AXHIP_ACT_NONE};
+    return pick_tile<true, true, int8_t>(names, g, 1);
+}
+}  // namespace axhip
+
+extern "C" int axhip_sgemm(int transa, int transb, int64_t M, int64_t N, int64_t K, float alpha,
+                           const float *A, int64_t lda, const float *B, int64_t ldb, float beta,
+                           float *C, int64_t ldc, const float *bias, int act) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (int rc = validate("sgemm", transa, transb, M, N, K, A, lda, B, ldb, C, ldc, act)) return rc;
+    if (M == 0 || N == 0) return AXHIP_OK;
+    if (M <= 8 && !transa && !transb && alpha == 1.0f && beta == 0.0f)
+        return axhip_sgemm_skinny(M, N, K, A, lda, B, ldb, C, ldc, bias, act);
+    SgemmArgs g{A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, alpha, beta, nullptr, bias, act};
+    return dispatch_f32(g, transa, transb, 1);
+}
+
+extern "C" int axhip_sgemm_strided_batched(int transa, int transb, int64_t M, int64_t N, int64_t K,
+                                           float alpha, const float *A, int64_t lda,
+                                           int64_t stride_a, const float *B, int64_t ldb,
+                                           int64_t stride_b, float beta, float *C, int64_t ldc,
+                                           int64_t stride_c, int64_t batch) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (int rc = validate("sgemm_strided_batched", transa, transb, M, N, K, A, lda, B, ldb, C, ldc,
+                          AXHIP_ACT_NONE))
+        return rc;
+    if (batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0)
+        return fail(AXHIP_ERR_SHAPE, "sgemm_strided_batched: negative batch or stride");
+    if (M == 0 || N == 0 || batch == 0) return AXHIP_OK;
+    SgemmArgs g{A, B, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c,
+                alpha, beta, nullptr, nullptr, AXHIP_ACT_NONE};
+    return dispatch_f32(g, transa, transb, batch);
+}

@@ -1,0 +1,219 @@
+// Skinny-M (1 <= M <= 8) fp32 route: C[M,N] = act(A[M,K] * B[K,N] + bias[n]).
+//
+// The work is one pass over B (K*N*4 bytes): HBM-bound.  A workgroup of 256 threads owns 64
+// columns (16 lanes x float4 = 256 contiguous bytes per B row) and a K range; its 16 lane
+// groups take rows k, k+16, ... of that range, so one wave-wide load instruction covers four
+// 256-byte row segments and eight of them are kept in flight per lane.  The M activations of
+// a k row are wave-uniform only per lane group, so they come from LDS (staged once per
+// workgroup).  Lane groups are summed through LDS in a fixed order; when K is split over
+// several workgroups the partial tiles go to a workspace and a second kernel adds them in
+// split order and applies bias and activation — no atomics, so results are bit-identical
+// run to run.
+#include "common.h"
+
+namespace {
+using namespace axhip;
+
+constexpr int COLS = 64;        // columns per workgroup
+constexpr int KGROUPS = 16;     // lane groups per workgroup, each 16 lanes x float4
+constexpr int UNROLL = 8;
+
+template <int MR, bool VEC>
+__global__ void __launch_bounds__(256)
+k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, int64_t ldb,
+         float *__restrict__ dst, int64_t dst_ld, int64_t dst_split_stride, int64_t N, int64_t K,
+         int64_t k_per_split, const float *__restrict__ bias, int act, int finish) {
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    // sm: [MR][k_per_split] activations, then [KGROUPS][MR][COLS] partial sums
+    const int tid = threadIdx.x;
+    const int cg = tid & 15;            // column group: columns 4*cg .. 4*cg+3 of the 64
+    const int kg = tid >> 4;            // lane group
+    const int64_t n0 = (int64_t)blockIdx.x * COLS;
+    const int64_t k_begin = (int64_t)blockIdx.y * k_per_split;
+    int64_t k_end = k_begin + k_per_split;
+    if (k_end > K) k_end = K;
+    const int64_t klen = k_end - k_begin;
+
+    float *xs = sm;
+    for (int64_t i = tid; i < (int64_t)MR * klen; i += 256) {
+        int64_t m = i / klen, k = i - m * klen;
+        xs[m * k_per_split + k] = A[m * lda + k_begin + k];
+    }
+    __syncthreads();
+
+    float acc[MR][4];
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[m][e] = 0.0f;
+
+    const int64_t col = n0 + 4 * cg;
+    const float *bp = B + col;
+    int64_t k = kg;
+    if (VEC) {
+        if (col < N) {      // N % 4 == 0: a float4 is entirely inside or outside
+            for (; k + (UNROLL - 1) * KGROUPS < klen; k += UNROLL * KGROUPS) {
+                v4f w[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++)
+                    w[u] = *reinterpret_cast<const v4f *>(bp + (k_begin + k + u * KGROUPS) * ldb);
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                    for (int m = 0; m < MR; m++) {
+                        const float xv = xs[m * k_per_split + k + u * KGROUPS];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[m][e] = __builtin_fmaf(xv, w[u][e], acc[m][e]);
+                    }
+            }
+            for (; k < klen; k += KGROUPS) {
+                v4f w = *reinterpret_cast<const v4f *>(bp + (k_begin + k) * ldb);
+#pragma unroll
+                for (int m = 0; m < MR; m++) {
+                    const float xv = xs[m * k_per_split + k];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[m][e] = __builtin_fmaf(xv, w[e], acc[m][e]);
+                }
+            }
+        }
+    } else {
+        for (; k < klen; k += KGROUPS) {
+            float w[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) w[e] = (col + e < N) ? bp[(k_begin + k) * ldb + e] : 0.0f;
+#pragma unroll
+            for (int m = 0; m < MR; m++) {
+                const float xv = xs[m * k_per_split + k];
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[m][e] = __builtin_fmaf(xv, w[e], acc[m][e]);
+            }
+        }
+    }
+
+    float *red = sm + (int64_t)MR * k_per_split;
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+        *reinterpret_cast<v4f *>(red + (kg * MR + m) * COLS + 4 * cg) =
+            v4f{acc[m][0], acc[m][1], acc[m][2], acc[m][3]};
+    __syncthreads();
+
+    for (int i = tid; i < MR * COLS; i += 256) {
+        const int m = i / COLS, c = i % COLS;
+        float s = 0.0f;
+#pragma unroll
+        for (int g2 = 0; g2 < KGROUPS; g2++) s += red[(g2 * MR + m) * COLS + c];
+        const int64_t n = n0 + c;
+        if (n < N) {
+            if (finish) {
+                if (bias) s += bias[n];
+                s = apply_act(s, act);
+            }
+            dst[blockIdx.y * dst_split_stride + m * dst_ld + n] = s;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+k_skinny_finish(const float *__restrict__ part, int64_t split_stride, int splits, int64_t M,
+                int64_t N, float *__restrict__ C, int64_t ldc, const float *__restrict__ bias,
+                int act) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= M * N) return;
+    const int64_t m = i / N, n = i - m * N;
+    float s = 0.0f;
+    for (int p = 0; p < splits; p++) s += part[p * split_stride + i];
+    if (bias) s += bias[n];
+    C[m * ldc + n] = apply_act(s, act);
+}
+
+template <int MR>
+int launch_m(bool vec, dim3 grid, size_t smem, const float *A, int64_t lda, const float *B,
+             int64_t ldb, float *dst, int64_t dst_ld, int64_t dst_split, int64_t N, int64_t K,
+             int64_t kps, const float *bias, int act, int finish) {
+    if (vec)
+        hipLaunchKernelGGL((k_skinny<MR, true>), grid, dim3(256), smem, kStream, A, lda, B, ldb, dst,
+                           dst_ld, dst_split, N, K, kps, bias, act, finish);
+    else
+        hipLaunchKernelGGL((k_skinny<MR, false>), grid, dim3(256), smem, kStream, A, lda, B, ldb,
+                           dst, dst_ld, dst_split, N, K, kps, bias, act, finish);
+    return check_launch("sgemm_skinny");
+}
+
+}  // namespace
+
+extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                                  const float *B, int64_t ldb, float *C, int64_t ldc,
+                                  const float *bias, int act) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!A || !B || !C) return fail(AXHIP_ERR_NULL_ARG, "sgemm_skinny: NULL matrix");
+    if (M < 1 || M > 8) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: M=%lld outside 1..8", (long long)M);
+    if (N < 0 || K < 0 || lda < K || ldb < N || ldc < N)
+        return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: bad dimension or leading dimension");
+    if (act < AXHIP_ACT_NONE || act > AXHIP_ACT_GELU)
+        return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: unknown activation %d", act);
+    if (N == 0) return AXHIP_OK;
+
+    const int64_t col_blocks = (N + COLS - 1) / COLS;
+    // enough workgroups to cover 256 CUs a few times over, each with at least 128 k rows
+    int64_t splits = (1024 + col_blocks - 1) / col_blocks;
+    const int64_t max_splits = K >= 128 ? K / 128 : 1;
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    int64_t kps = (K + splits - 1) / splits;
+    kps = (kps + KGROUPS - 1) / KGROUPS * KGROUPS;
+    // the activations of one split must fit LDS next to the reduction buffer
+    const int64_t red_floats = (int64_t)KGROUPS * M * COLS;
+    const int64_t max_kps = ((int64_t)(96 * 1024 / 4) - red_floats) / M / KGROUPS * KGROUPS;
+    if (kps > max_kps) kps = max_kps;
+    if (kps < KGROUPS) kps = KGROUPS;
+    splits = K > 0 ? (K + kps - 1) / kps : 1;
+    if (splits > 65535) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: K=%lld too large", (long long)K);
+
+    const bool vec = (N % 4 == 0) && (ldb % 4 == 0) && ((uintptr_t)B % 16 == 0);
+    const size_t smem = (size_t)(M * kps + red_floats) * sizeof(float);
+    float *dst = C;
+    int64_t dst_ld = ldc, dst_split = 0;
+    int finish = 1;
+    if (splits > 1) {
+        dst = static_cast<float *>(axhip::workspace((size_t)splits * M * N * sizeof(float)));
+        if (!dst) return AXHIP_ERR_ALLOC;
+        dst_ld = N;
+        dst_split = M * N;
+        finish = 0;
+    }
+    static bool attr_set = false;
+    if (!attr_set) {
+        const void *ks[] = {
+            (const void *)k_skinny<1, true>, (const void *)k_skinny<2, true>, (const void *)k_skinny<3, true>,
+            (const void *)k_skinny<4, true>, (const void *)k_skinny<5, true>, (const void *)k_skinny<6, true>,
+            (const void *)k_skinny<7, true>, (const void *)k_skinny<8, true>,
+            (const void *)k_skinny<1, false>, (const void *)k_skinny<2, false>, (const void *)k_skinny<3, false>,
+            (const void *)k_skinny<4, false>, (const void *)k_skinny<5, false>, (const void *)k_skinny<6, false>,
+            (const void *)k_skinny<7, false>, (const void *)k_skinny<8, false>};
+        for (const void *k : ks)
+            AXHIP_HIP_TRY(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024),
+                          "hipFuncSetAttribute");
+        attr_set = true;
+    }
+    dim3 grid((unsigned)col_blocks, (unsigned)splits);
+    note_kernel(vec ? "sgemm_skinny_vec4" : "sgemm_skinny_scalar");
+    int rc;
+    switch (M) {
+#define AX_CASE(m)                                                                            \
+    case m:                                                                                   \
+        rc = launch_m<m>(vec, grid, smem, A, lda, B, ldb, dst, dst_ld, dst_split, N, K, kps,  \
+                         bias, act, finish);                                                  \
+        break;
+        AX_CASE(1) AX_CASE(2) AX_CASE(3) AX_CASE(4) AX_CASE(5) AX_CASE(6) AX_CASE(7) AX_CASE(8)
+#undef AX_CASE
+        default: rc = AXHIP_ERR_SHAPE;
+    }
+    if (rc) return rc;
+    if (splits > 1) {
+        const int64_t total = M * N;
+        hipLaunchKernelGGL(k_skinny_finish, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                           kStream, dst, dst_split, (int)splits, M, N, C, ldc, bias, act);
+        return check_launch("sgemm_skinny_finish");
+    }
+    return AXHIP_OK;
+}

@@ -1,0 +1,181 @@
+// Lifecycle, memory and timing entry points of libaxhip.so.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "common.h"
+
+namespace {
+thread_local char t_err[512] = "";
+thread_local const char *t_kernel = "";
+int g_ready = 0;            // 1 once a gfx950-class device was initialised
+int g_devices = -1;
+char g_name[128] = "";
+void *g_ws = nullptr;
+size_t g_ws_bytes = 0;
+}  // namespace
+
+namespace axhip {
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_err, sizeof t_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+void note_kernel(const char *name) { t_kernel = name; }
+
+int ensure_ready() {
+    if (g_ready) return AXHIP_OK;
+    return axhip_init();
+}
+
+int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(AXHIP_ERR_BACKEND, "%s launch: %s", what, hipGetErrorString(e));
+    return AXHIP_OK;
+}
+
+void *workspace(size_t bytes) {
+    if (bytes <= g_ws_bytes) return g_ws;
+    if (g_ws) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(g_ws);
+        g_ws = nullptr;
+        g_ws_bytes = 0;
+    }
+    size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes;
+    if (hipMalloc(&g_ws, want) != hipSuccess) {
+        g_ws = nullptr;
+        fail(AXHIP_ERR_ALLOC, "workspace of %zu bytes: out of device memory", want);
+        return nullptr;
+    }
+    g_ws_bytes = want;
+    return g_ws;
+}
+
+}  // namespace axhip
+
+using axhip::fail;
+
+extern "C" {
+
+int axhip_device_count(void) {
+    if (g_devices >= 0) return g_devices;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) n = 0;
+    g_devices = n;
+    return n;
+}
+
+int axhip_init(void) {
+    if (g_ready) return AXHIP_OK;
+    if (axhip_device_count() <= 0)
+        return fail(AXHIP_ERR_BACKEND, "no HIP device visible: libaxhip has no CPU fallback");
+    AXHIP_HIP_TRY(hipSetDevice(0), "hipSetDevice");
+    hipDeviceProp_t prop;
+    AXHIP_HIP_TRY(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties");
+    snprintf(g_name, sizeof g_name, "%s", prop.gcnArchName);
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(AXHIP_ERR_BACKEND, "device 0 is %s; this library holds gfx950 code only",
+                    prop.gcnArchName);
+    g_ready = 1;
+    return AXHIP_OK;
+}
+
+void axhip_shutdown(void) {
+    if (!g_ready) return;
+    (void)hipDeviceSynchronize();
+    if (g_ws) (void)hipFree(g_ws);
+    g_ws = nullptr;
+    g_ws_bytes = 0;
+    g_ready = 0;
+}
+
+int axhip_synchronize(void) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    AXHIP_HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    return AXHIP_OK;
+}
+
+const char *axhip_last_error(void) { return t_err; }
+const char *axhip_device_name(void) { return g_name; }
+const char *axhip_last_kernel(void) { return t_kernel; }
+
+void *axhip_malloc(size_t bytes) {
+    if (axhip::ensure_ready()) return nullptr;
+    void *p = nullptr;
+    if (bytes == 0) bytes = 4;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        fail(AXHIP_ERR_ALLOC, "hipMalloc(%zu) failed", bytes);
+        return nullptr;
+    }
+    if (hipMemsetAsync(p, 0, bytes, axhip::kStream) != hipSuccess) {
+        (void)hipFree(p);
+        fail(AXHIP_ERR_BACKEND, "zero-fill of %zu bytes failed", bytes);
+        return nullptr;
+    }
+    return p;
+}
+
+void axhip_free(void *p) {
+    if (p) (void)hipFree(p);
+}
+
+int axhip_memset(void *p, int v, size_t bytes) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!p) return fail(AXHIP_ERR_NULL_ARG, "memset: NULL");
+    AXHIP_HIP_TRY(hipMemsetAsync(p, v, bytes, axhip::kStream), "hipMemsetAsync");
+    return AXHIP_OK;
+}
+
+int axhip_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!dst || !src) return fail(AXHIP_ERR_NULL_ARG, "memcpy_h2d: NULL");
+    AXHIP_HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice), "hipMemcpy h2d");
+    return AXHIP_OK;
+}
+
+int axhip_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!dst || !src) return fail(AXHIP_ERR_NULL_ARG, "memcpy_d2h: NULL");
+    AXHIP_HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost), "hipMemcpy d2h");
+    return AXHIP_OK;
+}
+
+int axhip_memcpy_d2d(void *dst, const void *src, size_t bytes) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!dst || !src) return fail(AXHIP_ERR_NULL_ARG, "memcpy_d2d: NULL");
+    AXHIP_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, axhip::kStream),
+                  "hipMemcpy d2d");
+    return AXHIP_OK;
+}
+
+void *axhip_event_create(void) {
+    if (axhip::ensure_ready()) return nullptr;
+    hipEvent_t ev;
+    if (hipEventCreate(&ev) != hipSuccess) return nullptr;
+    return (void *)ev;
+}
+
+void axhip_event_destroy(void *ev) {
+    if (ev) (void)hipEventDestroy((hipEvent_t)ev);
+}
+
+int axhip_event_record(void *ev) {
+    if (!ev) return fail(AXHIP_ERR_NULL_ARG, "event_record: NULL");
+    AXHIP_HIP_TRY(hipEventRecord((hipEvent_t)ev, axhip::kStream), "hipEventRecord");
+    return AXHIP_OK;
+}
+
+int axhip_event_elapsed_ms(void *start, void *stop, float *ms) {
+    if (!start || !stop || !ms) return fail(AXHIP_ERR_NULL_ARG, "event_elapsed: NULL");
+    AXHIP_HIP_TRY(hipEventSynchronize((hipEvent_t)stop), "hipEventSynchronize");
+    AXHIP_HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop),
+                  "hipEventElapsedTime");
+    return AXHIP_OK;
+}
+
+}  // extern "C"

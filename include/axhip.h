@@ -1,0 +1,133 @@
+/* axhip.h — C ABI of libaxhip.so, the MI355X (gfx950) GEMM kernels for Axiom.
+ *
+ * Plain pointers and sizes only.  Every pointer named "device" is HIP device memory
+ * obtained from axhip_malloc (or any hipMalloc in the same process).  All matrices are
+ * row-major.  Work is queued on the HIP null stream and is asynchronous with respect to
+ * the host unless stated; axhip_memcpy_d2h and axhip_synchronize wait for it.
+ *
+ * Return value: 0 (AXHIP_OK) on success, otherwise one of the AXHIP_ERR_* codes, whose
+ * numeric values equal Axiom's ax_status_t (include/axiom/types.h:89-103) so the host
+ * adapter can return them unchanged.  axhip_last_error() holds a description.
+ * There is no CPU fallback anywhere in this library: without a usable GPU every compute
+ * entry point fails with AXHIP_ERR_BACKEND.
+ *
+ * Each entry point cites the reference interface it stands in for (paths relative to the
+ * Axiom tree).
+ */
+#ifndef AXHIP_H
+#define AXHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    AXHIP_OK = 0,
+    AXHIP_ERR_NULL_ARG = 1,
+    AXHIP_ERR_ALLOC = 2,
+    AXHIP_ERR_SHAPE = 3,          /* AX_ERR_SHAPE_MISMATCH */
+    AXHIP_ERR_INVALID_AXIS = 5,
+    AXHIP_ERR_BACKEND = 9,
+    AXHIP_ERR_NOT_IMPLEMENTED = 10
+};
+
+/* fused epilogue activation */
+enum { AXHIP_ACT_NONE = 0, AXHIP_ACT_RELU = 1, AXHIP_ACT_GELU = 2 };
+
+/* ---- lifecycle: the device-owner hooks of struct ax_backend_ops
+ *      (include/axiom/internal/backend_ops.h:267-296; CUDA versions in
+ *      src/compute/backends/cuda/backend.cu:56-116) ------------------------------ */
+int         axhip_init(void);                 /* .init          */
+void        axhip_shutdown(void);             /* .shutdown      */
+int         axhip_synchronize(void);          /* .synchronize   */
+int         axhip_device_count(void);         /* .device_count  */
+const char *axhip_last_error(void);           /* thread-local message of the last failure */
+const char *axhip_device_name(void);          /* gcnArchName of device 0, "" without a GPU */
+
+/* ---- memory: .storage_alloc/.storage_free/.memcpy_* hooks
+ *      (src/compute/backends/cuda/memory.cu:78-140).  axhip_malloc returns zero-filled
+ *      memory like the reference's allocator (memory.cu:90), or NULL. ---------------- */
+void *axhip_malloc(size_t bytes);
+void  axhip_free(void *device_ptr);
+int   axhip_memset(void *device_ptr, int byte_value, size_t bytes);
+int   axhip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes);
+int   axhip_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes);   /* blocking */
+int   axhip_memcpy_d2d(void *device_dst, const void *device_src, size_t bytes);
+
+/* ---- fp32 GEMM.  Replaces cuda_gemm / cuda_gemm_ex / cuda_gemm_nt / cuda_gemm_tn
+ *      (src/compute/backends/cuda/ops_gemm.cu:15-126) and the cpu_opt drivers
+ *      opt_gemm / opt_gemm_nt / opt_gemm_relu / opt_gemm_ex
+ *      (src/compute/backends/cpu_opt.c:3446, 4842, 7401, 7442), with the bias add of
+ *      k_bias_add (cuda/ops_fused.cu:260-297) and the GELU of k_gelu
+ *      (cuda/ops_activations.cu:22) folded into the write-back.
+ *
+ *      C[M,N] = act( alpha * op(A) * op(B) + beta * C + bias[n] )
+ *      transa = 0: A is [M,K] (lda >= K);  1: A is [K,M] (lda >= M)
+ *      transb = 0: B is [K,N] (ldb >= N);  1: B is [N,K] (ldb >= K)
+ *      bias may be NULL; beta == 0 never reads C (C may be uninitialised).
+ *      True fp32 MFMA arithmetic; M <= 8 with transa = transb = 0 takes the
+ *      weight-streaming route below. ------------------------------------------------- */
+int axhip_sgemm(int transa, int transb, int64_t M, int64_t N, int64_t K, float alpha,
+                const float *A, int64_t lda, const float *B, int64_t ldb, float beta,
+                float *C, int64_t ldc, const float *bias, int act);
+
+/* Strided-batched form.  Replaces cublasSgemmStridedBatched as used for the per-head
+ * products in src/compute/backends/cuda/ops_attention.cu:326-334 (score = scale*Q*K^T)
+ * and :378-386 (O = P*V).  Matrix i of each operand starts at ptr + i*stride (elements). */
+int axhip_sgemm_strided_batched(int transa, int transb, int64_t M, int64_t N, int64_t K,
+                                float alpha, const float *A, int64_t lda, int64_t stride_a,
+                                const float *B, int64_t ldb, int64_t stride_b, float beta,
+                                float *C, int64_t ldc, int64_t stride_c, int64_t batch);
+
+/* Skinny-M route (1 <= M <= 8): C[M,N] = act(A[M,K] * B[K,N] + bias[n]), B streamed once
+ * for all M rows.  The GPU counterpart of the small/skinny-M AXPY route of opt_gemm
+ * (src/compute/backends/cpu_opt.c:3499-3567).  Results are deterministic run to run. */
+int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                       const float *B, int64_t ldb, float *C, int64_t ldc,
+                       const float *bias, int act);
+
+/* ---- int8 -------------------------------------------------------------------------- */
+/* W8A8: acc[m,n] = sum_k (int32)x[m,k] * (int32)w[n,k]   (exact, int32 MFMA)
+ *       out[m,n] = act( (float)acc * (x_scale * w_scales[n]) + bias[n] )
+ * x is [M,K] int8, w is [N,K] int8 — the data/scales layout of ax_qweight_t
+ * (include/axiom/quantize.h:50-55).  bias, out and acc_out may each be NULL (at least one
+ * of out / acc_out must be given).  Extends ax_qgemm_w8a32 (src/core/quantize.c:100-177)
+ * to int8 activations with int32 accumulation; there is no reference counterpart. */
+int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
+                     const float *bias, int act, float *out, int32_t *acc_out,
+                     int64_t M, int64_t N, int64_t K);
+
+/* W8A32: out[m,n] = w_scales[n] * sum_k a[m,k] * (float)w[n,k], fp32 accumulation.
+ * Device-memory form of ax_qgemm_w8a32 (src/core/quantize.c:100-177). */
+int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w_scales, float *out,
+                      int64_t M, int64_t N, int64_t K);
+
+/* Per-row symmetric int8 quantization on the device: the arithmetic of
+ * ax_qweight_create_from_fp32 (src/core/quantize.c:36-54). w is [N,K] fp32. */
+int axhip_quantize_rows(const float *w, int64_t N, int64_t K, int8_t *q, float *scales);
+
+/* ---- elementwise vtable slots ------------------------------------------------------- */
+/* .bias_add: out[o,a,i] = in[o,a,i] + bias[a]   (cuda/ops_fused.cu:260-297,
+ * cpu_opt.c:7148-7194); in/out may alias. */
+int axhip_bias_add(const float *in, const float *bias, int64_t outer, int64_t axis_len,
+                   int64_t inner, float *out);
+int axhip_relu(const float *in, float *out, int64_t n);       /* .relu    */
+int axhip_gelu(const float *in, float *out, int64_t n);       /* .gelu_op (tanh form) */
+int axhip_fill_f32(float *dst, float value, int64_t n);       /* .fill    */
+
+/* ---- timing on the library's stream (for benchmarks) -------------------------------- */
+void *axhip_event_create(void);
+void  axhip_event_destroy(void *ev);
+int   axhip_event_record(void *ev);
+int   axhip_event_elapsed_ms(void *start, void *stop, float *ms);   /* waits for stop */
+
+/* Name of the kernel variant the last GEMM-type call launched (for profiles/tests). */
+const char *axhip_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AXHIP_H */

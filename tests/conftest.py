@@ -31,3 +31,12 @@ def reflib():
     if not ref_available():
         pytest.skip("oracle/_ref/libaxref.so not built (reference tree absent)")
     return RefLib()
+
+
+@pytest.fixture(scope="session")
+def hip():
+    """libaxhip.so on a real GPU.  No fallback: a missing library or GPU is an error."""
+    from axiom_amd import AxHip
+    h = AxHip()
+    h.init()
+    return h

@@ -1,0 +1,375 @@
+"""GPU parity: the HIP path, called through the C ABI of libaxhip.so, against the CPU oracle
+on identical seeded inputs.  int32 accumulators and int8 outputs: bit-exact.  fp32: the gates
+stated next to each assert."""
+import numpy as np
+import pytest
+
+from fills import property_case, xorshift32_unit
+
+pytestmark = pytest.mark.gpu
+
+REL_FP32 = 1e-4      # max |gpu - cpu| / max |cpu|                      (fp32 GEMM vs the CPU path)
+BOUND_FP32 = 1e-5    # |gpu - c64| <= BOUND * sum_k |a_ik||b_kj|        (vs fp64 ground truth)
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def check_fp32(oracle, got, a, b, transb=False, ref=None):
+    c64 = oracle.gemm_f64(a, b, transb)
+    cabs = oracle.gemm_abs_f64(a, b, transb)
+    assert (np.abs(got - c64) <= BOUND_FP32 * cabs + 1e-30).all(), \
+        f"fp64 bound violated: {(np.abs(got - c64) / (cabs + 1e-30)).max()}"
+    if ref is not None:
+        assert np.abs(got - ref).max() <= REL_FP32 * max(np.abs(ref).max(), 1e-30)
+
+
+# ------------------------------------------------------------------ int8 W8A8
+INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300), (33, 64, 1000),
+               (128, 128, 256), (128, 256, 128), (256, 512, 384), (384, 128, 4096),
+               (2048, 4096, 512), (256, 4096, 4096)]
+
+
+@pytest.mark.parametrize("M,N,K", INT8_SHAPES)
+def test_w8a8_accumulators_bit_exact(hip, oracle, M, N, K):
+    say("w8a8", M, N, K)
+    oracle.seed(M * 7 + N * 3 + K)
+    x, w = oracle.int8((M, K)), oracle.int8((N, K))
+    ws = oracle.uniform((N,), 1e-3, 1e-2)
+    bias = oracle.normal((N,), 0.0, 0.02)
+    xs = float(np.float32(0.0173))
+    dx, dw, dws, db = hip.array(x), hip.array(w), hip.array(ws), hip.array(bias)
+    want_acc = oracle.qgemm_w8a8_acc(x, w)
+    for act in (0, 1, 2):
+        out, acc = hip.qgemm_w8a8(dx, xs, dw, dws, db, act)
+        say("  kernel", hip.last_kernel(), "act", act)
+        assert np.array_equal(acc.numpy(), want_acc)
+        want = oracle.w8a8_epilogue(want_acc, xs, ws, bias, act)
+        got = out.numpy()
+        if act != 2:
+            assert np.array_equal(got, want)              # same op order: bit-identical
+        else:                                             # tanhf differs between libms
+            assert np.abs(got - want).max() <= 1e-6 * max(1.0, np.abs(want).max())
+    out, _ = hip.qgemm_w8a8(dx, xs, dw, dws, None, 0, want_acc=False)
+    assert np.array_equal(out.numpy(), oracle.w8a8_epilogue(want_acc, xs, ws, None, 0))
+    _, acc = hip.qgemm_w8a8(dx, xs, dw, None, None, 0, want_out=False)
+    assert np.array_equal(acc.numpy(), want_acc)
+
+
+def test_w8a8_extreme_values_and_golden(hip, oracle, golden):
+    x = np.full((128, 8192), -127, np.int8)
+    w = np.full((128, 8192), -127, np.int8)
+    _, acc = hip.qgemm_w8a8(hip.array(x), 1.0, hip.array(w), None, want_out=False)
+    assert (acc.numpy() == 127 * 127 * 8192).all()
+    for K in (8, 32, 128, 512, 1024):                     # the reference's W8A32 with unit scales
+        oracle.seed(1000 + K)
+        x, w = oracle.int8((4, K)), oracle.int8((64, K))
+        _, acc = hip.qgemm_w8a8(hip.array(x), 1.0, hip.array(w), None, want_out=False)
+        assert np.array_equal(acc.numpy().astype(np.float64), golden[f"acc_K{K}"].astype(np.float64))
+
+
+def test_w8a8_8192_cube_properties(hip, oracle):
+    """Full size of the headline config: exact row/column checksums and 4096 sampled entries."""
+    M = N = K = 8192
+    oracle.seed(8192)
+    x, w = oracle.int8((M, K)), oracle.int8((N, K))
+    ws = oracle.uniform((N,), 1e-3, 1e-2)
+    bias = oracle.normal((N,), 0.0, 0.02)
+    xs = float(np.float32(0.011))
+    say("w8a8 8192^3 launch")
+    out, acc = hip.qgemm_w8a8(hip.array(x), xs, hip.array(w), hip.array(ws), hip.array(bias), 0)
+    say("  kernel", hip.last_kernel())
+    a = acc.numpy()
+    xi, wi = x.astype(np.int64), w.astype(np.int64)
+    assert np.array_equal(a.astype(np.int64).sum(axis=0), wi @ xi.sum(axis=0))   # column sums
+    assert np.array_equal(a.astype(np.int64).sum(axis=1), xi @ wi.sum(axis=0))   # row sums
+    rng = np.random.default_rng(1)
+    ms, ns = rng.integers(0, M, 4096), rng.integers(0, N, 4096)
+    exact = np.einsum("ik,ik->i", xi[ms], wi[ns])
+    assert np.array_equal(a[ms, ns].astype(np.int64), exact)
+    o = out.numpy()
+    want = oracle.w8a8_epilogue(np.ascontiguousarray(a[:64]), xs, ws, bias, 0)
+    assert np.array_equal(o[:64], want)
+
+
+# ------------------------------------------------------------------ fp32 GEMM
+F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), (64, 64, 32),
+              (128, 128, 64), (130, 260, 700), (256, 384, 512), (33, 40, 100), (96, 96, 96),
+              (2048, 1024, 256)]
+
+
+@pytest.mark.parametrize("M,N,K", F32_SHAPES)
+def test_sgemm_nn_nt_tn(hip, oracle, M, N, K):
+    say("sgemm", M, N, K)
+    oracle.seed(M + 31 * N + 977 * K)
+    a, b = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1)
+    ref = oracle.gemm_opt(a, b)
+    da, db = hip.array(a), hip.array(b)
+    got = hip.sgemm(da, db).numpy()
+    say("  nn", hip.last_kernel())
+    check_fp32(oracle, got, a, b, ref=ref)
+    bt = np.ascontiguousarray(b.T)
+    got = hip.sgemm(da, hip.array(bt), transb=True).numpy()
+    say("  nt", hip.last_kernel())
+    check_fp32(oracle, got, a, bt, transb=True, ref=oracle.gemm_opt_nt(a, bt))
+    at = np.ascontiguousarray(a.T)
+    got = hip.sgemm(hip.array(at), db, transa=True).numpy()
+    say("  tn", hip.last_kernel())
+    check_fp32(oracle, got, a, b, ref=ref)
+
+
+def test_sgemm_known_answers(hip, golden):
+    a = np.arange(1, 7, dtype=np.float32).reshape(2, 3)
+    b = np.arange(7, 13, dtype=np.float32).reshape(3, 2)
+    assert hip.sgemm(hip.array(a), hip.array(b)).numpy().reshape(-1).tolist() == [58, 64, 139, 154]
+    c = hip.sgemm(hip.array(np.array([[1, 2], [3, 4]], np.float32)),
+                  hip.array(np.array([[5, 6], [7, 8]], np.float32))).numpy()
+    assert c.reshape(-1).tolist() == [19, 22, 43, 50]
+    rng = np.random.default_rng(0)
+    m = rng.uniform(-1, 1, (200, 200)).astype(np.float32)
+    assert np.array_equal(hip.sgemm(hip.array(m), hip.array(np.eye(200, dtype=np.float32))).numpy(), m)
+    assert not hip.sgemm(hip.array(np.zeros((70, 300), np.float32)), hip.array(m[:, :100].repeat(3, 0)[:300])).numpy().any()
+    u, v = m[:33, :1].copy(), m[:1, :65].copy()
+    assert np.array_equal(hip.sgemm(hip.array(u), hip.array(v)).numpy(), u * v)      # K = 1
+
+
+@pytest.mark.parametrize("M,K,N", [(37, 73, 19), (64, 128, 32), (32, 2048, 16), (1, 784, 64), (7, 300, 130)])
+def test_sgemm_against_reference_outputs(hip, oracle, golden, M, K, N):
+    oracle.seed(M * 1000 + N)
+    a, b = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1)
+    ref = golden[f"gemm_{M}x{K}x{N}_opt"]
+    got = hip.sgemm(hip.array(a), hip.array(b)).numpy()
+    # the reference's own GPU-vs-CPU gate is 1e-3 abs (tests/test_cuda.c:235); ours is tighter
+    assert np.abs(got - ref).max() <= REL_FP32 * np.abs(ref).max()
+    got = hip.sgemm(hip.array(a), hip.array(np.ascontiguousarray(b.T)), transb=True).numpy()
+    assert np.abs(got - golden[f"gemm_nt_{M}x{K}x{N}_opt"]).max() <= REL_FP32 * np.abs(ref).max()
+
+
+def test_sgemm_property_cases(hip, oracle, golden):
+    for i in range(60):                                   # tests/test_property.c:176-208
+        M, N, K, a, b = property_case(i)
+        got = hip.sgemm(hip.array(a), hip.array(b)).numpy()
+        cn = oracle.gemm_naive(a, b)
+        assert (np.abs(got - cn) <= 1e-3 + 1e-4 * np.abs(cn)).all(), (i, M, N, K)
+        assert abs(got.astype(np.float64).sum() - golden["prop_sums"][i, 1]) <= \
+            1e-5 * max(1.0, golden["prop_sums"][i, 2])
+
+
+def test_sgemm_config0_1024_cube(hip, oracle, golden):
+    oracle.seed(0)
+    a, b = oracle.uniform((1024, 1024), -1, 1), oracle.uniform((1024, 1024), -1, 1)
+    da, db = hip.array(a), hip.array(b)
+    dc = hip.sgemm(da, db)
+    say("1024^3", hip.last_kernel())
+    c = dc.numpy()
+    check_fp32(oracle, c, a, b, ref=oracle.gemm_opt(a, b))
+    assert np.abs(c[0] - golden["gemm_1024_row0"]).max() <= REL_FP32 * 60
+    s, sabs = golden["gemm_1024_sums"]
+    assert abs(c.astype(np.float64).sum() - s) <= 1e-6 * sabs
+    # determinism (tests/test_optimization_paths.c:265-292): repeated runs are bit-identical
+    for _ in range(5):
+        assert np.array_equal(hip.sgemm(da, db).numpy(), c)
+
+
+def test_sgemm_alpha_beta_bias_act(hip, oracle):
+    oracle.seed(21)
+    M, N, K = 130, 200, 96
+    a, b = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1)
+    c0 = oracle.uniform((M, N), -1, 1)
+    bias = oracle.normal((N,), 0, 0.5)
+    c64 = oracle.gemm_f64(a, b)
+    da, db, dbias = hip.array(a), hip.array(b), hip.array(bias)
+    got = hip.sgemm(da, db, alpha=0.5, beta=2.0, c=hip.array(c0)).numpy()
+    assert np.abs(got - (0.5 * c64 + 2.0 * c0)).max() <= 1e-5 * K
+    got = hip.sgemm(da, db, alpha=1.0, beta=1.0, c=hip.array(c0)).numpy()      # gemm_ex accumulate
+    assert np.abs(got - (c64 + c0)).max() <= 1e-5 * K
+    lin = hip.sgemm(da, db, bias=dbias).numpy()
+    assert np.abs(lin - oracle.dense(a, b, bias, 0)).max() <= REL_FP32 * np.abs(c64).max()
+    relu = hip.sgemm(da, db, bias=dbias, act=1).numpy()
+    assert np.array_equal(relu, np.maximum(lin, 0))
+    assert np.abs(relu - oracle.dense(a, b, bias, 1)).max() <= REL_FP32 * np.abs(c64).max()
+    gelu = hip.sgemm(da, db, bias=dbias, act=2).numpy()
+    assert np.abs(gelu - oracle.gelu(lin)).max() <= 1e-5 + 1e-5 * np.abs(lin).max()
+    # beta = 0 must not read C: poison it with NaN
+    poison = hip.array(np.full((M, N), np.nan, np.float32))
+    assert np.isfinite(hip.sgemm(da, db, c=poison).numpy()).all()
+
+
+def test_config3_ffn_block(hip, oracle):
+    """tokens 2048, d_model 1024, d_ff 4096: GEMM1 + bias + GELU -> GEMM2 + bias."""
+    oracle.seed(3)
+    x = oracle.normal((2048, 1024))
+    w1, w2 = oracle.normal((1024, 4096), 0, 0.02), oracle.normal((4096, 1024), 0, 0.02)
+    b1, b2 = oracle.normal((4096,), 0, 0.02), oracle.normal((1024,), 0, 0.02)
+    say("ffn launch")
+    dh = hip.sgemm(hip.array(x), hip.array(w1), bias=hip.array(b1), act=2)
+    say("  ", hip.last_kernel())
+    dy = hip.sgemm(dh, hip.array(w2), bias=hip.array(b2))
+    h_ref = oracle.dense(x, w1, b1, 2)
+    y_ref = oracle.dense(h_ref, w2, b2, 0)
+    h, y = dh.numpy(), dy.numpy()
+    assert np.abs(h - h_ref).max() <= 1e-5 + REL_FP32 * np.abs(h_ref).max()
+    assert np.abs(y - y_ref).max() <= REL_FP32 * np.abs(y_ref).max()
+
+
+# ------------------------------------------------------------------ skinny-M route
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_skinny_against_oracle(hip, oracle, M):
+    oracle.seed(100 + M)
+    for (K, N) in [(784, 4096), (4096, 4096), (4096, 10), (1, 5), (130, 67), (16, 64), (3000, 1000)]:
+        say("skinny", M, K, N)
+        a, b = oracle.uniform((M, K), 0, 1), oracle.kaiming((K, N), K)
+        bias = oracle.normal((N,), 0, 0.1)
+        da, db, dbias = hip.array(a), hip.array(b), hip.array(bias)
+        got = hip.sgemm_skinny(da, db).numpy()
+        check_fp32(oracle, got, a, b, ref=oracle.gemm_opt(a, b))
+        fused = hip.sgemm_skinny(da, db, dbias, 1).numpy()
+        assert np.array_equal(fused, np.maximum(got + bias[None, :], 0))
+        via = hip.sgemm(da, db, bias=dbias, act=1).numpy()          # auto-routed
+        assert hip.last_kernel().startswith("sgemm_skinny")
+        assert np.array_equal(via, fused)
+        assert np.array_equal(hip.sgemm_skinny(da, db).numpy(), got)  # deterministic
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 8])
+def test_config1_mlp_inference(hip, oracle, M):
+    """x[M,784] -> dense 4096 -> ReLU -> dense 4096 -> ReLU -> dense 10; Kaiming-uniform weights
+    drawn in layer order after seeding (src/core/layer.c:66-99), biases zero."""
+    oracle.seed(1234)
+    w1, w2, w3 = oracle.kaiming((784, 4096), 784), oracle.kaiming((4096, 4096), 4096), oracle.kaiming((4096, 10), 4096)
+    z1, z2, z3 = np.zeros(4096, np.float32), np.zeros(4096, np.float32), np.zeros(10, np.float32)
+    x = oracle.uniform((M, 784), 0, 1)
+    ref = oracle.dense(oracle.dense(oracle.dense(x, w1, z1, 1), w2, z2, 1), w3, z3, 0)
+    h1 = hip.sgemm(hip.array(x), hip.array(w1), bias=hip.array(z1), act=1)
+    h2 = hip.sgemm(h1, hip.array(w2), bias=hip.array(z2), act=1)
+    y = hip.sgemm(h2, hip.array(w3), bias=hip.array(z3)).numpy()
+    assert y.shape == (M, 10)
+    assert np.abs(y - ref).max() <= REL_FP32 * np.abs(ref).max()
+
+
+# ------------------------------------------------------------------ strided batched
+def test_strided_batched_qkt_and_pv(hip, oracle):
+    oracle.seed(55)
+    Bn, S, D = 6, 512, 64
+    q, k, v = oracle.normal((Bn, S, D)), oracle.normal((Bn, S, D)), oracle.normal((Bn, S, D))
+    dq, dk, dv = hip.array(q), hip.array(k), hip.array(v)
+    ds = hip.sgemm_batched(dq, dk, transb=True, alpha=0.125)
+    say("qkt", hip.last_kernel())
+    s = ds.numpy()
+    do = hip.sgemm_batched(ds, dv)
+    say("pv", hip.last_kernel())
+    o = do.numpy()
+    for h in range(Bn):
+        s_ref = oracle.gemm_opt_nt(q[h], k[h]) * np.float32(0.125)
+        assert np.abs(s[h] - s_ref).max() <= REL_FP32 * np.abs(s_ref).max()
+        o_ref = oracle.gemm_opt(s[h], v[h])
+        assert np.abs(o[h] - o_ref).max() <= REL_FP32 * np.abs(o_ref).max()
+    # ragged batch member shapes
+    a, b = oracle.normal((3, 37, 29)), oracle.normal((3, 29, 41))
+    c = hip.sgemm_batched(hip.array(a), hip.array(b)).numpy()
+    for h in range(3):
+        check_fp32(oracle, c[h], a[h], b[h])
+
+
+def test_config4b_attention_shapes_full_size(hip, oracle):
+    """512 heads of [512,64]: sampled heads against the oracle, all heads by a linearity check."""
+    oracle.seed(44)
+    Bn, S, D = 512, 512, 64
+    q, k, v = oracle.normal((Bn, S, D)), oracle.normal((Bn, S, D)), oracle.normal((Bn, S, D))
+    dq, dk, dv = hip.array(q), hip.array(k), hip.array(v)
+    ds = hip.sgemm_batched(dq, dk, transb=True)
+    do = hip.sgemm_batched(ds, dv)
+    s, o = ds.numpy(), do.numpy()
+    for h in (0, 1, 255, 511):
+        s_ref = oracle.gemm_opt_nt(q[h], k[h])
+        assert np.abs(s[h] - s_ref).max() <= REL_FP32 * np.abs(s_ref).max()
+        o_ref = oracle.gemm_opt(s[h], v[h])
+        assert np.abs(o[h] - o_ref).max() <= REL_FP32 * np.abs(o_ref).max()
+    # every head: row sums of S equal Q . (sum of K rows), to fp32 accumulation accuracy
+    ksum = k.astype(np.float64).sum(axis=1)
+    want = np.einsum("hsd,hd->hs", q.astype(np.float64), ksum)
+    got = s.astype(np.float64).sum(axis=2)
+    scale = np.einsum("hsd,hd->hs", np.abs(q).astype(np.float64), np.abs(k).astype(np.float64).sum(axis=1))
+    assert (np.abs(got - want) <= 1e-5 * scale).all()
+
+
+# ------------------------------------------------------------------ W8A32
+W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 1024), (3, 17, 45),
+                (1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024),
+                (64, 1024, 4096), (1, 4096, 4096), (5, 33, 100)]
+
+
+@pytest.mark.parametrize("M,N,K", W8A32_SHAPES)
+def test_w8a32_against_oracle(hip, oracle, golden, M, N, K):
+    say("w8a32", M, N, K)
+    a = xorshift32_unit(M * K, 7).reshape(M, K) if M * K < 70000 else None
+    if a is None:
+        oracle.seed(M + N + K)
+        a, w = oracle.uniform((M, K), -1, 1), oracle.uniform((N, K), -1, 1)
+    else:
+        w = xorshift32_unit(N * K, 13).reshape(N, K)
+    q, s = oracle.quantize_rows(w)
+    got = hip.qgemm_w8a32(hip.array(a), hip.array(q), hip.array(s)).numpy()
+    say("  ", hip.last_kernel())
+    ref = oracle.qgemm_w8a32(a, q, s)
+    key = f"w8a32_{M}x{N}x{K}_out"
+    if key in golden.files:
+        assert np.array_equal(ref, golden[key])
+    # the reference's own gate (tests/test_quantize.c:107-111) ...
+    diff = np.abs(got - ref)
+    assert not ((diff > 1e-2) & (diff / np.maximum(np.abs(ref), 1e-30) > 1e-3)).any()
+    # ... and ours: fp32 accumulation-order noise only
+    assert diff.max() <= REL_FP32 * max(np.abs(ref).max(), 1e-30)
+
+
+def test_device_quantizer_bit_exact(hip, oracle, golden):
+    for (N, K) in ((8, 8), (128, 128), (64, 1024), (5, 333)):
+        w = xorshift32_unit(N * K, 42).reshape(N, K)
+        dq, ds = hip.quantize_rows(hip.array(w))
+        q, s = oracle.quantize_rows(w)
+        assert np.array_equal(dq.numpy(), q) and np.array_equal(ds.numpy(), s)
+    dq, ds = hip.quantize_rows(hip.array(golden["quant_ties_w"]))
+    assert np.array_equal(dq.numpy(), golden["quant_ties_q"])
+    dq, ds = hip.quantize_rows(hip.array(golden["quant_hand_w"]))
+    assert np.array_equal(dq.numpy(), golden["quant_hand_q"]) and np.array_equal(ds.numpy(), golden["quant_hand_s"])
+
+
+# ------------------------------------------------------------------ elementwise + errors
+def test_elementwise_slots(hip, oracle, golden):
+    oracle.seed(8)
+    x = oracle.normal((37, 1001), 0, 2)
+    dx = hip.array(x)
+    out = hip.empty(x.shape)
+    hip.check(hip.L.axhip_relu(dx.ptr, out.ptr, x.size))
+    assert np.array_equal(out.numpy(), np.maximum(x, 0))
+    hip.check(hip.L.axhip_gelu(dx.ptr, out.ptr, x.size))
+    assert np.abs(out.numpy() - oracle.gelu(x)).max() <= 1e-6
+    g = hip.array(golden["gelu_x"])
+    go = hip.empty(g.shape)
+    hip.check(hip.L.axhip_gelu(g.ptr, go.ptr, g.shape[0]))
+    assert np.abs(go.numpy() - golden["gelu_y"]).max() <= 2e-6          # the reference's ax_gelu
+    hip.check(hip.L.axhip_fill_f32(out.ptr, 2.5, x.size))
+    assert (out.numpy() == 2.5).all()
+    bias = oracle.normal((1001,), 0, 1)
+    hip.check(hip.L.axhip_bias_add(dx.ptr, hip.array(bias).ptr, 37, 1001, 1, out.ptr))
+    assert np.array_equal(out.numpy(), x + bias[None, :])
+    rb = oracle.normal((37,), 0, 1)
+    hip.check(hip.L.axhip_bias_add(dx.ptr, hip.array(rb).ptr, 1, 37, 1001, out.ptr))
+    assert np.array_equal(out.numpy(), x + rb[:, None])
+    z = hip.empty((1000,))                                               # zero-filled allocation
+    assert not z.numpy().any()
+
+
+def test_error_paths(hip):
+    L = hip.L
+    a = hip.empty((8, 8))
+    assert L.axhip_sgemm(0, 0, 8, 8, 8, 1.0, None, 8, a.ptr, 8, 0.0, a.ptr, 8, None, 0) == 1
+    assert L.axhip_sgemm(0, 0, 8, 8, 8, 1.0, a.ptr, 4, a.ptr, 8, 0.0, a.ptr, 8, None, 0) == 3
+    assert L.axhip_sgemm(1, 1, 8, 8, 8, 1.0, a.ptr, 8, a.ptr, 8, 0.0, a.ptr, 8, None, 0) == 10
+    assert L.axhip_sgemm_skinny(9, 8, 8, a.ptr, 8, a.ptr, 8, a.ptr, 8, None, 0) == 3
+    assert L.axhip_qgemm_w8a8(a.ptr, 1.0, a.ptr, None, None, 0, None, None, 8, 8, 8) == 1
+    assert L.axhip_qgemm_w8a8(a.ptr, 1.0, a.ptr, None, None, 7, None, a.ptr, 8, 8, 8) == 3
+    assert "activation" in hip.last_error()
+    assert L.axhip_sgemm(0, 0, 0, 8, 8, 1.0, a.ptr, 8, a.ptr, 8, 0.0, a.ptr, 8, None, 0) == 0   # empty
+    hip.sync()
