@@ -1,0 +1,155 @@
+/* Dense / ReLU / GELU / Sequential, forward only (Axiom's src/core/layer.c:48-103, 181-300). */
+#include <stdlib.h>
+
+#include "axiom/init.h"
+#include "axiom/layer.h"
+#include "axiom/ops.h"
+
+static ax_tensor_t *dense_bias(ax_dense_t *d) { return (d->use_bias && d->bias) ? d->bias : NULL; }
+
+static ax_tensor_t *dense_forward(ax_layer_t *self, ax_tensor_t *x) {
+    ax_dense_t *d = (ax_dense_t *)self;
+    return ax_matmul_bias(x, d->weight, dense_bias(d));
+}
+
+static void dense_destroy(ax_layer_t *self) {
+    ax_dense_t *d = (ax_dense_t *)self;
+    ax_tensor_destroy(d->weight);
+    ax_tensor_destroy(d->bias);
+    free(d);
+}
+
+/* weight [in,out] Kaiming-uniform with fan_in = in, drawn at creation; bias zeros (layer.c:66-99) */
+ax_layer_t *ax_dense_create(int64_t in_features, int64_t out_features, bool use_bias) {
+    if (in_features <= 0 || out_features <= 0) {
+        ax_err_set(AX_ERR_INVALID_SHAPE, "ax_dense_create: features must be positive");
+        return NULL;
+    }
+    ax_dense_t *d = calloc(1, sizeof *d);
+    if (!d) {
+        ax_err_set(AX_ERR_ALLOC, "ax_dense_create: out of memory");
+        return NULL;
+    }
+    d->base.ops.forward = dense_forward;
+    d->base.ops.destroy = dense_destroy;
+    d->base.type = AX_LAYER_DENSE;
+    d->base.training = true;
+    d->base.input_features = in_features;
+    d->base.output_features = out_features;
+    d->use_bias = use_bias;
+    int64_t wshape[2] = {in_features, out_features};
+    d->weight = ax_tensor_create(wshape, 2, AX_FLOAT32);
+    if (!d->weight) {
+        free(d);
+        return NULL;
+    }
+    ax_init_kaiming_uniform(d->weight, in_features);
+    d->weight->requires_grad = true;
+    d->base.params[0] = d->weight;
+    d->base.n_params = 1;
+    if (use_bias) {
+        d->bias = ax_tensor_zeros(&out_features, 1, AX_FLOAT32);
+        if (!d->bias) {
+            ax_tensor_destroy(d->weight);
+            free(d);
+            return NULL;
+        }
+        d->bias->requires_grad = true;
+        d->base.params[1] = d->bias;
+        d->base.n_params = 2;
+    }
+    return &d->base;
+}
+
+static ax_tensor_t *relu_forward(ax_layer_t *self, ax_tensor_t *x) { (void)self; return ax_relu(x); }
+static ax_tensor_t *gelu_forward(ax_layer_t *self, ax_tensor_t *x) { (void)self; return ax_gelu(x); }
+static void plain_destroy(ax_layer_t *self) { free(self); }
+
+static ax_layer_t *activation_layer(ax_layer_type_t type, ax_tensor_t *(*fwd)(ax_layer_t *, ax_tensor_t *)) {
+    ax_layer_t *l = calloc(1, sizeof *l);
+    if (!l) {
+        ax_err_set(AX_ERR_ALLOC, "activation layer: out of memory");
+        return NULL;
+    }
+    l->ops.forward = fwd;
+    l->ops.destroy = plain_destroy;
+    l->type = type;
+    l->training = true;
+    return l;
+}
+
+ax_layer_t *ax_relu_layer_create(void) { return activation_layer(AX_LAYER_RELU, relu_forward); }
+ax_layer_t *ax_gelu_layer_create(void) { return activation_layer(AX_LAYER_GELU, gelu_forward); }
+
+static ax_tensor_t *sequential_forward(ax_layer_t *self, ax_tensor_t *input) {
+    ax_sequential_t *seq = (ax_sequential_t *)self;
+    ax_tensor_t *x = input, *prev = NULL;
+    for (int i = 0; i < seq->n_layers; i++) {
+        ax_layer_t *l = seq->layers[i];
+        ax_layer_type_t next_type = (i + 1 < seq->n_layers) ? seq->layers[i + 1]->type : AX_LAYER_TYPE_COUNT;
+        ax_tensor_t *y;
+        if (l->type == AX_LAYER_DENSE && next_type == AX_LAYER_RELU) {
+            ax_dense_t *d = (ax_dense_t *)l;
+            y = ax_matmul_bias_relu(x, d->weight, dense_bias(d));
+            i++;
+        } else if (l->type == AX_LAYER_DENSE && next_type == AX_LAYER_GELU) {
+            ax_dense_t *d = (ax_dense_t *)l;
+            y = ax_matmul_bias_gelu(x, d->weight, dense_bias(d));
+            i++;
+        } else {
+            y = ax_layer_forward(l, x);
+        }
+        if (prev) ax_tensor_destroy(prev);      /* inference: nobody else holds the intermediate */
+        if (!y) return NULL;
+        prev = x = y;
+    }
+    return x;
+}
+
+static void sequential_destroy(ax_layer_t *self) {
+    ax_sequential_t *seq = (ax_sequential_t *)self;
+    for (int i = 0; i < seq->n_layers; i++) ax_layer_destroy(seq->layers[i]);
+    free(seq);
+}
+
+ax_layer_t *ax_sequential_create(void) {
+    ax_sequential_t *seq = calloc(1, sizeof *seq);
+    if (!seq) {
+        ax_err_set(AX_ERR_ALLOC, "ax_sequential_create: out of memory");
+        return NULL;
+    }
+    seq->base.ops.forward = sequential_forward;
+    seq->base.ops.destroy = sequential_destroy;
+    seq->base.type = AX_LAYER_SEQUENTIAL;
+    seq->base.training = true;
+    return &seq->base;
+}
+
+ax_layer_t *ax_sequential_add(ax_layer_t *seq_base, ax_layer_t *layer) {
+    ax_sequential_t *seq = (ax_sequential_t *)seq_base;
+    if (!seq || !layer || seq->base.type != AX_LAYER_SEQUENTIAL || seq->n_layers >= AX_SEQ_MAX_LAYERS) return NULL;
+    seq->layers[seq->n_layers++] = layer;
+    return seq_base;
+}
+
+ax_tensor_t *ax_layer_forward(ax_layer_t *layer, ax_tensor_t *input) {
+    if (!layer || !layer->ops.forward) return NULL;
+    return layer->ops.forward(layer, input);
+}
+
+int ax_layer_get_params(ax_layer_t *layer, ax_tensor_t **params, int max_params) {
+    if (!layer) return 0;
+    int count = 0;
+    if (layer->type == AX_LAYER_SEQUENTIAL) {
+        ax_sequential_t *seq = (ax_sequential_t *)layer;
+        for (int i = 0; i < seq->n_layers && count < max_params; i++)
+            count += ax_layer_get_params(seq->layers[i], params + count, max_params - count);
+        return count;
+    }
+    for (int i = 0; i < layer->n_params && count < max_params; i++) params[count++] = layer->params[i];
+    return count;
+}
+
+void ax_layer_destroy(ax_layer_t *layer) {
+    if (layer && layer->ops.destroy) layer->ops.destroy(layer);
+}

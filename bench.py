@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X GEMM backend.  Prints ONE JSON line on stdout.
+
+Headline workload (BASELINE.json configs[4], the shape the int8 target is quoted on): the
+W8A8 quantized GEMM at M=N=K=8192 with its fused dequantize + bias write-back.  One "step"
+is one such GEMM over inputs already resident in HBM; `value` is TOP/s (2*M*N*K per step).
+The `secondary` object carries the other configurations the metric names: fp32 GEMM TFLOP/s
+and the skinny-M route's GB/s, each with its own roofline fraction.  RESULT lines in the
+reference's benchmark format (benchmarks/bench_common.h:25-42) go to stderr.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, TOP/s
+PEAK_FP32_TFLOPS = 157.3     # MI355X fp32 matrix, TFLOP/s
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
+
+
+def result_line(suite, case, metric, value):
+    print(f"RESULT {suite} {case} {metric} {value:.6g}", file=sys.stderr, flush=True)
+
+
+def rand_i8(rng, shape):
+    return rng.integers(-127, 128, shape, dtype=np.int8)
+
+
+def time_calls(hip, fn, steps, warmup):
+    """(host ms per step between device syncs, event ms per step on the kernels' stream)."""
+    for _ in range(warmup):
+        fn()
+    hip.sync()
+    e0, e1 = hip.L.axhip_event_create(), hip.L.axhip_event_create()
+    t0 = time.perf_counter()
+    hip.check(hip.L.axhip_event_record(e0))
+    for _ in range(steps):
+        fn()
+    hip.check(hip.L.axhip_event_record(e1))
+    hip.sync()
+    host_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms = C.c_float()
+    hip.check(hip.L.axhip_event_elapsed_ms(e0, e1, C.byref(ms)))
+    hip.L.axhip_event_destroy(e0)
+    hip.L.axhip_event_destroy(e1)
+    return host_ms, ms.value / steps
+
+
+def headline(hip, steps, warmup):
+    M = N = K = 8192
+    rng = np.random.default_rng(0)
+    x, w = hip.array(rand_i8(rng, (M, K))), hip.array(rand_i8(rng, (N, K)))
+    ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+    bias = hip.array(rng.normal(0.0, 0.02, N).astype(np.float32))
+    out = hip.empty((M, N))
+
+    def step():
+        hip.check(hip.L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, bias.ptr, 0, out.ptr, None, M, N, K))
+
+    host_ms, ev_ms = time_calls(hip, step, steps, warmup)
+    ops = 2.0 * M * N * K
+    return {"M": M, "N": N, "K": K, "host_ms": host_ms, "event_ms": ev_ms, "ops": ops,
+            "kernel": hip.last_kernel(),
+            "algorithmic_bytes": M * K + N * K + 4 * M * N + 8 * N}
+
+
+def secondary(hip):
+    """The metric's other configurations, each timed with HIP events on the kernels' stream."""
+    rng = np.random.default_rng(1)
+    res = {}
+
+    def f32(a_shape, b_shape):
+        return (hip.array(rng.uniform(-1, 1, a_shape).astype(np.float32)),
+                hip.array(rng.uniform(-1, 1, b_shape).astype(np.float32)))
+
+    # config 0: fp32 1024^3
+    a, b = f32((1024, 1024), (1024, 1024))
+    c = hip.empty((1024, 1024))
+    _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm(
+        0, 0, 1024, 1024, 1024, 1.0, a.ptr, 1024, b.ptr, 1024, 0.0, c.ptr, 1024, None, 0)), 50, 5)
+    tf = 2 * 1024 ** 3 / ms / 1e9
+    res["fp32_gemm_1024"] = {"us": ms * 1e3, "TFLOP/s": tf, "frac_of_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS,
+                             "kernel": hip.last_kernel()}
+    result_line("axhip", "f32_nn_1024x1024x1024", "gflops", tf * 1e3)
+
+    # config 3: FFN block 2048 x 1024 x 4096, bias + GELU fused into GEMM1, bias into GEMM2
+    x, w1 = f32((2048, 1024), (1024, 4096))
+    w2 = hip.array(rng.normal(0, 0.02, (4096, 1024)).astype(np.float32))
+    b1 = hip.array(rng.normal(0, 0.02, 4096).astype(np.float32))
+    b2 = hip.array(rng.normal(0, 0.02, 1024).astype(np.float32))
+    hbuf, y = hip.empty((2048, 4096)), hip.empty((2048, 1024))
+
+    def ffn():
+        hip.check(hip.L.axhip_sgemm(0, 0, 2048, 4096, 1024, 1.0, x.ptr, 1024, w1.ptr, 4096, 0.0,
+                                    hbuf.ptr, 4096, b1.ptr, 2))
+        hip.check(hip.L.axhip_sgemm(0, 0, 2048, 1024, 4096, 1.0, hbuf.ptr, 4096, w2.ptr, 1024, 0.0,
+                                    y.ptr, 1024, b2.ptr, 0))
+    _, ms = time_calls(hip, ffn, 20, 3)
+    tf = 2 * 2 * 2048 * 1024 * 4096 / ms / 1e9
+    res["fp32_ffn_2048x1024x4096"] = {"us": ms * 1e3, "TFLOP/s": tf,
+                                      "frac_of_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS}
+    result_line("axhip", "f32_ffn_2048x1024x4096", "gflops", tf * 1e3)
+    del x, w1, w2, hbuf, y
+
+    # config 2: int8 M=256, N=K=4096 (HBM/latency-bound)
+    xi, wi = hip.array(rand_i8(rng, (256, 4096))), hip.array(rand_i8(rng, (4096, 4096)))
+    ws = hip.array(rng.uniform(1e-3, 1e-2, 4096).astype(np.float32))
+    bi = hip.array(rng.normal(0, 0.02, 4096).astype(np.float32))
+    oi = hip.empty((256, 4096))
+    _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_qgemm_w8a8(
+        xi.ptr, 0.01, wi.ptr, ws.ptr, bi.ptr, 0, oi.ptr, None, 256, 4096, 4096)), 50, 5)
+    nbytes = 4096 * 4096 + 256 * 4096 + 4 * 256 * 4096 + 8 * 4096
+    res["int8_qgemm_256x4096x4096"] = {"us": ms * 1e3, "TOP/s": 2 * 256 * 4096 * 4096 / ms / 1e9,
+                                       "GB/s": nbytes / ms / 1e6,
+                                       "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS,
+                                       "kernel": hip.last_kernel()}
+    del xi, wi, oi
+
+    # config 1: bs=1 MLP 784 -> 4096 -> 4096 -> 10 through the skinny-M route, M in {1,2,4,8}.
+    # 8 rotating weight sets (641 MB) so every pass streams from HBM, not the 256 MB Infinity Cache.
+    sets = []
+    for _ in range(8):
+        sets.append((hip.array(rng.uniform(-0.09, 0.09, (784, 4096)).astype(np.float32)),
+                     hip.array(rng.uniform(-0.04, 0.04, (4096, 4096)).astype(np.float32)),
+                     hip.array(rng.uniform(-0.04, 0.04, (4096, 10)).astype(np.float32))))
+    zeros = hip.empty((4096,))
+    weight_bytes = 4 * (784 * 4096 + 4096 * 4096 + 4096 * 10)
+    mlp = {}
+    for M in (1, 2, 4, 8):
+        xin = hip.array(rng.uniform(0, 1, (M, 784)).astype(np.float32))
+        h1, h2, yo = hip.empty((M, 4096)), hip.empty((M, 4096)), hip.empty((M, 10))
+        it = [0]
+
+        def mlp_step():
+            w1_, w2_, w3_ = sets[it[0] % 8]
+            it[0] += 1
+            L = hip.L
+            hip.check(L.axhip_sgemm(0, 0, M, 4096, 784, 1.0, xin.ptr, 784, w1_.ptr, 4096, 0.0, h1.ptr, 4096, zeros.ptr, 1))
+            hip.check(L.axhip_sgemm(0, 0, M, 4096, 4096, 1.0, h1.ptr, 4096, w2_.ptr, 4096, 0.0, h2.ptr, 4096, zeros.ptr, 1))
+            hip.check(L.axhip_sgemm(0, 0, M, 10, 4096, 1.0, h2.ptr, 4096, w3_.ptr, 10, 0.0, yo.ptr, 10, zeros.ptr, 0))
+
+        def layer2_only():
+            _, w2_, _ = sets[it[0] % 8]
+            it[0] += 1
+            hip.check(hip.L.axhip_sgemm(0, 0, M, 4096, 4096, 1.0, h1.ptr, 4096, w2_.ptr, 4096, 0.0, h2.ptr, 4096, zeros.ptr, 1))
+
+        _, ms = time_calls(hip, mlp_step, 64, 8)
+        _, ms2 = time_calls(hip, layer2_only, 64, 8)
+        gbs, gbs2 = weight_bytes / ms / 1e6, 4 * 4096 * 4096 / ms2 / 1e6
+        mlp[f"M{M}"] = {"mlp_us": ms * 1e3, "mlp_GB/s": gbs, "mlp_frac_of_hbm_peak": gbs / PEAK_HBM_GBS,
+                        "layer2_us": ms2 * 1e3, "layer2_GB/s": gbs2,
+                        "layer2_frac_of_hbm_peak": gbs2 / PEAK_HBM_GBS}
+        result_line("axhip", f"mlp3_bs{M}", "latency_us", ms * 1e3)
+    res["skinny_mlp_784_4096_4096_10"] = mlp
+    del sets
+
+    # config 4b: strided-batched attention-shaped products, 512 heads of [512,64]
+    Bn, S, D = 512, 512, 64
+    q = hip.array(rng.normal(0, 1, (Bn, S, D)).astype(np.float32))
+    k = hip.array(rng.normal(0, 1, (Bn, S, D)).astype(np.float32))
+    v = hip.array(rng.normal(0, 1, (Bn, S, D)).astype(np.float32))
+    s, o = hip.empty((Bn, S, S)), hip.empty((Bn, S, D))
+    _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm_strided_batched(
+        0, 1, S, S, D, 1.0, q.ptr, D, S * D, k.ptr, D, S * D, 0.0, s.ptr, S, S * S, Bn)), 10, 2)
+    nbytes = 4 * (2 * Bn * S * D + Bn * S * S)
+    res["fp32_batched_qkt"] = {"us": ms * 1e3, "TFLOP/s": 2 * Bn * S * S * D / ms / 1e9,
+                               "GB/s": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm_strided_batched(
+        0, 0, S, D, S, 1.0, s.ptr, S, S * S, v.ptr, D, S * D, 0.0, o.ptr, D, S * D, Bn)), 10, 2)
+    res["fp32_batched_pv"] = {"us": ms * 1e3, "TFLOP/s": 2 * Bn * S * S * D / ms / 1e9,
+                              "GB/s": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    return res
+
+
+def cpu_baseline():
+    """The reference's own CPU path on this box's host cores.  Checker/baseline code only."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_bind as ob
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    rng = np.random.default_rng(2)
+    M, N, K = 4096, 8192, 8192          # half of the headline's rows: ~10 s of CPU work
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    q = rand_i8(rng, (N, K))
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    if ob.ref_available():
+        lib, kind = ob.RefLib(), "reference"
+        run = lambda: lib.qgemm_w8a32(a, q, s)
+    else:
+        lib, kind = ob.Oracle(), "port"
+        run = lambda: lib.qgemm_w8a32(a, q, s)
+    t0 = time.perf_counter()
+    run()
+    dt = time.perf_counter() - t0
+    tops = 2.0 * M * N * K / dt / 1e12
+    result_line("cpu", f"q8a32_{M}x{N}x{K}", "gflops", tops * 1e3)
+    return {"value": tops, "unit": "TOP/s", "cores": cores, "kind": kind,
+            "sample": f"ax_qgemm_w8a32 (the reference's only quantized GEMM: int8 weights x fp32 "
+                      f"activations, fp32 accumulate; it has no W8A8) on M={M} of the headline's 8192 "
+                      f"rows, N=K=8192, one run of {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    from axiom_amd import AxHip
+    hip = AxHip()
+    hip.init()
+
+    h = headline(hip, args.steps, args.warmup)
+    tops = h["ops"] / h["host_ms"] / 1e9
+    achieved = h["ops"] / h["event_ms"] / 1e9
+    result_line("axhip", "q8a8_8192x8192x8192", "gflops", tops * 1e3)
+    line = {
+        "metric": "int8 qgemm TOP/s on 1 MI355X (W8A8, M=N=K=8192, fused dequant+bias)",
+        "value": tops, "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": h["host_ms"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8 (int32 accumulate, fp32 epilogue)", "data": "synthetic",
+        "config": {"workload": "configs[4]: int8 qgemm M=N=K=8192, W int8 [N,K] + per-channel fp32 "
+                               "scales, X int8 + per-tensor scale, bias, fp32 out",
+                   "M": h["M"], "N": h["N"], "K": h["K"], "device": hip.L.axhip_device_name().decode()},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                     "frac": achieved / PEAK_INT8_TOPS, "traffic": None, "kernel": h["kernel"],
+                     "kernel_us": h["event_ms"] * 1e3, "algorithmic_ops": h["ops"],
+                     "algorithmic_bytes": h["algorithmic_bytes"]},
+    }
+    if not args.no_secondary:
+        line["secondary"] = secondary(hip)
+    hip.sync()
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

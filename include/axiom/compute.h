@@ -1,0 +1,72 @@
+/* axiom/compute.h — backend selection and the ax_compute_* dispatch wrappers of the GEMM path
+ * (include/axiom/compute.h:46-317, src/compute/dispatch.c).  Every wrapper initialises the
+ * compute layer on first use, returns AX_ERR_BACKEND when no backend is active and
+ * AX_ERR_NOT_IMPLEMENTED when the active backend leaves the slot NULL, and bumps
+ * out->storage->generation on success. */
+#ifndef AX_COMPUTE_H
+#define AX_COMPUTE_H
+
+#include "types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ax_backend_ops ax_backend_ops_t;   /* layout: axiom/internal/backend_ops.h */
+typedef struct ax_tensor ax_tensor_t;
+
+typedef struct {            /* conv_gemm slot argument; unused here, kept for the vtable's types */
+    const float *input;
+    int64_t C_in, H, W;
+    int kh, kw, sh, sw, ph, pw;
+    int64_t out_h, out_w;
+} ax_conv_params_t;
+
+typedef enum {
+    AX_BACKEND_CPU_NAIVE = 0,   /* ids kept for numeric compatibility; this build registers */
+    AX_BACKEND_CPU_SIMD,        /* no CPU backend: there is no CPU compute path             */
+    AX_BACKEND_CPU_BLAS,
+    AX_BACKEND_CUDA,
+    AX_BACKEND_HIP,             /* ax_hip_ops */
+    AX_BACKEND_COUNT
+} ax_backend_id_t;
+
+/* fused-epilogue selector of the appended gemm_bias_act slot */
+typedef enum { AX_ACT_NONE = 0, AX_ACT_RELU = 1, AX_ACT_GELU = 2 } ax_activation_t;
+
+ax_status_t     ax_compute_init(void);        /* registers ax_hip_ops, fires its init hook, selects it */
+void            ax_compute_shutdown(void);
+ax_status_t     ax_compute_set_backend(ax_backend_id_t id);
+ax_backend_id_t ax_compute_get_backend(void);
+const char     *ax_compute_backend_name(void);
+ax_status_t     ax_compute_register_backend(ax_backend_id_t id, const ax_backend_ops_t *ops);
+const ax_backend_ops_t *ax_compute_get_ops(void);
+const ax_backend_ops_t *ax_backend_for_device(ax_device_t device);
+
+ax_status_t ax_compute_gemm(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_gemm_nt(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_gemm_tn(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_gemm_relu(const ax_tensor_t *a, const ax_tensor_t *b, const ax_tensor_t *bias, ax_tensor_t *out);
+ax_status_t ax_compute_gemm_ex(const ax_tensor_t *a, const ax_tensor_t *b, float alpha, float beta, ax_tensor_t *out);
+ax_status_t ax_compute_bias_add(const ax_tensor_t *in, const ax_tensor_t *bias, int axis, ax_tensor_t *out);
+ax_status_t ax_compute_relu(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_fill(ax_tensor_t *t, double value);
+ax_status_t ax_compute_copy(const ax_tensor_t *src, ax_tensor_t *dst);
+int ax_compute_has_gemm_relu(void);
+int ax_compute_has_gemm_nt(void);
+int ax_compute_has_gemm_tn(void);
+int ax_compute_has_gemm_ex(void);
+int ax_compute_has_bias_add(void);
+
+/* Not in the reference: its vtable has a gelu_op slot but no wrapper reaches it
+ * (src/core/activations.c:267 always runs on the host pointer), and it has no fused
+ * bias+activation GEMM beyond gemm_relu. */
+ax_status_t ax_compute_gelu(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_gemm_bias_act(const ax_tensor_t *a, const ax_tensor_t *b, const ax_tensor_t *bias,
+                                     ax_activation_t act, ax_tensor_t *out);
+int ax_compute_has_gemm_bias_act(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

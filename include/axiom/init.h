@@ -1,0 +1,15 @@
+/* axiom/init.h — weight initialisers used by Dense (include/axiom/init.h, src/core/init.c:84-94).
+ * Values are drawn on the host in element order and copied to the tensor's device. */
+#ifndef AX_INIT_H
+#define AX_INIT_H
+#include "tensor.h"
+#ifdef __cplusplus
+extern "C" {
+#endif
+void ax_init_kaiming_uniform(ax_tensor_t *t, int64_t fan_in);     /* U(+-sqrt(6/fan_in)) */
+void ax_init_normal(ax_tensor_t *t, float mean, float std);
+void ax_init_uniform(ax_tensor_t *t, float low, float high);
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,125 @@
+/* axiom/internal/backend_ops.h — the backend vtable: the drop-in boundary.
+ *
+ * Slot order, names and signatures reproduce struct ax_backend_ops of Axiom 0.10.0
+ * (include/axiom/internal/backend_ops.h:30-298) up to and including memcpy_d2d, so that a
+ * pointer to ax_hip_ops can be handed to the reference's ax_compute_register_backend()
+ * (src/compute/dispatch.c:302-315) unchanged.  tests/golden/abi_layout.json records the
+ * reference's offsets and tests/test_host_core.py compares them with this header.
+ * Any slot may be NULL; dispatch answers AX_ERR_NOT_IMPLEMENTED for those.
+ *
+ * One slot is appended after the reference's last member (gemm_bias_act); the reference
+ * never reads that far, this repository's dispatch layer does. */
+#ifndef AX_INTERNAL_BACKEND_OPS_H
+#define AX_INTERNAL_BACKEND_OPS_H
+
+#include "axiom/compute.h"
+#include "axiom/tensor.h"
+#include "axiom/types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef const ax_tensor_t *ax_tin_t;     /* borrowed input  */
+typedef ax_tensor_t *ax_tout_t;          /* borrowed output, pre-allocated by the caller */
+
+struct ax_backend_ops {
+    const char *name;
+
+    /* broadcasting binary, unary and scalar elementwise slots — not provided by ax_hip_ops */
+    ax_status_t (*add)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
+    ax_status_t (*sub)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
+    ax_status_t (*mul)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
+    ax_status_t (*div_op)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
+    ax_status_t (*neg)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*abs_op)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*exp_op)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*log_op)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*sqrt_op)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*square)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*add_scalar)(ax_tin_t in, double scalar, ax_tout_t out);
+    ax_status_t (*mul_scalar)(ax_tin_t in, double scalar, ax_tout_t out);
+
+    /* GEMM family: out fully overwritten, a/b/out 2-D fp32 */
+    ax_status_t (*gemm)(ax_tin_t a, ax_tin_t b, ax_tout_t out);        /* [M,K] x [K,N]   */
+    ax_status_t (*gemm_nt)(ax_tin_t a, ax_tin_t b, ax_tout_t out);     /* [M,K] x [N,K]^T */
+    ax_status_t (*gemm_tn)(ax_tin_t a, ax_tin_t b, ax_tout_t out);     /* [K,M]^T x [K,N] */
+
+    /* fused attention-training slots — out of scope, NULL in ax_hip_ops */
+    ax_status_t (*dwqkv_split_acc)(ax_tin_t x_flat, ax_tin_t dQKV, ax_tout_t dWq, ax_tout_t dWk,
+                                   ax_tout_t dWv);
+    ax_status_t (*dwqkv_split_acc_hm)(ax_tin_t x_flat, ax_tin_t dQh, ax_tin_t dKh, ax_tin_t dVh,
+                                      int64_t B, int64_t S, int64_t H, int64_t dk, ax_tout_t dWq,
+                                      ax_tout_t dWk, ax_tout_t dWv);
+    ax_status_t (*qkv_head_gemm)(ax_tin_t X, ax_tin_t Wqkv, ax_tin_t bqkv, int64_t B, int64_t S,
+                                 int64_t H, int64_t dk, ax_tout_t Qh, ax_tout_t Kh, ax_tout_t Vh);
+    ax_status_t (*dattn_head_gemm_nt)(ax_tin_t dout, ax_tin_t Wo, int64_t B, int64_t S, int64_t H,
+                                      int64_t dk, ax_tout_t dO_head);
+    ax_status_t (*mha_output_proj_fused)(ax_tin_t attn_flat, ax_tin_t Wo, ax_tin_t bo, ax_tin_t dout,
+                                         ax_tout_t y, ax_tout_t dattn, ax_tout_t dWo_acc,
+                                         ax_tout_t dbo_acc);
+
+    ax_status_t (*gemm_relu)(ax_tin_t a, ax_tin_t b, ax_tin_t bias /* [N] or NULL */, ax_tout_t out);
+    ax_status_t (*gemm_ex)(ax_tin_t a, ax_tin_t b, float alpha, float beta, ax_tout_t out);
+
+    ax_status_t (*add_relu)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
+    ax_status_t (*axpy)(ax_tin_t x, float alpha, ax_tout_t y);
+    ax_status_t (*softmax_rowwise)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*bias_add)(ax_tin_t in, ax_tin_t bias, int axis, ax_tout_t out);
+    ax_status_t (*conv_gemm)(ax_tin_t weight, const ax_conv_params_t *params, ax_tout_t out);
+    ax_status_t (*conv_gemm_nt_dw)(ax_tin_t grad_out, const ax_conv_params_t *params, ax_tout_t dw);
+
+    ax_status_t (*sum)(ax_tin_t in, int axis, ax_tout_t out);
+    ax_status_t (*mean)(ax_tin_t in, int axis, ax_tout_t out);
+    ax_status_t (*max_op)(ax_tin_t in, int axis, ax_tout_t out);
+    ax_status_t (*min_op)(ax_tin_t in, int axis, ax_tout_t out);
+    ax_status_t (*argmax)(ax_tin_t in, int axis, ax_tout_t out);
+    ax_status_t (*equal)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
+    ax_status_t (*greater)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
+
+    ax_status_t (*fill)(ax_tout_t t, double value);
+    ax_status_t (*copy)(ax_tin_t src, ax_tout_t dst);
+
+    ax_status_t (*relu)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*sigmoid)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*tanh_op)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*leaky_relu)(ax_tin_t in, float alpha, ax_tout_t out);
+    ax_status_t (*elu_op)(ax_tin_t in, float alpha, ax_tout_t out);
+    ax_status_t (*gelu_op)(ax_tin_t in, ax_tout_t out);
+    ax_status_t (*swish_op)(ax_tin_t in, ax_tout_t out);
+
+    ax_status_t (*adam_update)(ax_tout_t weight, ax_tout_t grad, ax_tout_t m, ax_tout_t v, float lr,
+                               float beta1, float beta2, float eps, float weight_decay, float bc1,
+                               float bc2, bool decoupled);
+    ax_status_t (*sgd_update)(ax_tout_t weight, ax_tout_t grad, ax_tout_t momentum_buf, float lr,
+                              float momentum, float weight_decay, bool nesterov);
+
+    /* device-owner hooks: a backend that owns a non-CPU device fills these */
+    ax_device_t device;                         /* AX_DEVICE_COUNT: owns none */
+    ax_status_t (*init)(void);
+    void (*shutdown)(void);
+    void (*synchronize)(void);
+    int (*device_count)(void);
+    void *(*storage_alloc)(size_t size_bytes);  /* zero-filled, or NULL */
+    void (*storage_free)(void *ptr);
+    ax_status_t (*memcpy_h2d)(void *dst, const void *src, size_t bytes);
+    ax_status_t (*memcpy_d2h)(void *dst, const void *src, size_t bytes);
+    ax_status_t (*memcpy_d2d)(void *dst, const void *src, size_t bytes);
+
+    /* ---- appended by this repository (absent from the reference's struct) ---- */
+    /* out = act(a x b + bias[n]); bias may be NULL; act is an ax_activation_t */
+    ax_status_t (*gemm_bias_act)(ax_tin_t a, ax_tin_t b, ax_tin_t bias, int act, ax_tout_t out);
+};
+
+/* The MI355X backend.  `device` is AX_DEVICE_HIP. */
+extern const ax_backend_ops_t ax_hip_ops;
+
+/* The same table with `device` set to `as_device`, for hosts whose device enum has no HIP
+ * entry (the unmodified reference: pass its AX_DEVICE_CUDA = 1).  Returns a pointer to
+ * static storage, rewritten by each call. */
+const ax_backend_ops_t *ax_hip_ops_for_device(ax_device_t as_device);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

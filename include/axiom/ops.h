@@ -1,0 +1,23 @@
+/* axiom/ops.h — tensor-level matmul family and the two activations of the path
+ * (include/axiom/ops.h, src/core/ops.c:285-440; activations.c).  Each returns a new tensor on
+ * the inputs' device (NULL + ax_err on failure).  Inference only: no grad_fn is attached.
+ *
+ * ax_matmul_bias adds bias[n] to column n.  (The reference passes axis 0 to its bias_add for
+ * an [M,N] + [N] add, src/core/ops.c:357, which its backends reject or apply down rows; the
+ * intended column-wise add is implemented here, as in the reference's own opt_gemm_relu.) */
+#ifndef AX_OPS_H
+#define AX_OPS_H
+#include "tensor.h"
+#ifdef __cplusplus
+extern "C" {
+#endif
+ax_tensor_t *ax_matmul(ax_tensor_t *a, ax_tensor_t *b);                              /* [M,K]x[K,N] */
+ax_tensor_t *ax_matmul_bias(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bias);     /* a may be [B,S,K] */
+ax_tensor_t *ax_matmul_bias_relu(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bias);
+ax_tensor_t *ax_matmul_bias_gelu(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bias); /* not in the reference */
+ax_tensor_t *ax_relu(ax_tensor_t *a);
+ax_tensor_t *ax_gelu(ax_tensor_t *a);                                                /* tanh form */
+#ifdef __cplusplus
+}
+#endif
+#endif

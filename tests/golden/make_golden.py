@@ -113,3 +113,15 @@ G["gelu_y"] = r.gelu(xg.reshape(1, -1)).reshape(-1)
 
 np.savez_compressed(os.path.join(HERE, "golden.npz"), **G)
 print("wrote", len(G), "arrays,", os.path.getsize(os.path.join(HERE, "golden.npz")), "bytes")
+
+# ---- struct layout of the reference's boundary types -----------------------------------
+import subprocess  # noqa: E402
+import tempfile  # noqa: E402
+
+with tempfile.TemporaryDirectory() as tmp:
+    exe = os.path.join(tmp, "abi_probe")
+    subprocess.check_call(["gcc", "-std=gnu11", "-I/root/reference/include",
+                           os.path.join(HERE, "abi_probe.c"), "-o", exe])
+    layout = subprocess.check_output([exe]).decode()
+open(os.path.join(HERE, "abi_layout.json"), "w").write(layout)
+print("wrote abi_layout.json")

@@ -1,0 +1,231 @@
+"""GPU tests of the host side: the Axiom C API of libaxiom_hip.so driving ax_hip_ops, and the
+backend object dropped into the unmodified reference library through its own
+ax_compute_register_backend()."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-4     # fp32: max |gpu - cpu| / max |cpu|
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def ax():
+    from axiom_amd.axiom import Axiom
+    a = Axiom()
+    assert a.L.ax_init() == 0, a.err()
+    assert a.L.ax_compute_backend_name() == b"hip"
+    a.L.ax_set_default_device(2)
+    yield a
+    a.L.ax_set_default_device(0)
+
+
+def close(got, ref, rel=REL):
+    return np.abs(got - ref).max() <= rel * max(np.abs(ref).max(), 1e-30)
+
+
+def test_dispatch_wrappers(ax, oracle):
+    L = ax.L
+    assert L.ax_device_count(2) >= 1 and L.ax_device_is_available(2) == 1
+    assert all(f() == 1 for f in (L.ax_compute_has_gemm_relu, L.ax_compute_has_gemm_nt, L.ax_compute_has_gemm_tn,
+                                  L.ax_compute_has_gemm_ex, L.ax_compute_has_bias_add, L.ax_compute_has_gemm_bias_act))
+    oracle.seed(5)
+    M, K, N = 70, 130, 90
+    a, b = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1)
+    bias = oracle.normal((N,), 0, 0.5)
+    ref = oracle.gemm_opt(a, b)
+    ta, tb, tbias = ax.from_numpy(a), ax.from_numpy(b), ax.from_numpy(bias)
+    out = ax.empty((M, N))
+    gen0 = out.contents.storage.contents.generation
+    assert L.ax_compute_gemm(ta, tb, out) == 0
+    assert out.contents.storage.contents.generation == gen0 + 1          # dispatch.c:347-350
+    assert close(ax.to_numpy(out), ref)
+    tbt = ax.from_numpy(np.ascontiguousarray(b.T))
+    assert L.ax_compute_gemm_nt(ta, tbt, out) == 0 and close(ax.to_numpy(out), ref)
+    tat = ax.from_numpy(np.ascontiguousarray(a.T))
+    assert L.ax_compute_gemm_tn(tat, tb, out) == 0 and close(ax.to_numpy(out), ref)
+    assert L.ax_compute_gemm_relu(ta, tb, tbias, out) == 0
+    assert close(ax.to_numpy(out), oracle.dense(a, b, bias, 1))
+    assert L.ax_compute_gemm_relu(ta, tb, None, out) == 0
+    assert close(ax.to_numpy(out), oracle.dense(a, b, None, 1))
+    assert L.ax_compute_gemm_bias_act(ta, tb, tbias, 2, out) == 0
+    assert np.abs(ax.to_numpy(out) - oracle.dense(a, b, bias, 2)).max() <= 1e-5 + REL * np.abs(ref).max()
+    # gemm_ex: alpha/beta, beta = 1 accumulates (cpu_opt.c:7442-7497)
+    c0 = oracle.uniform((M, N), -1, 1)
+    tc = ax.from_numpy(c0)
+    assert L.ax_compute_gemm_ex(ta, tb, 1.0, 1.0, tc) == 0 and close(ax.to_numpy(tc), ref + c0)
+    assert L.ax_compute_gemm_ex(ta, tb, 0.5, 0.0, tc) == 0 and close(ax.to_numpy(tc), 0.5 * ref)
+    # bias_add along either axis of [M,N] (cpu_opt.c:7148-7194)
+    lin = ax.from_numpy(ref)
+    assert L.ax_compute_bias_add(lin, tbias, 1, out) == 0
+    assert np.array_equal(ax.to_numpy(out), ref + bias[None, :])
+    rb = oracle.normal((M,), 0, 1)
+    trb = ax.from_numpy(rb)
+    assert L.ax_compute_bias_add(lin, trb, 0, out) == 0
+    assert np.array_equal(ax.to_numpy(out), ref + rb[:, None])
+    assert L.ax_compute_bias_add(lin, tbias, 0, out) == 3          # [N] bias against axis 0 of [M,N]
+    assert L.ax_compute_bias_add(lin, tbias, 2, out) == 5          # AX_ERR_INVALID_AXIS
+    assert L.ax_compute_relu(lin, out) == 0 and np.array_equal(ax.to_numpy(out), np.maximum(ref, 0))
+    assert L.ax_compute_gelu(lin, out) == 0 and np.abs(ax.to_numpy(out) - oracle.gelu(ref)).max() <= 2e-6 * max(1, np.abs(ref).max())
+    assert L.ax_compute_fill(out, 1.5) == 0 and (ax.to_numpy(out) == 1.5).all()
+    assert L.ax_compute_copy(lin, out) == 0 and np.array_equal(ax.to_numpy(out), ref)
+    # errors follow the reference backend's convention (cuda/ops_gemm.cu:16-23)
+    bad = ax.empty((M, N + 1))
+    assert L.ax_compute_gemm(ta, tb, bad) == 3
+    t3 = ax.empty((2, 3, 4))
+    assert L.ax_compute_gemm(t3, tb, out) == 3
+    host = ax.from_numpy(a, device=0)
+    assert L.ax_compute_gemm(host, tb, out) == 9 and b"hip device" in L.ax_err_last_message()
+    ax.free(ta, tb, tbias, out, tbt, tat, tc, lin, trb, bad, t3, host)
+
+
+def test_reference_gpu_vs_cpu_template(ax, oracle):
+    """tests/test_cuda.c:213-244: 64x128 . 128x32, rand(-0.1,0.1), every element within 1e-3."""
+    L = ax.L
+    L.ax_set_seed(7)
+    sa, _ = ax.shape_arg((64, 128))
+    sb, _ = ax.shape_arg((128, 32))
+    a, b = L.ax_tensor_rand(sa, 2, -0.1, 0.1), L.ax_tensor_rand(sb, 2, -0.1, 0.1)
+    assert a.contents.storage.contents.device == 2
+    c = L.ax_matmul(a, b)
+    got = ax.to_numpy(c)
+    oracle.seed(7)
+    an, bn = oracle.uniform((64, 128), -0.1, 0.1), oracle.uniform((128, 32), -0.1, 0.1)
+    assert np.array_equal(ax.to_numpy(a), an) and np.array_equal(ax.to_numpy(b), bn)
+    assert np.abs(got - oracle.gemm_opt(an, bn)).max() <= 1e-3
+    assert close(got, oracle.gemm_opt(an, bn))
+    cpu = L.ax_tensor_to_cpu(c)
+    assert cpu.contents.storage.contents.device == 0 and np.array_equal(ax.to_numpy(cpu), got)
+    ax.free(a, b, c, cpu)
+
+
+def test_matmul_bias_adds_to_columns(ax, oracle):
+    L = ax.L
+    oracle.seed(9)
+    x, w, bias = oracle.normal((6, 5, 48)), oracle.normal((48, 40), 0, 0.1), oracle.normal((40,), 0, 1)
+    tx, tw, tb = ax.from_numpy(x), ax.from_numpy(w), ax.from_numpy(bias)
+    y = L.ax_matmul_bias(tx, tw, tb)                       # [B,S,K] input is flattened and viewed back
+    assert [y.contents.shape[i] for i in range(y.contents.ndim)] == [6, 5, 40]
+    ref = oracle.dense(x.reshape(30, 48), w, bias, 0).reshape(6, 5, 40)
+    assert close(ax.to_numpy(y), ref)
+    tx2 = ax.from_numpy(x.reshape(30, 48))
+    y2 = L.ax_matmul_bias_relu(tx2, tw, tb)
+    assert close(ax.to_numpy(y2), np.maximum(ref.reshape(30, 40), 0))
+    assert not L.ax_matmul_bias_relu(tx, tw, tb)           # 3-D input: rejected like the reference (ops.c:405)
+    g = L.ax_gelu(y2)
+    assert np.abs(ax.to_numpy(g) - oracle.gelu(ax.to_numpy(y2))).max() <= 2e-6
+    ax.free(tx, tw, tb, y, tx2, y2, g)
+
+
+@pytest.mark.parametrize("M", [1, 8, 64])
+def test_config1_sequential_mlp(ax, oracle, M):
+    """Sequential(Dense 784-4096, ReLU, Dense 4096-4096, ReLU, Dense 4096-10) built after
+    ax_set_seed: the weights equal the oracle's draw, the output equals the oracle's MLP."""
+    L = ax.L
+    L.ax_set_seed(1234)
+    seq = L.ax_sequential_create()
+    for (i, o, relu) in ((784, 4096, True), (4096, 4096, True), (4096, 10, False)):
+        assert L.ax_sequential_add(seq, L.ax_dense_create(i, o, True))
+        if relu:
+            assert L.ax_sequential_add(seq, L.ax_relu_layer_create())
+    oracle.seed(1234)
+    w1, w2, w3 = oracle.kaiming((784, 4096), 784), oracle.kaiming((4096, 4096), 4096), oracle.kaiming((4096, 10), 4096)
+    from axiom_amd.axiom import TP
+    params = (TP * 8)()
+    assert L.ax_layer_get_params(seq, params, 8) == 6
+    assert np.array_equal(ax.to_numpy(params[2]), w2) and params[2].contents.storage.contents.device == 2
+    x = oracle.uniform((M, 784), 0, 1)
+    tx = ax.from_numpy(x)
+    y = L.ax_layer_forward(seq, tx)
+    assert y, ax.err()
+    ref = oracle.dense(oracle.dense(oracle.dense(x, w1, None, 1), w2, None, 1), w3, None, 0)
+    assert close(ax.to_numpy(y), ref)
+    ax.free(tx, y)
+    L.ax_layer_destroy(seq)
+
+
+def test_config3_ffn_through_layers(ax, oracle):
+    L = ax.L
+    L.ax_set_seed(3)
+    seq = L.ax_sequential_create()
+    d1, d2 = L.ax_dense_create(1024, 4096, True), L.ax_dense_create(4096, 1024, True)
+    for layer in (d1, L.ax_gelu_layer_create(), d2):
+        L.ax_sequential_add(seq, layer)
+    from axiom_amd.axiom import TP
+    params = (TP * 4)()
+    L.ax_layer_get_params(seq, params, 4)
+    oracle.seed(33)
+    w1, b1 = oracle.normal((1024, 4096), 0, 0.02), oracle.normal((4096,), 0, 0.02)
+    w2, b2 = oracle.normal((4096, 1024), 0, 0.02), oracle.normal((1024,), 0, 0.02)
+    hooks = L.ax_backend_for_device(2)
+    assert hooks
+    for t, v in zip(params, (w1, b1, w2, b2)):            # overwrite the parameters in place
+        src = ax.from_numpy(v)
+        assert L.ax_compute_copy(src, t) == 0
+        ax.free(src)
+    x = oracle.normal((4, 512, 1024))
+    tx = ax.from_numpy(x)
+    y = L.ax_layer_forward(seq, tx)
+    assert [y.contents.shape[i] for i in range(3)] == [4, 512, 1024]
+    h = oracle.dense(x.reshape(2048, 1024), w1, b1, 2)
+    ref = oracle.dense(h, w2, b2, 0).reshape(4, 512, 1024)
+    assert close(ax.to_numpy(y), ref)
+    ax.free(tx, y)
+    L.ax_layer_destroy(seq)
+
+
+def test_quantized_entry_points(ax, oracle):
+    L = ax.L
+    oracle.seed(13)
+    M, N, K = 8, 768, 768
+    w, a = oracle.uniform((N, K), -1, 1), oracle.uniform((M, K), -1, 1)
+    qw = L.ax_qweight_create_from_fp32(w, N, K)
+    q, s = oracle.quantize_rows(w)
+    ref = oracle.qgemm_w8a32(a, q, s)
+    out = np.zeros((M, N), np.float32)
+    assert L.ax_qgemm_w8a32(a, qw, out, M) == 0           # reference signature: host pointers
+    assert close(out, ref)
+    dq = L.ax_qweight_to_device(qw, 2)
+    ta, tout = ax.from_numpy(a), ax.empty((M, N))
+    assert L.ax_qgemm_w8a32_dev(ta.contents.storage.contents.data, dq, tout.contents.storage.contents.data, M) == 0
+    assert close(ax.to_numpy(tout), ref)
+    # W8A8 on device-resident operands
+    from axiom_amd import AxHip
+    hip = AxHip()
+    x8 = oracle.int8((M, K))
+    bias = oracle.normal((N,), 0, 0.02)
+    dx, db = hip.array(x8), hip.array(bias)
+    dout, dacc = hip.empty((M, N)), hip.empty((M, N), np.int32)
+    assert L.ax_qgemm_w8a8_dev(dx.ptr, 0.02, dq, db.ptr, 1, dout.ptr, dacc.ptr, M) == 0
+    acc = oracle.qgemm_w8a8_acc(x8, q)
+    assert np.array_equal(dacc.numpy(), acc)
+    assert np.array_equal(dout.numpy(), oracle.w8a8_epilogue(acc, np.float32(0.02), s, bias, 1))
+    assert L.ax_qgemm_w8a8_dev(None, 0.02, dq, None, 0, dout.ptr, None, M) == 1
+    L.ax_qweight_device_destroy(dq, 2)
+    L.ax_qweight_destroy(qw)
+    ax.free(ta, tout)
+
+
+def test_backend_dropped_into_the_unmodified_reference(oracle):
+    """Load the reference library itself, register ax_hip_ops through the reference's own
+    ax_compute_register_backend (src/compute/dispatch.c:302-315) in its GPU slot, and run the
+    reference's tensors, ops and Sequential on the MI355X."""
+    import subprocess
+    import sys
+    ref_so = os.path.join(ROOT, "oracle", "_ref", "libaxref.so")
+    if not os.path.exists(ref_so):
+        pytest.skip("oracle/_ref/libaxref.so was not built (needs the reference tree)")
+    # a fresh process: the reference's ax_* symbols must be the first ones in scope
+    r = subprocess.run([sys.executable, "-u", os.path.join(ROOT, "tests", "dropin_check.py")],
+                       capture_output=True, text=True, timeout=170)
+    say(r.stdout[-3000:], r.stderr[-3000:])
+    assert r.returncode == 0
+    assert "DROPIN OK" in r.stdout

@@ -1,0 +1,170 @@
+"""The C host core (libaxiom_hip.so) without a GPU: struct layout against the reference,
+RNG / initialisers / quantizer against the oracle and the golden vectors, tensor plumbing on
+the CPU device, and the error convention.  No compute runs here."""
+import ctypes as C
+import json
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from fills import xorshift32_unit
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def ax():
+    from axiom_amd.axiom import Axiom
+    return Axiom()
+
+
+def test_boundary_structs_match_the_reference_layout(tmp_path):
+    """Offsets of ax_tensor_t, ax_storage_t, ax_qweight_t, the layer structs and every vtable slot
+    up to memcpy_d2d equal those measured from the reference's own headers."""
+    exe = str(tmp_path / "abi_probe")
+    subprocess.check_call(["gcc", "-std=gnu11", "-I" + os.path.join(ROOT, "include"),
+                           os.path.join(ROOT, "tests", "golden", "abi_probe.c"), "-o", exe])
+    mine = json.loads(subprocess.check_output([exe]).decode())
+    ref = json.load(open(os.path.join(ROOT, "tests", "golden", "abi_layout.json")))
+    assert len(ref) > 110
+    assert {k: v for k, v in mine.items() if ref.get(k) != v} == {}
+    assert mine == ref
+
+
+def test_python_struct_mirrors_match_too():
+    from axiom_amd import axiom as m
+    ref = json.load(open(os.path.join(ROOT, "tests", "golden", "abi_layout.json")))
+    assert C.sizeof(m.Tensor) == ref["sizeof(ax_tensor_t)"] and C.sizeof(m.Storage) == ref["sizeof(ax_storage_t)"]
+    assert m.Tensor.offset.offset == ref["ax_tensor_t.offset"] and m.Tensor.layout.offset == ref["ax_tensor_t.layout"]
+    assert m.Storage.generation.offset == ref["ax_storage_t.generation"]
+    assert C.sizeof(m.QWeight) == ref["sizeof(ax_qweight_t)"]
+
+
+def test_exports_every_declared_function(ax):
+    from axiom_amd.axiom import DATA_SYMBOLS, SIGNATURES
+    declared = set()
+    inc = os.path.join(ROOT, "include", "axiom")
+    for dirpath, _, files in os.walk(inc):
+        for f in files:
+            text = re.sub(r"/\*.*?\*/", "", open(os.path.join(dirpath, f)).read(), flags=re.S)
+            text = re.sub(r"static inline[^{]*\{.*?\n\}", "", text, flags=re.S)
+            declared |= set(re.findall(r"\b(ax_[a-z0-9_]+)\s*\(", text))
+    declared = {d for d in declared if not d.endswith("_t")} - {"ax_dtype_size"}   # types; static inline
+    for name in sorted(declared):
+        assert hasattr(ax.L, name), f"{name} declared under include/axiom but not exported"
+    assert declared - {"ax_err_set"} == set(SIGNATURES), (declared ^ set(SIGNATURES))   # variadic: not bound
+    for name in DATA_SYMBOLS:
+        C.c_void_p.in_dll(ax.L, name)
+    plugin = C.CDLL(os.path.join(ROOT, "axiom_amd", "lib", "libax_hip_plugin.so"))
+    C.c_void_p.in_dll(plugin, "ax_hip_ops")
+    assert hasattr(plugin, "ax_hip_ops_for_device")
+
+
+def test_rng_and_initialisers_match_oracle_and_golden(ax, oracle, golden):
+    L = ax.L
+    for seed in (0, 42):
+        L.ax_rng_seed(seed)
+        assert [L.ax_rng_uint64() for _ in range(8)] == list(golden[f"rng_u64_seed{seed}"])
+        L.ax_rng_seed(seed)
+        got = np.array([L.ax_rng_uniform(-1.0, 1.0) for _ in range(8)], np.float32)
+        assert np.array_equal(got, golden[f"rng_uniform_seed{seed}"])
+        L.ax_rng_seed(seed)
+        assert [L.ax_rng_bounded(255) for _ in range(32)] == list(golden[f"rng_bounded255_seed{seed}"])
+    L.ax_rng_seed(0)
+    assert np.array_equal(np.array([L.ax_rng_normal() for _ in range(8)], np.float32), golden["rng_normal_seed0"])
+    # ax_set_seed + ax_tensor_rand: the 1024^3 config's inputs (golden probe from the reference)
+    L.ax_set_default_device(0)
+    L.ax_set_seed(0)
+    sh, nd = ax.shape_arg((1024, 1024))
+    a = L.ax_tensor_rand(sh, nd, -1.0, 1.0)
+    b = L.ax_tensor_rand(sh, nd, -1.0, 1.0)
+    an, bn = ax.to_numpy(a), ax.to_numpy(b)
+    assert an[0, 0] == golden["gemm_1024_probe"][0] and bn[0, 0] == golden["gemm_1024_probe"][1]
+    oracle.seed(0)
+    assert np.array_equal(an, oracle.uniform((1024, 1024), -1, 1))
+    ax.free(a, b)
+    # Dense: weight [in,out] Kaiming-uniform drawn at creation, bias zeros
+    L.ax_set_seed(1234)
+    d = L.ax_dense_create(784, 64, True)
+    params = (C.POINTER(type(a.contents)) * 4)()
+    assert L.ax_layer_get_params(d, params, 4) == 2
+    w, bias = ax.to_numpy(params[0]), ax.to_numpy(params[1])
+    oracle.seed(1234)
+    assert np.array_equal(w, oracle.kaiming((784, 64), 784)) and not bias.any() and bias.shape == (64,)
+    L.ax_layer_destroy(d)
+
+
+def test_quantizer_matches_reference_vectors(ax, oracle, golden):
+    L = ax.L
+    for key in ("hand", "ties"):
+        w = golden[f"quant_{key}_w"]
+        qw = L.ax_qweight_create_from_fp32(w, *w.shape)
+        q = np.ctypeslib.as_array(C.cast(qw.contents.data, C.POINTER(C.c_int8)), w.shape).copy()
+        s = np.ctypeslib.as_array(C.cast(qw.contents.scales, C.POINTER(C.c_float)), (w.shape[0],)).copy()
+        assert np.array_equal(q, golden[f"quant_{key}_q"]) and np.array_equal(s, golden[f"quant_{key}_s"])
+        L.ax_qweight_destroy(qw)
+    w = xorshift32_unit(64 * 1024, 42).reshape(64, 1024)
+    qw = L.ax_qweight_create_from_fp32(w, 64, 1024)
+    q = np.ctypeslib.as_array(C.cast(qw.contents.data, C.POINTER(C.c_int8)), w.shape).copy()
+    assert np.array_equal(q, golden["quant_64x1024_q"])
+    deq = np.empty_like(w)
+    L.ax_qweight_dequantize(qw, deq)
+    oq, os_ = oracle.quantize_rows(w)
+    assert np.array_equal(deq, oracle.dequantize_rows(oq, os_))
+    L.ax_qweight_destroy(qw)
+    assert not L.ax_qweight_create_from_fp32(w, 0, 5)
+
+
+def test_tensor_plumbing_on_cpu_device(ax):
+    L = ax.L
+    x = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    t = ax.from_numpy(x, device=0)
+    assert L.ax_tensor_numel(t) == 24 and L.ax_tensor_is_contiguous(t)
+    assert [t.contents.strides[i] for i in range(3)] == [12, 4, 1]
+    sh, nd = ax.shape_arg((6, 4))
+    v = L.ax_tensor_reshape(t, sh, nd)
+    assert t.contents.storage.contents.refcount == 2
+    assert np.array_equal(ax.to_numpy(v), x.reshape(6, 4))
+    sh_bad, _ = ax.shape_arg((5, 5))
+    assert not L.ax_tensor_reshape(t, sh_bad, 2) and L.ax_err_last_status() == 3
+    ax.free(v)
+    assert t.contents.storage.contents.refcount == 1
+    z = L.ax_tensor_zeros(sh, nd, 0)
+    assert not ax.to_numpy(z).any() and z.contents.storage.contents.generation == 1
+    c = L.ax_tensor_to_cpu(t)
+    assert np.array_equal(ax.to_numpy(c), x)
+    ax.free(t, z, c)
+
+
+def test_error_convention_and_no_cpu_compute(ax):
+    L = ax.L
+    L.ax_err_clear()
+    assert L.ax_err_last_status() == 0 and L.ax_err_last_message() == b""
+    assert L.ax_status_name(3) == b"shape mismatch" and L.ax_status_name(99) == b"unknown error"
+    assert not L.ax_matmul(None, None) and L.ax_err_last_status() == 1           # AX_ERR_NULL_ARG
+    a, b = ax.from_numpy(np.ones((2, 3)), 0), ax.from_numpy(np.ones((4, 2)), 0)
+    assert not L.ax_matmul(a, b) and L.ax_err_last_status() == 3
+    assert b"inner dims" in L.ax_err_last_message()
+    assert L.ax_compute_set_backend(0) == 9                                      # no CPU backend exists
+    assert L.ax_compute_register_backend(99, None) == 9 and L.ax_compute_register_backend(4, None) == 1
+    assert L.ax_device_count(0) == 1
+    if L.ax_device_count(2) == 0:
+        # no GPU: nothing is active, every wrapper refuses instead of computing on the host
+        b2 = ax.from_numpy(np.ones((3, 2)), 0)
+        out = ax.from_numpy(np.zeros((2, 2)), 0)
+        assert L.ax_compute_gemm(a, b2, out) == 9
+        assert not L.ax_matmul(a, b2)
+        assert not ax.to_numpy(out).any()
+        w = np.ones((4, 8), np.float32)
+        qw = L.ax_qweight_create_from_fp32(w, 4, 8)
+        assert L.ax_qgemm_w8a32(np.ones((1, 8), np.float32), qw, np.zeros((1, 4), np.float32), 1) == 9
+        L.ax_qweight_destroy(qw)
+        sh, nd = ax.shape_arg((4,))
+        L.ax_set_default_device(2)
+        assert not L.ax_tensor_create(sh, nd, 0)
+        L.ax_set_default_device(0)
+        ax.free(b2, out)
+    ax.free(a, b)
