@@ -3,8 +3,11 @@
 //   acc[m,n] = sum_k x[m,k] * w[n,k]          x: [M,K] int8, w: [N,K] int8 (both K-contiguous)
 //   out[m,n] = act((float)acc * (x_scale*w_scale[n]) + bias[n])
 //
-// One workgroup owns a BM x BN tile of the output and walks K in slabs of 128 bytes.
-// Slabs are fetched with 16-byte global loads (8 consecutive lanes cover one 128-byte row
+// Two kernels.  k_qgemm_w8a8_256 (further down) serves large aligned shapes; the template
+// below serves everything else, including ragged and unaligned shapes through its guarded form.
+//
+// Template kernel: one workgroup owns a BM x BN tile of the output and walks K in slabs of 128
+// bytes.  Slabs are fetched with 16-byte global loads (8 consecutive lanes cover one 128-byte row
 // segment), staged through registers into a double-buffered LDS tile, and consumed by
 // v_mfma_i32_32x32x32_i8: lane l supplies row (l & 31), bytes [16*(l>>5), +16) of each
 // 32-byte k-step.  Because A and B fragments use the same byte placement the integer dot
@@ -184,6 +187,237 @@ int launch(const char *name, const int8_t *x, float x_scale, const int8_t *w,
     return check_launch(name);
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Large aligned shapes (M, N multiples of 256, K a multiple of 128): 256x256 tile, 8 waves as
+// 2 (M) x 4 (N), wave tile 128x64, K slabs of 128 bytes, two LDS stages laid out
+// [X stage0][X stage1][W stage0][W stage1] (32 KiB each).
+//
+// The inner loop holds no vector-ALU instruction other than the MFMAs.  On gfx950 a VALU
+// instruction issued by any wave of a SIMD while that SIMD streams MFMAs costs about a
+// whole MFMA slot, so pointer arithmetic inside the loop serialises memory traffic with
+// the matrix core.  Therefore:
+//   * global -> LDS copies are global_load_lds_dwordx4 (no register staging) addressed by a
+//     scalar base pointer, advanced with scalar adds, plus a per-lane byte offset computed once;
+//   * LDS -> register fragment reads use per-lane addresses computed once plus immediate offsets;
+//   * waits and barriers are scalar.
+// Each load instruction of a wave fills 1 KiB of LDS = 8 rows x 128 bytes, so every row
+// segment is one full 128-byte cache line (half-line segments run the texture path at
+// about 60% of that rate).  Lane l of the instruction writes LDS row (l>>3), physical 16-byte
+// chunk (l&7); it fetches logical chunk (l&7) ^ ((row>>1)&7) so that the XOR swizzle, which
+// keeps ds_read_b128 conflict-free, is applied on the global side.
+// Fragments are double-buffered in registers: the reads of k-step ks+1 are in flight while
+// the 8 MFMAs of k-step ks execute.
+//
+// The MFMA takes the W fragment as its first operand: a lane then holds 4 consecutive n of
+// one output row m, and the write-back is 16-byte stores with the per-channel scale and bias
+// fetched as float4.
+#define AXI8_LGKM(n) __builtin_amdgcn_s_waitcnt(0x3F | (3 << 14) | (7 << 4) | ((n) << 8))
+#define AXI8_VM0() __builtin_amdgcn_s_waitcnt(0 | (0 << 14) | (7 << 4) | (15 << 8))
+#define AXI8_DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
+#define AXI8_LOAD_LDS(m0val, voff, base)                                                     \
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0val), \
+                 "v"(voff), "s"(base)                                                        \
+                 : "memory")
+
+template <int ACT>
+__global__ void __launch_bounds__(512)
+k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
+                 int64_t K, float x_scale, const float *__restrict__ w_scales,
+                 const float *__restrict__ bias, float *__restrict__ out,
+                 int32_t *__restrict__ acc_out) {
+    constexpr int BM = 256, BN = 256, BKB = 128, WAVES_N = 4, WTM = 128, WTN = 64, TM = 4, TN = 2;
+    constexpr int OPER = BM * BKB;   // bytes of one operand in one stage
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    int tm, tn;
+    tile_of_block(blockIdx.x, (int)(M / BM), (int)(N / BN), tm, tn);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int slabs = (int)(K / BKB);
+
+    // load instruction j (0..3) of wave w fills rows (j*8+w)*8 .. +8 of an operand stage
+    unsigned voff[4];
+    {
+        const int sw = (wave & 1) * 4 + (lane >> 4);      // (row >> 1) & 7 of this lane's row
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            voff[j] = (unsigned)(((j * 8 + wave) * 8 + (lane >> 3)) * K + (((lane & 7) ^ sw) << 4));
+    }
+    const int8_t *gx = X + m0 * K, *gw = W + n0 * K;
+    const unsigned lds_w = (unsigned)(uintptr_t)lds + wave * 1024;
+
+    // fragment reads: lane (frow, fhalf) of tile i takes row i*32+frow, logical chunk ks*2+fhalf
+    const int frow = lane & 31, fhalf = lane >> 5;
+    unsigned rx[4], rw[4];
+    {
+        const int sw = (frow >> 1) & 7;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const unsigned inrow = (unsigned)(frow * BKB + (((ks * 2 + fhalf) ^ sw) << 4));
+            rx[ks] = (unsigned)(uintptr_t)lds + wm * WTM * BKB + inrow;
+            rw[ks] = (unsigned)(uintptr_t)lds + 2 * OPER + wn * WTN * BKB + inrow;
+        }
+    }
+
+    // Per-channel scale (premultiplied by x_scale) and bias of this tile's 256 columns go to LDS
+    // now, so the write-back does not wait on global loads.
+    typedef float v4f_t __attribute__((ext_vector_type(4)));
+    float *lds_scale = reinterpret_cast<float *>(lds + 4 * OPER), *lds_bias = lds_scale + BN;
+    if (out && tid < 128) {
+        const int c4 = (tid & 63) * 4;
+        v4f_t v = {0.f, 0.f, 0.f, 0.f};
+        if (tid < 64) {
+            v = *reinterpret_cast<const v4f_t *>(w_scales + n0 + c4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = x_scale * v[e];
+            *reinterpret_cast<v4f_t *>(lds_scale + c4) = v;
+        } else {
+            if (bias) v = *reinterpret_cast<const v4f_t *>(bias + n0 + c4);
+            *reinterpret_cast<v4f_t *>(lds_bias + c4) = v;
+        }
+    }
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
+
+#define AXI8_ISSUE(stage)                                                                 \
+    do {                                                                                  \
+        AXI8_LOAD_LDS(lds_w + (stage) * OPER + 0 * 8192, voff[0], gx);                    \
+        AXI8_LOAD_LDS(lds_w + (stage) * OPER + 1 * 8192, voff[1], gx);                    \
+        AXI8_LOAD_LDS(lds_w + (stage) * OPER + 2 * 8192, voff[2], gx);                    \
+        AXI8_LOAD_LDS(lds_w + (stage) * OPER + 3 * 8192, voff[3], gx);                    \
+        AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + 0 * 8192, voff[0], gw);         \
+        AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + 1 * 8192, voff[1], gw);         \
+        AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + 2 * 8192, voff[2], gw);         \
+        AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + 3 * 8192, voff[3], gw);         \
+        gx += BKB;                                                                        \
+        gw += BKB;                                                                        \
+    } while (0)
+
+#define AXI8_FRAGS(buf, stage, ks)                                          \
+    do {                                                                    \
+        AXI8_DS_READ(fx[buf][0], rx[ks], (stage) * OPER + 0 * 4096);        \
+        AXI8_DS_READ(fx[buf][1], rx[ks], (stage) * OPER + 1 * 4096);        \
+        AXI8_DS_READ(fw[buf][0], rw[ks], (stage) * OPER + 0 * 4096);        \
+        AXI8_DS_READ(fw[buf][1], rw[ks], (stage) * OPER + 1 * 4096);        \
+        AXI8_DS_READ(fx[buf][2], rx[ks], (stage) * OPER + 2 * 4096);        \
+        AXI8_DS_READ(fx[buf][3], rx[ks], (stage) * OPER + 3 * 4096);        \
+    } while (0)
+
+#define AXI8_MFMAS(buf)                                                                         \
+    do {                                                                                        \
+        _Pragma("unroll") for (int i = 0; i < TM; i++)                                          \
+            _Pragma("unroll") for (int j = 0; j < TN; j++)                                      \
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[buf][j], fx[buf][i],       \
+                                                                  acc[i][j], 0, 0, 0);          \
+        __builtin_amdgcn_sched_barrier(0);                                                      \
+    } while (0)
+
+    // One slab resident in `stage`; `more`: prefetch the next slab into the other stage.
+#define AXI8_SLAB(stage, more)                                   \
+    do {                                                         \
+        if (more) AXI8_ISSUE(1 - (stage));                       \
+        AXI8_FRAGS(0, stage, 0);                                 \
+        AXI8_FRAGS(1, stage, 1);                                 \
+        AXI8_LGKM(6); __builtin_amdgcn_sched_barrier(0);         \
+        AXI8_MFMAS(0);                                           \
+        AXI8_FRAGS(0, stage, 2);                                 \
+        AXI8_LGKM(6); __builtin_amdgcn_sched_barrier(0);         \
+        AXI8_MFMAS(1);                                           \
+        AXI8_FRAGS(1, stage, 3);                                 \
+        AXI8_LGKM(6); __builtin_amdgcn_sched_barrier(0);         \
+        AXI8_MFMAS(0);                                           \
+        AXI8_LGKM(0); __builtin_amdgcn_sched_barrier(0);         \
+        AXI8_MFMAS(1);                                           \
+        AXI8_VM0();                                              \
+        __builtin_amdgcn_s_barrier();                            \
+        __builtin_amdgcn_sched_barrier(0);                       \
+    } while (0)
+
+    v4i fx[2][TM], fw[2][TN];
+    AXI8_ISSUE(0);
+    AXI8_VM0();
+    __builtin_amdgcn_s_barrier();
+
+    for (int s = 0; s < slabs; s += 2) {           // `more` is wave-uniform: scalar branches only
+        AXI8_SLAB(0, s + 1 < slabs);
+        if (s + 1 < slabs) AXI8_SLAB(1, s + 2 < slabs);
+    }
+
+    // Write-back.  With W as the MFMA's first operand, register v of lane l holds
+    // m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3): four consecutive n per lane.
+    const int64_t row0 = m0 + wm * WTM + frow, col0 = n0 + wn * WTN + 4 * fhalf;
+    if (acc_out) {
+        int32_t *dst = acc_out + row0 * N + col0;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    *reinterpret_cast<v4i *>(dst + (int64_t)i * 32 * N + j * 32 + 8 * g) =
+                        v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+    }
+    if (out) {
+        float *dst = out + row0 * N + col0;
+        const float *sp = lds_scale + wn * WTN + 4 * fhalf, *bp = lds_bias + wn * WTN + 4 * fhalf;
+        const bool has_bias = bias != nullptr;
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const v4f_t sc = *reinterpret_cast<const v4f_t *>(sp + j * 32 + 8 * g);
+                const v4f_t bv = *reinterpret_cast<const v4f_t *>(bp + j * 32 + 8 * g);
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    v4f_t r;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float f = (float)acc[i][j][4 * g + e];
+                        // a fused multiply-add with bias = 0 would round differently from the plain product
+                        r[e] = apply_act(has_bias ? __builtin_fmaf(f, sc[e], bv[e]) : f * sc[e], ACT);
+                    }
+                    *reinterpret_cast<v4f_t *>(dst + (int64_t)i * 32 * N + j * 32 + 8 * g) = r;
+                }
+            }
+    }
+}
+#undef AXI8_ISSUE
+#undef AXI8_FRAGS
+#undef AXI8_MFMAS
+#undef AXI8_SLAB
+
+int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
+               const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N,
+               int64_t K) {
+    constexpr int smem = 4 * 256 * 128 + 2 * 256 * 4;   // two stages of both operands + scale and bias
+    typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
+                           const float *, float *, int32_t *);
+    static const kern_t kerns[3] = {k_qgemm_w8a8_256<AXHIP_ACT_NONE>, k_qgemm_w8a8_256<AXHIP_ACT_RELU>,
+                                    k_qgemm_w8a8_256<AXHIP_ACT_GELU>};
+    static bool attr_set = false;
+    if (!attr_set) {
+        for (kern_t kf : kerns)
+            AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kf),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, smem),
+                          "hipFuncSetAttribute");
+        attr_set = true;
+    }
+    const int64_t tiles = (M / 256) * (N / 256);
+    if (tiles > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: too many tiles");
+    note_kernel("qgemm_w8a8_256x256_dma");
+    hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles), dim3(512), smem, kStream, x, w, M, N, K,
+                       x_scale, w_scales, bias, out, acc_out);
+    return check_launch("qgemm_w8a8_256x256_dma");
+}
+
 }  // namespace
 
 extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
@@ -198,9 +432,11 @@ extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
         return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: unknown activation %d", act);
     if (M == 0 || N == 0) return AXHIP_OK;
     const bool aligned = ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) && (K % BK == 0) && K > 0;
-    if (aligned && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128)
-        return launch<256, 256, 2, 4, false>("qgemm_w8a8_256x256", x, x_scale, w, w_scales, bias,
-                                             act, out, acc_out, M, N, K);
+    const bool vec_out = (!out || (((uintptr_t)out | (uintptr_t)w_scales | (uintptr_t)bias) & 15) == 0) &&
+                         (((uintptr_t)acc_out & 15) == 0);
+    if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128 &&
+        K < (int64_t(1) << 24))   // per-lane 32-bit byte offsets span 256 rows
+        return launch_256(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K);
     if (aligned && M % 128 == 0 && N % 128 == 0)
         return launch<128, 128, 2, 2, false>("qgemm_w8a8_128x128", x, x_scale, w, w_scales, bias,
                                              act, out, acc_out, M, N, K);
