@@ -17,6 +17,9 @@ void note_kernel(const char *name);
 int check_launch(const char *what);
 // A device workspace of at least `bytes`, owned by the runtime (grown on demand), or NULL.
 void *workspace(size_t bytes);
+// `n` zero-initialised device ints owned by the runtime.  Kernels that use them as arrival counters
+// leave them at zero when they finish.
+int *strip_counters(size_t n);
 
 constexpr hipStream_t kStream = nullptr;
 

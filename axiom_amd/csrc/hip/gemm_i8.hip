@@ -437,9 +437,13 @@ extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
     if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128 &&
         K < (int64_t(1) << 24))   // per-lane 32-bit byte offsets span 256 rows
         return launch_256(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K);
-    if (aligned && M % 128 == 0 && N % 128 == 0)
+    // fewer than ~3/4 of the 256 CUs busy with 128x128 tiles: quarter the tile instead
+    if (aligned && M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 192)
         return launch<128, 128, 2, 2, false>("qgemm_w8a8_128x128", x, x_scale, w, w_scales, bias,
                                              act, out, acc_out, M, N, K);
+    if (aligned && M % 64 == 0 && N % 64 == 0)
+        return launch<64, 64, 2, 2, false>("qgemm_w8a8_64x64", x, x_scale, w, w_scales, bias, act,
+                                           out, acc_out, M, N, K);
     return launch<64, 64, 2, 2, true>("qgemm_w8a8_64x64_guarded", x, x_scale, w, w_scales, bias,
                                       act, out, acc_out, M, N, K);
 }

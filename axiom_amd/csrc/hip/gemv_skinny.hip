@@ -5,10 +5,12 @@
 // groups take rows k, k+16, ... of that range, so one wave-wide load instruction covers four
 // 256-byte row segments and eight of them are kept in flight per lane.  The M activations of
 // a k row are wave-uniform only per lane group, so they come from LDS (staged once per
-// workgroup).  Lane groups are summed through LDS in a fixed order; when K is split over
-// several workgroups the partial tiles go to a workspace and a second kernel adds them in
-// split order and applies bias and activation — no atomics, so results are bit-identical
-// run to run.
+// workgroup); the first batch of weight loads is issued before that staging so HBM latency
+// overlaps it.  Lane groups are summed through LDS in a fixed order.  When K is split over
+// several workgroups each writes its partial tile to a workspace and bumps a per-strip
+// counter; the workgroup that arrives last adds the partials in split order (not arrival
+// order) and applies bias and activation.  The sum order is fixed, so results are
+// bit-identical run to run, and there is no second launch.
 #include "common.h"
 
 namespace {
@@ -22,7 +24,8 @@ template <int MR, bool VEC>
 __global__ void __launch_bounds__(256)
 k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, int64_t ldb,
          float *__restrict__ dst, int64_t dst_ld, int64_t dst_split_stride, int64_t N, int64_t K,
-         int64_t k_per_split, const float *__restrict__ bias, int act, int finish) {
+         int64_t k_per_split, const float *__restrict__ bias, int act, int splits,
+         float *__restrict__ C, int64_t ldc, int *__restrict__ counters) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
     // sm: [MR][k_per_split] activations, then [KGROUPS][MR][COLS] partial sums
     const int tid = threadIdx.x;
@@ -34,10 +37,22 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
     if (k_end > K) k_end = K;
     const int64_t klen = k_end - k_begin;
 
+    const int64_t col = n0 + 4 * cg;
+    const float *bp = B + col;
+    int64_t k = kg;
+    // first batch of weights in flight before anything else (VEC form, full batch available)
+    const bool pre = VEC && col < N && (UNROLL - 1) * KGROUPS + kg < klen;
+    v4f w0[UNROLL];
+    if (pre) {
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++)
+            w0[u] = *reinterpret_cast<const v4f *>(bp + (k_begin + k + u * KGROUPS) * ldb);
+    }
+
     float *xs = sm;
     for (int64_t i = tid; i < (int64_t)MR * klen; i += 256) {
-        int64_t m = i / klen, k = i - m * klen;
-        xs[m * k_per_split + k] = A[m * lda + k_begin + k];
+        int64_t m = i / klen, kk = i - m * klen;
+        xs[m * k_per_split + kk] = A[m * lda + k_begin + kk];
     }
     __syncthreads();
 
@@ -47,11 +62,19 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
 #pragma unroll
         for (int e = 0; e < 4; e++) acc[m][e] = 0.0f;
 
-    const int64_t col = n0 + 4 * cg;
-    const float *bp = B + col;
-    int64_t k = kg;
     if (VEC) {
         if (col < N) {      // N % 4 == 0: a float4 is entirely inside or outside
+            if (pre) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                    for (int m = 0; m < MR; m++) {
+                        const float xv = xs[m * k_per_split + k + u * KGROUPS];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[m][e] = __builtin_fmaf(xv, w0[u][e], acc[m][e]);
+                    }
+                k += UNROLL * KGROUPS;
+            }
             for (; k + (UNROLL - 1) * KGROUPS < klen; k += UNROLL * KGROUPS) {
                 v4f w[UNROLL];
 #pragma unroll
@@ -97,6 +120,7 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
             v4f{acc[m][0], acc[m][1], acc[m][2], acc[m][3]};
     __syncthreads();
 
+    float *part = dst + (int64_t)blockIdx.y * dst_split_stride;   // == C itself when splits == 1
     for (int i = tid; i < MR * COLS; i += 256) {
         const int m = i / COLS, c = i % COLS;
         float s = 0.0f;
@@ -104,38 +128,70 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
         for (int g2 = 0; g2 < KGROUPS; g2++) s += red[(g2 * MR + m) * COLS + c];
         const int64_t n = n0 + c;
         if (n < N) {
-            if (finish) {
+            if (splits == 1) {
                 if (bias) s += bias[n];
-                s = apply_act(s, act);
+                part[m * dst_ld + n] = apply_act(s, act);
+            } else {
+                // device-scope store: written through to the point all XCDs' L2s agree on
+                __hip_atomic_store(reinterpret_cast<int *>(part + m * dst_ld + n), __float_as_int(s),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            dst[blockIdx.y * dst_split_stride + m * dst_ld + n] = s;
         }
     }
-}
+    if (splits == 1) return;
 
-__global__ void __launch_bounds__(256)
-k_skinny_finish(const float *__restrict__ part, int64_t split_stride, int splits, int64_t M,
-                int64_t N, float *__restrict__ C, int64_t ldc, const float *__restrict__ bias,
-                int act) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= M * N) return;
-    const int64_t m = i / N, n = i - m * N;
-    float s = 0.0f;
-    for (int p = 0; p < splits; p++) s += part[p * split_stride + i];
-    if (bias) s += bias[n];
-    C[m * ldc + n] = apply_act(s, act);
+    // Publish this partial, then find out whether every split of this column strip is in.
+    // Partials, counter and the reads below are all device-scope accesses, so no cache-wide
+    // write-back or invalidate is needed (a __threadfence here costs ~150 us per launch: it
+    // flushes the XCD's whole L2); the wait makes this thread's stores complete before the
+    // barrier, the barrier orders them before thread 0's increment.
+    __shared__ int last_flag;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) {
+        const int arrived = __hip_atomic_fetch_add(counters + blockIdx.x, 1, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+        last_flag = (arrived == splits - 1);
+    }
+    __syncthreads();
+    if (!last_flag) return;
+    for (int i = tid; i < MR * COLS; i += 256) {
+        const int m = i / COLS, c = i % COLS;
+        const int64_t n = n0 + c;
+        if (n >= N) continue;
+        const float *pp = dst + m * dst_ld + n;
+        float s = 0.0f;
+        int p = 0;
+        for (; p + 8 <= splits; p += 8) {           // loads independent, additions in split order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                v[u] = __int_as_float(__hip_atomic_load(reinterpret_cast<const int *>(pp + (int64_t)(p + u) * dst_split_stride),
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+#pragma unroll
+            for (int u = 0; u < 8; u++) s += v[u];
+        }
+        for (; p < splits; p++)
+            s += __int_as_float(__hip_atomic_load(reinterpret_cast<const int *>(pp + (int64_t)p * dst_split_stride),
+                                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        if (bias) s += bias[n];
+        C[m * ldc + n] = apply_act(s, act);
+    }
+    if (tid == 0)                                   // ready for the next launch
+        __hip_atomic_store(counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int MR>
 int launch_m(bool vec, dim3 grid, size_t smem, const float *A, int64_t lda, const float *B,
              int64_t ldb, float *dst, int64_t dst_ld, int64_t dst_split, int64_t N, int64_t K,
-             int64_t kps, const float *bias, int act, int finish) {
+             int64_t kps, const float *bias, int act, int splits, float *C, int64_t ldc,
+             int *counters) {
     if (vec)
         hipLaunchKernelGGL((k_skinny<MR, true>), grid, dim3(256), smem, kStream, A, lda, B, ldb, dst,
-                           dst_ld, dst_split, N, K, kps, bias, act, finish);
+                           dst_ld, dst_split, N, K, kps, bias, act, splits, C, ldc, counters);
     else
         hipLaunchKernelGGL((k_skinny<MR, false>), grid, dim3(256), smem, kStream, A, lda, B, ldb,
-                           dst, dst_ld, dst_split, N, K, kps, bias, act, finish);
+                           dst, dst_ld, dst_split, N, K, kps, bias, act, splits, C, ldc, counters);
     return check_launch("sgemm_skinny");
 }
 
@@ -155,7 +211,8 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
 
     const int64_t col_blocks = (N + COLS - 1) / COLS;
     // enough workgroups to cover 256 CUs a few times over, each with at least 128 k rows
-    int64_t splits = (1024 + col_blocks - 1) / col_blocks;
+    const int64_t want_blocks = M <= 2 ? 1024 : 512;   // partial traffic grows with M
+    int64_t splits = (want_blocks + col_blocks - 1) / col_blocks;
     const int64_t max_splits = K >= 128 ? K / 128 : 1;
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
@@ -173,13 +230,13 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
     const size_t smem = (size_t)(M * kps + red_floats) * sizeof(float);
     float *dst = C;
     int64_t dst_ld = ldc, dst_split = 0;
-    int finish = 1;
+    int *counters = nullptr;
     if (splits > 1) {
         dst = static_cast<float *>(axhip::workspace((size_t)splits * M * N * sizeof(float)));
-        if (!dst) return AXHIP_ERR_ALLOC;
+        counters = axhip::strip_counters((size_t)col_blocks);
+        if (!dst || !counters) return AXHIP_ERR_ALLOC;
         dst_ld = N;
         dst_split = M * N;
-        finish = 0;
     }
     static bool attr_set = false;
     if (!attr_set) {
@@ -202,18 +259,11 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
 #define AX_CASE(m)                                                                            \
     case m:                                                                                   \
         rc = launch_m<m>(vec, grid, smem, A, lda, B, ldb, dst, dst_ld, dst_split, N, K, kps,  \
-                         bias, act, finish);                                                  \
+                         bias, act, (int)splits, C, ldc, counters);                           \
         break;
         AX_CASE(1) AX_CASE(2) AX_CASE(3) AX_CASE(4) AX_CASE(5) AX_CASE(6) AX_CASE(7) AX_CASE(8)
 #undef AX_CASE
         default: rc = AXHIP_ERR_SHAPE;
     }
-    if (rc) return rc;
-    if (splits > 1) {
-        const int64_t total = M * N;
-        hipLaunchKernelGGL(k_skinny_finish, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                           kStream, dst, dst_split, (int)splits, M, N, C, ldc, bias, act);
-        return check_launch("sgemm_skinny_finish");
-    }
-    return AXHIP_OK;
+    return rc;
 }

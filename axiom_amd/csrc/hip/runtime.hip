@@ -13,6 +13,8 @@ int g_devices = -1;
 char g_name[128] = "";
 void *g_ws = nullptr;
 size_t g_ws_bytes = 0;
+int *g_ctr = nullptr;
+size_t g_ctr_n = 0;
 }  // namespace
 
 namespace axhip {
@@ -56,6 +58,25 @@ void *workspace(size_t bytes) {
     return g_ws;
 }
 
+int *strip_counters(size_t n) {
+    if (n <= g_ctr_n) return g_ctr;
+    if (g_ctr) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(g_ctr);
+        g_ctr = nullptr;
+        g_ctr_n = 0;
+    }
+    size_t want = n < 4096 ? 4096 : n;
+    if (hipMalloc(reinterpret_cast<void **>(&g_ctr), want * sizeof(int)) != hipSuccess ||
+        hipMemset(g_ctr, 0, want * sizeof(int)) != hipSuccess) {
+        g_ctr = nullptr;
+        fail(AXHIP_ERR_ALLOC, "arrival counters (%zu ints): out of device memory", want);
+        return nullptr;
+    }
+    g_ctr_n = want;
+    return g_ctr;
+}
+
 }  // namespace axhip
 
 using axhip::fail;
@@ -89,8 +110,11 @@ void axhip_shutdown(void) {
     if (!g_ready) return;
     (void)hipDeviceSynchronize();
     if (g_ws) (void)hipFree(g_ws);
+    if (g_ctr) (void)hipFree(g_ctr);
     g_ws = nullptr;
     g_ws_bytes = 0;
+    g_ctr = nullptr;
+    g_ctr_n = 0;
     g_ready = 0;
 }
 
