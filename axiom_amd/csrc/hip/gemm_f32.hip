@@ -267,10 +267,283 @@ int validate(const char *who, int transa, int transb, int64_t M, int64_t N, int6
     return AXHIP_OK;
 }
 
+
+// =====================================================================================
+// Fast path for aligned shapes: direct-to-LDS loads and an inner loop with no vector-ALU
+// instruction other than the MFMAs (a VALU instruction issued on a SIMD that is streaming MFMAs
+// costs about one MFMA slot, so address arithmetic in the loop serialises with the matrix core).
+//
+// K slabs of 32 floats, two LDS stages.  An operand whose K index is contiguous in memory is
+// staged as rows of 128 bytes (one full cache line per row per slab); a wave's load
+// instruction fills 1 KiB = 8 rows, lane l -> row (l>>3), physical 16-byte chunk (l&7), and
+// fetches logical chunk (l&7) ^ ((row>>1)&7): the bank swizzle is applied on the global side.
+// A fragment read is one ds_read_b128 (4 consecutive k).  An operand whose M/N index is
+// contiguous is staged k-row by k-row: one load instruction carries RPI = 256/R k-rows of R
+// floats (1 KiB), groups are spaced 1024 + 32*RPI bytes apart so that the two lane halves of a
+// fragment read (k and k+4) land 128 bytes apart modulo 256 and never share a bank; a fragment
+// is four ds_read_b32.  Global addresses are a scalar base (advanced by scalar adds) plus a
+// per-lane byte offset computed once; LDS addresses are per-lane constants plus immediates.
+// The MFMA takes the B fragment first, so a lane owns four consecutive n of one row m and the
+// write-back moves 16 bytes per lane.
+#define AXF_LGKM(n) __builtin_amdgcn_s_waitcnt(0x3F | (3 << 14) | (7 << 4) | (((n) > 15 ? 15 : (n)) << 8))
+#define AXF_VM0() __builtin_amdgcn_s_waitcnt(0 | (0 << 14) | (7 << 4) | (15 << 8))
+#define AXF_LOAD_LDS(m0val, voff, base)                                                       \
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0val), \
+                 "v"(voff), "s"(base)                                                         \
+                 : "memory")
+
+template <int R, bool KC, int NW>
+struct DmaOperand {
+    static constexpr int RPI = KC ? 0 : 256 / R;                       // k-rows per load instruction
+    static constexpr int PITCH = KC ? 1024 : 1024 + 32 * (256 / R);    // LDS bytes per load instruction
+    static constexpr int NINSTR = KC ? R / 8 : 32 / (256 / R);         // load instructions per slab
+    static constexpr int IPW = NINSTR / NW;                            // ... per wave
+    static constexpr int BYTES = NINSTR * PITCH;                       // one stage
+    static constexpr int READS = KC ? 1 : 4;                           // ds_reads per 32-wide tile per k-block
+    static_assert(IPW * NW == NINSTR && IPW >= 1, "slab must divide over the waves");
+
+    // byte offset, from the operand's slab origin, of what lane `lane` of instruction q fetches
+    __device__ static unsigned lane_offset(int q, int lane, int64_t ld) {
+        if (KC) {
+            const int row = q * 8 + (lane >> 3);
+            return (unsigned)(row * ld * 4 + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+        }
+        constexpr int LPR = 64 / (256 / R);                            // lanes per k-row
+        return (unsigned)((q * (256 / R) + lane / LPR) * ld * 4 + (lane % LPR) * 16);
+    }
+    // LDS byte address (within a stage) a lane reads its fragments from, for k-block index kbi
+    // (KC) or for all k-blocks (MC, kbi ignored); `first` = first row/column of the wave's tile
+    __device__ static unsigned frag_base(int first, int frow, int fhalf, int kbi) {
+        if (KC) return (unsigned)((first + frow) * 128 + (((kbi * 2 + fhalf) ^ ((frow >> 1) & 7)) << 4));
+        return (unsigned)(fhalf * (4 / (256 / R)) * PITCH + (first + frow) * 4);
+    }
+    // immediate offset of k = kbi*8 + j (MC only)
+    static constexpr int k_imm(int k) { return KC ? 0 : (k / (256 / R)) * PITCH + (k % (256 / R)) * R * 4; }
+};
+
+template <bool KC> struct Frag;
+template <> struct Frag<true> {
+    v4f q;
+    __device__ __forceinline__ float get(int j) const { return q[j]; }
+};
+template <> struct Frag<false> {
+    float s0, s1, s2, s3;
+    __device__ __forceinline__ float get(int j) const { return j == 0 ? s0 : j == 1 ? s1 : j == 2 ? s2 : s3; }
+};
+
+#define AXF_DS128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
+#define AXF_DS32(dst, addr, off) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g) {
+    constexpr int NW = WAVES_M * WAVES_N;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
+    using OA = DmaOperand<BM, A_KC, NW>;
+    using OB = DmaOperand<BN, B_KC, NW>;
+    constexpr int A0 = 0, A1 = OA::BYTES, B0 = 2 * OA::BYTES, B1 = 2 * OA::BYTES + OB::BYTES;
+    constexpr int NREADS = TM * OA::READS + TN * OB::READS;
+    static_assert(B1 + OB::BYTES <= 160 * 1024 && B1 + OB::BYTES < 65536 * 3, "LDS budget");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    int tm, tn;
+    tile_of_block(blockIdx.x, (int)(g.M / BM), (int)(g.N / BN), tm, tn);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t batch = blockIdx.y;
+    const float *A = static_cast<const float *>(g.A) + batch * g.stride_a;
+    const float *B = static_cast<const float *>(g.B) + batch * g.stride_b;
+    float *C = g.C + batch * g.stride_c;
+    const int slabs = (int)(g.K / 32);
+
+    // ---- global -> LDS ----
+    unsigned va[OA::IPW], vb[OB::IPW];
+#pragma unroll
+    for (int j = 0; j < OA::IPW; j++) va[j] = OA::lane_offset(j * NW + wave, lane, g.lda);
+#pragma unroll
+    for (int j = 0; j < OB::IPW; j++) vb[j] = OB::lane_offset(j * NW + wave, lane, g.ldb);
+    const char *ga = reinterpret_cast<const char *>(A_KC ? A + m0 * g.lda : A + m0);
+    const char *gb = reinterpret_cast<const char *>(B_KC ? B + n0 * g.ldb : B + n0);
+    const int64_t step_a = A_KC ? 128 : 128 * g.lda, step_b = B_KC ? 128 : 128 * g.ldb;   // bytes per slab
+    const unsigned lds0 = (unsigned)(uintptr_t)lds_raw;
+    const unsigned dma_a = lds0 + wave * OA::PITCH, dma_b = lds0 + wave * OB::PITCH;
+
+    // ---- LDS -> fragments ----
+    const int frow = lane & 31, fhalf = lane >> 5;
+    unsigned ra[2][4], rb[2][4];        // [stage][k-block]: the stage base does not fit a 16-bit immediate
+#pragma unroll
+    for (int kbi = 0; kbi < 4; kbi++) {
+        ra[0][kbi] = lds0 + A0 + OA::frag_base(wm * WTM, frow, fhalf, kbi);
+        rb[0][kbi] = lds0 + B0 + OB::frag_base(wn * WTN, frow, fhalf, kbi);
+        ra[1][kbi] = ra[0][kbi] + (A1 - A0);
+        rb[1][kbi] = rb[0][kbi] + (B1 - B0);
+    }
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    Frag<A_KC> fa[2][TM];
+    Frag<B_KC> fb[2][TN];
+
+#define AXF_ISSUE(SA, SB)                                                                        \
+    do {                                                                                         \
+        _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                                      \
+            AXF_LOAD_LDS(dma_a + (SA) + j * NW * OA::PITCH, va[j], ga);                          \
+        _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                                      \
+            AXF_LOAD_LDS(dma_b + (SB) + j * NW * OB::PITCH, vb[j], gb);                          \
+        ga += step_a;                                                                            \
+        gb += step_b;                                                                            \
+    } while (0)
+
+// fragments of k-block KBI of stage ST
+#define AXF_FRAGS(BUF, ST, KBI)                                                                  \
+    do {                                                                                         \
+        _Pragma("unroll") for (int t = 0; t < TM; t++) {                                         \
+            if constexpr (A_KC) {                                                                \
+                AXF_DS128(fa[BUF][t].q, ra[ST][KBI], t * 4096);                                  \
+            } else {                                                                             \
+                AXF_DS32(fa[BUF][t].s0, ra[ST][0], OA::k_imm((KBI) * 8 + 0) + t * 128);          \
+                AXF_DS32(fa[BUF][t].s1, ra[ST][0], OA::k_imm((KBI) * 8 + 1) + t * 128);          \
+                AXF_DS32(fa[BUF][t].s2, ra[ST][0], OA::k_imm((KBI) * 8 + 2) + t * 128);          \
+                AXF_DS32(fa[BUF][t].s3, ra[ST][0], OA::k_imm((KBI) * 8 + 3) + t * 128);          \
+            }                                                                                    \
+        }                                                                                        \
+        _Pragma("unroll") for (int t = 0; t < TN; t++) {                                         \
+            if constexpr (B_KC) {                                                                \
+                AXF_DS128(fb[BUF][t].q, rb[ST][KBI], t * 4096);                                  \
+            } else {                                                                             \
+                AXF_DS32(fb[BUF][t].s0, rb[ST][0], OB::k_imm((KBI) * 8 + 0) + t * 128);          \
+                AXF_DS32(fb[BUF][t].s1, rb[ST][0], OB::k_imm((KBI) * 8 + 1) + t * 128);          \
+                AXF_DS32(fb[BUF][t].s2, rb[ST][0], OB::k_imm((KBI) * 8 + 2) + t * 128);          \
+                AXF_DS32(fb[BUF][t].s3, rb[ST][0], OB::k_imm((KBI) * 8 + 3) + t * 128);          \
+            }                                                                                    \
+        }                                                                                        \
+    } while (0)
+
+#define AXF_MFMAS(BUF)                                                                           \
+    do {                                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+        _Pragma("unroll") for (int e = 0; e < 4; e++)                                            \
+            _Pragma("unroll") for (int i = 0; i < TM; i++)                                       \
+                _Pragma("unroll") for (int j = 0; j < TN; j++)                                   \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[BUF][j].get(e),          \
+                                                                     fa[BUF][i].get(e), acc[i][j], 0, 0, 0); \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    } while (0)
+
+#define AXF_SLAB(ST, NA, NB, more)                                                               \
+    do {                                                                                         \
+        if (more) AXF_ISSUE(NA, NB);                                                             \
+        AXF_FRAGS(0, ST, 0);                                                                     \
+        AXF_FRAGS(1, ST, 1);                                                                     \
+        AXF_LGKM(NREADS);                                                                        \
+        AXF_MFMAS(0);                                                                            \
+        AXF_FRAGS(0, ST, 2);                                                                     \
+        AXF_LGKM(NREADS);                                                                        \
+        AXF_MFMAS(1);                                                                            \
+        AXF_FRAGS(1, ST, 3);                                                                     \
+        AXF_LGKM(NREADS);                                                                        \
+        AXF_MFMAS(0);                                                                            \
+        AXF_LGKM(0);                                                                             \
+        AXF_MFMAS(1);                                                                            \
+        AXF_VM0();                                                                               \
+        __builtin_amdgcn_s_barrier();                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    } while (0)
+
+    AXF_ISSUE(A0, B0);
+    AXF_VM0();
+    __builtin_amdgcn_s_barrier();
+    for (int s = 0; s < slabs; s += 2) {
+        AXF_SLAB(0, A1, B1, s + 1 < slabs);
+        if (s + 1 < slabs) AXF_SLAB(1, A0, B0, s + 2 < slabs);
+    }
+#undef AXF_ISSUE
+#undef AXF_FRAGS
+#undef AXF_MFMAS
+#undef AXF_SLAB
+
+    // register v of lane l: m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3)
+    const int64_t row0 = m0 + wm * WTM + frow, col0 = n0 + wn * WTN + 4 * fhalf;
+    float *dst = C + row0 * g.ldc + col0;
+    const float *bp = g.bias ? g.bias + col0 : nullptr;
+    const bool use_beta = g.beta != 0.0f;
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int gq = 0; gq < 4; gq++) {
+            v4f bv = {0.f, 0.f, 0.f, 0.f};
+            if (bp) bv = *reinterpret_cast<const v4f *>(bp + j * 32 + 8 * gq);
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                float *cp = dst + (int64_t)i * 32 * g.ldc + j * 32 + 8 * gq;
+                v4f r;
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = acc[i][j][4 * gq + e];
+                if (g.alpha != 1.0f) r *= g.alpha;
+                if (use_beta) r += g.beta * *reinterpret_cast<const v4f *>(cp);
+                if (bp) r += bv;
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = apply_act(r[e], g.act);
+                *reinterpret_cast<v4f *>(cp) = r;
+            }
+        }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
+    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, A_KC, B_KC>;
+    constexpr int NW = WAVES_M * WAVES_N;
+    constexpr int smem = 2 * (DmaOperand<BM, A_KC, NW>::BYTES + DmaOperand<BN, B_KC, NW>::BYTES);
+    static bool attr_set = false;
+    if (!attr_set) {
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem),
+                      "hipFuncSetAttribute");
+        attr_set = true;
+    }
+    const int64_t tiles = (g.M / BM) * (g.N / BN);
+    note_kernel(name);
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)batch), dim3(NW * 64), smem, kStream, g);
+    return check_launch(name);
+}
+
+// Chooses the largest tile that still gives every CU work; returns -1 when the shape does not
+// qualify for the fast path (the caller then uses the register-staged kernel).
+template <bool A_KC, bool B_KC>
+int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
+    const bool ok = g.K % 32 == 0 && g.K > 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
+                    ((uintptr_t)g.C % 16 == 0) && ((uintptr_t)g.bias % 16 == 0) && g.lda % 4 == 0 &&
+                    g.ldb % 4 == 0 && g.ldc % 4 == 0 && g.stride_a % 4 == 0 && g.stride_b % 4 == 0 &&
+                    g.stride_c % 4 == 0 && g.lda < (1 << 20) && g.ldb < (1 << 20) && batch <= 65535 &&
+                    g.M % 64 == 0 && g.N % 64 == 0;
+    if (!ok) return -1;
+    auto count = [&](int64_t t) { return (g.M / t) * (g.N / t) * batch; };
+    if (g.M % 256 == 0 && g.N % 256 == 0 && count(256) >= 224)
+        return launch_dma<256, 256, 2, 4, A_KC, B_KC>(names[0], g, batch);
+    if (g.M % 128 == 0 && g.N % 128 == 0 && count(128) >= 224)
+        return launch_dma<128, 128, 2, 2, A_KC, B_KC>(names[1], g, batch);
+    return launch_dma<64, 64, 2, 2, A_KC, B_KC>(names[2], g, batch);
+}
+
 int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     static const char *const nn[3] = {"sgemm_nn_128x128", "sgemm_nn_64x64", "sgemm_nn_64x64_guarded"};
     static const char *const nt[3] = {"sgemm_nt_128x128", "sgemm_nt_64x64", "sgemm_nt_64x64_guarded"};
     static const char *const tn[3] = {"sgemm_tn_128x128", "sgemm_tn_64x64", "sgemm_tn_64x64_guarded"};
+    static const char *const nn_d[3] = {"sgemm_nn_256x256_dma", "sgemm_nn_128x128_dma", "sgemm_nn_64x64_dma"};
+    static const char *const nt_d[3] = {"sgemm_nt_256x256_dma", "sgemm_nt_128x128_dma", "sgemm_nt_64x64_dma"};
+    static const char *const tn_d[3] = {"sgemm_tn_256x256_dma", "sgemm_tn_128x128_dma", "sgemm_tn_64x64_dma"};
+    int rc = -1;
+    if (!transa && !transb) rc = try_dma<true, false>(nn_d, g, batch);
+    else if (!transa && transb) rc = try_dma<true, true>(nt_d, g, batch);
+    else if (transa && !transb) rc = try_dma<false, false>(tn_d, g, batch);
+    if (rc >= 0) return rc;
     if (!transa && !transb) return pick_tile<true, false, float>(nn, g, batch);
     if (!transa && transb) return pick_tile<true, true, float>(nt, g, batch);
     if (transa && !transb) return pick_tile<false, false, float>(tn, g, batch);
