@@ -273,7 +273,7 @@ int validate(const char *who, int transa, int transb, int64_t M, int64_t N, int6
 // instruction other than the MFMAs (a VALU instruction issued on a SIMD that is streaming MFMAs
 // costs about one MFMA slot, so address arithmetic in the loop serialises with the matrix core).
 //
-// K slabs of 32 floats, two LDS stages.  An operand whose K index is contiguous in memory is
+// K slabs of 32 floats, two to four LDS stages.  An operand whose K index is contiguous in memory is
 // staged as rows of 128 bytes (one full cache line per row per slab); a wave's load
 // instruction fills 1 KiB = 8 rows, lane l -> row (l>>3), physical 16-byte chunk (l&7), and
 // fetches logical chunk (l&7) ^ ((row>>1)&7): the bank swizzle is applied on the global side.
@@ -286,7 +286,7 @@ int validate(const char *who, int transa, int transb, int64_t M, int64_t N, int6
 // The MFMA takes the B fragment first, so a lane owns four consecutive n of one row m and the
 // write-back moves 16 bytes per lane.
 #define AXF_LGKM(n) __builtin_amdgcn_s_waitcnt(0x3F | (3 << 14) | (7 << 4) | (((n) > 15 ? 15 : (n)) << 8))
-#define AXF_VM0() __builtin_amdgcn_s_waitcnt(0 | (0 << 14) | (7 << 4) | (15 << 8))
+#define AXF_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 #define AXF_LOAD_LDS(m0val, voff, base)                                                       \
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0val), \
                  "v"(voff), "s"(base)                                                         \
@@ -334,15 +334,19 @@ template <> struct Frag<false> {
 #define AXF_DS128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 #define AXF_DS32(dst, addr, off) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g) {
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
     using OA = DmaOperand<BM, A_KC, NW>;
     using OB = DmaOperand<BN, B_KC, NW>;
-    constexpr int A0 = 0, A1 = OA::BYTES, B0 = 2 * OA::BYTES, B1 = 2 * OA::BYTES + OB::BYTES;
+    // LDS: NST stages of A, then NST stages of B
+    constexpr int B_BASE = NST * OA::BYTES;
     constexpr int NREADS = TM * OA::READS + TN * OB::READS;
-    static_assert(B1 + OB::BYTES <= 160 * 1024 && B1 + OB::BYTES < 65536 * 3, "LDS budget");
+    // loads a wave may leave in flight at the end of a slab: everything but the next slab's
+    constexpr int VM_KEEP = (NST - 2) * (OA::IPW + OB::IPW);
+    static_assert(NST >= 2 && NST <= 4 && VM_KEEP < 64, "stage count");
+    static_assert(B_BASE + NST * OB::BYTES <= 160 * 1024, "LDS budget");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -371,14 +375,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
 
     // ---- LDS -> fragments ----
     const int frow = lane & 31, fhalf = lane >> 5;
-    unsigned ra[2][4], rb[2][4];        // [stage][k-block]: the stage base does not fit a 16-bit immediate
+    unsigned ra[NST][4], rb[NST][4];    // [stage][k-block]: the stage base does not fit a 16-bit immediate
 #pragma unroll
-    for (int kbi = 0; kbi < 4; kbi++) {
-        ra[0][kbi] = lds0 + A0 + OA::frag_base(wm * WTM, frow, fhalf, kbi);
-        rb[0][kbi] = lds0 + B0 + OB::frag_base(wn * WTN, frow, fhalf, kbi);
-        ra[1][kbi] = ra[0][kbi] + (A1 - A0);
-        rb[1][kbi] = rb[0][kbi] + (B1 - B0);
-    }
+    for (int st = 0; st < NST; st++)
+#pragma unroll
+        for (int kbi = 0; kbi < 4; kbi++) {
+            ra[st][kbi] = lds0 + st * OA::BYTES + OA::frag_base(wm * WTM, frow, fhalf, kbi);
+            rb[st][kbi] = lds0 + B_BASE + st * OB::BYTES + OB::frag_base(wn * WTN, frow, fhalf, kbi);
+        }
 
     v16f acc[TM][TN];
 #pragma unroll
@@ -391,12 +395,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
     Frag<A_KC> fa[2][TM];
     Frag<B_KC> fb[2][TN];
 
-#define AXF_ISSUE(SA, SB)                                                                        \
+// loads of the next unread slab into stage ST
+#define AXF_ISSUE(ST)                                                                            \
     do {                                                                                         \
         _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                                      \
-            AXF_LOAD_LDS(dma_a + (SA) + j * NW * OA::PITCH, va[j], ga);                          \
+            AXF_LOAD_LDS(dma_a + (ST) * OA::BYTES + j * NW * OA::PITCH, va[j], ga);              \
         _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                                      \
-            AXF_LOAD_LDS(dma_b + (SB) + j * NW * OB::PITCH, vb[j], gb);                          \
+            AXF_LOAD_LDS(dma_b + B_BASE + (ST) * OB::BYTES + j * NW * OB::PITCH, vb[j], gb);     \
         ga += step_a;                                                                            \
         gb += step_b;                                                                            \
     } while (0)
@@ -437,9 +442,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
         __builtin_amdgcn_sched_barrier(0);                                                       \
     } while (0)
 
-#define AXF_SLAB(ST, NA, NB, more)                                                               \
+// one slab out of stage ST; `more`: slab s+NST-1 exists and is fetched into the stage read last
+#define AXF_SLAB(ST, more)                                                                       \
     do {                                                                                         \
-        if (more) AXF_ISSUE(NA, NB);                                                             \
+        if (more) AXF_ISSUE(((ST) + NST - 1) % NST);                                             \
         AXF_FRAGS(0, ST, 0);                                                                     \
         AXF_FRAGS(1, ST, 1);                                                                     \
         AXF_LGKM(NREADS);                                                                        \
@@ -452,17 +458,28 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
         AXF_MFMAS(0);                                                                            \
         AXF_LGKM(0);                                                                             \
         AXF_MFMAS(1);                                                                            \
-        AXF_VM0();                                                                               \
+        if (VM_KEEP > 0 && (more)) AXF_VM(VM_KEEP); else AXF_VM(0);                              \
         __builtin_amdgcn_s_barrier();                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     } while (0)
 
-    AXF_ISSUE(A0, B0);
-    AXF_VM0();
+    AXF_ISSUE(0);
+    if constexpr (NST > 2) { if (slabs > 1) AXF_ISSUE(1); }
+    if constexpr (NST > 3) { if (slabs > 2) AXF_ISSUE(2); }
+    AXF_VM(0);
     __builtin_amdgcn_s_barrier();
-    for (int s = 0; s < slabs; s += 2) {
-        AXF_SLAB(0, A1, B1, s + 1 < slabs);
-        if (s + 1 < slabs) AXF_SLAB(1, A0, B0, s + 2 < slabs);
+    for (int s = 0; s < slabs; s += NST) {
+        AXF_SLAB(0, s + NST - 1 < slabs);
+        if (s + 1 >= slabs) break;
+        AXF_SLAB(1, s + NST < slabs);
+        if constexpr (NST > 2) {
+            if (s + 2 >= slabs) break;
+            AXF_SLAB(2, s + NST + 1 < slabs);
+        }
+        if constexpr (NST > 3) {
+            if (s + 3 >= slabs) break;
+            AXF_SLAB(3, s + NST + 2 < slabs);
+        }
     }
 #undef AXF_ISSUE
 #undef AXF_FRAGS
@@ -470,37 +487,86 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
 #undef AXF_SLAB
 
     // register v of lane l: m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3)
-    const int64_t row0 = m0 + wm * WTM + frow, col0 = n0 + wn * WTN + 4 * fhalf;
-    float *dst = C + row0 * g.ldc + col0;
-    const float *bp = g.bias ? g.bias + col0 : nullptr;
     const bool use_beta = g.beta != 0.0f;
+    if constexpr (EPI == 0) {
+        const int64_t row0 = m0 + wm * WTM + frow, col0 = n0 + wn * WTN + 4 * fhalf;
+        float *dst = C + row0 * g.ldc + col0;
+        const float *bp = g.bias ? g.bias + col0 : nullptr;
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+        for (int j = 0; j < TN; j++)
 #pragma unroll
-        for (int gq = 0; gq < 4; gq++) {
+            for (int gq = 0; gq < 4; gq++) {
+                v4f bv = {0.f, 0.f, 0.f, 0.f};
+                if (bp) bv = *reinterpret_cast<const v4f *>(bp + j * 32 + 8 * gq);
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    float *cp = dst + (int64_t)i * 32 * g.ldc + j * 32 + 8 * gq;
+                    v4f r;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r[e] = acc[i][j][4 * gq + e];
+                    if (g.alpha != 1.0f) r *= g.alpha;
+                    if (use_beta) r += g.beta * *reinterpret_cast<const v4f *>(cp);
+                    if (bp) r += bv;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r[e] = apply_act(r[e], g.act);
+                    *reinterpret_cast<v4f *>(cp) = r;
+                }
+            }
+    } else {
+        // Each wave turns its 32x32 sub-tiles through a private 4 KiB of LDS (the stages are
+        // dead after the loop's last barrier) so that a store instruction writes 8 rows of 128
+        // contiguous bytes instead of 32 rows of 32.  Rows of 128 bytes, 16-byte chunk c of row
+        // r kept at chunk c ^ ((r>>1)&7): both the write (16 rows, one chunk column) and the
+        // read (2 rows, all chunks) of a 16-lane group then touch every bank once.
+        unsigned char *turn = lds_raw + wave * 4096;
+        const int rrow = lane >> 3, rchunk = lane & 7;
+        const int64_t col0 = n0 + wn * WTN + 4 * rchunk;
+        float *dst = C + (m0 + wm * WTM + rrow) * g.ldc + col0;
+        const float *bp = g.bias ? g.bias + col0 : nullptr;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
             v4f bv = {0.f, 0.f, 0.f, 0.f};
-            if (bp) bv = *reinterpret_cast<const v4f *>(bp + j * 32 + 8 * gq);
+            if (bp) bv = *reinterpret_cast<const v4f *>(bp + j * 32);
 #pragma unroll
             for (int i = 0; i < TM; i++) {
-                float *cp = dst + (int64_t)i * 32 * g.ldc + j * 32 + 8 * gq;
-                v4f r;
 #pragma unroll
-                for (int e = 0; e < 4; e++) r[e] = acc[i][j][4 * gq + e];
-                if (g.alpha != 1.0f) r *= g.alpha;
-                if (use_beta) r += g.beta * *reinterpret_cast<const v4f *>(cp);
-                if (bp) r += bv;
+                for (int gq = 0; gq < 4; gq++) {
+                    v4f r;
 #pragma unroll
-                for (int e = 0; e < 4; e++) r[e] = apply_act(r[e], g.act);
-                *reinterpret_cast<v4f *>(cp) = r;
+                    for (int e = 0; e < 4; e++) r[e] = acc[i][j][4 * gq + e];
+                    *reinterpret_cast<v4f *>(turn + frow * 128 + (((2 * gq + fhalf) ^ ((frow >> 1) & 7)) << 4)) = r;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                v4f r[4];
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    const int row = p * 8 + rrow;
+                    r[p] = *reinterpret_cast<const v4f *>(turn + row * 128 + ((rchunk ^ ((row >> 1) & 7)) << 4));
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    float *cp = dst + (int64_t)(i * 32 + p * 8) * g.ldc + j * 32;
+                    v4f o = r[p];
+                    if (g.alpha != 1.0f) o *= g.alpha;
+                    if (use_beta) o += g.beta * *reinterpret_cast<const v4f *>(cp);
+                    if (bp) o += bv;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[e] = apply_act(o[e], g.act);
+                    *reinterpret_cast<v4f *>(cp) = o;
+                }
             }
         }
+    }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI = 1>
 int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
-    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, A_KC, B_KC>;
+    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI>;
     constexpr int NW = WAVES_M * WAVES_N;
-    constexpr int smem = 2 * (DmaOperand<BM, A_KC, NW>::BYTES + DmaOperand<BN, B_KC, NW>::BYTES);
+    constexpr int smem = NST * (DmaOperand<BM, A_KC, NW>::BYTES + DmaOperand<BN, B_KC, NW>::BYTES);
     static bool attr_set = false;
     if (!attr_set) {
         AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -514,31 +580,37 @@ int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
     return check_launch(name);
 }
 
-// Chooses the largest tile that still gives every CU work; returns -1 when the shape does not
-// qualify for the fast path (the caller then uses the register-staged kernel).
+// Chooses the largest tile that still leaves about eight waves per CU; returns -1 when the
+// shape does not qualify for the fast path (the caller then uses the register-staged kernel).
+// names: 128x256, 128x128, 128x64, 64x64.
 template <bool A_KC, bool B_KC>
-int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
+int try_dma(const char *const names[4], const SgemmArgs &g, int64_t batch) {
     const bool ok = g.K % 32 == 0 && g.K > 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                     ((uintptr_t)g.C % 16 == 0) && ((uintptr_t)g.bias % 16 == 0) && g.lda % 4 == 0 &&
                     g.ldb % 4 == 0 && g.ldc % 4 == 0 && g.stride_a % 4 == 0 && g.stride_b % 4 == 0 &&
                     g.stride_c % 4 == 0 && g.lda < (1 << 20) && g.ldb < (1 << 20) && batch <= 65535 &&
-                    g.M % 64 == 0 && g.N % 64 == 0;
+                    g.M % 64 == 0 && g.N % 64 == 0 && (g.M / 64) * (g.N / 64) <= 0x7fffffff;
     if (!ok) return -1;
-    auto count = [&](int64_t t) { return (g.M / t) * (g.N / t) * batch; };
-    if (g.M % 256 == 0 && g.N % 256 == 0 && count(256) >= 224)
-        return launch_dma<256, 256, 2, 4, A_KC, B_KC>(names[0], g, batch);
-    if (g.M % 128 == 0 && g.N % 128 == 0 && count(128) >= 224)
-        return launch_dma<128, 128, 2, 2, A_KC, B_KC>(names[1], g, batch);
-    return launch_dma<64, 64, 2, 2, A_KC, B_KC>(names[2], g, batch);
+    auto count = [&](int64_t bm, int64_t bn) { return (g.M / bm) * (g.N / bn) * batch; };
+    if (g.M % 128 == 0 && g.N % 256 == 0 && count(128, 256) >= 256)
+        return launch_dma<128, 256, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
+    if (g.M % 128 == 0 && g.N % 128 == 0 && count(128, 128) >= 512)
+        return launch_dma<128, 128, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
+    // a tile that spans whole rows of C (ldc == 64) already writes contiguous memory
+    if (g.M % 128 == 0 && count(128, 64) >= 512)
+        return g.ldc == 64 ? launch_dma<128, 64, 2, 2, 3, A_KC, B_KC, 0>(names[2], g, batch)
+                           : launch_dma<128, 64, 2, 2, 3, A_KC, B_KC, 1>(names[2], g, batch);
+    return g.ldc == 64 ? launch_dma<64, 64, 2, 2, 3, A_KC, B_KC, 0>(names[3], g, batch)
+                       : launch_dma<64, 64, 2, 2, 3, A_KC, B_KC, 1>(names[3], g, batch);
 }
 
 int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     static const char *const nn[3] = {"sgemm_nn_128x128", "sgemm_nn_64x64", "sgemm_nn_64x64_guarded"};
     static const char *const nt[3] = {"sgemm_nt_128x128", "sgemm_nt_64x64", "sgemm_nt_64x64_guarded"};
     static const char *const tn[3] = {"sgemm_tn_128x128", "sgemm_tn_64x64", "sgemm_tn_64x64_guarded"};
-    static const char *const nn_d[3] = {"sgemm_nn_256x256_dma", "sgemm_nn_128x128_dma", "sgemm_nn_64x64_dma"};
-    static const char *const nt_d[3] = {"sgemm_nt_256x256_dma", "sgemm_nt_128x128_dma", "sgemm_nt_64x64_dma"};
-    static const char *const tn_d[3] = {"sgemm_tn_256x256_dma", "sgemm_tn_128x128_dma", "sgemm_tn_64x64_dma"};
+    static const char *const nn_d[4] = {"sgemm_nn_128x256_dma", "sgemm_nn_128x128_dma", "sgemm_nn_128x64_dma", "sgemm_nn_64x64_dma"};
+    static const char *const nt_d[4] = {"sgemm_nt_128x256_dma", "sgemm_nt_128x128_dma", "sgemm_nt_128x64_dma", "sgemm_nt_64x64_dma"};
+    static const char *const tn_d[4] = {"sgemm_tn_128x256_dma", "sgemm_tn_128x128_dma", "sgemm_tn_128x64_dma", "sgemm_tn_64x64_dma"};
     int rc = -1;
     if (!transa && !transb) rc = try_dma<true, false>(nn_d, g, batch);
     else if (!transa && transb) rc = try_dma<true, true>(nt_d, g, batch);

@@ -96,7 +96,9 @@ def test_w8a8_8192_cube_properties(hip, oracle):
 # ------------------------------------------------------------------ fp32 GEMM
 F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), (64, 64, 32),
               (128, 128, 64), (130, 260, 700), (256, 384, 512), (33, 40, 100), (96, 96, 96),
-              (2048, 1024, 256)]
+              (2048, 1024, 256),
+              # one shape per tile of the direct-to-LDS fast path: 128x256, 128x128, 128x64
+              (2048, 4096, 64), (4096, 2176, 64), (4096, 1088, 32), (128, 64, 4096)]
 
 
 @pytest.mark.parametrize("M,N,K", F32_SHAPES)
@@ -172,9 +174,10 @@ def test_sgemm_config0_1024_cube(hip, oracle, golden):
         assert np.array_equal(hip.sgemm(da, db).numpy(), c)
 
 
-def test_sgemm_alpha_beta_bias_act(hip, oracle):
+@pytest.mark.parametrize("M,N,K", [(130, 200, 96), (256, 320, 96), (2048, 4096, 32)])
+def test_sgemm_alpha_beta_bias_act(hip, oracle, M, N, K):
+    say("sgemm epilogue", M, N, K)
     oracle.seed(21)
-    M, N, K = 130, 200, 96
     a, b = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1)
     c0 = oracle.uniform((M, N), -1, 1)
     bias = oracle.normal((N,), 0, 0.5)
