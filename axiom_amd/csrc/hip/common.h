@@ -57,6 +57,36 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     tn = in_band / rows;
 }
 
+// Write-back of one 32x32 MFMA result tile held in the layout "lane l owns row (l & 31), and
+// for g = 0..3 the four consecutive columns 8*g + 4*(l >> 5) + e": the wave turns the tile
+// through 4 KiB of LDS private to it so that each store instruction writes 8 rows of 128
+// contiguous bytes (whole cache lines) instead of 32 rows of 32 bytes.  LDS rows are 128 bytes
+// with 16-byte chunk c of row r kept at chunk c ^ ((r >> 1) & 7): both the write (16 rows, one
+// chunk column per 16-lane group) and the read (2 rows, all chunks) touch every bank once.
+// V4 is a 16-byte vector; dst points at the tile's element (0, 0), ld in elements.
+template <typename V4, typename T>
+__device__ __forceinline__ void turn_tile_and_store(unsigned char *turn, int lane, const V4 (&r)[4],
+                                                    T *dst, int64_t ld) {
+    static_assert(sizeof(V4) == 16 && sizeof(T) == 4, "32-bit elements in 16-byte vectors");
+    const int frow = lane & 31, fhalf = lane >> 5;
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+        *reinterpret_cast<V4 *>(turn + frow * 128 + (((2 * g + fhalf) ^ ((frow >> 1) & 7)) << 4)) = r[g];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    V4 o[4];
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const int row = p * 8 + (lane >> 3);
+        o[p] = *reinterpret_cast<const V4 *>(turn + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int p = 0; p < 4; p++)
+        *reinterpret_cast<V4 *>(dst + (int64_t)(p * 8 + (lane >> 3)) * ld + (lane & 7) * 4) = o[p];
+}
+
 }  // namespace axhip
 
 #define AXHIP_HIP_TRY(expr, what)                                                         \

@@ -353,40 +353,47 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 
     // Write-back.  With W as the MFMA's first operand, register v of lane l holds
     // m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3): four consecutive n per lane.
-    const int64_t row0 = m0 + wm * WTM + frow, col0 = n0 + wn * WTN + 4 * fhalf;
+    // The stages are dead after the loop's last barrier; each wave turns its tiles through
+    // 4 KiB of them to store whole 128-byte rows.
+    unsigned char *turn = lds + wave * 4096;
+    const int64_t trow = m0 + wm * WTM, tcol = n0 + wn * WTN;
     if (acc_out) {
-        int32_t *dst = acc_out + row0 * N + col0;
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < TN; j++)
+            for (int j = 0; j < TN; j++) {
+                v4i r[4];
 #pragma unroll
                 for (int g = 0; g < 4; g++)
-                    *reinterpret_cast<v4i *>(dst + (int64_t)i * 32 * N + j * 32 + 8 * g) =
-                        v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    r[g] = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                turn_tile_and_store(turn, lane, r, acc_out + (trow + i * 32) * N + tcol + j * 32, N);
+            }
     }
     if (out) {
-        float *dst = out + row0 * N + col0;
         const float *sp = lds_scale + wn * WTN + 4 * fhalf, *bp = lds_bias + wn * WTN + 4 * fhalf;
         const bool has_bias = bias != nullptr;
 #pragma unroll
-        for (int j = 0; j < TN; j++)
+        for (int j = 0; j < TN; j++) {
+            v4f_t sc[4], bv[4];
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const v4f_t sc = *reinterpret_cast<const v4f_t *>(sp + j * 32 + 8 * g);
-                const v4f_t bv = *reinterpret_cast<const v4f_t *>(bp + j * 32 + 8 * g);
+                sc[g] = *reinterpret_cast<const v4f_t *>(sp + j * 32 + 8 * g);
+                bv[g] = *reinterpret_cast<const v4f_t *>(bp + j * 32 + 8 * g);
+            }
 #pragma unroll
-                for (int i = 0; i < TM; i++) {
-                    v4f_t r;
+            for (int i = 0; i < TM; i++) {
+                v4f_t r[4];
+#pragma unroll
+                for (int g = 0; g < 4; g++)
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const float f = (float)acc[i][j][4 * g + e];
                         // a fused multiply-add with bias = 0 would round differently from the plain product
-                        r[e] = apply_act(has_bias ? __builtin_fmaf(f, sc[e], bv[e]) : f * sc[e], ACT);
+                        r[g][e] = apply_act(has_bias ? __builtin_fmaf(f, sc[g][e], bv[g][e]) : f * sc[g][e], ACT);
                     }
-                    *reinterpret_cast<v4f_t *>(dst + (int64_t)i * 32 * N + j * 32 + 8 * g) = r;
-                }
+                turn_tile_and_store(turn, lane, r, out + (trow + i * 32) * N + tcol + j * 32, N);
             }
+        }
     }
 }
 #undef AXI8_ISSUE
