@@ -206,8 +206,8 @@ int launch(const char *name, const int8_t *x, float x_scale, const int8_t *w,
 // about 60% of that rate).  Lane l of the instruction writes LDS row (l>>3), physical 16-byte
 // chunk (l&7); it fetches logical chunk (l&7) ^ ((row>>1)&7) so that the XOR swizzle, which
 // keeps ds_read_b128 conflict-free, is applied on the global side.
-// Fragments are double-buffered in registers: the reads of k-step ks+1 are in flight while
-// the 8 MFMAs of k-step ks execute.
+// Fragments are double-buffered in registers: the reads of k-step ks+1 are issued one by one
+// between the 8 MFMAs of k-step ks, and so are the loads of the slab after next.
 //
 // The MFMA takes the W fragment as its first operand: a lane then holds 4 consecutive n of
 // one output row m, and the write-back is 16-byte stores with the per-channel scale and bias
@@ -287,16 +287,12 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
 
+#define AXI8_LOAD_X(stage, j) AXI8_LOAD_LDS(lds_w + (stage) * OPER + (j) * 8192, voff[j], gx)
+#define AXI8_LOAD_W(stage, j) AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + (j) * 8192, voff[j], gw)
 #define AXI8_ISSUE(stage)                                                                 \
     do {                                                                                  \
-        AXI8_LOAD_LDS(lds_w + (stage) * OPER + 0 * 8192, voff[0], gx);                    \
-        AXI8_LOAD_LDS(lds_w + (stage) * OPER + 1 * 8192, voff[1], gx);                    \
-        AXI8_LOAD_LDS(lds_w + (stage) * OPER + 2 * 8192, voff[2], gx);                    \
-        AXI8_LOAD_LDS(lds_w + (stage) * OPER + 3 * 8192, voff[3], gx);                    \
-        AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + 0 * 8192, voff[0], gw);         \
-        AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + 1 * 8192, voff[1], gw);         \
-        AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + 2 * 8192, voff[2], gw);         \
-        AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + 3 * 8192, voff[3], gw);         \
+        AXI8_LOAD_X(stage, 0); AXI8_LOAD_X(stage, 1); AXI8_LOAD_X(stage, 2); AXI8_LOAD_X(stage, 3); \
+        AXI8_LOAD_W(stage, 0); AXI8_LOAD_W(stage, 1); AXI8_LOAD_W(stage, 2); AXI8_LOAD_W(stage, 3); \
         gx += BKB;                                                                        \
         gw += BKB;                                                                        \
     } while (0)
@@ -311,45 +307,79 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         AXI8_DS_READ(fx[buf][3], rx[ks], (stage) * OPER + 3 * 4096);        \
     } while (0)
 
-#define AXI8_MFMAS(buf)                                                                         \
+// MFMA m (0..7) of a k-step: tile row m>>1, tile column m&1
+#define AXI8_M(buf, m)                                                                          \
     do {                                                                                        \
-        _Pragma("unroll") for (int i = 0; i < TM; i++)                                          \
-            _Pragma("unroll") for (int j = 0; j < TN; j++)                                      \
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[buf][j], fx[buf][i],       \
-                                                                  acc[i][j], 0, 0, 0);          \
+        acc[(m) >> 1][(m) & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(                         \
+            fw[buf][(m) & 1], fx[buf][(m) >> 1], acc[(m) >> 1][(m) & 1], 0, 0, 0);              \
         __builtin_amdgcn_sched_barrier(0);                                                      \
     } while (0)
 
-    // One slab resident in `stage`; `more`: prefetch the next slab into the other stage.
-#define AXI8_SLAB(stage, more)                                   \
-    do {                                                         \
-        if (more) AXI8_ISSUE(1 - (stage));                       \
-        AXI8_FRAGS(0, stage, 0);                                 \
-        AXI8_FRAGS(1, stage, 1);                                 \
-        AXI8_LGKM(6); __builtin_amdgcn_sched_barrier(0);         \
-        AXI8_MFMAS(0);                                           \
-        AXI8_FRAGS(0, stage, 2);                                 \
-        AXI8_LGKM(6); __builtin_amdgcn_sched_barrier(0);         \
-        AXI8_MFMAS(1);                                           \
-        AXI8_FRAGS(1, stage, 3);                                 \
-        AXI8_LGKM(6); __builtin_amdgcn_sched_barrier(0);         \
-        AXI8_MFMAS(0);                                           \
-        AXI8_LGKM(0); __builtin_amdgcn_sched_barrier(0);         \
-        AXI8_MFMAS(1);                                           \
-        AXI8_VM0();                                              \
-        __builtin_amdgcn_s_barrier();                            \
-        __builtin_amdgcn_sched_barrier(0);                       \
+// The 8 MFMAs of the k-step held in fragment buffer `buf`.  Between them, so that their issue
+// falls into the shadow of the MFMA before: (RD) the 6 fragment reads of k-step rks of stage
+// rstage into the other buffer, in the order the next block consumes them; (LD) the 8 loads of
+// the next unfetched slab into stage lstage.
+#define AXI8_BLOCK(buf, RD, rstage, rks, LD, lstage)                                            \
+    do {                                                                                        \
+        AXI8_M(buf, 0);                                                                         \
+        if (RD) AXI8_DS_READ(fx[1 - (buf)][0], rx[rks], (rstage) * OPER + 0 * 4096);            \
+        if (LD) AXI8_LOAD_X(lstage, 0);                                                         \
+        AXI8_M(buf, 1);                                                                         \
+        if (RD) AXI8_DS_READ(fw[1 - (buf)][0], rw[rks], (rstage) * OPER + 0 * 4096);            \
+        if (LD) AXI8_LOAD_X(lstage, 1);                                                         \
+        AXI8_M(buf, 2);                                                                         \
+        if (RD) AXI8_DS_READ(fw[1 - (buf)][1], rw[rks], (rstage) * OPER + 1 * 4096);            \
+        if (LD) AXI8_LOAD_X(lstage, 2);                                                         \
+        AXI8_M(buf, 3);                                                                         \
+        if (RD) AXI8_DS_READ(fx[1 - (buf)][1], rx[rks], (rstage) * OPER + 1 * 4096);            \
+        if (LD) AXI8_LOAD_X(lstage, 3);                                                         \
+        AXI8_M(buf, 4);                                                                         \
+        if (RD) AXI8_DS_READ(fx[1 - (buf)][2], rx[rks], (rstage) * OPER + 2 * 4096);            \
+        if (LD) AXI8_LOAD_W(lstage, 0);                                                         \
+        AXI8_M(buf, 5);                                                                         \
+        if (RD) AXI8_DS_READ(fx[1 - (buf)][3], rx[rks], (rstage) * OPER + 3 * 4096);            \
+        if (LD) AXI8_LOAD_W(lstage, 1);                                                         \
+        AXI8_M(buf, 6);                                                                         \
+        if (LD) AXI8_LOAD_W(lstage, 2);                                                         \
+        AXI8_M(buf, 7);                                                                         \
+        if (LD) { AXI8_LOAD_W(lstage, 3); gx += BKB; gw += BKB; }                               \
+        __builtin_amdgcn_sched_barrier(0);                                                      \
+    } while (0)
+
+#define AXI8_WAIT_FRAGS() do { AXI8_LGKM(0); __builtin_amdgcn_sched_barrier(0); } while (0)
+
+    // One slab resident in `stage`, its k-step 0 already (being) read into buffer 0.  After the
+    // third k-step every wave has read all it needs of this stage and waits for its own loads
+    // of the next slab; past the barrier the stage is free, so the last k-step's MFMAs cover
+    // the first fragment reads of the next slab (after the last slab they fetch stale bytes
+    // nobody uses) and, when more2, the loads of the slab after.
+#define AXI8_SLAB(stage, more2)                                              \
+    do {                                                                     \
+        AXI8_WAIT_FRAGS();                                                   \
+        AXI8_BLOCK(0, 1, stage, 1, 0, 0);                                    \
+        AXI8_WAIT_FRAGS();                                                   \
+        AXI8_BLOCK(1, 1, stage, 2, 0, 0);                                    \
+        AXI8_WAIT_FRAGS();                                                   \
+        AXI8_BLOCK(0, 1, stage, 3, 0, 0);                                    \
+        AXI8_WAIT_FRAGS();                                                   \
+        AXI8_VM0();                                                          \
+        __builtin_amdgcn_s_barrier();                                        \
+        __builtin_amdgcn_sched_barrier(0);                                   \
+        AXI8_BLOCK(1, 1, 1 - (stage), 0, more2, stage);                      \
     } while (0)
 
     v4i fx[2][TM], fw[2][TN];
     AXI8_ISSUE(0);
     AXI8_VM0();
     __builtin_amdgcn_s_barrier();
+    if (slabs > 1) AXI8_ISSUE(1);
+    AXI8_FRAGS(0, 0, 0);
 
-    for (int s = 0; s < slabs; s += 2) {           // `more` is wave-uniform: scalar branches only
-        AXI8_SLAB(0, s + 1 < slabs);
-        if (s + 1 < slabs) AXI8_SLAB(1, s + 2 < slabs);
+    for (int s = 0; s < slabs; s += 2) {           // the flags are wave-uniform: scalar branches only
+        AXI8_SLAB(0, s + 2 < slabs);
+        if (s + 1 < slabs) AXI8_SLAB(1, s + 3 < slabs);
     }
+    AXI8_WAIT_FRAGS();      // the stale reads must land before their registers are reused
 
     // Write-back.  With W as the MFMA's first operand, register v of lane l holds
     // m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3): four consecutive n per lane.
@@ -398,7 +428,11 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 }
 #undef AXI8_ISSUE
 #undef AXI8_FRAGS
-#undef AXI8_MFMAS
+#undef AXI8_M
+#undef AXI8_BLOCK
+#undef AXI8_WAIT_FRAGS
+#undef AXI8_LOAD_X
+#undef AXI8_LOAD_W
 #undef AXI8_SLAB
 
 int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
