@@ -9,6 +9,8 @@ and the skinny-M route's GB/s, each with its own roofline fraction.  RESULT line
 reference's benchmark format (benchmarks/bench_common.h:25-42) go to stderr.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu]
+    python bench.py --counter-probe     # for hardware-counter runs: 3 headline launches and 3
+                                        # launches of a copy-shaped kernel of known size, no output line
 """
 import argparse
 import ctypes as C
@@ -35,8 +37,23 @@ def rand_i8(rng, shape):
     return rng.integers(-127, 128, shape, dtype=np.int8)
 
 
-def time_calls(hip, fn, steps, warmup):
-    """(host ms per step between device syncs, event ms per step on the kernels' stream)."""
+def time_calls(hip, fn, steps=None, warmup=None, seconds=0.3):
+    """(host ms per step between device syncs, event ms per step on the kernels' stream).
+    Without explicit counts, warms up for `seconds` and times `seconds` worth of launches: the
+    GPU raises its clock only after some tens of milliseconds of load and settles at its
+    power-limited clock after a few hundred, and sustained throughput is what is reported."""
+    if steps is None or warmup is None:
+        for _ in range(3):
+            fn()
+        hip.sync()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            fn()
+        hip.sync()
+        per = max((time.perf_counter() - t0) / 10, 1e-6)
+        n = int(min(max(seconds / per, 20), 20000))
+        steps = n if steps is None else steps
+        warmup = n if warmup is None else warmup
     for _ in range(warmup):
         fn()
     hip.sync()
@@ -86,7 +103,7 @@ def secondary(hip):
     a, b = f32((1024, 1024), (1024, 1024))
     c = hip.empty((1024, 1024))
     _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm(
-        0, 0, 1024, 1024, 1024, 1.0, a.ptr, 1024, b.ptr, 1024, 0.0, c.ptr, 1024, None, 0)), 50, 5)
+        0, 0, 1024, 1024, 1024, 1.0, a.ptr, 1024, b.ptr, 1024, 0.0, c.ptr, 1024, None, 0)))
     tf = 2 * 1024 ** 3 / ms / 1e9
     res["fp32_gemm_1024"] = {"us": ms * 1e3, "TFLOP/s": tf, "frac_of_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS,
                              "kernel": hip.last_kernel()}
@@ -104,7 +121,7 @@ def secondary(hip):
                                     hbuf.ptr, 4096, b1.ptr, 2))
         hip.check(hip.L.axhip_sgemm(0, 0, 2048, 1024, 4096, 1.0, hbuf.ptr, 4096, w2.ptr, 1024, 0.0,
                                     y.ptr, 1024, b2.ptr, 0))
-    _, ms = time_calls(hip, ffn, 20, 3)
+    _, ms = time_calls(hip, ffn)
     tf = 2 * 2 * 2048 * 1024 * 4096 / ms / 1e9
     res["fp32_ffn_2048x1024x4096"] = {"us": ms * 1e3, "TFLOP/s": tf,
                                       "frac_of_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS}
@@ -117,7 +134,7 @@ def secondary(hip):
     bi = hip.array(rng.normal(0, 0.02, 4096).astype(np.float32))
     oi = hip.empty((256, 4096))
     _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_qgemm_w8a8(
-        xi.ptr, 0.01, wi.ptr, ws.ptr, bi.ptr, 0, oi.ptr, None, 256, 4096, 4096)), 50, 5)
+        xi.ptr, 0.01, wi.ptr, ws.ptr, bi.ptr, 0, oi.ptr, None, 256, 4096, 4096)))
     nbytes = 4096 * 4096 + 256 * 4096 + 4 * 256 * 4096 + 8 * 4096
     res["int8_qgemm_256x4096x4096"] = {"us": ms * 1e3, "TOP/s": 2 * 256 * 4096 * 4096 / ms / 1e9,
                                        "GB/s": nbytes / ms / 1e6,
@@ -153,8 +170,8 @@ def secondary(hip):
             it[0] += 1
             hip.check(hip.L.axhip_sgemm(0, 0, M, 4096, 4096, 1.0, h1.ptr, 4096, w2_.ptr, 4096, 0.0, h2.ptr, 4096, zeros.ptr, 1))
 
-        _, ms = time_calls(hip, mlp_step, 64, 8)
-        _, ms2 = time_calls(hip, layer2_only, 64, 8)
+        _, ms = time_calls(hip, mlp_step)
+        _, ms2 = time_calls(hip, layer2_only)
         gbs, gbs2 = weight_bytes / ms / 1e6, 4 * 4096 * 4096 / ms2 / 1e6
         mlp[f"M{M}"] = {"mlp_us": ms * 1e3, "mlp_GB/s": gbs, "mlp_frac_of_hbm_peak": gbs / PEAK_HBM_GBS,
                         "layer2_us": ms2 * 1e3, "layer2_GB/s": gbs2,
@@ -170,15 +187,37 @@ def secondary(hip):
     v = hip.array(rng.normal(0, 1, (Bn, S, D)).astype(np.float32))
     s, o = hip.empty((Bn, S, S)), hip.empty((Bn, S, D))
     _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm_strided_batched(
-        0, 1, S, S, D, 1.0, q.ptr, D, S * D, k.ptr, D, S * D, 0.0, s.ptr, S, S * S, Bn)), 10, 2)
+        0, 1, S, S, D, 1.0, q.ptr, D, S * D, k.ptr, D, S * D, 0.0, s.ptr, S, S * S, Bn)))
     nbytes = 4 * (2 * Bn * S * D + Bn * S * S)
     res["fp32_batched_qkt"] = {"us": ms * 1e3, "TFLOP/s": 2 * Bn * S * S * D / ms / 1e9,
                                "GB/s": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
     _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm_strided_batched(
-        0, 0, S, D, S, 1.0, s.ptr, S, S * S, v.ptr, D, S * D, 0.0, o.ptr, D, S * D, Bn)), 10, 2)
+        0, 0, S, D, S, 1.0, s.ptr, S, S * S, v.ptr, D, S * D, 0.0, o.ptr, D, S * D, Bn)))
     res["fp32_batched_pv"] = {"us": ms * 1e3, "TFLOP/s": 2 * Bn * S * S * D / ms / 1e9,
                               "GB/s": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
     return res
+
+
+def counter_probe(hip):
+    """Workload for per-dispatch hardware counters (HBM bytes fetched / written): the headline
+    kernel, and for scale the elementwise ReLU kernel over 64 Mi floats, which reads 256 MiB
+    and writes 256 MiB exactly once (a plain copy as far as memory traffic goes)."""
+    M = N = K = 8192
+    rng = np.random.default_rng(0)
+    x, w = hip.array(rand_i8(rng, (M, K))), hip.array(rand_i8(rng, (N, K)))
+    ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+    bias = hip.array(rng.normal(0.0, 0.02, N).astype(np.float32))
+    out = hip.empty((M, N))
+    for _ in range(3):
+        hip.check(hip.L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, bias.ptr, 0, out.ptr, None, M, N, K))
+    hip.sync()
+    n = 64 << 20
+    src, dst = hip.empty((n,)), hip.empty((n,))
+    for _ in range(3):
+        hip.check(hip.L.axhip_relu(src.ptr, dst.ptr, n))
+    hip.sync()
+    print(f"counter probe: 3 x {hip.last_kernel()} over {n} floats after 3 x qgemm_w8a8 8192^3",
+          file=sys.stderr, flush=True)
 
 
 def cpu_baseline():
@@ -211,10 +250,11 @@ def cpu_baseline():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--counter-probe", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -222,6 +262,9 @@ def main():
     from axiom_amd import AxHip
     hip = AxHip()
     hip.init()
+    if args.counter_probe:
+        counter_probe(hip)
+        return
 
     h = headline(hip, args.steps, args.warmup)
     tops = h["ops"] / h["host_ms"] / 1e9
