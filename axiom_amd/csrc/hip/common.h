@@ -11,6 +11,8 @@ namespace axhip {
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // 0 when the runtime is initialised on a usable GPU, else an AXHIP_ERR_* code (message set).
 int ensure_ready();
+// Compute units of the device (valid once ensure_ready() has returned 0).
+int cu_count();
 // Remembers which kernel variant a GEMM-type entry point chose.
 void note_kernel(const char *name);
 // Checks the launch that was just issued on the null stream.

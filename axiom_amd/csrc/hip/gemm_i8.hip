@@ -213,7 +213,8 @@ int launch(const char *name, const int8_t *x, float x_scale, const int8_t *w,
 // one output row m, and the write-back is 16-byte stores with the per-channel scale and bias
 // fetched as float4.
 #define AXI8_LGKM(n) __builtin_amdgcn_s_waitcnt(0x3F | (3 << 14) | (7 << 4) | ((n) << 8))
-#define AXI8_VM0() __builtin_amdgcn_s_waitcnt(0 | (0 << 14) | (7 << 4) | (15 << 8))
+#define AXI8_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
+#define AXI8_VM0() AXI8_VM(0)
 #define AXI8_DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 #define AXI8_LOAD_LDS(m0val, voff, base)                                                     \
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0val), \
@@ -232,9 +233,7 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-    int tm, tn;
-    tile_of_block(blockIdx.x, (int)(M / BM), (int)(N / BN), tm, tn);
-    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int tiles_m = (int)(M / BM), tiles_n = (int)(N / BN), total = tiles_m * tiles_n;
     const int slabs = (int)(K / BKB);
 
     // load instruction j (0..3) of wave w fills rows (j*8+w)*8 .. +8 of an operand stage
@@ -245,7 +244,7 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         for (int j = 0; j < 4; j++)
             voff[j] = (unsigned)(((j * 8 + wave) * 8 + (lane >> 3)) * K + (((lane & 7) ^ sw) << 4));
     }
-    const int8_t *gx = X + m0 * K, *gw = W + n0 * K;
+    const int8_t *gx = X, *gw = W;
     const unsigned lds_w = (unsigned)(uintptr_t)lds + wave * 1024;
 
     // fragment reads: lane (frow, fhalf) of tile i takes row i*32+frow, logical chunk ks*2+fhalf
@@ -261,31 +260,9 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         }
     }
 
-    // Per-channel scale (premultiplied by x_scale) and bias of this tile's 256 columns go to LDS
-    // now, so the write-back does not wait on global loads.
     typedef float v4f_t __attribute__((ext_vector_type(4)));
     float *lds_scale = reinterpret_cast<float *>(lds + 4 * OPER), *lds_bias = lds_scale + BN;
-    if (out && tid < 128) {
-        const int c4 = (tid & 63) * 4;
-        v4f_t v = {0.f, 0.f, 0.f, 0.f};
-        if (tid < 64) {
-            v = *reinterpret_cast<const v4f_t *>(w_scales + n0 + c4);
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = x_scale * v[e];
-            *reinterpret_cast<v4f_t *>(lds_scale + c4) = v;
-        } else {
-            if (bias) v = *reinterpret_cast<const v4f_t *>(bias + n0 + c4);
-            *reinterpret_cast<v4f_t *>(lds_bias + c4) = v;
-        }
-    }
-
     v16i acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
 
 #define AXI8_LOAD_X(stage, j) AXI8_LOAD_LDS(lds_w + (stage) * OPER + (j) * 8192, voff[j], gx)
 #define AXI8_LOAD_W(stage, j) AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + (j) * 8192, voff[j], gw)
@@ -368,62 +345,127 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         AXI8_BLOCK(1, 1, 1 - (stage), 0, more2, stage);                      \
     } while (0)
 
+    // Persistent: one workgroup per CU walks tiles t = blockIdx.x, + gridDim.x, ... (the same
+    // tile a non-persistent launch would hand that CU next).  With an even slab count the last
+    // slab of a tile sits in stage 1, so the first slab of the next tile is fetched into stage 0
+    // before the write-back starts and the stores drain under the next tile's first slabs: loads
+    // and stores complete in issue order, so "at most 32 outstanding" (the write-back's stores of
+    // one wave) means the 8 loads issued before them have landed.
+    const bool carry = (slabs & 1) == 0 && acc_out == nullptr;
+    bool fetched = false;
+    v4f_t col_v = {0.f, 0.f, 0.f, 0.f};      // waves 0/1: scales / biases of 4 columns of the coming tile
+    auto fetch_cols = [&](int64_t n0) {
+        if (out && tid < 128) {
+            const int c4 = (tid & 63) * 4;
+            col_v = v4f_t{0.f, 0.f, 0.f, 0.f};
+            if (tid < 64) col_v = *reinterpret_cast<const v4f_t *>(w_scales + n0 + c4);
+            else if (bias) col_v = *reinterpret_cast<const v4f_t *>(bias + n0 + c4);
+        }
+    };
     v4i fx[2][TM], fw[2][TN];
-    AXI8_ISSUE(0);
-    AXI8_VM0();
-    __builtin_amdgcn_s_barrier();
-    if (slabs > 1) AXI8_ISSUE(1);
-    AXI8_FRAGS(0, 0, 0);
 
-    for (int s = 0; s < slabs; s += 2) {           // the flags are wave-uniform: scalar branches only
-        AXI8_SLAB(0, s + 2 < slabs);
-        if (s + 1 < slabs) AXI8_SLAB(1, s + 3 < slabs);
-    }
-    AXI8_WAIT_FRAGS();      // the stale reads must land before their registers are reused
-
-    // Write-back.  With W as the MFMA's first operand, register v of lane l holds
-    // m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3): four consecutive n per lane.
-    // The stages are dead after the loop's last barrier; each wave turns its tiles through
-    // 4 KiB of them to store whole 128-byte rows.
-    unsigned char *turn = lds + wave * 4096;
-    const int64_t trow = m0 + wm * WTM, tcol = n0 + wn * WTN;
-    if (acc_out) {
+    for (int t = blockIdx.x; t < total; t += gridDim.x) {
+        int tm, tn;
+        tile_of_block(t, tiles_m, tiles_n, tm, tn);
+        const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+        if (!fetched) {
+            gx = X + m0 * K;
+            gw = W + n0 * K;
+            AXI8_ISSUE(0);
+            fetch_cols(n0);
+        }
+        // Per-channel scale (premultiplied by x_scale) and bias of this tile's 256 columns go to
+        // LDS, so the write-back does not wait on global loads.
+        if (out && tid < 128) {
+            const int c4 = (tid & 63) * 4;
+            if (tid < 64) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) col_v[e] = x_scale * col_v[e];
+                *reinterpret_cast<v4f_t *>(lds_scale + c4) = col_v;
+            } else {
+                *reinterpret_cast<v4f_t *>(lds_bias + c4) = col_v;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
+
+        if (fetched) AXI8_VM(32); else AXI8_VM(0);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        if (slabs > 1) AXI8_ISSUE(1);
+        AXI8_FRAGS(0, 0, 0);
+
+        for (int s = 0; s < slabs; s += 2) {       // the flags are wave-uniform: scalar branches only
+            AXI8_SLAB(0, s + 2 < slabs);
+            if (s + 1 < slabs) AXI8_SLAB(1, s + 3 < slabs);
+        }
+        AXI8_WAIT_FRAGS();      // the stale reads must land before their registers are reused
+
+        const int t_next = t + (int)gridDim.x;
+        fetched = carry && t_next < total;
+        if (fetched) {
+            int tm2, tn2;
+            tile_of_block(t_next, tiles_m, tiles_n, tm2, tn2);
+            gx = X + (int64_t)tm2 * BM * K;
+            gw = W + (int64_t)tn2 * BN * K;
+            AXI8_ISSUE(0);
+            fetch_cols((int64_t)tn2 * BN);
+        }
+
+        // Write-back.  With W as the MFMA's first operand, register v of lane l holds
+        // m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3): four consecutive n per lane.
+        // Stage 1 of X is dead after the loop's last barrier; each wave turns its tiles through
+        // 4 KiB of it to store whole 128-byte rows.
+        unsigned char *turn = lds + OPER + wave * 4096;
+        const int64_t trow = m0 + wm * WTM, tcol = n0 + wn * WTN;
+        if (acc_out) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    v4i r[4];
+#pragma unroll
+                    for (int g = 0; g < 4; g++)
+                        r[g] = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    turn_tile_and_store(turn, lane, r, acc_out + (trow + i * 32) * N + tcol + j * 32, N);
+                }
+        }
+        if (out) {
+            const float *sp = lds_scale + wn * WTN + 4 * fhalf, *bp = lds_bias + wn * WTN + 4 * fhalf;
+            const bool has_bias = bias != nullptr;
+#pragma unroll
             for (int j = 0; j < TN; j++) {
-                v4i r[4];
+                v4f_t sc[4], bv[4];
 #pragma unroll
-                for (int g = 0; g < 4; g++)
-                    r[g] = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                turn_tile_and_store(turn, lane, r, acc_out + (trow + i * 32) * N + tcol + j * 32, N);
-            }
-    }
-    if (out) {
-        const float *sp = lds_scale + wn * WTN + 4 * fhalf, *bp = lds_bias + wn * WTN + 4 * fhalf;
-        const bool has_bias = bias != nullptr;
+                for (int g = 0; g < 4; g++) {
+                    sc[g] = *reinterpret_cast<const v4f_t *>(sp + j * 32 + 8 * g);
+                    bv[g] = *reinterpret_cast<const v4f_t *>(bp + j * 32 + 8 * g);
+                }
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            v4f_t sc[4], bv[4];
+                for (int i = 0; i < TM; i++) {
+                    v4f_t r[4];
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                sc[g] = *reinterpret_cast<const v4f_t *>(sp + j * 32 + 8 * g);
-                bv[g] = *reinterpret_cast<const v4f_t *>(bp + j * 32 + 8 * g);
-            }
+                    for (int g = 0; g < 4; g++)
 #pragma unroll
-            for (int i = 0; i < TM; i++) {
-                v4f_t r[4];
-#pragma unroll
-                for (int g = 0; g < 4; g++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const float f = (float)acc[i][j][4 * g + e];
-                        // a fused multiply-add with bias = 0 would round differently from the plain product
-                        r[g][e] = apply_act(has_bias ? __builtin_fmaf(f, sc[g][e], bv[g][e]) : f * sc[g][e], ACT);
-                    }
-                turn_tile_and_store(turn, lane, r, out + (trow + i * 32) * N + tcol + j * 32, N);
+                        for (int e = 0; e < 4; e++) {
+                            const float f = (float)acc[i][j][4 * g + e];
+                            // a fused multiply-add with bias = 0 would round differently from the plain product
+                            r[g][e] = apply_act(has_bias ? __builtin_fmaf(f, sc[g][e], bv[g][e]) : f * sc[g][e], ACT);
+                        }
+                    turn_tile_and_store(turn, lane, r, out + (trow + i * 32) * N + tcol + j * 32, N);
+                }
             }
         }
+        // Every wave is done with lds_scale / lds_bias and the turn area before the next tile
+        // overwrites them.  Only LDS traffic is ordered here: waiting for the stores as well
+        // (as __syncthreads would) is exactly what the persistent loop avoids.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
 }
 #undef AXI8_ISSUE
@@ -454,7 +496,8 @@ int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_s
     const int64_t tiles = (M / 256) * (N / 256);
     if (tiles > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: too many tiles");
     note_kernel("qgemm_w8a8_256x256_dma");
-    hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles), dim3(512), smem, kStream, x, w, M, N, K,
+    const int64_t grid = tiles < cu_count() ? tiles : cu_count();     // one persistent workgroup per CU
+    hipLaunchKernelGGL(kerns[act], dim3((unsigned)grid), dim3(512), smem, kStream, x, w, M, N, K,
                        x_scale, w_scales, bias, out, acc_out);
     return check_launch("qgemm_w8a8_256x256_dma");
 }

@@ -11,6 +11,7 @@ thread_local const char *t_kernel = "";
 int g_ready = 0;            // 1 once a gfx950-class device was initialised
 int g_devices = -1;
 char g_name[128] = "";
+int g_cu_count = 0;
 void *g_ws = nullptr;
 size_t g_ws_bytes = 0;
 int *g_ctr = nullptr;
@@ -26,6 +27,8 @@ int fail(int code, const char *fmt, ...) {
     va_end(ap);
     return code;
 }
+
+int cu_count() { return g_cu_count; }
 
 void note_kernel(const char *name) { t_kernel = name; }
 
@@ -99,6 +102,7 @@ int axhip_init(void) {
     hipDeviceProp_t prop;
     AXHIP_HIP_TRY(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties");
     snprintf(g_name, sizeof g_name, "%s", prop.gcnArchName);
+    g_cu_count = prop.multiProcessorCount;
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(AXHIP_ERR_BACKEND, "device 0 is %s; this library holds gfx950 code only",
                     prop.gcnArchName);
