@@ -27,6 +27,11 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, TOP/s
 PEAK_FP32_TFLOPS = 157.3     # MI355X fp32 matrix, TFLOP/s
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
+# Bytes that cross the L2 boundary per headline launch, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of `bench.py --counter-probe`, each scaled by what the same counter reads for
+# the probe's copy-shaped kernel of known size (profiles/qgemm_w8a8_256_8192cube_hbm_counters.txt):
+# 806.3 MB fetched (the counter under-reads by 2.000) + 268.4 MB written (scale 1.000).
+HEADLINE_TRAFFIC_BYTES = 806.3e6 + 268.4e6
 
 
 def result_line(suite, case, metric, value):
@@ -279,7 +284,9 @@ def main():
                                "scales, X int8 + per-tensor scale, bias, fp32 out",
                    "M": h["M"], "N": h["N"], "K": h["K"], "device": hip.L.axhip_device_name().decode()},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                     "frac": achieved / PEAK_INT8_TOPS, "traffic": None, "kernel": h["kernel"],
+                     "frac": achieved / PEAK_INT8_TOPS,
+                     "traffic": HEADLINE_TRAFFIC_BYTES if h["kernel"] == "qgemm_w8a8_256x256_dma" else None,
+                     "kernel": h["kernel"],
                      "kernel_us": h["event_ms"] * 1e3, "algorithmic_ops": h["ops"],
                      "algorithmic_bytes": h["algorithmic_bytes"]},
     }
