@@ -19,6 +19,8 @@ using namespace axhip;
 constexpr int COLS = 64;        // columns per workgroup
 constexpr int KGROUPS = 16;     // lane groups per workgroup, each 16 lanes x float4
 constexpr int UNROLL = 8;
+// workgroups to aim for: enough to cover 256 CUs a few times over; partial-sum traffic grows with M
+int64_t g_want_blocks_m12 = 1024, g_want_blocks_m38 = 512;
 
 template <int MR, bool VEC>
 __global__ void __launch_bounds__(256)
@@ -100,6 +102,23 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
             }
         }
     } else {
+        // all loads of a batch of rows are issued before the first use, as in the vector form
+        for (; k + (UNROLL - 1) * KGROUPS < klen; k += UNROLL * KGROUPS) {
+            float w[UNROLL][4];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    w[u][e] = (col + e < N) ? bp[(k_begin + k + u * KGROUPS) * ldb + e] : 0.0f;
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                for (int m = 0; m < MR; m++) {
+                    const float xv = xs[m * k_per_split + k + u * KGROUPS];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[m][e] = __builtin_fmaf(xv, w[u][e], acc[m][e]);
+                }
+        }
         for (; k < klen; k += KGROUPS) {
             float w[4];
 #pragma unroll
@@ -211,7 +230,7 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
 
     const int64_t col_blocks = (N + COLS - 1) / COLS;
     // enough workgroups to cover 256 CUs a few times over, each with at least 128 k rows
-    const int64_t want_blocks = M <= 2 ? 1024 : 512;   // partial traffic grows with M
+    const int64_t want_blocks = M <= 2 ? g_want_blocks_m12 : g_want_blocks_m38;
     int64_t splits = (want_blocks + col_blocks - 1) / col_blocks;
     const int64_t max_splits = K >= 128 ? K / 128 : 1;
     if (splits > max_splits) splits = max_splits;
