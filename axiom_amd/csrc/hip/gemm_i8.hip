@@ -477,6 +477,220 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 #undef AXI8_LOAD_W
 #undef AXI8_SLAB
 
+// ---------------------------------------------------------------------------------------
+// Mid-size aligned shapes (M, N multiples of the tile, K a multiple of 128) that cannot fill
+// the chip with 256x256 tiles: the same direct-to-LDS, VALU-free loop over smaller tiles with
+// NST LDS stages, so NST-1 slabs of loads are in flight per workgroup (a 64x64 tile has only
+// 128 MFMA cycles of work per slab and wave: the loop is bound by load latency and by the
+// CU's L1 bandwidth, not by the matrix core).  LDS: NST stages of X (BM rows x 128 B), NST
+// stages of W, then BN scales and BN biases.  Not persistent.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int ACT>
+__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64)
+k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
+                 int64_t K, float x_scale, const float *__restrict__ w_scales,
+                 const float *__restrict__ bias, float *__restrict__ out,
+                 int32_t *__restrict__ acc_out) {
+    constexpr int NW = WAVES_M * WAVES_N, BKB = 128;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
+    constexpr int XS = BM * BKB, WS = BN * BKB;          // bytes of one stage of each operand
+    constexpr int W_BASE = NST * XS;
+    constexpr int IPW_X = BM / 8 / NW, IPW_W = BN / 8 / NW;   // load instructions per wave and slab
+    constexpr int NREADS = TM + TN;
+    constexpr int VM_KEEP = (NST - 2) * (IPW_X + IPW_W);
+    static_assert(IPW_X * 8 * NW == BM && IPW_W * 8 * NW == BN, "slab must divide over the waves");
+    static_assert(NST >= 2 && NST <= 4 && VM_KEEP < 64, "stage count");
+    static_assert((NST - 1) * XS + (TM - 1) * 4096 < 65536 && (NST - 1) * WS + (TN - 1) * 4096 < 65536,
+                  "ds_read immediates are 16 bits");
+    static_assert(NW * 4096 <= NST * XS, "write-back turn area");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    int tm, tn;
+    tile_of_block(blockIdx.x, (int)(M / BM), (int)(N / BN), tm, tn);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int slabs = (int)(K / BKB);
+
+    // load instruction q fills rows q*8 .. q*8+7 of an operand stage; wave w issues q = j*NW + w
+    unsigned vx[IPW_X], vw[IPW_W];
+#pragma unroll
+    for (int j = 0; j < IPW_X; j++) {
+        const int row = (j * NW + wave) * 8 + (lane >> 3);
+        vx[j] = (unsigned)(row * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+    }
+#pragma unroll
+    for (int j = 0; j < IPW_W; j++) {
+        const int row = (j * NW + wave) * 8 + (lane >> 3);
+        vw[j] = (unsigned)(row * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+    }
+    const int8_t *gx = X + m0 * K, *gw = W + n0 * K;
+    const unsigned lds0 = (unsigned)(uintptr_t)lds, lds_w = lds0 + wave * 1024;
+
+    const int frow = lane & 31, fhalf = lane >> 5;
+    unsigned rx[4], rw[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+        const unsigned inrow = (unsigned)(frow * BKB + (((ks * 2 + fhalf) ^ ((frow >> 1) & 7)) << 4));
+        rx[ks] = lds0 + wm * WTM * BKB + inrow;
+        rw[ks] = lds0 + W_BASE + wn * WTN * BKB + inrow;
+    }
+
+    typedef float v4f_t __attribute__((ext_vector_type(4)));
+    float *lds_scale = reinterpret_cast<float *>(lds + NST * (XS + WS)), *lds_bias = lds_scale + BN;
+    if (out) {
+        for (int c = tid; c < BN; c += NW * 64) {
+            lds_scale[c] = x_scale * w_scales[n0 + c];
+            lds_bias[c] = bias ? bias[n0 + c] : 0.0f;
+        }
+    }
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
+    v4i fx[2][TM], fw[2][TN];
+
+#define AXI8G_ISSUE(ST)                                                                          \
+    do {                                                                                         \
+        _Pragma("unroll") for (int j = 0; j < IPW_X; j++)                                        \
+            AXI8_LOAD_LDS(lds_w + (ST) * XS + j * NW * 1024, vx[j], gx);                         \
+        _Pragma("unroll") for (int j = 0; j < IPW_W; j++)                                        \
+            AXI8_LOAD_LDS(lds_w + W_BASE + (ST) * WS + j * NW * 1024, vw[j], gw);                \
+        gx += BKB;                                                                               \
+        gw += BKB;                                                                               \
+    } while (0)
+#define AXI8G_FRAGS(buf, ST, ks)                                                                 \
+    do {                                                                                         \
+        _Pragma("unroll") for (int t = 0; t < TM; t++)                                           \
+            AXI8_DS_READ(fx[buf][t], rx[ks], (ST) * XS + t * 4096);                              \
+        _Pragma("unroll") for (int t = 0; t < TN; t++)                                           \
+            AXI8_DS_READ(fw[buf][t], rw[ks], (ST) * WS + t * 4096);                              \
+    } while (0)
+#define AXI8G_MFMAS(buf)                                                                         \
+    do {                                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+        _Pragma("unroll") for (int i = 0; i < TM; i++)                                           \
+            _Pragma("unroll") for (int j = 0; j < TN; j++)                                       \
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[buf][j], fx[buf][i],        \
+                                                                  acc[i][j], 0, 0, 0);           \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    } while (0)
+    // one slab out of stage ST; `more`: slab s+NST-1 exists and is fetched into the stage read last
+#define AXI8G_SLAB(ST, more)                                                                     \
+    do {                                                                                         \
+        if (more) AXI8G_ISSUE(((ST) + NST - 1) % NST);                                           \
+        AXI8G_FRAGS(0, ST, 0);                                                                   \
+        AXI8G_FRAGS(1, ST, 1);                                                                   \
+        AXI8_LGKM(NREADS);                                                                       \
+        AXI8G_MFMAS(0);                                                                          \
+        AXI8G_FRAGS(0, ST, 2);                                                                   \
+        AXI8_LGKM(NREADS);                                                                       \
+        AXI8G_MFMAS(1);                                                                          \
+        AXI8G_FRAGS(1, ST, 3);                                                                   \
+        AXI8_LGKM(NREADS);                                                                       \
+        AXI8G_MFMAS(0);                                                                          \
+        AXI8_LGKM(0);                                                                            \
+        AXI8G_MFMAS(1);                                                                          \
+        if (VM_KEEP > 0 && (more)) AXI8_VM(VM_KEEP); else AXI8_VM(0);                            \
+        __builtin_amdgcn_s_barrier();                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    } while (0)
+
+    AXI8G_ISSUE(0);
+    if constexpr (NST > 2) { if (slabs > 1) AXI8G_ISSUE(1); }
+    if constexpr (NST > 3) { if (slabs > 2) AXI8G_ISSUE(2); }
+    AXI8_VM(0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    for (int s = 0; s < slabs; s += NST) {
+        AXI8G_SLAB(0, s + NST - 1 < slabs);
+        if (s + 1 < slabs) {
+            AXI8G_SLAB(1, s + NST < slabs);
+            if constexpr (NST > 2) {
+                if (s + 2 < slabs) {
+                    AXI8G_SLAB(2, s + NST + 1 < slabs);
+                    if constexpr (NST > 3) {
+                        if (s + 3 < slabs) AXI8G_SLAB(3, s + NST + 2 < slabs);
+                    }
+                }
+            }
+        }
+    }
+#undef AXI8G_ISSUE
+#undef AXI8G_FRAGS
+#undef AXI8G_MFMAS
+#undef AXI8G_SLAB
+
+    // write-back as in the 256x256 kernel: through 4 KiB of dead stage per wave
+    unsigned char *turn = lds + wave * 4096;
+    const int64_t trow = m0 + wm * WTM, tcol = n0 + wn * WTN;
+    if (acc_out) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                v4i r[4];
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    r[g] = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                turn_tile_and_store(turn, lane, r, acc_out + (trow + i * 32) * N + tcol + j * 32, N);
+            }
+    }
+    if (out) {
+        const float *sp = lds_scale + wn * WTN + 4 * fhalf, *bp = lds_bias + wn * WTN + 4 * fhalf;
+        const bool has_bias = bias != nullptr;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            v4f_t sc[4], bv[4];
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                sc[g] = *reinterpret_cast<const v4f_t *>(sp + j * 32 + 8 * g);
+                bv[g] = *reinterpret_cast<const v4f_t *>(bp + j * 32 + 8 * g);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                v4f_t r[4];
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float f = (float)acc[i][j][4 * g + e];
+                        r[g][e] = apply_act(has_bias ? __builtin_fmaf(f, sc[g][e], bv[g][e]) : f * sc[g][e], ACT);
+                    }
+                turn_tile_and_store(turn, lane, r, out + (trow + i * 32) * N + tcol + j * 32, N);
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+int launch_dma(const char *name, const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
+               const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K) {
+    constexpr int smem = NST * (BM + BN) * 128 + 2 * BN * 4;
+    typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
+                           const float *, float *, int32_t *);
+    static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU>};
+    static bool attr_set = false;
+    if (!attr_set) {
+        for (kern_t kf : kerns)
+            AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kf),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, smem),
+                          "hipFuncSetAttribute");
+        attr_set = true;
+    }
+    const int64_t tiles = (M / BM) * (N / BN);
+    if (tiles > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: too many tiles");
+    note_kernel(name);
+    hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles), dim3(WAVES_M * WAVES_N * 64), smem, kStream, x, w,
+                       M, N, K, x_scale, w_scales, bias, out, acc_out);
+    return check_launch(name);
+}
+
 int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
                const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N,
                int64_t K) {
@@ -521,6 +735,14 @@ extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
     if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128 &&
         K < (int64_t(1) << 24))   // per-lane 32-bit byte offsets span 256 rows
         return launch_256(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K);
+    // aligned but too few 256x256 tiles: direct-to-LDS kernel over smaller tiles
+    if (aligned && vec_out && K % 128 == 0 && M % 64 == 0 && N % 64 == 0 && K < (int64_t(1) << 24)) {
+        if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 512)
+            return launch_dma<128, 128, 2, 2, 3>("qgemm_w8a8_128x128_dma", x, x_scale, w, w_scales, bias,
+                                                 act, out, acc_out, M, N, K);
+        return launch_dma<64, 64, 2, 2, 4>("qgemm_w8a8_64x64_dma", x, x_scale, w, w_scales, bias, act,
+                                           out, acc_out, M, N, K);
+    }
     // fewer than ~3/4 of the 256 CUs busy with 128x128 tiles: quarter the tile instead
     if (aligned && M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 192)
         return launch<128, 128, 2, 2, false>("qgemm_w8a8_128x128", x, x_scale, w, w_scales, bias,
