@@ -69,17 +69,23 @@ def test_w8a8_extreme_values_and_golden(hip, oracle, golden):
         assert np.array_equal(acc.numpy().astype(np.float64), golden[f"acc_K{K}"].astype(np.float64))
 
 
-def test_w8a8_8192_cube_properties(hip, oracle):
-    """Full size of the headline config: exact row/column checksums and 4096 sampled entries."""
-    M = N = K = 8192
-    oracle.seed(8192)
+@pytest.mark.parametrize("M,N,K", [(8192, 8192, 8192), (4096, 8192, 384), (4096, 8192, 512), (2048, 4096, 128)])
+def test_w8a8_persistent_tiles_properties(hip, oracle, M, N, K):
+    """Shapes served by the persistent 256x256 kernel, several tiles per workgroup, with an even
+    slab count (next tile's first slab fetched under the write-back), an odd one, and one slab;
+    the first is the full size of the headline config.  Exact row/column checksums and 4096
+    sampled entries of the accumulators; the fp32 output of the out-only call (the form the
+    benchmark times) against the epilogue applied to those accumulators."""
+    oracle.seed(M + N + K)
     x, w = oracle.int8((M, K)), oracle.int8((N, K))
     ws = oracle.uniform((N,), 1e-3, 1e-2)
     bias = oracle.normal((N,), 0.0, 0.02)
     xs = float(np.float32(0.011))
-    say("w8a8 8192^3 launch")
-    out, acc = hip.qgemm_w8a8(hip.array(x), xs, hip.array(w), hip.array(ws), hip.array(bias), 0)
+    dx, dw, dws, db = hip.array(x), hip.array(w), hip.array(ws), hip.array(bias)
+    say("w8a8 persistent", M, N, K)
+    out, acc = hip.qgemm_w8a8(dx, xs, dw, dws, db, 0)
     say("  kernel", hip.last_kernel())
+    assert hip.last_kernel() == "qgemm_w8a8_256x256_dma"
     a = acc.numpy()
     xi, wi = x.astype(np.int64), w.astype(np.int64)
     assert np.array_equal(a.astype(np.int64).sum(axis=0), wi @ xi.sum(axis=0))   # column sums
@@ -88,9 +94,15 @@ def test_w8a8_8192_cube_properties(hip, oracle):
     ms, ns = rng.integers(0, M, 4096), rng.integers(0, N, 4096)
     exact = np.einsum("ik,ik->i", xi[ms], wi[ns])
     assert np.array_equal(a[ms, ns].astype(np.int64), exact)
-    o = out.numpy()
-    want = oracle.w8a8_epilogue(np.ascontiguousarray(a[:64]), xs, ws, bias, 0)
-    assert np.array_equal(o[:64], want)
+    want = oracle.w8a8_epilogue(a, xs, ws, bias, 0)
+    assert np.array_equal(out.numpy(), want)
+    _, acc_only = hip.qgemm_w8a8(dx, xs, dw, None, None, 0, want_out=False)
+    assert np.array_equal(acc_only.numpy(), a)
+    for act in (0, 1):
+        out_only, _ = hip.qgemm_w8a8(dx, xs, dw, dws, db, act, want_acc=False)
+        assert np.array_equal(out_only.numpy(), np.maximum(want, 0) if act else want)
+    out_nb, _ = hip.qgemm_w8a8(dx, xs, dw, dws, None, 0, want_acc=False)
+    assert np.array_equal(out_nb.numpy(), oracle.w8a8_epilogue(a, xs, ws, None, 0))
 
 
 # ------------------------------------------------------------------ fp32 GEMM
@@ -119,6 +131,32 @@ def test_sgemm_nn_nt_tn(hip, oracle, M, N, K):
     got = hip.sgemm(hip.array(at), db, transa=True).numpy()
     say("  tn", hip.last_kernel())
     check_fp32(oracle, got, a, b, ref=ref)
+
+
+@pytest.mark.parametrize("M,N,K,pad,off", [(256, 384, 128, 64, 32), (2048, 4096, 64, 128, 64),
+                                           (256, 384, 128, 3, 1), (70, 50, 90, 5, 2)])
+def test_sgemm_submatrix_views(hip, oracle, M, N, K, pad, off):
+    """Operands and result are windows of larger row-major arrays (leading dimension > row
+    length, first element `off` floats into the allocation): multiples of 4 keep the
+    direct-to-LDS path, odd values must fall back to the guarded kernel; memory outside the C
+    window must stay untouched."""
+    oracle.seed(M + N + K + pad)
+    big_a, big_b = oracle.uniform((M, K + pad), -1, 1), oracle.uniform((K, N + pad), -1, 1)
+    big_bt = oracle.uniform((N, K + pad), -1, 1)
+    big_c = oracle.uniform((M, N + pad), -1, 1)
+    a, b = np.ascontiguousarray(big_a[:, off:off + K]), np.ascontiguousarray(big_b[:, off:off + N])
+    bt = np.ascontiguousarray(big_bt[:, off:off + K])
+    da, db, dbt = hip.array(big_a), hip.array(big_b), hip.array(big_bt)
+    for transb, dbb, ldb, href in ((0, db, N + pad, b), (1, dbt, K + pad, bt)):
+        dc = hip.array(big_c)
+        hip.check(hip.L.axhip_sgemm(0, transb, M, N, K, 1.0, da.ptr + 4 * off, K + pad, dbb.ptr + 4 * off, ldb,
+                                    0.0, dc.ptr + 4 * off, N + pad, None, 0))
+        say("  view", (M, N, K, pad, off), "transb", transb, hip.last_kernel())
+        got = dc.numpy()
+        check_fp32(oracle, np.ascontiguousarray(got[:, off:off + N]), a, href, transb=bool(transb))
+        mask = np.ones_like(big_c, bool)
+        mask[:, off:off + N] = False
+        assert np.array_equal(got[mask], big_c[mask])
 
 
 def test_sgemm_known_answers(hip, golden):
