@@ -592,16 +592,18 @@ int try_dma(const char *const names[4], const SgemmArgs &g, int64_t batch) {
                     g.M % 64 == 0 && g.N % 64 == 0 && (g.M / 64) * (g.N / 64) <= 0x7fffffff;
     if (!ok) return -1;
     auto count = [&](int64_t bm, int64_t bn) { return (g.M / bm) * (g.N / bn) * batch; };
-    if (g.M % 128 == 0 && g.N % 256 == 0 && count(128, 256) >= 256)
-        return launch_dma<128, 256, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
-    if (g.M % 128 == 0 && g.N % 128 == 0 && count(128, 128) >= 512)
-        return launch_dma<128, 128, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
-    // a tile that spans whole rows of C (ldc == 64) already writes contiguous memory
-    if (g.M % 128 == 0 && count(128, 64) >= 512)
-        return g.ldc == 64 ? launch_dma<128, 64, 2, 2, 3, A_KC, B_KC, 0>(names[2], g, batch)
-                           : launch_dma<128, 64, 2, 2, 3, A_KC, B_KC, 1>(names[2], g, batch);
-    return g.ldc == 64 ? launch_dma<64, 64, 2, 2, 3, A_KC, B_KC, 0>(names[3], g, batch)
-                       : launch_dma<64, 64, 2, 2, 3, A_KC, B_KC, 1>(names[3], g, batch);
+    // Two stages everywhere: sustained timings show no gain from three or four.  With only a
+    // few slabs per tile (K <= 128) a workgroup's life is mostly its loads and its write-back,
+    // and small tiles (several workgroups per CU) do slightly better.
+    if (g.K > 128) {
+        if (g.M % 128 == 0 && g.N % 256 == 0 && count(128, 256) >= 256)
+            return launch_dma<128, 256, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
+        if (g.M % 128 == 0 && g.N % 128 == 0 && count(128, 128) >= 512)
+            return launch_dma<128, 128, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
+        if (g.M % 128 == 0 && count(128, 64) >= 512)
+            return launch_dma<128, 64, 2, 2, 2, A_KC, B_KC, 1>(names[2], g, batch);
+    }
+    return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[3], g, batch);
 }
 
 int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
