@@ -334,9 +334,14 @@ template <> struct Frag<false> {
 #define AXF_DS128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 #define AXF_DS32(dst, addr, off) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI>
-__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g) {
-    constexpr int NW = WAVES_M * WAVES_N;
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI, int WAVES_K>
+__global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(SgemmArgs g) {
+    // WAVES_K == 2: a second set of waves shares each tile; set 0 multiplies k-blocks 0 and 1 of
+    // every slab, set 1 k-blocks 2 and 3, and the two accumulators are added through LDS at the
+    // end.  For 64x64 tiles with one workgroup per CU this puts two waves on every SIMD, so one
+    // wave's LDS and barrier waits are covered by the other's MFMAs.
+    constexpr int NW = WAVES_M * WAVES_N * WAVES_K;
+    static_assert(WAVES_K == 1 || WAVES_K == 2, "k split");
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
     using OA = DmaOperand<BM, A_KC, NW>;
     using OB = DmaOperand<BN, B_KC, NW>;
@@ -351,7 +356,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int wk = wave / (WAVES_M * WAVES_N), wmn = wave % (WAVES_M * WAVES_N);
+    const int wm = wmn / WAVES_N, wn = wmn % WAVES_N;
     int tm, tn;
     tile_of_block(blockIdx.x, (int)(g.M / BM), (int)(g.N / BN), tm, tn);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
@@ -380,8 +386,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
     for (int st = 0; st < NST; st++)
 #pragma unroll
         for (int kbi = 0; kbi < 4; kbi++) {
-            ra[st][kbi] = lds0 + st * OA::BYTES + OA::frag_base(wm * WTM, frow, fhalf, kbi);
-            rb[st][kbi] = lds0 + B_BASE + st * OB::BYTES + OB::frag_base(wn * WTN, frow, fhalf, kbi);
+            // with a k split, entries 0 and 1 address this wave set's own two k-blocks
+            const int kb = WAVES_K == 2 ? 2 * wk + (kbi & 1) : kbi;
+            ra[st][kbi] = lds0 + st * OA::BYTES + OA::frag_base(wm * WTM, frow, fhalf, kb) +
+                          (WAVES_K == 2 && !A_KC ? wk * OA::k_imm(16) : 0);
+            rb[st][kbi] = lds0 + B_BASE + st * OB::BYTES + OB::frag_base(wn * WTN, frow, fhalf, kb) +
+                          (WAVES_K == 2 && !B_KC ? wk * OB::k_imm(16) : 0);
         }
 
     v16f acc[TM][TN];
@@ -450,12 +460,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
         AXF_FRAGS(1, ST, 1);                                                                     \
         AXF_LGKM(NREADS);                                                                        \
         AXF_MFMAS(0);                                                                            \
-        AXF_FRAGS(0, ST, 2);                                                                     \
-        AXF_LGKM(NREADS);                                                                        \
-        AXF_MFMAS(1);                                                                            \
-        AXF_FRAGS(1, ST, 3);                                                                     \
-        AXF_LGKM(NREADS);                                                                        \
-        AXF_MFMAS(0);                                                                            \
+        if constexpr (WAVES_K == 1) {                                                            \
+            AXF_FRAGS(0, ST, 2);                                                                 \
+            AXF_LGKM(NREADS);                                                                    \
+            AXF_MFMAS(1);                                                                        \
+            AXF_FRAGS(1, ST, 3);                                                                 \
+            AXF_LGKM(NREADS);                                                                    \
+            AXF_MFMAS(0);                                                                        \
+        }                                                                                        \
         AXF_LGKM(0);                                                                             \
         AXF_MFMAS(1);                                                                            \
         if (VM_KEEP > 0 && (more)) AXF_VM(VM_KEEP); else AXF_VM(0);                              \
@@ -485,6 +497,25 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
 #undef AXF_FRAGS
 #undef AXF_MFMAS
 #undef AXF_SLAB
+
+    if constexpr (WAVES_K == 2) {
+        static_assert(TM == 1 && TN == 1, "the k split is for one 32x32 tile per wave");
+        float *sum = reinterpret_cast<float *>(lds_raw + wmn * 4096);   // the stages are dead now
+        if (wk == 1) {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                *reinterpret_cast<v4f *>(sum + (q * 64 + lane) * 4) =
+                    v4f{acc[0][0][4 * q], acc[0][0][4 * q + 1], acc[0][0][4 * q + 2], acc[0][0][4 * q + 3]};
+        }
+        __syncthreads();
+        if (wk == 1) return;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const v4f t = *reinterpret_cast<const v4f *>(sum + (q * 64 + lane) * 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[0][0][4 * q + e] += t[e];
+        }
+    }
 
     // register v of lane l: m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3)
     const bool use_beta = g.beta != 0.0f;
@@ -518,7 +549,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
         // contiguous bytes instead of 32 rows of 32.  Rows of 128 bytes, 16-byte chunk c of row
         // r kept at chunk c ^ ((r>>1)&7): both the write (16 rows, one chunk column) and the
         // read (2 rows, all chunks) of a 16-lane group then touch every bank once.
-        unsigned char *turn = lds_raw + wave * 4096;
+        unsigned char *turn = lds_raw + wmn * 4096;
         const int rrow = lane >> 3, rchunk = lane & 7;
         const int64_t col0 = n0 + wn * WTN + 4 * rchunk;
         float *dst = C + (m0 + wm * WTM + rrow) * g.ldc + col0;
@@ -562,10 +593,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm_dma(SgemmArgs g
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI = 1>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI = 1, int WAVES_K = 1>
 int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
-    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI>;
-    constexpr int NW = WAVES_M * WAVES_N;
+    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K>;
+    constexpr int NW = WAVES_M * WAVES_N * WAVES_K;
     constexpr int smem = NST * (DmaOperand<BM, A_KC, NW>::BYTES + DmaOperand<BN, B_KC, NW>::BYTES);
     static bool attr_set = false;
     if (!attr_set) {
@@ -582,9 +613,9 @@ int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
 
 // Chooses the largest tile that still leaves about eight waves per CU; returns -1 when the
 // shape does not qualify for the fast path (the caller then uses the register-staged kernel).
-// names: 128x256, 128x128, 128x64, 64x64.
+// names: 128x256, 128x128, 128x64, 64x64, 64x64 with the k split.
 template <bool A_KC, bool B_KC>
-int try_dma(const char *const names[4], const SgemmArgs &g, int64_t batch) {
+int try_dma(const char *const names[5], const SgemmArgs &g, int64_t batch) {
     const bool ok = g.K % 32 == 0 && g.K > 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                     ((uintptr_t)g.C % 16 == 0) && ((uintptr_t)g.bias % 16 == 0) && g.lda % 4 == 0 &&
                     g.ldb % 4 == 0 && g.ldc % 4 == 0 && g.stride_a % 4 == 0 && g.stride_b % 4 == 0 &&
@@ -602,6 +633,8 @@ int try_dma(const char *const names[4], const SgemmArgs &g, int64_t batch) {
             return launch_dma<128, 128, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
         if (g.M % 128 == 0 && count(128, 64) >= 512)
             return launch_dma<128, 64, 2, 2, 2, A_KC, B_KC, 1>(names[2], g, batch);
+        // 64x64 with the k split: 8 waves per tile, two per SIMD even at one workgroup per CU
+        return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[4], g, batch);
     }
     return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[3], g, batch);
 }
@@ -610,9 +643,12 @@ int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     static const char *const nn[3] = {"sgemm_nn_128x128", "sgemm_nn_64x64", "sgemm_nn_64x64_guarded"};
     static const char *const nt[3] = {"sgemm_nt_128x128", "sgemm_nt_64x64", "sgemm_nt_64x64_guarded"};
     static const char *const tn[3] = {"sgemm_tn_128x128", "sgemm_tn_64x64", "sgemm_tn_64x64_guarded"};
-    static const char *const nn_d[4] = {"sgemm_nn_128x256_dma", "sgemm_nn_128x128_dma", "sgemm_nn_128x64_dma", "sgemm_nn_64x64_dma"};
-    static const char *const nt_d[4] = {"sgemm_nt_128x256_dma", "sgemm_nt_128x128_dma", "sgemm_nt_128x64_dma", "sgemm_nt_64x64_dma"};
-    static const char *const tn_d[4] = {"sgemm_tn_128x256_dma", "sgemm_tn_128x128_dma", "sgemm_tn_128x64_dma", "sgemm_tn_64x64_dma"};
+    static const char *const nn_d[5] = {"sgemm_nn_128x256_dma", "sgemm_nn_128x128_dma", "sgemm_nn_128x64_dma",
+                                         "sgemm_nn_64x64_dma", "sgemm_nn_64x64k2_dma"};
+    static const char *const nt_d[5] = {"sgemm_nt_128x256_dma", "sgemm_nt_128x128_dma", "sgemm_nt_128x64_dma",
+                                         "sgemm_nt_64x64_dma", "sgemm_nt_64x64k2_dma"};
+    static const char *const tn_d[5] = {"sgemm_tn_128x256_dma", "sgemm_tn_128x128_dma", "sgemm_tn_128x64_dma",
+                                         "sgemm_tn_64x64_dma", "sgemm_tn_64x64k2_dma"};
     int rc = -1;
     if (!transa && !transb) rc = try_dma<true, false>(nn_d, g, batch);
     else if (!transa && transb) rc = try_dma<true, true>(nt_d, g, batch);
