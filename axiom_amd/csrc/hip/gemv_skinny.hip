@@ -52,10 +52,10 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
     }
 
     float *xs = sm;
-    for (int64_t i = tid; i < (int64_t)MR * klen; i += 256) {
-        int64_t m = i / klen, kk = i - m * klen;
-        xs[m * k_per_split + kk] = A[m * lda + k_begin + kk];
-    }
+    const int klen32 = (int)klen;
+#pragma unroll
+    for (int m = 0; m < MR; m++)            // no division by the run-time split length
+        for (int kk = tid; kk < klen32; kk += 256) xs[m * (int)k_per_split + kk] = A[m * lda + k_begin + kk];
     __syncthreads();
 
     float acc[MR][4];
@@ -174,27 +174,45 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
     }
     __syncthreads();
     if (!last_flag) return;
-    for (int i = tid; i < MR * COLS; i += 256) {
-        const int m = i / COLS, c = i % COLS;
-        const int64_t n = n0 + c;
-        if (n >= N) continue;
-        const float *pp = dst + m * dst_ld + n;
-        float s = 0.0f;
-        int p = 0;
-        for (; p + 8 <= splits; p += 8) {           // loads independent, additions in split order
-            float v[8];
+    // Each thread owns up to OUTS outputs.  All partials of a chunk of splits are requested
+    // before the first is used (one trip to memory per chunk, not per split); they are added
+    // in split order.
+    constexpr int OUTS = (MR * COLS + 255) / 256, CHUNK = 16;
+    const float *pp[OUTS];
+    float s[OUTS];
+    bool ok[OUTS];
 #pragma unroll
-            for (int u = 0; u < 8; u++)
-                v[u] = __int_as_float(__hip_atomic_load(reinterpret_cast<const int *>(pp + (int64_t)(p + u) * dst_split_stride),
-                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    for (int o = 0; o < OUTS; o++) {
+        const int i = tid + o * 256, m = i / COLS, c = i % COLS;
+        ok[o] = i < MR * COLS && n0 + c < N;
+        pp[o] = dst + m * dst_ld + n0 + c;
+        s[o] = 0.0f;
+    }
+    for (int p0 = 0; p0 < splits; p0 += CHUNK) {
+        float v[OUTS][CHUNK];
 #pragma unroll
-            for (int u = 0; u < 8; u++) s += v[u];
-        }
-        for (; p < splits; p++)
-            s += __int_as_float(__hip_atomic_load(reinterpret_cast<const int *>(pp + (int64_t)p * dst_split_stride),
-                                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        if (bias) s += bias[n];
-        C[m * ldc + n] = apply_act(s, act);
+        for (int o = 0; o < OUTS; o++)
+#pragma unroll
+            for (int u = 0; u < CHUNK; u++)
+                v[o][u] = (ok[o] && p0 + u < splits)
+                              ? __int_as_float(__hip_atomic_load(
+                                    reinterpret_cast<const int *>(pp[o] + (int64_t)(p0 + u) * dst_split_stride),
+                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                              : 0.0f;
+#pragma unroll
+        for (int o = 0; o < OUTS; o++)
+#pragma unroll
+            for (int u = 0; u < CHUNK; u++)
+                if (p0 + u < splits) s[o] += v[o][u];
+    }
+#pragma unroll
+    for (int o = 0; o < OUTS; o++) {
+        if (!ok[o]) continue;
+        const int i = tid + o * 256, m = i / COLS;
+        const int64_t n = n0 + i % COLS;
+        float r = s[o];
+        if (bias) r += bias[n];
+        C[m * ldc + n] = apply_act(r, act);
     }
     if (tid == 0)                                   // ready for the next launch
         __hip_atomic_store(counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
