@@ -42,7 +42,20 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
     const int64_t col = n0 + 4 * cg;
     const float *bp = B + col;
     int64_t k = kg;
-    // first batch of weights in flight before anything else (VEC form, full batch available)
+    // Activations of this split go to LDS.  Their loads (L2 hits, every workgroup reads the same
+    // few rows) are issued first and the first batch of weights right behind them: loads return
+    // in issue order, so the staging then waits only for the activations while the weights are
+    // on their way from HBM.
+    const int klen32 = (int)klen;
+    float xr[MR][2];
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int kk = tid + c * 256;
+            xr[m][c] = kk < klen32 ? A[m * lda + k_begin + kk] : 0.0f;
+        }
+    // first batch of weights (VEC form, full batch available)
     const bool pre = VEC && col < N && (UNROLL - 1) * KGROUPS + kg < klen;
     v4f w0[UNROLL];
     if (pre) {
@@ -52,10 +65,16 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
     }
 
     float *xs = sm;
-    const int klen32 = (int)klen;
 #pragma unroll
-    for (int m = 0; m < MR; m++)            // no division by the run-time split length
-        for (int kk = tid; kk < klen32; kk += 256) xs[m * (int)k_per_split + kk] = A[m * lda + k_begin + kk];
+    for (int m = 0; m < MR; m++) {
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int kk = tid + c * 256;
+            if (kk < klen32) xs[m * (int)k_per_split + kk] = xr[m][c];
+        }
+        for (int kk = tid + 512; kk < klen32; kk += 256)      // splits longer than 512 rows
+            xs[m * (int)k_per_split + kk] = A[m * lda + k_begin + kk];
+    }
     __syncthreads();
 
     float acc[MR][4];
