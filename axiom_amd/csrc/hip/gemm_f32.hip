@@ -475,13 +475,17 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         __builtin_amdgcn_sched_barrier(0);                                                       \
     } while (0)
 
+    // When K is exactly NST slabs the whole of it fits the stages: everything is fetched at once
+    // (one load latency per tile instead of two) and the loop issues nothing.
+    const bool ring = slabs != NST;
     AXF_ISSUE(0);
     if constexpr (NST > 2) { if (slabs > 1) AXF_ISSUE(1); }
     if constexpr (NST > 3) { if (slabs > 2) AXF_ISSUE(2); }
+    if (!ring) AXF_ISSUE(NST - 1);
     AXF_VM(0);
     __builtin_amdgcn_s_barrier();
     for (int s = 0; s < slabs; s += NST) {
-        AXF_SLAB(0, s + NST - 1 < slabs);
+        AXF_SLAB(0, ring && s + NST - 1 < slabs);
         if (s + 1 >= slabs) break;
         AXF_SLAB(1, s + NST < slabs);
         if constexpr (NST > 2) {
