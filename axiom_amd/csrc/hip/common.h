@@ -22,6 +22,8 @@ void *workspace(size_t bytes);
 // `n` zero-initialised device ints owned by the runtime.  Kernels that use them as arrival counters
 // leave them at zero when they finish.
 int *strip_counters(size_t n);
+// At least `n` device floats, all 1.0f, owned by the runtime (grown on demand).
+float *ones_vector(size_t n);
 
 constexpr hipStream_t kStream = nullptr;
 

@@ -617,9 +617,9 @@ int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
 
 // Chooses the largest tile that still leaves about eight waves per CU; returns -1 when the
 // shape does not qualify for the fast path (the caller then uses the register-staged kernel).
-// names: 128x256, 128x128, 128x64, 64x64, 64x64 with the k split.
+// names: 128x256, 64x64, 64x64 with the k split.
 template <bool A_KC, bool B_KC>
-int try_dma(const char *const names[5], const SgemmArgs &g, int64_t batch) {
+int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
     const bool ok = g.K % 32 == 0 && g.K > 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                     ((uintptr_t)g.C % 16 == 0) && ((uintptr_t)g.bias % 16 == 0) && g.lda % 4 == 0 &&
                     g.ldb % 4 == 0 && g.ldc % 4 == 0 && g.stride_a % 4 == 0 && g.stride_b % 4 == 0 &&
@@ -627,32 +627,26 @@ int try_dma(const char *const names[5], const SgemmArgs &g, int64_t batch) {
                     g.M % 64 == 0 && g.N % 64 == 0 && (g.M / 64) * (g.N / 64) <= 0x7fffffff;
     if (!ok) return -1;
     auto count = [&](int64_t bm, int64_t bn) { return (g.M / bm) * (g.N / bn) * batch; };
-    // Two stages everywhere: sustained timings show no gain from three or four.  With only a
-    // few slabs per tile (K <= 128) a workgroup's life is mostly its loads and its write-back,
-    // and small tiles (several workgroups per CU) do slightly better.
+    // Sustained timings over the benchmark shapes: 128x256 (8 waves, one workgroup per CU) wins
+    // once it fills the chip; below that 64x64 tiles with the k split beat 128x128 and 128x64
+    // everywhere, and two stages are as good as three or four.  With only a few slabs per tile
+    // (K <= 128) a workgroup's life is mostly its loads and its write-back: plain 64x64 tiles,
+    // several workgroups per CU.
     if (g.K > 128) {
         if (g.M % 128 == 0 && g.N % 256 == 0 && count(128, 256) >= 256)
             return launch_dma<128, 256, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
-        if (g.M % 128 == 0 && g.N % 128 == 0 && count(128, 128) >= 512)
-            return launch_dma<128, 128, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
-        if (g.M % 128 == 0 && count(128, 64) >= 512)
-            return launch_dma<128, 64, 2, 2, 2, A_KC, B_KC, 1>(names[2], g, batch);
-        // 64x64 with the k split: 8 waves per tile, two per SIMD even at one workgroup per CU
-        return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[4], g, batch);
+        return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[2], g, batch);
     }
-    return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[3], g, batch);
+    return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
 }
 
 int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     static const char *const nn[3] = {"sgemm_nn_128x128", "sgemm_nn_64x64", "sgemm_nn_64x64_guarded"};
     static const char *const nt[3] = {"sgemm_nt_128x128", "sgemm_nt_64x64", "sgemm_nt_64x64_guarded"};
     static const char *const tn[3] = {"sgemm_tn_128x128", "sgemm_tn_64x64", "sgemm_tn_64x64_guarded"};
-    static const char *const nn_d[5] = {"sgemm_nn_128x256_dma", "sgemm_nn_128x128_dma", "sgemm_nn_128x64_dma",
-                                         "sgemm_nn_64x64_dma", "sgemm_nn_64x64k2_dma"};
-    static const char *const nt_d[5] = {"sgemm_nt_128x256_dma", "sgemm_nt_128x128_dma", "sgemm_nt_128x64_dma",
-                                         "sgemm_nt_64x64_dma", "sgemm_nt_64x64k2_dma"};
-    static const char *const tn_d[5] = {"sgemm_tn_128x256_dma", "sgemm_tn_128x128_dma", "sgemm_tn_128x64_dma",
-                                         "sgemm_tn_64x64_dma", "sgemm_tn_64x64k2_dma"};
+    static const char *const nn_d[3] = {"sgemm_nn_128x256_dma", "sgemm_nn_64x64_dma", "sgemm_nn_64x64k2_dma"};
+    static const char *const nt_d[3] = {"sgemm_nt_128x256_dma", "sgemm_nt_64x64_dma", "sgemm_nt_64x64k2_dma"};
+    static const char *const tn_d[3] = {"sgemm_tn_128x256_dma", "sgemm_tn_64x64_dma", "sgemm_tn_64x64k2_dma"};
     int rc = -1;
     if (!transa && !transb) rc = try_dma<true, false>(nn_d, g, batch);
     else if (!transa && transb) rc = try_dma<true, true>(nt_d, g, batch);

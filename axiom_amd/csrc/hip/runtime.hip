@@ -16,6 +16,8 @@ void *g_ws = nullptr;
 size_t g_ws_bytes = 0;
 int *g_ctr = nullptr;
 size_t g_ctr_n = 0;
+float *g_ones = nullptr;
+size_t g_ones_n = 0;
 }  // namespace
 
 namespace axhip {
@@ -59,6 +61,30 @@ void *workspace(size_t bytes) {
     }
     g_ws_bytes = want;
     return g_ws;
+}
+
+float *ones_vector(size_t n) {
+    if (n <= g_ones_n) return g_ones;
+    if (g_ones) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(g_ones);
+        g_ones = nullptr;
+        g_ones_n = 0;
+    }
+    size_t want = n < 65536 ? 65536 : n;
+    if (hipMalloc(reinterpret_cast<void **>(&g_ones), want * sizeof(float)) != hipSuccess) {
+        g_ones = nullptr;
+        fail(AXHIP_ERR_ALLOC, "ones vector (%zu floats): out of device memory", want);
+        return nullptr;
+    }
+    g_ones_n = want;      // set before the fill so a failure below still leaves a consistent size
+    if (axhip_fill_f32(g_ones, 1.0f, (int64_t)want) != AXHIP_OK) {
+        (void)hipFree(g_ones);
+        g_ones = nullptr;
+        g_ones_n = 0;
+        return nullptr;
+    }
+    return g_ones;
 }
 
 int *strip_counters(size_t n) {
@@ -115,6 +141,9 @@ void axhip_shutdown(void) {
     (void)hipDeviceSynchronize();
     if (g_ws) (void)hipFree(g_ws);
     if (g_ctr) (void)hipFree(g_ctr);
+    if (g_ones) (void)hipFree(g_ones);
+    g_ones = nullptr;
+    g_ones_n = 0;
     g_ws = nullptr;
     g_ws_bytes = 0;
     g_ctr = nullptr;

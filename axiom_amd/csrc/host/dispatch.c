@@ -141,6 +141,8 @@ ax_status_t ax_compute_relu(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPAT
 ax_status_t ax_compute_gelu(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(gelu_op, out, gelu_op(in, out)); }
 ax_status_t ax_compute_fill(ax_tensor_t *t, double value) { AX_DISPATCH(fill, t, fill(t, value)); }
 ax_status_t ax_compute_copy(const ax_tensor_t *src, ax_tensor_t *dst) { AX_DISPATCH(copy, dst, copy(src, dst)); }
+ax_status_t ax_compute_sum(const ax_tensor_t *in, int axis, ax_tensor_t *out) { AX_DISPATCH(sum, out, sum(in, axis, out)); }
+ax_status_t ax_compute_axpy(const ax_tensor_t *x, float alpha, ax_tensor_t *y) { AX_DISPATCH(axpy, y, axpy(x, alpha, y)); }
 ax_status_t ax_compute_gemm_bias_act(const ax_tensor_t *a, const ax_tensor_t *b, const ax_tensor_t *bias,
                                      ax_activation_t act, ax_tensor_t *out) {
     AX_DISPATCH(gemm_bias_act, out, gemm_bias_act(a, b, bias, (int)act, out));

@@ -209,6 +209,50 @@ static ax_status_t hip_bias_add(const ax_tensor_t *in, const ax_tensor_t *bias, 
     return lift(axhip_bias_add(ip, bp, outer, in->shape[axis], inner, op), "hip bias_add");
 }
 
+/* out = sum of `in` over `axis` (-1: over everything, out holds one element); the output must
+ * hold numel(in) / shape[axis] elements (cuda_sum, cuda/ops_reduce.cu:262-295). */
+static ax_status_t hip_sum(const ax_tensor_t *in, int axis, ax_tensor_t *out) {
+    float *ip, *op;
+    int64_t n, no;
+    ax_status_t st;
+    if (!in || !out) return AX_ERR_NULL_ARG;
+    if ((st = as_flat(in, "hip sum", &ip, &n)) || (st = as_flat(out, "hip sum", &op, &no))) return st;
+    if (axis == -1) {
+        if (no != 1) {
+            ax_err_set(AX_ERR_SHAPE_MISMATCH, "hip sum: full reduction needs a one-element output");
+            return AX_ERR_SHAPE_MISMATCH;
+        }
+        return lift(axhip_sum_all(ip, n, op), "hip sum");
+    }
+    if (axis < 0 || axis >= in->ndim) {
+        ax_err_set(AX_ERR_INVALID_AXIS, "axis %d out of range", axis);
+        return AX_ERR_INVALID_AXIS;
+    }
+    int64_t outer = 1, inner = 1;
+    for (int d = 0; d < axis; d++) outer *= in->shape[d];
+    for (int d = axis + 1; d < in->ndim; d++) inner *= in->shape[d];
+    if (no != outer * inner) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "hip sum: output holds %lld elements, expected %lld",
+                   (long long)no, (long long)(outer * inner));
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    return lift(axhip_sum_axis(ip, outer, in->shape[axis], inner, op), "hip sum");
+}
+
+/* y += alpha * x over matching element counts (cuda_axpy, cuda/ops_fused.cu:193-211) */
+static ax_status_t hip_axpy(const ax_tensor_t *x, float alpha, ax_tensor_t *y) {
+    float *xp, *yp;
+    int64_t nx, ny;
+    ax_status_t st;
+    if (!x || !y) return AX_ERR_NULL_ARG;
+    if ((st = as_flat(x, "hip axpy", &xp, &nx)) || (st = as_flat(y, "hip axpy", &yp, &ny))) return st;
+    if (nx != ny) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "hip axpy requires matching numel");
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    return lift(axhip_axpy(xp, alpha, yp, nx), "hip axpy");
+}
+
 /* ---- device-owner hooks ---- */
 static ax_status_t hook_init(void) { return lift(axhip_init(), "hip init"); }
 static void hook_shutdown(void) { axhip_shutdown(); }
@@ -229,6 +273,7 @@ static ax_status_t hook_d2d(void *d, const void *s, size_t n) { return lift(axhi
         .name = "hip", .gemm = hip_gemm, .gemm_nt = hip_gemm_nt, .gemm_tn = hip_gemm_tn,        \
         .gemm_relu = hip_gemm_relu, .gemm_ex = hip_gemm_ex, .bias_add = hip_bias_add,           \
         .fill = hip_fill, .copy = hip_copy, .relu = hip_relu, .gelu_op = hip_gelu,              \
+        .sum = hip_sum, .axpy = hip_axpy,                                                       \
         .device = (dev), .init = hook_init, .shutdown = hook_shutdown,                          \
         .synchronize = hook_synchronize, .device_count = hook_device_count,                     \
         .storage_alloc = hook_alloc, .storage_free = hook_free, .memcpy_h2d = hook_h2d,         \

@@ -131,6 +131,26 @@ def secondary(hip):
     res["fp32_ffn_2048x1024x4096"] = {"us": ms * 1e3, "TFLOP/s": tf,
                                       "frac_of_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS}
     result_line("axhip", "f32_ffn_2048x1024x4096", "gflops", tf * 1e3)
+
+    # dense backward of the FFN block's first layer (X [2048,1024], W [1024,4096], dY [2048,4096]):
+    # dA = dY W^T (NT), dW = X^T dY (TN), dBias = sum(dY, 0)
+    dyb = hip.array(rng.normal(0, 1, (2048, 4096)).astype(np.float32))
+    da, dw, dbias = hip.empty((2048, 1024)), hip.empty((1024, 4096)), hip.empty((4096,))
+    L = hip.L
+    _, ms = time_calls(hip, lambda: hip.check(L.axhip_sgemm(0, 1, 2048, 1024, 4096, 1.0, dyb.ptr, 4096, w1.ptr, 4096,
+                                                           0.0, da.ptr, 1024, None, 0)))
+    k_nt = hip.last_kernel()
+    _, ms2 = time_calls(hip, lambda: hip.check(L.axhip_sgemm(1, 0, 1024, 4096, 2048, 1.0, x.ptr, 1024, dyb.ptr, 4096,
+                                                            0.0, dw.ptr, 4096, None, 0)))
+    k_tn = hip.last_kernel()
+    _, ms3 = time_calls(hip, lambda: hip.check(L.axhip_sum_axis(dyb.ptr, 1, 2048, 4096, dbias.ptr)))
+    fl = 2 * 2048 * 1024 * 4096
+    res["fp32_dense_backward_2048x1024x4096"] = {
+        "dA_nt_us": ms * 1e3, "dA_TFLOP/s": fl / ms / 1e9, "dA_kernel": k_nt,
+        "dW_tn_us": ms2 * 1e3, "dW_TFLOP/s": fl / ms2 / 1e9, "dW_kernel": k_tn,
+        "dBias_us": ms3 * 1e3, "dBias_GB/s": 4 * 2048 * 4096 / ms3 / 1e6,
+        "frac_of_fp32_mfma_peak": 2 * fl / (ms + ms2) / 1e9 / PEAK_FP32_TFLOPS}
+    del dyb, da, dw
     del x, w1, w2, hbuf, y
 
     # config 2: int8 M=256, N=K=4096 (HBM/latency-bound)

@@ -118,6 +118,18 @@ int axhip_relu(const float *in, float *out, int64_t n);       /* .relu    */
 int axhip_gelu(const float *in, float *out, int64_t n);       /* .gelu_op (tanh form) */
 int axhip_fill_f32(float *dst, float value, int64_t n);       /* .fill    */
 
+/* ---- reductions and accumulation used by the dense layer's backward pass -------------- */
+/* .sum over one axis of a contiguous fp32 tensor viewed as [outer, axis_len, inner]:
+ * out[o,i] = sum_a in[o,a,i]  (cuda_sum, cuda/ops_reduce.cu:262-295; opt_sum,
+ * cpu_opt.c:4614-4660).  outer = 1 gives the bias gradient sum(grad_out, axis=0)
+ * (src/core/autograd_ops.c:724-757). */
+int axhip_sum_axis(const float *in, int64_t outer, int64_t axis_len, int64_t inner, float *out);
+/* .sum with axis = -1: out[0] = sum of all n elements (cuda/ops_reduce.cu:268-275). */
+int axhip_sum_all(const float *in, int64_t n, float *out);
+/* .axpy: y[i] = fma(alpha, x[i], y[i])  (cuda_axpy, cuda/ops_fused.cu:193-211; opt_axpy,
+ * cpu_opt.c:7287-7307). */
+int axhip_axpy(const float *x, float alpha, float *y, int64_t n);
+
 /* ---- timing on the library's stream (for benchmarks) -------------------------------- */
 void *axhip_event_create(void);
 void  axhip_event_destroy(void *ev);

@@ -52,6 +52,11 @@ ax_status_t ax_compute_bias_add(const ax_tensor_t *in, const ax_tensor_t *bias, 
 ax_status_t ax_compute_relu(const ax_tensor_t *in, ax_tensor_t *out);
 ax_status_t ax_compute_fill(ax_tensor_t *t, double value);
 ax_status_t ax_compute_copy(const ax_tensor_t *src, ax_tensor_t *dst);
+/* Reduction and accumulation the dense layer's backward pass is made of
+ * (src/core/autograd_ops.c:603-757): dA = gemm_nt(dY, W), dW = gemm_tn(X, dY),
+ * dBias = sum(dY, 0), and axpy to add into a gradient that already exists. */
+ax_status_t ax_compute_sum(const ax_tensor_t *in, int axis, ax_tensor_t *out);
+ax_status_t ax_compute_axpy(const ax_tensor_t *x, float alpha, ax_tensor_t *y);
 int ax_compute_has_gemm_relu(void);
 int ax_compute_has_gemm_nt(void);
 int ax_compute_has_gemm_tn(void);

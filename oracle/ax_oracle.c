@@ -447,3 +447,31 @@ void axo_w8a8_epilogue(const int32_t *acc, float x_scale, const float *w_scales,
             out[m * N + n] = v;
         }
 }
+
+/* ---- reductions / accumulation of the dense backward pass ------------------------------ */
+void axo_sum_axis0(const float *in, int64_t rows, int64_t cols, float *out) {
+    for (int64_t j = 0; j < cols; j++) {
+        float s = 0.0f;
+        for (int64_t i = 0; i < rows; i++) s += in[i * cols + j];
+        out[j] = s;
+    }
+}
+
+void axo_sum_axis_f64(const float *in, int64_t outer, int64_t axis_len, int64_t inner, double *out,
+                      double *out_abs) {
+    for (int64_t o = 0; o < outer; o++)
+        for (int64_t i = 0; i < inner; i++) {
+            double s = 0.0, sa = 0.0;
+            for (int64_t a = 0; a < axis_len; a++) {
+                const double v = (double)in[(o * axis_len + a) * inner + i];
+                s += v;
+                sa += fabs(v);
+            }
+            out[o * inner + i] = s;
+            if (out_abs) out_abs[o * inner + i] = sa;
+        }
+}
+
+void axo_axpy(const float *x, float alpha, float *y, int64_t n) {
+    for (int64_t i = 0; i < n; i++) y[i] = fmaf(alpha, x[i], y[i]);
+}

@@ -58,6 +58,15 @@ void axo_gemm_opt(const float *a, const float *b, float *c, int64_t M, int64_t N
 void axo_gemm_opt_nt(const float *a, const float *b, float *c, int64_t M, int64_t N, int64_t K);
 /* cpu_opt.c:7148-7194 with the mathematically intended axis: c[m,n] += bias[n]. */
 void axo_bias_add_cols(float *c, const float *bias, int64_t M, int64_t N);
+/* Bias gradient: out[j] = sum_i in[i*cols + j], each column added row by row in fp32 — the
+ * order of both the scalar loop in autograd_ops.c:740-752 and the per-lane accumulators of
+ * simd_axis0_sum (cpu_opt.c opt_sum, axis 0), so this restatement is bit-exact with them.
+ * Pinned against oracle/_ref (ax_compute_sum) in tests/test_oracle.py. */
+void axo_sum_axis0(const float *in, int64_t rows, int64_t cols, float *out);
+/* fp64 ground truth of any axis: out[o,i] = sum_a in[o,a,i], and the sum of |in| for the bound. */
+void axo_sum_axis_f64(const float *in, int64_t outer, int64_t axis_len, int64_t inner, double *out, double *out_abs);
+/* cpu_opt.c:7287-7307 (vector body): y[i] = fma(alpha, x[i], y[i]). */
+void axo_axpy(const float *x, float alpha, float *y, int64_t n);
 /* cpu_opt.c:7401-7440: c = max(c + bias[n], 0); bias may be NULL. */
 void axo_bias_relu(float *c, const float *bias, int64_t M, int64_t N);
 /* activations.c:24-25,267-316 (scalar tail form): 0.5x(1+tanh(0.79788456(x+0.044715x^3))). */

@@ -122,5 +122,48 @@ for M in (1, 8, 128):
     assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max(), M
     print("sequential M=%d ok" % M, flush=True)
 
+# 3. the reference's own autograd node for the dense layer (matmul_bias_backward,
+#    src/core/autograd_ops.c:603-757) run on the MI355X: gemm_nt, gemm_tn, sum and copy slots.
+#    The node's backward function is the first member of ax_grad_fn_t (include/axiom/autograd.h:48-50).
+L.ax_matmul_bias.restype = TP
+L.ax_matmul_bias.argtypes = [TP, TP, TP]
+BACKWARD = C.CFUNCTYPE(None, C.c_void_p, TP)
+
+
+def dense_backward(x, w, b, dy):
+    sh = lambda a: (i64 * a.ndim)(*a.shape)
+    ts = [L.ax_tensor_from_array(np.ascontiguousarray(a, np.float32).ctypes.data, sh(a), a.ndim, 0)
+          for a in (x, w, b, dy)]
+    tx, tw, tb, tdy = ts
+    for t in (tx, tw, tb):
+        t.contents.requires_grad = True
+    L.ax_enable_grad()
+    y = L.ax_matmul_bias(tx, tw, tb)
+    assert y and y.contents.grad_fn, L.ax_err_last_message()
+    fn = BACKWARD(C.cast(y.contents.grad_fn, C.POINTER(C.c_void_p))[0])
+    fn(y.contents.grad_fn, tdy)
+    L.ax_no_grad()
+    grads = []
+    for t in (tx, tw, tb):
+        g = t.contents.grad
+        assert g, "gradient was not produced"
+        grads.append(fetch(g) if g.contents.storage.contents.device != 0 else ref.numpy(g))
+    return grads
+
+
+for (M, K, N) in [(48, 40, 24), (256, 512, 384)]:
+    x = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    w = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    b = rng.uniform(-1, 1, N).astype(np.float32)
+    dy = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    on_cpu()
+    want = dense_backward(x, w, b, dy)
+    on_gpu()
+    got = dense_backward(x, w, b, dy)
+    for name, g, r_ in zip(("dX", "dW", "dBias"), got, want):
+        assert g.shape == r_.shape, name
+        assert np.abs(g - r_).max() <= 1e-4 * np.abs(r_).max(), (name, M, K, N)
+    print("dense backward", M, K, N, "ok", flush=True)
+
 on_cpu()
 print("DROPIN OK", flush=True)

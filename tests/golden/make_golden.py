@@ -111,6 +111,28 @@ xg = np.linspace(-6, 6, 1201, dtype=np.float32)
 G["gelu_x"] = xg
 G["gelu_y"] = r.gelu(xg.reshape(1, -1)).reshape(-1)
 
+# ---- dense backward building blocks (src/core/autograd_ops.c:603-757): dA = dY W^T (gemm_nt),
+# dW = X^T dY (gemm_tn), dBias = sum(dY, 0), accumulation by axpy
+L.ax_rng_seed(4242)
+Mb, Kb, Nb = 48, 40, 24                                   # tokens, in features, out features
+xb = ref_uniform(Mb * Kb, -1.0, 1.0).reshape(Mb, Kb)
+wb = ref_uniform(Kb * Nb, -1.0, 1.0).reshape(Kb, Nb)      # Dense weight is [in, out]
+dyb = ref_uniform(Mb * Nb, -1.0, 1.0).reshape(Mb, Nb)
+G["dense_bwd_dA"] = r.gemm(dyb, wb, backend=1, nt=True)   # [M,N] x [K,N]^T
+G["dense_bwd_dW"] = r.gemm_tn(xb, dyb, backend=1)         # [M,K]^T x [M,N]
+G["dense_bwd_db"] = r.sum(dyb, 0, backend=1)
+G["dense_bwd_db_naive"] = r.sum(dyb, 0, backend=0)
+L.ax_rng_seed(4343)
+s2 = ref_uniform(37 * 19, -1.0, 1.0).reshape(37, 19)
+s3 = ref_uniform(4 * 9 * 10, -1.0, 1.0).reshape(4, 9, 10)
+for name, arr in (("sum2d", s2), ("sum3d", s3)):
+    for axis in [-1] + list(range(arr.ndim)):
+        G[f"{name}_axis{axis}"] = r.sum(arr, axis, backend=1)
+        G[f"{name}_axis{axis}_naive"] = r.sum(arr, axis, backend=0)
+xa, ya = ref_uniform(1003, -1.0, 1.0), ref_uniform(1003, -1.0, 1.0)
+G["axpy_1003"] = r.axpy(xa, 0.37, ya, backend=1)
+G["axpy_1003_naive"] = r.axpy(xa, 0.37, ya, backend=0)
+
 np.savez_compressed(os.path.join(HERE, "golden.npz"), **G)
 print("wrote", len(G), "arrays,", os.path.getsize(os.path.join(HERE, "golden.npz")), "bytes")
 

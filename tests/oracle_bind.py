@@ -52,6 +52,9 @@ class Oracle:
         L.axo_gemm_opt_nt.argtypes = [f32p, f32p, f32p, i64, i64, i64]
         L.axo_bias_add_cols.argtypes = [f32p, f32p, i64, i64]
         L.axo_bias_relu.argtypes = [f32p, C.c_void_p, i64, i64]
+        L.axo_sum_axis0.argtypes = [f32p, i64, i64, f32p]
+        L.axo_sum_axis_f64.argtypes = [f32p, i64, i64, i64, f64p, C.c_void_p]
+        L.axo_axpy.argtypes = [f32p, C.c_float, f32p, i64]
         L.axo_gelu_tanh.restype = C.c_float
         L.axo_gelu_tanh.argtypes = [C.c_float]
         L.axo_gelu_f64.restype = C.c_double
@@ -138,6 +141,27 @@ class Oracle:
         bp = bias.ctypes.data_as(C.c_void_p) if bias is not None else None
         self.L.axo_bias_relu(c, bp, c.shape[0], c.shape[1])
         return c
+
+    def sum_axis0(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        rows, cols = x.shape[0], int(np.prod(x.shape[1:]))
+        out = np.empty(cols, np.float32)
+        self.L.axo_sum_axis0(x.reshape(-1), rows, cols, out)
+        return out.reshape(x.shape[1:])
+
+    def sum_axis_f64(self, x, axis):
+        """(fp64 sums over `axis`, fp64 sums of |x| over `axis`)"""
+        x = np.ascontiguousarray(x, np.float32)
+        outer, inner = int(np.prod(x.shape[:axis])), int(np.prod(x.shape[axis + 1:]))
+        out, out_abs = np.empty(outer * inner, np.float64), np.empty(outer * inner, np.float64)
+        self.L.axo_sum_axis_f64(x.reshape(-1), outer, x.shape[axis], inner, out, out_abs.ctypes.data_as(C.c_void_p))
+        shape = x.shape[:axis] + x.shape[axis + 1:]
+        return out.reshape(shape), out_abs.reshape(shape)
+
+    def axpy(self, x, alpha, y):
+        y = np.ascontiguousarray(y, np.float32).copy()
+        self.L.axo_axpy(np.ascontiguousarray(x, np.float32).reshape(-1), alpha, y.reshape(-1), y.size)
+        return y
 
     def gelu(self, x):
         x = np.ascontiguousarray(x, np.float32).copy()
@@ -257,6 +281,8 @@ class RefLib:
         L.ax_compute_gemm_relu.argtypes = [TP, TP, TP, TP]
         L.ax_compute_gemm_relu.restype = C.c_int
         L.ax_compute_bias_add.argtypes = [TP, TP, C.c_int, TP]
+        L.ax_compute_sum.argtypes = [TP, C.c_int, TP]
+        L.ax_compute_axpy.argtypes = [TP, C.c_float, TP]
         L.ax_compute_bias_add.restype = C.c_int
         L.ax_gelu.restype = TP
         L.ax_gelu.argtypes = [TP]
@@ -319,6 +345,37 @@ class RefLib:
         assert st == 0, st
         out = self.numpy(to)
         self.free(ta, tb, to)
+        return out
+
+    def gemm_tn(self, a_km, b, backend=1):
+        """a_km is [K,M]; returns a_km^T x b, [M,N]."""
+        self.backend(backend)
+        ta, tb = self.tensor(a_km), self.tensor(b)
+        to = self.empty(a_km.shape[1], b.shape[1])
+        st = self.L.ax_compute_gemm_tn(ta, tb, to)
+        assert st == 0, st
+        out = self.numpy(to)
+        self.free(ta, tb, to)
+        return out
+
+    def sum(self, x, axis, backend=1):
+        self.backend(backend)
+        x = np.ascontiguousarray(x, np.float32)
+        shape = (1,) if axis == -1 else x.shape[:axis] + x.shape[axis + 1:]
+        t, to = self.tensor(x), self.empty(*shape)
+        st = self.L.ax_compute_sum(t, axis, to)
+        assert st == 0, st
+        out = self.numpy(to)
+        self.free(t, to)
+        return out
+
+    def axpy(self, x, alpha, y, backend=1):
+        self.backend(backend)
+        tx, ty = self.tensor(x), self.tensor(y)
+        st = self.L.ax_compute_axpy(tx, alpha, ty)
+        assert st == 0, st
+        out = self.numpy(ty)
+        self.free(tx, ty)
         return out
 
     def gemm_relu(self, a, b, bias):

@@ -87,6 +87,42 @@ def test_dispatch_wrappers(ax, oracle):
     ax.free(ta, tb, tbias, out, tbt, tat, tc, lin, trb, bad, t3, host)
 
 
+def test_dense_backward_through_dispatch(ax, oracle):
+    """The call sequence of the reference's matmul_bias_backward (src/core/autograd_ops.c:603-757)
+    on device tensors: gemm_nt, gemm_tn, sum(axis 0) + copy for fresh gradients, temp + axpy for
+    gradients that already hold a value."""
+    L = ax.L
+    oracle.seed(31)
+    M, K, N = 96, 160, 72
+    x, w, dy = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1), oracle.uniform((M, N), -1, 1)
+    tx, tw, tdy = ax.from_numpy(x), ax.from_numpy(w), ax.from_numpy(dy)
+    dA, dW, db, tmp = ax.empty((M, K)), ax.empty((K, N)), ax.empty((N,)), ax.empty((N,))
+    assert L.ax_compute_has_gemm_tn() == 1
+    assert L.ax_compute_gemm_nt(tdy, tw, dA) == 0 and close(ax.to_numpy(dA), oracle.gemm_opt_nt(dy, w))
+    xt = np.ascontiguousarray(x.T)
+    assert L.ax_compute_gemm_tn(tx, tdy, dW) == 0 and close(ax.to_numpy(dW), oracle.gemm_opt(xt, dy))
+    assert L.ax_compute_sum(tdy, 0, tmp) == 0 and L.ax_compute_copy(tmp, db) == 0
+    want_db = oracle.sum_axis0(dy)
+    assert np.abs(ax.to_numpy(db) - want_db).max() <= 1e-5 * np.abs(dy).sum(axis=0).max()
+    # second backward pass into the same gradients: += semantics
+    assert L.ax_compute_axpy(tmp, 1.0, db) == 0
+    assert np.array_equal(ax.to_numpy(db), ax.to_numpy(tmp) * 2)
+    g = ax.empty((K, N))
+    assert L.ax_compute_gemm_tn(tx, tdy, g) == 0 and L.ax_compute_axpy(g, 1.0, dW) == 0
+    assert close(ax.to_numpy(dW), 2 * oracle.gemm_opt(xt, dy))
+    # other axes, the full reduction, and the error codes of cuda_sum (cuda/ops_reduce.cu:262-295)
+    rows = ax.empty((M,))
+    assert L.ax_compute_sum(tdy, 1, rows) == 0
+    assert np.abs(ax.to_numpy(rows) - dy.astype(np.float64).sum(axis=1)).max() <= 1e-5 * np.abs(dy).sum(axis=1).max()
+    one = ax.empty((1,))
+    assert L.ax_compute_sum(tdy, -1, one) == 0
+    assert abs(float(ax.to_numpy(one)[0]) - dy.astype(np.float64).sum()) <= 1e-5 * np.abs(dy).sum()
+    assert L.ax_compute_sum(tdy, 2, rows) == 5                     # AX_ERR_INVALID_AXIS
+    assert L.ax_compute_sum(tdy, 0, rows) == 3                     # wrong output size
+    assert L.ax_compute_axpy(tmp, 1.0, rows) == 3                  # numel mismatch
+    ax.free(tx, tw, tdy, dA, dW, db, tmp, g, rows, one)
+
+
 def test_reference_gpu_vs_cpu_template(ax, oracle):
     """tests/test_cuda.c:213-244: 64x128 . 128x32, rand(-0.1,0.1), every element within 1e-3."""
     L = ax.L

@@ -109,7 +109,7 @@ def test_w8a8_persistent_tiles_properties(hip, oracle, M, N, K):
 F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), (64, 64, 32),
               (128, 128, 64), (130, 260, 700), (256, 384, 512), (33, 40, 100), (96, 96, 96),
               (2048, 1024, 256),
-              # one shape per tile of the direct-to-LDS fast path: 128x256, 128x128, 128x64
+              # shapes that take the 128x256 tile, and ones just short of it in N or in tile count
               (2048, 4096, 64), (4096, 2176, 64), (4096, 1088, 32), (128, 64, 4096)]
 
 
@@ -400,6 +400,83 @@ def test_elementwise_slots(hip, oracle, golden):
     assert np.array_equal(out.numpy(), x + rb[:, None])
     z = hip.empty((1000,))                                               # zero-filled allocation
     assert not z.numpy().any()
+
+
+# ------------------------------------------------------------------ dense backward blocks
+SUM_BOUND = 1e-5     # |gpu - sum64| <= SUM_BOUND * sum |x|   (fp32 sums in a fixed parallel order)
+
+
+@pytest.mark.parametrize("shape,axis", [((37, 19), 0), ((37, 19), 1), ((4, 9, 10), 0), ((4, 9, 10), 1),
+                                        ((4, 9, 10), 2), ((2048, 4096), 0), ((2048, 4096), 1),
+                                        ((1000, 7), 0), ((3, 100003), 1), ((1, 64), 0), ((5000, 64), 0)])
+def test_sum_axis(hip, oracle, golden, shape, axis):
+    say("sum", shape, axis)
+    oracle.seed(4343 if shape in ((37, 19), (4, 9, 10)) else sum(shape) + axis)
+    if shape == (4, 9, 10):
+        oracle.uniform((37, 19), -1, 1)        # the golden vectors draw the 2-D case first
+    x = oracle.uniform(shape, -1, 1)
+    outer, inner = int(np.prod(shape[:axis])), int(np.prod(shape[axis + 1:]))
+    out = hip.empty(shape[:axis] + shape[axis + 1:] or (1,))
+    hip.check(hip.L.axhip_sum_axis(hip.array(x).ptr, outer, shape[axis], inner, out.ptr))
+    got = out.numpy().reshape(shape[:axis] + shape[axis + 1:])
+    s64, sabs = oracle.sum_axis_f64(x, axis)
+    assert (np.abs(got - s64) <= SUM_BOUND * sabs + 1e-30).all()
+    if axis == 0:
+        ref = oracle.sum_axis0(x)              # the reference's own order, row by row
+        assert np.abs(got - ref).max() <= SUM_BOUND * sabs.max()
+    name = {(37, 19): "sum2d", (4, 9, 10): "sum3d"}.get(shape)
+    if name:
+        assert np.abs(got - golden[f"{name}_axis{axis}"]).max() <= SUM_BOUND * sabs.max()
+    # run-to-run determinism
+    hip.check(hip.L.axhip_sum_axis(hip.array(x).ptr, outer, shape[axis], inner, out.ptr))
+    assert np.array_equal(out.numpy().reshape(got.shape), got)
+
+
+@pytest.mark.parametrize("n", [1, 63, 4096, 4097, 1000003, 1 << 24])
+def test_sum_all_and_axpy(hip, oracle, n):
+    oracle.seed(n)
+    x = oracle.uniform((n,), -1, 1)
+    out = hip.empty((1,))
+    dx = hip.array(x)
+    hip.check(hip.L.axhip_sum_all(dx.ptr, n, out.ptr))
+    exact = x.astype(np.float64).sum()
+    assert abs(float(out.numpy()[0]) - exact) <= SUM_BOUND * np.abs(x).astype(np.float64).sum()
+    y = oracle.uniform((n,), -1, 1)
+    dy = hip.array(y)
+    hip.check(hip.L.axhip_axpy(dx.ptr, 0.37, dy.ptr, n))
+    assert np.array_equal(dy.numpy(), oracle.axpy(x, 0.37, y))        # one fused multiply-add: bit-exact
+
+
+@pytest.mark.parametrize("M,K,N", [(48, 40, 24), (130, 70, 50), (2048, 1024, 4096)])
+def test_dense_backward_blocks(hip, oracle, golden, M, K, N):
+    """The three products of the dense layer's backward pass (src/core/autograd_ops.c:603-757)
+    through the C ABI: dA = dY W^T (NT), dW = X^T dY (TN), dBias = sum(dY, 0); then the
+    accumulate-into-an-existing-gradient forms (temp + axpy, and beta = 1)."""
+    say("dense backward", M, K, N)
+    oracle.seed(4242 if (M, K, N) == (48, 40, 24) else M + K + N)
+    x, w, dy = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1), oracle.uniform((M, N), -1, 1)
+    dx_, dw_, ddy = hip.array(x), hip.array(w), hip.array(dy)
+    dA = hip.sgemm(ddy, dw_, transb=True).numpy()                     # [M,N] x [K,N]^T -> [M,K]
+    say("  dA", hip.last_kernel())
+    check_fp32(oracle, dA, dy, w, transb=True, ref=oracle.gemm_opt_nt(dy, w))
+    dW = hip.sgemm(dx_, ddy, transa=True).numpy()                     # [M,K]^T x [M,N] -> [K,N]
+    say("  dW", hip.last_kernel())
+    xt = np.ascontiguousarray(x.T)
+    check_fp32(oracle, dW, xt, dy, ref=oracle.gemm_opt(xt, dy))
+    db = hip.empty((N,))
+    hip.check(hip.L.axhip_sum_axis(ddy.ptr, 1, M, N, db.ptr))
+    s64, sabs = oracle.sum_axis_f64(dy, 0)
+    assert (np.abs(db.numpy() - s64) <= SUM_BOUND * sabs).all()
+    if (M, K, N) == (48, 40, 24):
+        for got, key in ((dA, "dense_bwd_dA"), (dW, "dense_bwd_dW"), (db.numpy(), "dense_bwd_db")):
+            assert np.abs(got - golden[key]).max() <= REL_FP32 * np.abs(golden[key]).max()
+    # gradient that already exists: temp + axpy (what the reference does) == gemm with beta = 1
+    g0 = oracle.uniform((K, N), -1, 1)
+    acc1 = hip.array(g0)
+    hip.check(hip.L.axhip_axpy(hip.array(dW).ptr, 1.0, acc1.ptr, K * N))
+    assert np.array_equal(acc1.numpy(), g0 + dW)
+    acc2 = hip.sgemm(dx_, ddy, transa=True, beta=1.0, c=hip.array(g0)).numpy()
+    assert np.abs(acc2 - (g0 + dW)).max() <= 1e-6 * max(1.0, np.abs(dW).max())
 
 
 def test_error_paths(hip):

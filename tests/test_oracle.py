@@ -205,6 +205,44 @@ def test_bias_relu_and_gelu(oracle, golden):
     assert oracle.L.axo_gelu_tanh(0.0) == 0.0 and abs(oracle.L.axo_gelu_tanh(10.0) - 10.0) < 1e-6
 
 
+# ---------------------------------------------------------------- dense backward blocks
+def test_dense_backward_blocks_match_reference_vectors(oracle, golden):
+    """dA = dY W^T, dW = X^T dY, dBias = sum(dY, 0), axpy: the restatement against what the
+    reference produced for the same seeded inputs (both of its CPU backends where they exist)."""
+    oracle.seed(4242)
+    M, K, N = 48, 40, 24
+    x, w, dy = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1), oracle.uniform((M, N), -1, 1)
+    dA = oracle.gemm_opt_nt(dy, w)
+    assert np.abs(dA - golden["dense_bwd_dA"]).max() <= 1e-5 * np.abs(golden["dense_bwd_dA"]).max()
+    dW = oracle.gemm_opt(np.ascontiguousarray(x.T), dy)
+    assert np.abs(dW - golden["dense_bwd_dW"]).max() <= 1e-5 * np.abs(golden["dense_bwd_dW"]).max()
+    db = oracle.sum_axis0(dy)
+    assert np.array_equal(db, golden["dense_bwd_db"]) and np.array_equal(db, golden["dense_bwd_db_naive"])
+    oracle.seed(4343)
+    s2, s3 = oracle.uniform((37, 19), -1, 1), oracle.uniform((4, 9, 10), -1, 1)
+    for name, arr in (("sum2d", s2), ("sum3d", s3)):
+        assert np.array_equal(oracle.sum_axis0(arr), golden[f"{name}_axis0"])        # bit-exact order
+        for axis in range(arr.ndim):
+            s64, sabs = oracle.sum_axis_f64(arr, axis)
+            for tag in ("", "_naive"):
+                ref = golden[f"{name}_axis{axis}{tag}"]
+                assert (np.abs(ref - s64) <= 1e-6 * sabs + 1e-30).all()
+        full = np.float64(arr.astype(np.float64).sum())
+        assert abs(golden[f"{name}_axis-1"][0] - full) <= 1e-6 * np.abs(arr).sum()
+    xa, ya = oracle.uniform((1003,), -1, 1), oracle.uniform((1003,), -1, 1)
+    got = oracle.axpy(xa, 0.37, ya)
+    # vector body is a fused multiply-add (bit-exact); the scalar tail of the SIMD backend and
+    # the naive backend may round the product first: allow one rounding of the product
+    for tag in ("", "_naive"):
+        ref = golden[f"axpy_1003{tag}"]
+        assert np.abs(got - ref).max() <= 2e-7
+    assert np.array_equal(got[:1000], golden["axpy_1003"][:1000])
+    # closed forms
+    assert np.array_equal(oracle.sum_axis0(np.ones((1000, 7), np.float32)), np.full(7, 1000, np.float32))
+    assert np.array_equal(oracle.axpy(np.ones(5, np.float32), 2.0, np.arange(5, dtype=np.float32)),
+                          np.arange(5, dtype=np.float32) + 2)
+
+
 # ---------------------------------------------------------------- live cross-check
 def test_oracle_equals_compiled_reference(oracle, reflib):
     oracle.seed(11)
