@@ -1,0 +1,280 @@
+// Scaled dot-product attention forward: O = softmax(scale * Q K^T [+ causal mask]) V per head,
+// Q, K, V, O [BH, S, dk] row-major fp32, L [BH, S] = log-sum-exp of each score row (or NULL).
+//
+// Fused kernel (dk = 64, S a multiple of 128): the score matrix never leaves the chip.  A
+// workgroup of 4 waves owns 128 query rows of one head, a wave 32 of them; keys and values
+// stream through LDS in blocks of 64 (direct-to-LDS loads, two stages).  Both products run on
+// v_mfma_f32_32x32x2_f32 with the query index on the MFMA's column side, so lane l of a wave
+// owns query (l & 31) in the score tile *and* in the output accumulator:
+//   S^T tile:  A = K rows (32 keys), B = the wave's Q rows (held in registers for the whole
+//              kernel); register v of lane l = score(query l&31, key 8*(v>>2) + 4*(l>>5) + (v&3)).
+//   softmax:   running maximum m and sum per query, the online form: the accumulator is
+//              rescaled by 2^(m_old - m_new) when the maximum moves.  Row reductions are within
+//              a lane plus one exchange with lane l^32.  Scores are kept in base-2 units
+//              (scale * log2(e) folded in) so the exponential is the hardware's 2^x.
+//   O^T tile:  A = V^T (lane reads V[key][d] with d = l&31), B = the probabilities exactly
+//              where the score MFMA left them: key(v, l>>5) above is also a legal pairing of
+//              the MFMA's two k indices, and a sum over keys does not care about their order.
+// K rows (256 bytes) are XOR-swizzled in 16-byte chunks, applied on the global address side of
+// the load, so a 16-lane ds_read_b128 touches every bank once; V is laid in groups of 4 rows
+// spaced 1152 bytes apart so the two lane halves (keys 4 apart) read different banks.
+//
+// Every other shape: scores through a workspace, one batched NT GEMM, a row softmax kernel and
+// one batched NN GEMM over as many heads at a time as fit 256 MiB (the structure of
+// ax_cuda_sdpa_fwd, cuda/ops_attention.cu:299-392).
+#include "common.h"
+
+namespace {
+using namespace axhip;
+
+#define AXS_LOAD_LDS(m0val, voff, base)                                                        \
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0val),  \
+                 "v"(voff), "s"(base)                                                          \
+                 : "memory")
+#define AXS_VM0() __builtin_amdgcn_s_waitcnt(0 | (0 << 14) | (7 << 4) | (15 << 8))
+
+constexpr int SD_DK = 64, SD_BQ = 128, SD_BKV = 64;
+constexpr int SD_KSTAGE = SD_BKV * SD_DK * 4;            // 16 KiB
+constexpr int SD_VGROUP = 1152;                          // 4 rows of 256 B + 128 B
+constexpr int SD_VSTAGE = (SD_BKV / 4) * SD_VGROUP;      // 18 KiB
+constexpr int SD_SMEM = 2 * SD_KSTAGE + 2 * SD_VSTAGE;
+
+template <bool CAUSAL>
+__global__ void __launch_bounds__(256)
+k_sdpa64(const float *__restrict__ Q, const float *__restrict__ K, const float *__restrict__ V,
+         float *__restrict__ O, float *__restrict__ L, int64_t S, float scale_log2e) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int64_t head = blockIdx.y;
+    const int64_t q0 = (int64_t)blockIdx.x * SD_BQ;
+    const float *Qh = Q + head * S * SD_DK, *Kh = K + head * S * SD_DK, *Vh = V + head * S * SD_DK;
+    const unsigned lds0 = (unsigned)(uintptr_t)lds;
+
+    // per-lane byte offsets of the direct-to-LDS loads: instruction i of this wave covers rows
+    // 4*(4*i + wave) .. +3 of a 64-row tile, lane l row + (l >> 4), 16-byte chunk (l & 15)
+    unsigned koff[4], voff[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = 4 * (4 * i + wave) + (lane >> 4), c = lane & 15;
+        koff[i] = (unsigned)(row * 256 + ((c ^ (row & 15)) << 4));
+        voff[i] = (unsigned)(row * 256 + (c << 4));
+    }
+
+    // ---- Q tile (128 rows) through the two K stages, then into registers ----
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        AXS_LOAD_LDS(lds0 + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * SD_DK));
+        AXS_LOAD_LDS(lds0 + SD_KSTAGE + (4 * i + wave) * 1024, koff[i],
+                     reinterpret_cast<const char *>(Qh + (q0 + 64) * SD_DK));
+    }
+    AXS_VM0();
+    __syncthreads();
+    v4f qf[8];                                   // k-block kb: dk 8*kb + 4*fhalf .. +3 of this lane's query
+    {
+        const int r = wave * 32 + frow;          // rows 64..127 sit in the second stage, same swizzle
+        const unsigned char *qrow = lds + (r >> 6) * SD_KSTAGE + (r & 63) * 256;
+#pragma unroll
+        for (int kb = 0; kb < 8; kb++)
+            qf[kb] = *reinterpret_cast<const v4f *>(qrow + (((kb * 2 + fhalf) ^ (r & 15)) << 4));
+    }
+    __syncthreads();
+
+    const int64_t nblocks = CAUSAL ? (q0 + SD_BQ) / SD_BKV : S / SD_BKV;
+    auto issue = [&](int64_t blk, int stage) {
+        const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * SD_DK);
+        const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * SD_DK);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            AXS_LOAD_LDS(lds0 + stage * SD_KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
+            AXS_LOAD_LDS(lds0 + 2 * SD_KSTAGE + stage * SD_VSTAGE + (4 * i + wave) * SD_VGROUP, voff[i], vg);
+        }
+    };
+    issue(0, 0);
+
+    v16f acc_o[2];
+#pragma unroll
+    for (int d = 0; d < 2; d++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc_o[d][v] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;       // l_run: this lane half's share of the row sum
+    const int64_t qg = q0 + wave * 32 + frow;    // this lane's query
+
+    for (int64_t blk = 0; blk < nblocks; blk++) {
+        const int stage = (int)(blk & 1);
+        AXS_VM0();
+        __syncthreads();                          // block blk has landed; stage^1 is free again
+        if (blk + 1 < nblocks) issue(blk + 1, stage ^ 1);
+        const unsigned char *ks = lds + stage * SD_KSTAGE;
+        const unsigned char *vs = lds + 2 * SD_KSTAGE + stage * SD_VSTAGE;
+
+        // ---- scores of 64 keys ----
+        v16f acc_s[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc_s[kt][v] = 0.0f;
+            const int r = kt * 32 + frow;
+            const unsigned char *krow = ks + r * 256;
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) {
+                const v4f kf = *reinterpret_cast<const v4f *>(krow + (((kb * 2 + fhalf) ^ (r & 15)) << 4));
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc_s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[kb][e], acc_s[kt], 0, 0, 0);
+            }
+        }
+
+        // ---- online softmax ----
+        float m_blk = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                float s = acc_s[kt][v] * scale_log2e;
+                if (CAUSAL) {
+                    const int64_t key = blk * SD_BKV + kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3);
+                    if (key > qg) s = -INFINITY;
+                }
+                acc_s[kt][v] = s;
+                m_blk = fmaxf(m_blk, s);
+            }
+        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
+        const float m_new = fmaxf(m_run, m_blk);      // finite: key 0 is visible to every query
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        float l_blk = 0.0f;
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const float p = __builtin_amdgcn_exp2f(acc_s[kt][v] - m_new);
+                acc_s[kt][v] = p;
+                l_blk += p;
+            }
+        l_run = l_run * alpha + l_blk;
+        m_run = m_new;
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc_o[d][v] *= alpha;
+
+        // ---- O^T += V^T P^T ----
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int key = kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3);
+                const float *vrow = reinterpret_cast<const float *>(vs + (key >> 2) * SD_VGROUP + (key & 3) * 256);
+#pragma unroll
+                for (int d = 0; d < 2; d++)
+                    acc_o[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[d * 32 + frow], acc_s[kt][v], acc_o[d], 0, 0, 0);
+            }
+    }
+
+    // ---- normalise and write: lane owns query qg, dk columns 32*d + 8*g + 4*fhalf .. +3 ----
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / l_tot;
+    float *orow = O + (head * S + qg) * SD_DK;
+#pragma unroll
+    for (int d = 0; d < 2; d++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            v4f r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) r[e] = acc_o[d][4 * g + e] * inv;
+            *reinterpret_cast<v4f *>(orow + d * 32 + 8 * g + 4 * fhalf) = r;
+        }
+    if (L && fhalf == 0) L[head * S + qg] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+}
+
+// One workgroup per score row: mask, maximum, exponentials, sum, normalise in place; L = max + log(sum).
+__global__ void __launch_bounds__(256)
+k_softmax_lse_rows(float *__restrict__ score, float *__restrict__ L, int64_t S, int causal) {
+    __shared__ float red[256];
+    const int64_t row = blockIdx.x;               // head * S + query
+    const int64_t qi = row % S;
+    float *p = score + row * S;
+    const int64_t n = causal ? qi + 1 : S;        // keys this query sees
+    float mx = -INFINITY;
+    for (int64_t j = threadIdx.x; j < n; j += 256) mx = fmaxf(mx, p[j]);
+    red[threadIdx.x] = mx;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + s]);
+        __syncthreads();
+    }
+    mx = red[0];
+    __syncthreads();
+    float sum = 0.0f;
+    for (int64_t j = threadIdx.x; j < S; j += 256) {
+        const float e = j < n ? expf(p[j] - mx) : 0.0f;
+        p[j] = e;
+        sum += e;
+    }
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    sum = red[0];
+    const float inv = 1.0f / sum;
+    for (int64_t j = threadIdx.x; j < n; j += 256) p[j] *= inv;
+    if (L && threadIdx.x == 0) L[row] = mx + logf(sum);
+}
+
+int sdpa_unfused(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH,
+                 int64_t S, int64_t dk, float scale, int causal) {
+    const size_t per_head = (size_t)S * (size_t)S * sizeof(float);
+    int64_t chunk = (int64_t)((size_t(256) << 20) / per_head);
+    if (chunk < 1) chunk = 1;
+    if (chunk > BH) chunk = BH;
+    if (chunk > 65535) chunk = 65535;
+    float *score = static_cast<float *>(workspace((size_t)chunk * per_head));
+    if (!score) return AXHIP_ERR_ALLOC;
+    for (int64_t h0 = 0; h0 < BH; h0 += chunk) {
+        const int64_t nb = BH - h0 < chunk ? BH - h0 : chunk;
+        const float *q = Q + h0 * S * dk, *k = K + h0 * S * dk, *v = V + h0 * S * dk;
+        int rc = axhip_sgemm_strided_batched(0, 1, S, S, dk, scale, q, dk, S * dk, k, dk, S * dk, 0.0f, score, S,
+                                             S * S, nb);
+        if (rc) return rc;
+        if (nb * S > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "sdpa: too many score rows per chunk");
+        hipLaunchKernelGGL(k_softmax_lse_rows, dim3((unsigned)(nb * S)), dim3(256), 0, kStream, score,
+                           L ? L + h0 * S : nullptr, S, causal);
+        if ((rc = check_launch("sdpa softmax"))) return rc;
+        rc = axhip_sgemm_strided_batched(0, 0, S, dk, S, 1.0f, score, S, S * S, v, dk, S * dk, 0.0f,
+                                         O + h0 * S * dk, dk, S * dk, nb);
+        if (rc) return rc;
+    }
+    note_kernel("sdpa_unfused");
+    return AXHIP_OK;
+}
+
+}  // namespace
+
+extern "C" int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH,
+                              int64_t S, int64_t dk, float scale, int causal) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!Q || !K || !V || !O) return fail(AXHIP_ERR_NULL_ARG, "sdpa_fwd: NULL tensor");
+    if (BH < 0 || S < 0 || dk <= 0) return fail(AXHIP_ERR_SHAPE, "sdpa_fwd: bad extent");
+    if (BH == 0 || S == 0) return AXHIP_OK;
+    const bool aligned = ((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O) & 15) == 0);
+    if (dk == SD_DK && S % SD_BQ == 0 && aligned && BH <= 65535 && S / SD_BQ <= 0x7fffffff) {
+        static bool attr_set = false;
+        if (!attr_set) {
+            AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sdpa64<false>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, SD_SMEM), "hipFuncSetAttribute");
+            AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sdpa64<true>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, SD_SMEM), "hipFuncSetAttribute");
+            attr_set = true;
+        }
+        const float sl2 = scale * 1.4426950408889634f;
+        dim3 grid((unsigned)(S / SD_BQ), (unsigned)BH);
+        if (causal) hipLaunchKernelGGL(k_sdpa64<true>, grid, dim3(256), SD_SMEM, kStream, Q, K, V, O, L, S, sl2);
+        else hipLaunchKernelGGL(k_sdpa64<false>, grid, dim3(256), SD_SMEM, kStream, Q, K, V, O, L, S, sl2);
+        axhip::note_kernel(causal ? "sdpa_fused_dk64_causal" : "sdpa_fused_dk64");
+        return check_launch("sdpa_fwd");
+    }
+    return sdpa_unfused(Q, K, V, O, L, BH, S, dk, scale, causal);
+}

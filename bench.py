@@ -220,6 +220,15 @@ def secondary(hip):
         0, 0, S, D, S, 1.0, s.ptr, S, S * S, v.ptr, D, S * D, 0.0, o.ptr, D, S * D, Bn)))
     res["fp32_batched_pv"] = {"us": ms * 1e3, "TFLOP/s": 2 * Bn * S * S * D / ms / 1e9,
                               "GB/s": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    # fused attention forward over the same heads (both products and the softmax in one kernel,
+    # no [512,512] score matrix in memory); flops counted as the two GEMMs'
+    l = hip.empty((Bn, S))
+    _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sdpa_fwd(q.ptr, k.ptr, v.ptr, o.ptr, l.ptr, Bn, S, D,
+                                                                  0.125, 0)))
+    res["fp32_sdpa_fwd_512x512x64"] = {"us": ms * 1e3, "TFLOP/s": 4 * Bn * S * S * D / ms / 1e9,
+                                       "frac_of_fp32_mfma_peak": 4 * Bn * S * S * D / ms / 1e9 / PEAK_FP32_TFLOPS,
+                                       "kernel": hip.last_kernel(),
+                                       "unfused_us": res["fp32_batched_qkt"]["us"] + res["fp32_batched_pv"]["us"]}
     return res
 
 

@@ -130,6 +130,17 @@ int axhip_sum_all(const float *in, int64_t n, float *out);
  * cpu_opt.c:7287-7307). */
 int axhip_axpy(const float *x, float alpha, float *y, int64_t n);
 
+/* ---- scaled dot-product attention forward --------------------------------------------- */
+/* O[h] = softmax(scale * Q[h] K[h]^T) V[h] for BH heads; Q, K, V, O are [BH, S, dk] row-major
+ * fp32 in device memory, L is [BH, S] (log-sum-exp of each score row, natural log) or NULL;
+ * causal != 0: query i sees keys j <= i.  Replaces ax_cuda_sdpa_fwd
+ * (cuda/ops_attention.cu:299-392) and the device form of ax_fused_attention_fwd /
+ * ax_fused_attention_fwd_causal (include/axiom/attention.h:273-283,
+ * src/core/fused_attention.c:559-573).  dk = 64 with S a multiple of 128 runs fused (no score
+ * matrix in memory); other shapes go through batched GEMMs and a row softmax. */
+int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L,
+                   int64_t BH, int64_t S, int64_t dk, float scale, int causal);
+
 /* ---- timing on the library's stream (for benchmarks) -------------------------------- */
 void *axhip_event_create(void);
 void  axhip_event_destroy(void *ev);

@@ -475,3 +475,69 @@ void axo_sum_axis_f64(const float *in, int64_t outer, int64_t axis_len, int64_t 
 void axo_axpy(const float *x, float alpha, float *y, int64_t n) {
     for (int64_t i = 0; i < n; i++) y[i] = fmaf(alpha, x[i], y[i]);
 }
+
+/* ---- scaled dot-product attention forward ---------------------------------------------- */
+void axo_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH,
+                  int64_t S, int64_t dk, float scale, int causal) {
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t h = 0; h < BH; h++) {
+        const float *q = Q + h * S * dk, *k = K + h * S * dk, *v = V + h * S * dk;
+        float *scores = (float *)malloc((size_t)S * sizeof(float));
+        for (int64_t i = 0; i < S; i++) {
+            const int64_t n = causal ? i + 1 : S;
+            float mx = -INFINITY;
+            for (int64_t j = 0; j < n; j++) {
+                float dot = 0.0f;
+                for (int64_t d = 0; d < dk; d++) dot += q[i * dk + d] * k[j * dk + d];
+                dot *= scale;
+                scores[j] = dot;
+                if (dot > mx) mx = dot;
+            }
+            float sum = 0.0f;
+            for (int64_t j = 0; j < n; j++) {
+                scores[j] = expf(scores[j] - mx);
+                sum += scores[j];
+            }
+            const float inv = 1.0f / sum;
+            for (int64_t d = 0; d < dk; d++) {
+                float acc = 0.0f;
+                for (int64_t j = 0; j < n; j++) acc += scores[j] * inv * v[j * dk + d];
+                O[(h * S + i) * dk + d] = acc;
+            }
+            if (L) L[h * S + i] = mx + logf(sum);
+        }
+        free(scores);
+    }
+}
+
+void axo_sdpa_fwd_f64(const float *Q, const float *K, const float *V, double *O, double *L, int64_t BH,
+                      int64_t S, int64_t dk, float scale, int causal) {
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t h = 0; h < BH; h++) {
+        const float *q = Q + h * S * dk, *k = K + h * S * dk, *v = V + h * S * dk;
+        double *scores = (double *)malloc((size_t)S * sizeof(double));
+        for (int64_t i = 0; i < S; i++) {
+            const int64_t n = causal ? i + 1 : S;
+            double mx = -INFINITY;
+            for (int64_t j = 0; j < n; j++) {
+                double dot = 0.0;
+                for (int64_t d = 0; d < dk; d++) dot += (double)q[i * dk + d] * (double)k[j * dk + d];
+                dot *= (double)scale;
+                scores[j] = dot;
+                if (dot > mx) mx = dot;
+            }
+            double sum = 0.0;
+            for (int64_t j = 0; j < n; j++) {
+                scores[j] = exp(scores[j] - mx);
+                sum += scores[j];
+            }
+            for (int64_t d = 0; d < dk; d++) {
+                double acc = 0.0;
+                for (int64_t j = 0; j < n; j++) acc += scores[j] * (double)v[j * dk + d];
+                O[(h * S + i) * dk + d] = acc / sum;
+            }
+            if (L) L[h * S + i] = mx + log(sum);
+        }
+        free(scores);
+    }
+}

@@ -67,6 +67,15 @@ void axo_sum_axis0(const float *in, int64_t rows, int64_t cols, float *out);
 void axo_sum_axis_f64(const float *in, int64_t outer, int64_t axis_len, int64_t inner, double *out, double *out_abs);
 /* cpu_opt.c:7287-7307 (vector body): y[i] = fma(alpha, x[i], y[i]). */
 void axo_axpy(const float *x, float alpha, float *y, int64_t n);
+/* Scaled dot-product attention forward, per head: O = softmax(scale * Q K^T [causal]) V,
+ * L = row max + log(row sum) or NULL.  The textbook evaluation the reference's own test uses as
+ * its yardstick (tests/test_attention.c:17-48, gate 1e-4); the reference's fused kernel
+ * (src/core/fused_attention.c:559-573) is pinned against it through oracle/_ref and the
+ * golden vectors in tests/test_oracle.py.  The _f64 form is the ground truth. */
+void axo_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH,
+                  int64_t S, int64_t dk, float scale, int causal);
+void axo_sdpa_fwd_f64(const float *Q, const float *K, const float *V, double *O, double *L, int64_t BH,
+                      int64_t S, int64_t dk, float scale, int causal);
 /* cpu_opt.c:7401-7440: c = max(c + bias[n], 0); bias may be NULL. */
 void axo_bias_relu(float *c, const float *bias, int64_t M, int64_t N);
 /* activations.c:24-25,267-316 (scalar tail form): 0.5x(1+tanh(0.79788456(x+0.044715x^3))). */

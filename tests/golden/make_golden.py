@@ -133,6 +133,16 @@ xa, ya = ref_uniform(1003, -1.0, 1.0), ref_uniform(1003, -1.0, 1.0)
 G["axpy_1003"] = r.axpy(xa, 0.37, ya, backend=1)
 G["axpy_1003_naive"] = r.axpy(xa, 0.37, ya, backend=0)
 
+# ---- scaled dot-product attention forward (src/core/fused_attention.c:559-573) at the shapes
+# of tests/test_attention.c:54-60,101-104 and one with dk = 64
+for (BH, S, dk, causal) in ((6, 24, 16, 0), (2, 16, 8, 1), (3, 128, 64, 0), (3, 128, 64, 1), (2, 40, 32, 1)):
+    L.ax_rng_seed(5000 + BH * 100 + S + dk + causal)
+    q = ref_uniform(BH * S * dk, -0.5, 0.5).reshape(BH, S, dk)
+    k = ref_uniform(BH * S * dk, -0.5, 0.5).reshape(BH, S, dk)
+    v = ref_uniform(BH * S * dk, -0.5, 0.5).reshape(BH, S, dk)
+    o, l = r.sdpa(q, k, v, float(np.float32(1.0) / np.sqrt(np.float32(dk))), bool(causal))
+    G[f"sdpa_{BH}x{S}x{dk}_c{causal}_O"], G[f"sdpa_{BH}x{S}x{dk}_c{causal}_L"] = o, l
+
 np.savez_compressed(os.path.join(HERE, "golden.npz"), **G)
 print("wrote", len(G), "arrays,", os.path.getsize(os.path.join(HERE, "golden.npz")), "bytes")
 

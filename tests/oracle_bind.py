@@ -55,6 +55,8 @@ class Oracle:
         L.axo_sum_axis0.argtypes = [f32p, i64, i64, f32p]
         L.axo_sum_axis_f64.argtypes = [f32p, i64, i64, i64, f64p, C.c_void_p]
         L.axo_axpy.argtypes = [f32p, C.c_float, f32p, i64]
+        L.axo_sdpa_fwd.argtypes = [f32p, f32p, f32p, f32p, f32p, i64, i64, i64, C.c_float, C.c_int]
+        L.axo_sdpa_fwd_f64.argtypes = [f32p, f32p, f32p, f64p, f64p, i64, i64, i64, C.c_float, C.c_int]
         L.axo_gelu_tanh.restype = C.c_float
         L.axo_gelu_tanh.argtypes = [C.c_float]
         L.axo_gelu_f64.restype = C.c_double
@@ -162,6 +164,15 @@ class Oracle:
         y = np.ascontiguousarray(y, np.float32).copy()
         self.L.axo_axpy(np.ascontiguousarray(x, np.float32).reshape(-1), alpha, y.reshape(-1), y.size)
         return y
+
+    def sdpa(self, q, k, v, scale, causal=False, f64=False):
+        """(O, L) for q, k, v of shape [BH, S, dk]; fp32 textbook evaluation, or the fp64 ground truth."""
+        BH, S, dk = q.shape
+        q, k, v = (np.ascontiguousarray(t, np.float32).reshape(-1) for t in (q, k, v))
+        dt = np.float64 if f64 else np.float32
+        o, l = np.empty(BH * S * dk, dt), np.empty(BH * S, dt)
+        (self.L.axo_sdpa_fwd_f64 if f64 else self.L.axo_sdpa_fwd)(q, k, v, o, l, BH, S, dk, scale, int(causal))
+        return o.reshape(BH, S, dk), l.reshape(BH, S)
 
     def gelu(self, x):
         x = np.ascontiguousarray(x, np.float32).copy()
@@ -281,6 +292,9 @@ class RefLib:
         L.ax_compute_gemm_relu.argtypes = [TP, TP, TP, TP]
         L.ax_compute_gemm_relu.restype = C.c_int
         L.ax_compute_bias_add.argtypes = [TP, TP, C.c_int, TP]
+        for name in ("ax_fused_attention_fwd", "ax_fused_attention_fwd_causal"):
+            getattr(L, name).restype = None
+            getattr(L, name).argtypes = [f32p, f32p, f32p, f32p, f32p, i64, i64, i64, C.c_float]
         L.ax_compute_sum.argtypes = [TP, C.c_int, TP]
         L.ax_compute_axpy.argtypes = [TP, C.c_float, TP]
         L.ax_compute_bias_add.restype = C.c_int
@@ -377,6 +391,15 @@ class RefLib:
         out = self.numpy(ty)
         self.free(tx, ty)
         return out
+
+    def sdpa(self, q, k, v, scale, causal=False):
+        """The reference's fused CPU attention (src/core/fused_attention.c:559-573): (O, L)."""
+        BH, S, dk = q.shape
+        q, k, v = (np.ascontiguousarray(t, np.float32).reshape(-1) for t in (q, k, v))
+        o, l = np.zeros(BH * S * dk, np.float32), np.zeros(BH * S, np.float32)
+        fn = self.L.ax_fused_attention_fwd_causal if causal else self.L.ax_fused_attention_fwd
+        fn(q, k, v, o, l, BH, S, dk, scale)
+        return o.reshape(BH, S, dk), l.reshape(BH, S)
 
     def gemm_relu(self, a, b, bias):
         self.backend(self.CPU_SIMD)

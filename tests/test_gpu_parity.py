@@ -393,10 +393,12 @@ def test_elementwise_slots(hip, oracle, golden):
     hip.check(hip.L.axhip_fill_f32(out.ptr, 2.5, x.size))
     assert (out.numpy() == 2.5).all()
     bias = oracle.normal((1001,), 0, 1)
-    hip.check(hip.L.axhip_bias_add(dx.ptr, hip.array(bias).ptr, 37, 1001, 1, out.ptr))
+    dbias = hip.array(bias)
+    hip.check(hip.L.axhip_bias_add(dx.ptr, dbias.ptr, 37, 1001, 1, out.ptr))
     assert np.array_equal(out.numpy(), x + bias[None, :])
     rb = oracle.normal((37,), 0, 1)
-    hip.check(hip.L.axhip_bias_add(dx.ptr, hip.array(rb).ptr, 1, 37, 1001, out.ptr))
+    drb = hip.array(rb)
+    hip.check(hip.L.axhip_bias_add(dx.ptr, drb.ptr, 1, 37, 1001, out.ptr))
     assert np.array_equal(out.numpy(), x + rb[:, None])
     z = hip.empty((1000,))                                               # zero-filled allocation
     assert not z.numpy().any()
@@ -417,7 +419,8 @@ def test_sum_axis(hip, oracle, golden, shape, axis):
     x = oracle.uniform(shape, -1, 1)
     outer, inner = int(np.prod(shape[:axis])), int(np.prod(shape[axis + 1:]))
     out = hip.empty(shape[:axis] + shape[axis + 1:] or (1,))
-    hip.check(hip.L.axhip_sum_axis(hip.array(x).ptr, outer, shape[axis], inner, out.ptr))
+    dx = hip.array(x)
+    hip.check(hip.L.axhip_sum_axis(dx.ptr, outer, shape[axis], inner, out.ptr))
     got = out.numpy().reshape(shape[:axis] + shape[axis + 1:])
     s64, sabs = oracle.sum_axis_f64(x, axis)
     assert (np.abs(got - s64) <= SUM_BOUND * sabs + 1e-30).all()
@@ -428,7 +431,7 @@ def test_sum_axis(hip, oracle, golden, shape, axis):
     if name:
         assert np.abs(got - golden[f"{name}_axis{axis}"]).max() <= SUM_BOUND * sabs.max()
     # run-to-run determinism
-    hip.check(hip.L.axhip_sum_axis(hip.array(x).ptr, outer, shape[axis], inner, out.ptr))
+    hip.check(hip.L.axhip_sum_axis(dx.ptr, outer, shape[axis], inner, out.ptr))
     assert np.array_equal(out.numpy().reshape(got.shape), got)
 
 
@@ -473,10 +476,74 @@ def test_dense_backward_blocks(hip, oracle, golden, M, K, N):
     # gradient that already exists: temp + axpy (what the reference does) == gemm with beta = 1
     g0 = oracle.uniform((K, N), -1, 1)
     acc1 = hip.array(g0)
-    hip.check(hip.L.axhip_axpy(hip.array(dW).ptr, 1.0, acc1.ptr, K * N))
+    ddw = hip.array(dW)
+    hip.check(hip.L.axhip_axpy(ddw.ptr, 1.0, acc1.ptr, K * N))
     assert np.array_equal(acc1.numpy(), g0 + dW)
     acc2 = hip.sgemm(dx_, ddy, transa=True, beta=1.0, c=hip.array(g0)).numpy()
     assert np.abs(acc2 - (g0 + dW)).max() <= 1e-6 * max(1.0, np.abs(dW).max())
+
+
+# ------------------------------------------------------------------ attention forward
+SDPA_TOL = 1e-5      # max |gpu - fp64 ground truth| on O (entries are convex combinations of V in [-0.5, 0.5))
+
+
+def run_sdpa(hip, q, k, v, scale, causal, want_l=True):
+    BH, S, dk = q.shape
+    o = hip.empty((BH, S, dk))
+    l = hip.empty((BH, S)) if want_l else None
+    dq, dk_, dv = hip.array(q), hip.array(k), hip.array(v)      # named: they must outlive the call
+    hip.check(hip.L.axhip_sdpa_fwd(dq.ptr, dk_.ptr, dv.ptr, o.ptr,
+                                   l.ptr if l is not None else None, BH, S, dk, scale, int(causal)))
+    return o.numpy(), (l.numpy() if l is not None else None)
+
+
+@pytest.mark.parametrize("BH,S,dk,causal", [(6, 24, 16, 0), (2, 16, 8, 1), (3, 128, 64, 0), (3, 128, 64, 1),
+                                            (2, 40, 32, 1), (5, 256, 64, 0), (5, 256, 64, 1), (2, 1, 64, 0),
+                                            (1, 129, 64, 1), (3, 384, 64, 1), (2, 77, 128, 0), (4, 512, 64, 0)])
+def test_sdpa_forward(hip, oracle, golden, BH, S, dk, causal):
+    say("sdpa", BH, S, dk, causal)
+    oracle.seed(5000 + BH * 100 + S + dk + causal)
+    q, k, v = (oracle.uniform((BH, S, dk), -0.5, 0.5) for _ in range(3))
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(dk)))
+    o, l = run_sdpa(hip, q, k, v, scale, causal)
+    say("  kernel", hip.last_kernel())
+    o64, l64 = oracle.sdpa(q, k, v, scale, causal, f64=True)
+    assert np.abs(o - o64).max() <= SDPA_TOL, np.abs(o - o64).max()
+    assert np.abs(l - l64).max() <= 1e-5 * max(1.0, np.abs(l64).max())
+    o32, _ = oracle.sdpa(q, k, v, scale, causal)
+    assert np.abs(o - o32).max() < 1e-4                                   # the reference test's own gate
+    key = f"sdpa_{BH}x{S}x{dk}_c{causal}_O"
+    if key in golden:
+        assert np.abs(o - golden[key]).max() < 1e-4
+        assert np.abs(l - golden[key[:-1] + "L"]).max() < 1e-4
+    o2, none = run_sdpa(hip, q, k, v, scale, causal, want_l=False)        # L = NULL, and determinism
+    assert none is None and np.array_equal(o2, o)
+
+
+def test_sdpa_large_scores_and_full_size(hip, oracle):
+    """Scores far from zero (the running maximum must absorb them), and the attention shape of
+    the benchmark (512 heads of [512, 64]) checked on sampled heads."""
+    oracle.seed(77)
+    q, k, v = (oracle.uniform((2, 256, 64), -1, 1) for _ in range(3))
+    q *= 30.0
+    o, l = run_sdpa(hip, q, k, v, 1.0, False)
+    o64, l64 = oracle.sdpa(q, k, v, 1.0, False, f64=True)
+    # |score| reaches ~300 here: one fp32 rounding of a score moves its exponential by 300 * 2^-24 = 2e-5 relative
+    assert np.isfinite(o).all() and np.abs(o - o64).max() <= 1e-4
+    assert np.abs(l - l64).max() <= 1e-5 * np.abs(l64).max()
+    BH, S, dk = 512, 512, 64
+    q, k, v = (oracle.normal((BH, S, dk), 0, 1) for _ in range(3))
+    scale = 0.125
+    for causal in (False, True):
+        o, l = run_sdpa(hip, q, k, v, scale, causal)
+        say("  full size", hip.last_kernel())
+        assert hip.last_kernel().startswith("sdpa_fused_dk64")
+        heads = [0, 1, 255, 511]
+        o64, l64 = oracle.sdpa(q[heads], k[heads], v[heads], scale, causal, f64=True)
+        assert np.abs(o[heads] - o64).max() <= 5e-5      # V ~ N(0,1): entries up to ~4
+        assert np.abs(l[heads] - l64).max() <= 1e-5 * np.abs(l64).max()
+        # each output row is a convex combination of value rows
+        assert (o.max(axis=1) <= v.max(axis=1) + 1e-4).all() and (o.min(axis=1) >= v.min(axis=1) - 1e-4).all()
 
 
 def test_error_paths(hip):

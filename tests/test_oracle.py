@@ -243,6 +243,58 @@ def test_dense_backward_blocks_match_reference_vectors(oracle, golden):
                           np.arange(5, dtype=np.float32) + 2)
 
 
+# ---------------------------------------------------------------- attention forward
+SDPA_GOLDEN = [(6, 24, 16, 0), (2, 16, 8, 1), (3, 128, 64, 0), (3, 128, 64, 1), (2, 40, 32, 1)]
+
+
+def sdpa_inputs(oracle, BH, S, dk, causal):
+    oracle.seed(5000 + BH * 100 + S + dk + causal)
+    return tuple(oracle.uniform((BH, S, dk), -0.5, 0.5) for _ in range(3))
+
+
+@pytest.mark.parametrize("BH,S,dk,causal", SDPA_GOLDEN)
+def test_sdpa_restatement_against_reference_vectors(oracle, golden, BH, S, dk, causal):
+    """The textbook evaluation (the yardstick of tests/test_attention.c) against what the
+    reference's fused CPU kernel produced, at the reference test's gate of 1e-4, and against
+    the fp64 ground truth; plus what the mathematics fixes."""
+    q, k, v = sdpa_inputs(oracle, BH, S, dk, causal)
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(dk)))
+    o, l = oracle.sdpa(q, k, v, scale, causal)
+    o64, l64 = oracle.sdpa(q, k, v, scale, causal, f64=True)
+    ref_o, ref_l = golden[f"sdpa_{BH}x{S}x{dk}_c{causal}_O"], golden[f"sdpa_{BH}x{S}x{dk}_c{causal}_L"]
+    assert np.abs(o - ref_o).max() < 1e-4 and np.abs(l - ref_l).max() < 1e-4
+    assert np.abs(o - o64).max() < 2e-6 and np.abs(ref_o - o64).max() < 1e-5
+    assert np.abs(l - l64).max() < 1e-5 and np.abs(ref_l - l64).max() < 1e-4
+    # numpy evaluation of the definition
+    s = np.einsum("hid,hjd->hij", q.astype(np.float64), k.astype(np.float64)) * scale
+    if causal:
+        s = np.where(np.tril(np.ones((S, S), bool))[None], s, -np.inf)
+    p = np.exp(s - s.max(axis=-1, keepdims=True))
+    want = np.einsum("hij,hjd->hid", p / p.sum(axis=-1, keepdims=True), v.astype(np.float64))
+    assert np.abs(o64 - want).max() < 1e-12
+    assert np.abs(l64 - (s.max(axis=-1) + np.log(p.sum(axis=-1)))).max() < 1e-12
+
+
+def test_sdpa_closed_forms(oracle):
+    # identical keys: uniform attention, O = mean of V, L = score + log S
+    BH, S, dk = 2, 33, 8
+    oracle.seed(9)
+    q, v = oracle.uniform((BH, S, dk), -1, 1), oracle.uniform((BH, S, dk), -1, 1)
+    k = np.repeat(oracle.uniform((BH, 1, dk), -1, 1), S, axis=1)
+    o, l = oracle.sdpa(q, k, v, 0.5)
+    assert np.abs(o - v.mean(axis=1, keepdims=True)).max() < 1e-6
+    score = 0.5 * np.einsum("hid,hd->hi", q, k[:, 0])
+    assert np.abs(l - (score + np.log(S))).max() < 1e-5
+    # causal: the first query sees only key 0; a one-hot dominant key selects its value row
+    o, l = oracle.sdpa(q, k, v, 0.5, causal=True)
+    assert np.abs(o[:, 0] - v[:, 0]).max() < 1e-7
+    q1 = np.zeros((1, 4, 4), np.float32); q1[0, :, 0] = 1
+    k1 = np.zeros((1, 4, 4), np.float32); k1[0, 2, 0] = 100
+    v1 = np.arange(16, dtype=np.float32).reshape(1, 4, 4)
+    o, _ = oracle.sdpa(q1, k1, v1, 1.0)
+    assert np.abs(o[0] - v1[0, 2]).max() < 1e-6
+
+
 # ---------------------------------------------------------------- live cross-check
 def test_oracle_equals_compiled_reference(oracle, reflib):
     oracle.seed(11)
