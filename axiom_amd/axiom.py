@@ -54,6 +54,8 @@ SIGNATURES = {
     "ax_compute_bias_add": (C.c_int, [TP, TP, C.c_int, TP]),
     "ax_compute_relu": (C.c_int, [TP, TP]), "ax_compute_gelu": (C.c_int, [TP, TP]),
     "ax_compute_fill": (C.c_int, [TP, C.c_double]), "ax_compute_copy": (C.c_int, [TP, TP]),
+    "ax_hip_sdpa_fwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, i64, i64, i64,
+                                 C.c_float, C.c_bool, C.c_void_p]),
     "ax_compute_sum": (C.c_int, [TP, C.c_int, TP]), "ax_compute_axpy": (C.c_int, [TP, C.c_float, TP]),
     "ax_compute_gemm_bias_act": (C.c_int, [TP, TP, TP, C.c_int, TP]),
     "ax_compute_has_gemm_relu": (C.c_int, []), "ax_compute_has_gemm_nt": (C.c_int, []),

@@ -282,6 +282,19 @@ static ax_status_t hook_d2d(void *d, const void *s, size_t n) { return lift(axhi
 
 const ax_backend_ops_t ax_hip_ops = AX_HIP_OPS_INIT(AX_DEVICE_HIP);
 
+/* Attention forward on device pointers, with the signature of the `sdpa_fwd` member of the
+ * reference's GPU extension table (include/axiom/internal/cuda_extension.h:86-92; its CUDA
+ * implementation is ax_cuda_sdpa_fwd, cuda/ops_attention.cu:299-392).  P_save (a copy of the
+ * probabilities for the save-aware backward) is not produced: the fused kernel never forms them. */
+ax_status_t ax_hip_sdpa_fwd(const float *Q, const float *K, const float *V, float *out, float *L,
+                            int64_t BH, int64_t S, int64_t dk, float scale, bool causal, float *P_save) {
+    if (P_save) {
+        ax_err_set(AX_ERR_NOT_IMPLEMENTED, "hip sdpa_fwd: P_save is not supported");
+        return AX_ERR_NOT_IMPLEMENTED;
+    }
+    return lift(axhip_sdpa_fwd(Q, K, V, out, L, BH, S, dk, scale, causal ? 1 : 0), "hip sdpa_fwd");
+}
+
 const ax_backend_ops_t *ax_hip_ops_for_device(ax_device_t as_device) {
     static ax_backend_ops_t alias = AX_HIP_OPS_INIT(AX_DEVICE_HIP);
     alias.device = as_device;

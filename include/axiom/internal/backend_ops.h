@@ -119,6 +119,12 @@ extern const ax_backend_ops_t ax_hip_ops;
  * static storage, rewritten by each call. */
 const ax_backend_ops_t *ax_hip_ops_for_device(ax_device_t as_device);
 
+/* Attention forward on device pointers: same arguments as the sdpa_fwd member of the
+ * reference's GPU extension table (include/axiom/internal/cuda_extension.h:86-92).  Q, K, V,
+ * out are [BH, S, dk] fp32, L is [BH, S] or NULL; P_save must be NULL. */
+ax_status_t ax_hip_sdpa_fwd(const float *Q, const float *K, const float *V, float *out, float *L,
+                            int64_t BH, int64_t S, int64_t dk, float scale, bool causal, float *P_save);
+
 #ifdef __cplusplus
 }
 #endif

@@ -123,6 +123,26 @@ def test_dense_backward_through_dispatch(ax, oracle):
     ax.free(tx, tw, tdy, dA, dW, db, tmp, g, rows, one)
 
 
+def test_attention_forward_extension_entry(ax, oracle):
+    """ax_hip_sdpa_fwd: the sdpa_fwd member of the reference's GPU extension table
+    (include/axiom/internal/cuda_extension.h:86-92) on device tensors of the host core."""
+    L = ax.L
+    oracle.seed(64)
+    BH, S, dk = 4, 256, 64
+    q, k, v = (oracle.uniform((BH, S, dk), -0.5, 0.5) for _ in range(3))
+    tq, tk, tv = ax.from_numpy(q), ax.from_numpy(k), ax.from_numpy(v)
+    to, tl = ax.empty((BH, S, dk)), ax.empty((BH, S))
+    ptr = lambda t: t.contents.storage.contents.data
+    for causal in (False, True):
+        assert L.ax_hip_sdpa_fwd(ptr(tq), ptr(tk), ptr(tv), ptr(to), ptr(tl), BH, S, dk, 0.125, causal, None) == 0
+        o64, l64 = oracle.sdpa(q, k, v, 0.125, causal, f64=True)
+        assert np.abs(ax.to_numpy(to) - o64).max() <= 1e-5
+        assert np.abs(ax.to_numpy(tl) - l64).max() <= 1e-5 * max(1.0, np.abs(l64).max())
+    assert L.ax_hip_sdpa_fwd(ptr(tq), ptr(tk), ptr(tv), ptr(to), None, BH, S, dk, 0.125, False, ptr(tl)) == 10
+    assert b"P_save" in L.ax_err_last_message()
+    ax.free(tq, tk, tv, to, tl)
+
+
 def test_reference_gpu_vs_cpu_template(ax, oracle):
     """tests/test_cuda.c:213-244: 64x128 . 128x32, rand(-0.1,0.1), every element within 1e-3."""
     L = ax.L
