@@ -236,16 +236,22 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     const int tiles_m = (int)(M / BM), tiles_n = (int)(N / BN), total = tiles_m * tiles_n;
     const int slabs = (int)(K / BKB);
 
-    // load instruction j (0..3) of wave w fills rows (j*8+w)*8 .. +8 of an operand stage
-    unsigned voff[4];
+    // Loads and stores retire in issue order within a wave, so a wave that has stores in flight
+    // cannot see its later loads complete before them.  The two are therefore kept on different
+    // waves: waves 0-3 issue every global->LDS load of the workgroup (and never store), waves
+    // 4-7 issue every global store (and never load), and the write-back of one tile drains to
+    // HBM underneath the next tile's slabs instead of stalling them.
+    const bool loader = wave < 4;
+    // load instruction j (0..7) of loader wave w fills rows (j*4+w)*8 .. +8 of an operand stage
+    unsigned voff[8];
     {
         const int sw = (wave & 1) * 4 + (lane >> 4);      // (row >> 1) & 7 of this lane's row
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-            voff[j] = (unsigned)(((j * 8 + wave) * 8 + (lane >> 3)) * K + (((lane & 7) ^ sw) << 4));
+        for (int j = 0; j < 8; j++)
+            voff[j] = (unsigned)(((j * 4 + (wave & 3)) * 8 + (lane >> 3)) * K + (((lane & 7) ^ sw) << 4));
     }
     const int8_t *gx = X, *gw = W;
-    const unsigned lds_w = (unsigned)(uintptr_t)lds + wave * 1024;
+    const unsigned lds_w = (unsigned)(uintptr_t)lds + (wave & 3) * 1024;
 
     // fragment reads: lane (frow, fhalf) of tile i takes row i*32+frow, logical chunk ks*2+fhalf
     const int frow = lane & 31, fhalf = lane >> 5;
@@ -261,15 +267,18 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     }
 
     typedef float v4f_t __attribute__((ext_vector_type(4)));
-    float *lds_scale = reinterpret_cast<float *>(lds + 4 * OPER), *lds_bias = lds_scale + BN;
+    float *lds_scale = reinterpret_cast<float *>(lds + 4 * OPER);     // [2 slots][scale 256 | bias 256]
     v16i acc[TM][TN];
 
-#define AXI8_LOAD_X(stage, j) AXI8_LOAD_LDS(lds_w + (stage) * OPER + (j) * 8192, voff[j], gx)
-#define AXI8_LOAD_W(stage, j) AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + (j) * 8192, voff[j], gw)
+#define AXI8_LOAD_X(stage, j) AXI8_LOAD_LDS(lds_w + (stage) * OPER + (j) * 4096, voff[j], gx)
+#define AXI8_LOAD_W(stage, j) AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + (j) * 4096, voff[j], gw)
+// a loader wave's 16 loads of the next unfetched slab
 #define AXI8_ISSUE(stage)                                                                 \
     do {                                                                                  \
         AXI8_LOAD_X(stage, 0); AXI8_LOAD_X(stage, 1); AXI8_LOAD_X(stage, 2); AXI8_LOAD_X(stage, 3); \
+        AXI8_LOAD_X(stage, 4); AXI8_LOAD_X(stage, 5); AXI8_LOAD_X(stage, 6); AXI8_LOAD_X(stage, 7); \
         AXI8_LOAD_W(stage, 0); AXI8_LOAD_W(stage, 1); AXI8_LOAD_W(stage, 2); AXI8_LOAD_W(stage, 3); \
+        AXI8_LOAD_W(stage, 4); AXI8_LOAD_W(stage, 5); AXI8_LOAD_W(stage, 6); AXI8_LOAD_W(stage, 7); \
         gx += BKB;                                                                        \
         gw += BKB;                                                                        \
     } while (0)
@@ -294,32 +303,32 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 
 // The 8 MFMAs of the k-step held in fragment buffer `buf`.  Between them, so that their issue
 // falls into the shadow of the MFMA before: (RD) the 6 fragment reads of k-step rks of stage
-// rstage into the other buffer, in the order the next block consumes them; (LD) the 8 loads of
-// the next unfetched slab into stage lstage.
+// rstage into the other buffer, in the order the next block consumes them; (LD, loader waves
+// only) the 16 loads of the next unfetched slab into stage lstage.
 #define AXI8_BLOCK(buf, RD, rstage, rks, LD, lstage)                                            \
     do {                                                                                        \
         AXI8_M(buf, 0);                                                                         \
         if (RD) AXI8_DS_READ(fx[1 - (buf)][0], rx[rks], (rstage) * OPER + 0 * 4096);            \
-        if (LD) AXI8_LOAD_X(lstage, 0);                                                         \
+        if (LD) { AXI8_LOAD_X(lstage, 0); AXI8_LOAD_W(lstage, 0); }                             \
         AXI8_M(buf, 1);                                                                         \
         if (RD) AXI8_DS_READ(fw[1 - (buf)][0], rw[rks], (rstage) * OPER + 0 * 4096);            \
-        if (LD) AXI8_LOAD_X(lstage, 1);                                                         \
+        if (LD) { AXI8_LOAD_X(lstage, 1); AXI8_LOAD_W(lstage, 1); }                             \
         AXI8_M(buf, 2);                                                                         \
         if (RD) AXI8_DS_READ(fw[1 - (buf)][1], rw[rks], (rstage) * OPER + 1 * 4096);            \
-        if (LD) AXI8_LOAD_X(lstage, 2);                                                         \
+        if (LD) { AXI8_LOAD_X(lstage, 2); AXI8_LOAD_W(lstage, 2); }                             \
         AXI8_M(buf, 3);                                                                         \
         if (RD) AXI8_DS_READ(fx[1 - (buf)][1], rx[rks], (rstage) * OPER + 1 * 4096);            \
-        if (LD) AXI8_LOAD_X(lstage, 3);                                                         \
+        if (LD) { AXI8_LOAD_X(lstage, 3); AXI8_LOAD_W(lstage, 3); }                             \
         AXI8_M(buf, 4);                                                                         \
         if (RD) AXI8_DS_READ(fx[1 - (buf)][2], rx[rks], (rstage) * OPER + 2 * 4096);            \
-        if (LD) AXI8_LOAD_W(lstage, 0);                                                         \
+        if (LD) { AXI8_LOAD_X(lstage, 4); AXI8_LOAD_W(lstage, 4); }                             \
         AXI8_M(buf, 5);                                                                         \
         if (RD) AXI8_DS_READ(fx[1 - (buf)][3], rx[rks], (rstage) * OPER + 3 * 4096);            \
-        if (LD) AXI8_LOAD_W(lstage, 1);                                                         \
+        if (LD) { AXI8_LOAD_X(lstage, 5); AXI8_LOAD_W(lstage, 5); }                             \
         AXI8_M(buf, 6);                                                                         \
-        if (LD) AXI8_LOAD_W(lstage, 2);                                                         \
+        if (LD) { AXI8_LOAD_X(lstage, 6); AXI8_LOAD_W(lstage, 6); }                             \
         AXI8_M(buf, 7);                                                                         \
-        if (LD) { AXI8_LOAD_W(lstage, 3); gx += BKB; gw += BKB; }                               \
+        if (LD) { AXI8_LOAD_X(lstage, 7); AXI8_LOAD_W(lstage, 7); gx += BKB; gw += BKB; }       \
         __builtin_amdgcn_sched_barrier(0);                                                      \
     } while (0)
 
@@ -339,30 +348,79 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         AXI8_WAIT_FRAGS();                                                   \
         AXI8_BLOCK(0, 1, stage, 3, 0, 0);                                    \
         AXI8_WAIT_FRAGS();                                                   \
-        AXI8_VM0();                                                          \
+        if (loader) AXI8_VM0();                                              \
         __builtin_amdgcn_s_barrier();                                        \
         __builtin_amdgcn_sched_barrier(0);                                   \
-        AXI8_BLOCK(1, 1, 1 - (stage), 0, more2, stage);                      \
+        AXI8_BLOCK(1, 1, 1 - (stage), 0, (more2) && loader, stage);          \
     } while (0)
 
     // Persistent: one workgroup per CU walks tiles t = blockIdx.x, + gridDim.x, ... (the same
     // tile a non-persistent launch would hand that CU next).  With an even slab count the last
-    // slab of a tile sits in stage 1, so the first slab of the next tile is fetched into stage 0
-    // before the write-back starts and the stores drain under the next tile's first slabs: loads
-    // and stores complete in issue order, so "at most 32 outstanding" (the write-back's stores of
-    // one wave) means the 8 loads issued before them have landed.
-    const bool carry = (slabs & 1) == 0 && acc_out == nullptr;
+    // slab of a tile sits in stage 1, so the loader waves fetch the first slab of the next tile
+    // into stage 0 before the write-back starts.
+    const bool carry = (slabs & 1) == 0;
     bool fetched = false;
-    v4f_t col_v = {0.f, 0.f, 0.f, 0.f};      // waves 0/1: scales / biases of 4 columns of the coming tile
-    auto fetch_cols = [&](int64_t n0) {
-        if (out && tid < 128) {
-            const int c4 = (tid & 63) * 4;
-            col_v = v4f_t{0.f, 0.f, 0.f, 0.f};
-            if (tid < 64) col_v = *reinterpret_cast<const v4f_t *>(w_scales + n0 + c4);
-            else if (bias) col_v = *reinterpret_cast<const v4f_t *>(bias + n0 + c4);
+    // Per-channel scale (premultiplied by x_scale) and bias of a tile's 256 columns go to LDS
+    // ahead of its write-back, into one of two slots so the coming tile's can be staged while
+    // the current tile's are still being read.  Wave 0 only, behind one scalar branch: the
+    // waits the compiler places around these loads must stay out of the storer waves' path,
+    // where they would wait for the stores in flight.
+    v4f_t col_s = {0.f, 0.f, 0.f, 0.f}, col_b = {0.f, 0.f, 0.f, 0.f};
+    auto load_cols = [&](int64_t n0) {            // issued a whole tile ahead of store_cols
+        if (out && wave == 0) {
+            col_s = *reinterpret_cast<const v4f_t *>(w_scales + n0 + lane * 4);
+            if (bias) col_b = *reinterpret_cast<const v4f_t *>(bias + n0 + lane * 4);
         }
     };
+    auto store_cols = [&](int slot) {
+        if (out && wave == 0) {
+            v4f_t v = col_s;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = x_scale * v[e];
+            float *dst = lds_scale + slot * 2 * BN + lane * 4;
+            *reinterpret_cast<v4f_t *>(dst) = v;
+            *reinterpret_cast<v4f_t *>(dst + BN) = col_b;
+        }
+    };
+    int slot = 0;
     v4i fx[2][TM], fw[2][TN];
+
+    // Write-back of one 32x32 sub-tile per wave and round.  With W as the MFMA's first operand,
+    // register v of lane l holds m = (l&31), n = 8*(v>>2) + 4*(l>>5) + (v&3) of the sub-tile:
+    // four consecutive n per lane.  Every wave writes its sub-tile (16-byte chunk c of row r at
+    // chunk c ^ ((r>>1)&7), conflict-free both ways) into its 4 KiB of a turn buffer; after the
+    // barrier storer wave 4+s reads the sub-tiles of waves 2s and 2s+1 back row-major and stores
+    // whole 128-byte rows.  The two turn buffers (stage 1 of X and of W, dead after the loop's
+    // last barrier) alternate, so one barrier per round is enough: a buffer is rewritten two
+    // rounds later, after every storer has passed the barrier in between.
+    int round = 0;
+    auto emit = [&](const auto (&r)[4], auto *base, int64_t m0, int64_t n0, int i, int j) {
+        typedef typename std::remove_const<typename std::remove_reference<decltype(r[0])>::type>::type V4;
+        unsigned char *buf = lds + ((round & 1) ? 3 * OPER : OPER);
+        round++;
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            *reinterpret_cast<V4 *>(buf + wave * 4096 + frow * 128 + (((2 * g + fhalf) ^ ((frow >> 1) & 7)) << 4)) = r[g];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+        if (!loader) {
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const int src = 2 * (wave - 4) + q;                     // wave whose sub-tile this is
+                auto *dst = base + (m0 + (src / WAVES_N) * WTM + i * 32) * N + n0 + (src % WAVES_N) * WTN + j * 32;
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    const int row = p * 8 + (lane >> 3);
+                    const V4 v = *reinterpret_cast<const V4 *>(buf + src * 4096 + row * 128 +
+                                                               (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+                    // streaming store: the 256 KB a tile writes must not evict the operand panels the
+                    // XCD's other workgroups are re-reading from its 4 MB L2 (plain stores: +30 us)
+                    __builtin_nontemporal_store(v, reinterpret_cast<V4 *>(dst + (int64_t)row * N + (lane & 7) * 4));
+                }
+            }
+        }
+    };
 
     for (int t = blockIdx.x; t < total; t += gridDim.x) {
         int tm, tn;
@@ -371,20 +429,16 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         if (!fetched) {
             gx = X + m0 * K;
             gw = W + n0 * K;
-            AXI8_ISSUE(0);
-            fetch_cols(n0);
+            if (loader) AXI8_ISSUE(0);
+            load_cols(n0);
+            store_cols(slot);
         }
-        // Per-channel scale (premultiplied by x_scale) and bias of this tile's 256 columns go to
-        // LDS, so the write-back does not wait on global loads.
-        if (out && tid < 128) {
-            const int c4 = (tid & 63) * 4;
-            if (tid < 64) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) col_v[e] = x_scale * col_v[e];
-                *reinterpret_cast<v4f_t *>(lds_scale + c4) = col_v;
-            } else {
-                *reinterpret_cast<v4f_t *>(lds_bias + c4) = col_v;
-            }
+        const int t_next = t + (int)gridDim.x;
+        const bool will_fetch = carry && t_next < total;
+        int tm2 = 0, tn2 = 0;
+        if (will_fetch) {
+            tile_of_block(t_next, tiles_m, tiles_n, tm2, tn2);
+            load_cols((int64_t)tn2 * BN);
         }
 #pragma unroll
         for (int i = 0; i < TM; i++)
@@ -393,10 +447,10 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 #pragma unroll
                 for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
 
-        if (fetched) AXI8_VM(32); else AXI8_VM(0);
+        if (loader) AXI8_VM0();
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
         __builtin_amdgcn_s_barrier();
-        if (slabs > 1) AXI8_ISSUE(1);
+        if (slabs > 1 && loader) AXI8_ISSUE(1);
         AXI8_FRAGS(0, 0, 0);
 
         for (int s = 0; s < slabs; s += 2) {       // the flags are wave-uniform: scalar branches only
@@ -405,23 +459,14 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         }
         AXI8_WAIT_FRAGS();      // the stale reads must land before their registers are reused
 
-        const int t_next = t + (int)gridDim.x;
-        fetched = carry && t_next < total;
+        fetched = will_fetch;
         if (fetched) {
-            int tm2, tn2;
-            tile_of_block(t_next, tiles_m, tiles_n, tm2, tn2);
+            store_cols(slot ^ 1);
             gx = X + (int64_t)tm2 * BM * K;
             gw = W + (int64_t)tn2 * BN * K;
-            AXI8_ISSUE(0);
-            fetch_cols((int64_t)tn2 * BN);
+            if (loader) AXI8_ISSUE(0);
         }
 
-        // Write-back.  With W as the MFMA's first operand, register v of lane l holds
-        // m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3): four consecutive n per lane.
-        // Stage 1 of X is dead after the loop's last barrier; each wave turns its tiles through
-        // 4 KiB of it to store whole 128-byte rows.
-        unsigned char *turn = lds + OPER + wave * 4096;
-        const int64_t trow = m0 + wm * WTM, tcol = n0 + wn * WTN;
         if (acc_out) {
 #pragma unroll
             for (int i = 0; i < TM; i++)
@@ -431,11 +476,11 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 #pragma unroll
                     for (int g = 0; g < 4; g++)
                         r[g] = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                    turn_tile_and_store(turn, lane, r, acc_out + (trow + i * 32) * N + tcol + j * 32, N);
+                    emit(r, acc_out, m0, n0, i, j);
                 }
         }
         if (out) {
-            const float *sp = lds_scale + wn * WTN + 4 * fhalf, *bp = lds_bias + wn * WTN + 4 * fhalf;
+            const float *sp = lds_scale + slot * 2 * BN + wn * WTN + 4 * fhalf, *bp = sp + BN;
             const bool has_bias = bias != nullptr;
 #pragma unroll
             for (int j = 0; j < TN; j++) {
@@ -456,13 +501,13 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
                             // a fused multiply-add with bias = 0 would round differently from the plain product
                             r[g][e] = apply_act(has_bias ? __builtin_fmaf(f, sc[g][e], bv[g][e]) : f * sc[g][e], ACT);
                         }
-                    turn_tile_and_store(turn, lane, r, out + (trow + i * 32) * N + tcol + j * 32, N);
+                    emit(r, out, m0, n0, i, j);
                 }
             }
         }
-        // Every wave is done with lds_scale / lds_bias and the turn area before the next tile
-        // overwrites them.  Only LDS traffic is ordered here: waiting for the stores as well
-        // (as __syncthreads would) is exactly what the persistent loop avoids.
+        slot ^= 1;
+        // Every wave is done with the turn buffers and this tile's scale/bias slot before the next
+        // tile overwrites them.  Only LDS traffic is ordered here, never the stores.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -694,7 +739,7 @@ int launch_dma(const char *name, const int8_t *x, float x_scale, const int8_t *w
 int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
                const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N,
                int64_t K) {
-    constexpr int smem = 4 * 256 * 128 + 2 * 256 * 4;   // two stages of both operands + scale and bias
+    constexpr int smem = 4 * 256 * 128 + 2 * 2 * 256 * 4;   // two stages of both operands + two slots of scale and bias
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
                            const float *, float *, int32_t *);
     static const kern_t kerns[3] = {k_qgemm_w8a8_256<AXHIP_ACT_NONE>, k_qgemm_w8a8_256<AXHIP_ACT_RELU>,
