@@ -30,8 +30,8 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
 # Bytes that cross the L2 boundary per headline launch, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of `bench.py --counter-probe`, each scaled by what the same counter reads for
 # the probe's copy-shaped kernel of known size (profiles/qgemm_w8a8_256_8192cube_hbm_counters.txt):
-# 806.8 MB fetched (the counter under-reads by 2.000) + 268.4 MB written (scale 1.000).
-HEADLINE_TRAFFIC_BYTES = 806.8e6 + 268.4e6
+# 806.5 MB fetched (the counter under-reads by 2.000) + 268.9 MB written (scale 1.000).
+HEADLINE_TRAFFIC_BYTES = 806.5e6 + 268.9e6
 
 
 def result_line(suite, case, metric, value):
