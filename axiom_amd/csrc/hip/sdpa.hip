@@ -1,7 +1,7 @@
 // Scaled dot-product attention forward: O = softmax(scale * Q K^T [+ causal mask]) V per head,
 // Q, K, V, O [BH, S, dk] row-major fp32, L [BH, S] = log-sum-exp of each score row (or NULL).
 //
-// Fused kernel (dk = 64, S a multiple of 128): the score matrix never leaves the chip.  A
+// Fused kernel (dk = 32, 64 or 128, S a multiple of 128): the score matrix never leaves the chip.  A
 // workgroup of 4 waves owns 128 query rows of one head, a wave 32 of them; keys and values
 // stream through LDS in blocks of 64 (direct-to-LDS loads, two stages).  Both products run on
 // v_mfma_f32_32x32x2_f32 with the query index on the MFMA's column side, so lane l of a wave
@@ -15,9 +15,10 @@
 //   O^T tile:  A = V^T (lane reads V[key][d] with d = l&31), B = the probabilities exactly
 //              where the score MFMA left them: key(v, l>>5) above is also a legal pairing of
 //              the MFMA's two k indices, and a sum over keys does not care about their order.
-// K rows (256 bytes) are XOR-swizzled in 16-byte chunks, applied on the global address side of
-// the load, so a 16-lane ds_read_b128 touches every bank once; V is laid in groups of 4 rows
-// spaced 1152 bytes apart so the two lane halves (keys 4 apart) read different banks.
+// K rows are XOR-swizzled in 16-byte chunks, applied on the global address side of the load, so
+// a 16-lane ds_read_b128 touches every bank once; V is laid out per load instruction with a
+// pitch (or, for dk = 32, a row order) that puts the two lane halves of a fragment read (keys 4
+// apart) on different banks.
 //
 // Every other shape: scores through a workspace, one batched NT GEMM, a row softmax kernel and
 // one batched NN GEMM over as many heads at a time as fit 256 MiB (the structure of
@@ -33,69 +34,101 @@ using namespace axhip;
                  : "memory")
 #define AXS_VM0() __builtin_amdgcn_s_waitcnt(0 | (0 << 14) | (7 << 4) | (15 << 8))
 
-constexpr int SD_DK = 64, SD_BQ = 128, SD_BKV = 64;
-constexpr int SD_KSTAGE = SD_BKV * SD_DK * 4;            // 16 KiB
-constexpr int SD_VGROUP = 1152;                          // 4 rows of 256 B + 128 B
-constexpr int SD_VSTAGE = (SD_BKV / 4) * SD_VGROUP;      // 18 KiB
-constexpr int SD_SMEM = 2 * SD_KSTAGE + 2 * SD_VSTAGE;
+constexpr int SD_BQ = 128, SD_BKV = 64;
 
-template <bool CAUSAL>
+// LDS geometry for head dimension DK (32, 64 or 128).  A direct-to-LDS load instruction moves
+// 1 KiB = RPI whole rows of DK floats.
+template <int DK>
+struct SdGeom {
+    static constexpr int ROWB = DK * 4;                 // bytes per row
+    static constexpr int CH = DK / 4;                   // 16-byte chunks per row
+    static constexpr int RPI = 1024 / ROWB;             // rows per load instruction
+    static constexpr int KSTAGE = SD_BKV * ROWB;        // K block, rows contiguous, chunks swizzled
+    // V block: load-instruction groups spaced so that keys k and k+4 (the two lane halves of a
+    // fragment read) fall 128 bytes apart modulo 256, i.e. on different halves of the banks
+    static constexpr int VGROUP = DK == 64 ? 1152 : DK == 128 ? 1088 : 1024;
+    static constexpr int VSTAGE = (SD_BKV / RPI) * VGROUP;
+    static constexpr int SMEM = 2 * KSTAGE + 2 * VSTAGE;
+    static constexpr int IPW = SD_BKV / RPI / 4;        // load instructions per wave and 64-row block
+    static_assert(DK == 32 || DK == 64 || DK == 128, "head dimension");
+    static_assert(2 * KSTAGE >= SD_BQ * ROWB, "the Q tile is staged through the two K stages");
+
+    // chunk swizzle key of a K/Q row: the 16 rows a ds_read_b128 serves together (same logical
+    // chunk) must land on 16 different 16-byte bank slots
+    __device__ static int swz(int row) { return CH >= 16 ? (row & 15) : ((row >> 1) & 7); }
+    // which row of its group the lane at group position `slot` fetches (V only; DK = 32 keeps
+    // rows k and k+4 next to each other)
+    __device__ static int v_row_of_slot(int slot) { return DK == 32 ? ((slot & 1) * 4 + (slot >> 1)) : slot; }
+    // byte offset of V row `key` inside a stage
+    __device__ static int v_addr(int key) {
+        if (DK == 64) return (key >> 2) * VGROUP + (key & 3) * ROWB;
+        if (DK == 128) return (key >> 1) * VGROUP + (key & 1) * ROWB;
+        return (key >> 3) * VGROUP + (((key & 3) * 2 + ((key >> 2) & 1))) * ROWB;
+    }
+};
+
+template <int DK, bool CAUSAL>
 __global__ void __launch_bounds__(256)
-k_sdpa64(const float *__restrict__ Q, const float *__restrict__ K, const float *__restrict__ V,
-         float *__restrict__ O, float *__restrict__ L, int64_t S, float scale_log2e) {
+k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__restrict__ V,
+       float *__restrict__ O, float *__restrict__ L, int64_t S, float scale_log2e) {
+    using G = SdGeom<DK>;
+    constexpr int KB = DK / 8;                   // 8-wide k-blocks of the score product
+    constexpr int DT = DK / 32;                  // 32-wide column tiles of the output
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int frow = lane & 31, fhalf = lane >> 5;
     const int64_t head = blockIdx.y;
     const int64_t q0 = (int64_t)blockIdx.x * SD_BQ;
-    const float *Qh = Q + head * S * SD_DK, *Kh = K + head * S * SD_DK, *Vh = V + head * S * SD_DK;
+    const float *Qh = Q + head * S * DK, *Kh = K + head * S * DK, *Vh = V + head * S * DK;
     const unsigned lds0 = (unsigned)(uintptr_t)lds;
 
-    // per-lane byte offsets of the direct-to-LDS loads: instruction i of this wave covers rows
-    // 4*(4*i + wave) .. +3 of a 64-row tile, lane l row + (l >> 4), 16-byte chunk (l & 15)
-    unsigned koff[4], voff[4];
+    // per-lane byte offsets of the direct-to-LDS loads: instruction i of this wave is number
+    // 4*i + wave of a 64-row block and covers rows RPI*(4*i + wave) .. + RPI-1
+    unsigned koff[G::IPW], voff[G::IPW];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int row = 4 * (4 * i + wave) + (lane >> 4), c = lane & 15;
-        koff[i] = (unsigned)(row * 256 + ((c ^ (row & 15)) << 4));
-        voff[i] = (unsigned)(row * 256 + (c << 4));
+    for (int i = 0; i < G::IPW; i++) {
+        const int slot = lane / G::CH, c = lane % G::CH;
+        const int krow = G::RPI * (4 * i + wave) + slot;
+        koff[i] = (unsigned)(krow * G::ROWB + ((c ^ G::swz(krow)) << 4));
+        const int vrow = G::RPI * (4 * i + wave) + G::v_row_of_slot(slot);
+        voff[i] = (unsigned)(vrow * G::ROWB + (c << 4));
     }
 
     // ---- Q tile (128 rows) through the two K stages, then into registers ----
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        AXS_LOAD_LDS(lds0 + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * SD_DK));
-        AXS_LOAD_LDS(lds0 + SD_KSTAGE + (4 * i + wave) * 1024, koff[i],
-                     reinterpret_cast<const char *>(Qh + (q0 + 64) * SD_DK));
+    for (int i = 0; i < G::IPW; i++) {
+        AXS_LOAD_LDS(lds0 + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * DK));
+        AXS_LOAD_LDS(lds0 + G::KSTAGE + (4 * i + wave) * 1024, koff[i],
+                     reinterpret_cast<const char *>(Qh + (q0 + 64) * DK));
     }
     AXS_VM0();
     __syncthreads();
-    v4f qf[8];                                   // k-block kb: dk 8*kb + 4*fhalf .. +3 of this lane's query
+    v4f qf[KB];                                  // k-block kb: dk 8*kb + 4*fhalf .. +3 of this lane's query
     {
         const int r = wave * 32 + frow;          // rows 64..127 sit in the second stage, same swizzle
-        const unsigned char *qrow = lds + (r >> 6) * SD_KSTAGE + (r & 63) * 256;
+        const unsigned char *qrow = lds + (r >> 6) * G::KSTAGE + (r & 63) * G::ROWB;
 #pragma unroll
-        for (int kb = 0; kb < 8; kb++)
-            qf[kb] = *reinterpret_cast<const v4f *>(qrow + (((kb * 2 + fhalf) ^ (r & 15)) << 4));
+        for (int kb = 0; kb < KB; kb++)
+            qf[kb] = *reinterpret_cast<const v4f *>(qrow + (((kb * 2 + fhalf) ^ G::swz(r & 63)) << 4));
     }
     __syncthreads();
 
     const int64_t nblocks = CAUSAL ? (q0 + SD_BQ) / SD_BKV : S / SD_BKV;
     auto issue = [&](int64_t blk, int stage) {
-        const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * SD_DK);
-        const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * SD_DK);
+        const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * DK);
+        const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * DK);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            AXS_LOAD_LDS(lds0 + stage * SD_KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
-            AXS_LOAD_LDS(lds0 + 2 * SD_KSTAGE + stage * SD_VSTAGE + (4 * i + wave) * SD_VGROUP, voff[i], vg);
+        for (int i = 0; i < G::IPW; i++) {
+            AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
+            AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff[i], vg);
         }
     };
     issue(0, 0);
 
-    v16f acc_o[2];
+    v16f acc_o[DT];
 #pragma unroll
-    for (int d = 0; d < 2; d++)
+    for (int d = 0; d < DT; d++)
 #pragma unroll
         for (int v = 0; v < 16; v++) acc_o[d][v] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;       // l_run: this lane half's share of the row sum
@@ -106,8 +139,8 @@ k_sdpa64(const float *__restrict__ Q, const float *__restrict__ K, const float *
         AXS_VM0();
         __syncthreads();                          // block blk has landed; stage^1 is free again
         if (blk + 1 < nblocks) issue(blk + 1, stage ^ 1);
-        const unsigned char *ks = lds + stage * SD_KSTAGE;
-        const unsigned char *vs = lds + 2 * SD_KSTAGE + stage * SD_VSTAGE;
+        const unsigned char *ks = lds + stage * G::KSTAGE;
+        const unsigned char *vs = lds + 2 * G::KSTAGE + stage * G::VSTAGE;
 
         // ---- scores of 64 keys ----
         v16f acc_s[2];
@@ -116,10 +149,10 @@ k_sdpa64(const float *__restrict__ Q, const float *__restrict__ K, const float *
 #pragma unroll
             for (int v = 0; v < 16; v++) acc_s[kt][v] = 0.0f;
             const int r = kt * 32 + frow;
-            const unsigned char *krow = ks + r * 256;
+            const unsigned char *krow = ks + r * G::ROWB;
 #pragma unroll
-            for (int kb = 0; kb < 8; kb++) {
-                const v4f kf = *reinterpret_cast<const v4f *>(krow + (((kb * 2 + fhalf) ^ (r & 15)) << 4));
+            for (int kb = 0; kb < KB; kb++) {
+                const v4f kf = *reinterpret_cast<const v4f *>(krow + (((kb * 2 + fhalf) ^ G::swz(r)) << 4));
 #pragma unroll
                 for (int e = 0; e < 4; e++)
                     acc_s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[kb][e], acc_s[kt], 0, 0, 0);
@@ -155,7 +188,7 @@ k_sdpa64(const float *__restrict__ Q, const float *__restrict__ K, const float *
         l_run = l_run * alpha + l_blk;
         m_run = m_new;
 #pragma unroll
-        for (int d = 0; d < 2; d++)
+        for (int d = 0; d < DT; d++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc_o[d][v] *= alpha;
 
@@ -165,9 +198,9 @@ k_sdpa64(const float *__restrict__ Q, const float *__restrict__ K, const float *
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int key = kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3);
-                const float *vrow = reinterpret_cast<const float *>(vs + (key >> 2) * SD_VGROUP + (key & 3) * 256);
+                const float *vrow = reinterpret_cast<const float *>(vs + G::v_addr(key));
 #pragma unroll
-                for (int d = 0; d < 2; d++)
+                for (int d = 0; d < DT; d++)
                     acc_o[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[d * 32 + frow], acc_s[kt][v], acc_o[d], 0, 0, 0);
             }
     }
@@ -175,9 +208,9 @@ k_sdpa64(const float *__restrict__ Q, const float *__restrict__ K, const float *
     // ---- normalise and write: lane owns query qg, dk columns 32*d + 8*g + 4*fhalf .. +3 ----
     const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = 1.0f / l_tot;
-    float *orow = O + (head * S + qg) * SD_DK;
+    float *orow = O + (head * S + qg) * DK;
 #pragma unroll
-    for (int d = 0; d < 2; d++)
+    for (int d = 0; d < DT; d++)
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             v4f r;
@@ -186,6 +219,25 @@ k_sdpa64(const float *__restrict__ Q, const float *__restrict__ K, const float *
             *reinterpret_cast<v4f *>(orow + d * 32 + 8 * g + 4 * fhalf) = r;
         }
     if (L && fhalf == 0) L[head * S + qg] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+}
+
+template <int DK>
+int launch_sdpa(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH, int64_t S,
+                float scale, int causal) {
+    using G = SdGeom<DK>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sdpa<DK, false>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, G::SMEM), "hipFuncSetAttribute");
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sdpa<DK, true>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, G::SMEM), "hipFuncSetAttribute");
+        attr_set = true;
+    }
+    const float sl2 = scale * 1.4426950408889634f;
+    dim3 grid((unsigned)(S / SD_BQ), (unsigned)BH);
+    if (causal) hipLaunchKernelGGL((k_sdpa<DK, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, S, sl2);
+    else hipLaunchKernelGGL((k_sdpa<DK, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, S, sl2);
+    return check_launch("sdpa_fwd");
 }
 
 // One workgroup per score row: mask, maximum, exponentials, sum, normalise in place; L = max + log(sum).
@@ -260,21 +312,19 @@ extern "C" int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, fl
     if (BH < 0 || S < 0 || dk <= 0) return fail(AXHIP_ERR_SHAPE, "sdpa_fwd: bad extent");
     if (BH == 0 || S == 0) return AXHIP_OK;
     const bool aligned = ((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O) & 15) == 0);
-    if (dk == SD_DK && S % SD_BQ == 0 && aligned && BH <= 65535 && S / SD_BQ <= 0x7fffffff) {
-        static bool attr_set = false;
-        if (!attr_set) {
-            AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sdpa64<false>),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, SD_SMEM), "hipFuncSetAttribute");
-            AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sdpa64<true>),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, SD_SMEM), "hipFuncSetAttribute");
-            attr_set = true;
+    if ((dk == 32 || dk == 64 || dk == 128) && S % SD_BQ == 0 && aligned && BH <= 65535 && S / SD_BQ <= 0x7fffffff) {
+        int rc;
+        if (dk == 32) {
+            rc = launch_sdpa<32>(Q, K, V, O, L, BH, S, scale, causal);
+            axhip::note_kernel(causal ? "sdpa_fused_dk32_causal" : "sdpa_fused_dk32");
+        } else if (dk == 64) {
+            rc = launch_sdpa<64>(Q, K, V, O, L, BH, S, scale, causal);
+            axhip::note_kernel(causal ? "sdpa_fused_dk64_causal" : "sdpa_fused_dk64");
+        } else {
+            rc = launch_sdpa<128>(Q, K, V, O, L, BH, S, scale, causal);
+            axhip::note_kernel(causal ? "sdpa_fused_dk128_causal" : "sdpa_fused_dk128");
         }
-        const float sl2 = scale * 1.4426950408889634f;
-        dim3 grid((unsigned)(S / SD_BQ), (unsigned)BH);
-        if (causal) hipLaunchKernelGGL(k_sdpa64<true>, grid, dim3(256), SD_SMEM, kStream, Q, K, V, O, L, S, sl2);
-        else hipLaunchKernelGGL(k_sdpa64<false>, grid, dim3(256), SD_SMEM, kStream, Q, K, V, O, L, S, sl2);
-        axhip::note_kernel(causal ? "sdpa_fused_dk64_causal" : "sdpa_fused_dk64");
-        return check_launch("sdpa_fwd");
+        return rc;
     }
     return sdpa_unfused(Q, K, V, O, L, BH, S, dk, scale, causal);
 }
