@@ -70,7 +70,7 @@ struct SdGeom {
 template <int DK, bool CAUSAL>
 __global__ void __launch_bounds__(256)
 k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__restrict__ V,
-       float *__restrict__ O, float *__restrict__ L, int64_t S, float scale_log2e) {
+       float *__restrict__ O, float *__restrict__ L, int64_t BH, int64_t S, float scale_log2e) {
     using G = SdGeom<DK>;
     constexpr int KB = DK / 8;                   // 8-wide k-blocks of the score product
     constexpr int DT = DK / 32;                  // 32-wide column tiles of the output
@@ -78,8 +78,18 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int frow = lane & 31, fhalf = lane >> 5;
-    const int64_t head = blockIdx.y;
-    const int64_t q0 = (int64_t)blockIdx.x * SD_BQ;
+    const int64_t nq = S / SD_BQ;
+    // Workgroups are handed to the 8 XCDs round-robin by linear index, and inside an XCD to its
+    // CUs in a fixed rotation, so every workgroup has to carry the same amount of work.  Eight
+    // heads form a group: workgroup r of a group works on head r % 8 (every query tile of a
+    // head then runs on the same XCD and shares its L2 copy of K and V) and on unit r / 8.
+    // A unit is one query tile, or, causal, the pair of tiles p and nq-1-p, which together
+    // visit nq+1 key blocks whatever p is (the middle tile of an odd nq stands alone).
+    const int64_t units = CAUSAL ? (nq + 1) / 2 : nq;
+    const int64_t lin = blockIdx.x, group = lin / (8 * units), left = BH - group * 8;
+    const int64_t r = lin - group * 8 * units, hpg = left < 8 ? left : 8;
+    const int64_t head = group * 8 + r % hpg, unit = r / hpg;
+    const int passes = (CAUSAL && unit != nq - 1 - unit) ? 2 : 1;
     const float *Qh = Q + head * S * DK, *Kh = K + head * S * DK, *Vh = V + head * S * DK;
     const unsigned lds0 = (unsigned)(uintptr_t)lds;
 
@@ -95,130 +105,141 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
         voff[i] = (unsigned)(vrow * G::ROWB + (c << 4));
     }
 
-    // ---- Q tile (128 rows) through the two K stages, then into registers ----
-#pragma unroll
-    for (int i = 0; i < G::IPW; i++) {
-        AXS_LOAD_LDS(lds0 + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * DK));
-        AXS_LOAD_LDS(lds0 + G::KSTAGE + (4 * i + wave) * 1024, koff[i],
-                     reinterpret_cast<const char *>(Qh + (q0 + 64) * DK));
-    }
-    AXS_VM0();
-    __syncthreads();
-    v4f qf[KB];                                  // k-block kb: dk 8*kb + 4*fhalf .. +3 of this lane's query
-    {
-        const int r = wave * 32 + frow;          // rows 64..127 sit in the second stage, same swizzle
-        const unsigned char *qrow = lds + (r >> 6) * G::KSTAGE + (r & 63) * G::ROWB;
-#pragma unroll
-        for (int kb = 0; kb < KB; kb++)
-            qf[kb] = *reinterpret_cast<const v4f *>(qrow + (((kb * 2 + fhalf) ^ G::swz(r & 63)) << 4));
-    }
-    __syncthreads();
-
-    const int64_t nblocks = CAUSAL ? (q0 + SD_BQ) / SD_BKV : S / SD_BKV;
-    auto issue = [&](int64_t blk, int stage) {
-        const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * DK);
-        const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * DK);
+    for (int pass = 0; pass < passes; pass++) {
+        const int64_t q0 = (CAUSAL && pass == 0 ? nq - 1 - unit : unit) * SD_BQ;
+        if (pass) __syncthreads();                   // the first tile's last key block has been read
+        // ---- Q tile (128 rows) through the two K stages, then into registers ----
 #pragma unroll
         for (int i = 0; i < G::IPW; i++) {
-            AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
-            AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff[i], vg);
+            AXS_LOAD_LDS(lds0 + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * DK));
+            AXS_LOAD_LDS(lds0 + G::KSTAGE + (4 * i + wave) * 1024, koff[i],
+                         reinterpret_cast<const char *>(Qh + (q0 + 64) * DK));
         }
-    };
-    issue(0, 0);
-
-    v16f acc_o[DT];
-#pragma unroll
-    for (int d = 0; d < DT; d++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) acc_o[d][v] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;       // l_run: this lane half's share of the row sum
-    const int64_t qg = q0 + wave * 32 + frow;    // this lane's query
-
-    for (int64_t blk = 0; blk < nblocks; blk++) {
-        const int stage = (int)(blk & 1);
         AXS_VM0();
-        __syncthreads();                          // block blk has landed; stage^1 is free again
-        if (blk + 1 < nblocks) issue(blk + 1, stage ^ 1);
-        const unsigned char *ks = lds + stage * G::KSTAGE;
-        const unsigned char *vs = lds + 2 * G::KSTAGE + stage * G::VSTAGE;
-
-        // ---- scores of 64 keys ----
-        v16f acc_s[2];
+        __syncthreads();
+        v4f qf[KB];                                  // k-block kb: dk 8*kb + 4*fhalf .. +3 of this lane's query
+        {
+            const int r = wave * 32 + frow;          // rows 64..127 sit in the second stage, same swizzle
+            const unsigned char *qrow = lds + (r >> 6) * G::KSTAGE + (r & 63) * G::ROWB;
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++) {
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc_s[kt][v] = 0.0f;
-            const int r = kt * 32 + frow;
-            const unsigned char *krow = ks + r * G::ROWB;
-#pragma unroll
-            for (int kb = 0; kb < KB; kb++) {
-                const v4f kf = *reinterpret_cast<const v4f *>(krow + (((kb * 2 + fhalf) ^ G::swz(r)) << 4));
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    acc_s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[kb][e], acc_s[kt], 0, 0, 0);
-            }
+            for (int kb = 0; kb < KB; kb++)
+                qf[kb] = *reinterpret_cast<const v4f *>(qrow + (((kb * 2 + fhalf) ^ G::swz(r & 63)) << 4));
         }
+        __syncthreads();
 
-        // ---- online softmax ----
-        float m_blk = -INFINITY;
+        const int64_t nblocks = CAUSAL ? (q0 + SD_BQ) / SD_BKV : S / SD_BKV;
+        auto issue = [&](int64_t blk, int stage) {
+            const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * DK);
+            const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * DK);
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                float s = acc_s[kt][v] * scale_log2e;
-                if (CAUSAL) {
-                    const int64_t key = blk * SD_BKV + kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3);
-                    if (key > qg) s = -INFINITY;
-                }
-                acc_s[kt][v] = s;
-                m_blk = fmaxf(m_blk, s);
+            for (int i = 0; i < G::IPW; i++) {
+                AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
+                AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff[i], vg);
             }
-        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
-        const float m_new = fmaxf(m_run, m_blk);      // finite: key 0 is visible to every query
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        float l_blk = 0.0f;
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const float p = __builtin_amdgcn_exp2f(acc_s[kt][v] - m_new);
-                acc_s[kt][v] = p;
-                l_blk += p;
-            }
-        l_run = l_run * alpha + l_blk;
-        m_run = m_new;
+        };
+        issue(0, 0);
+
+        v16f acc_o[DT];
 #pragma unroll
         for (int d = 0; d < DT; d++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc_o[d][v] *= alpha;
+            for (int v = 0; v < 16; v++) acc_o[d][v] = 0.0f;
+        float m_run = -INFINITY, l_run = 0.0f;       // l_run: this lane half's share of the row sum
+        const int64_t qg = q0 + wave * 32 + frow;    // this lane's query
 
-        // ---- O^T += V^T P^T ----
+        for (int64_t blk = 0; blk < nblocks; blk++) {
+            const int stage = (int)(blk & 1);
+            AXS_VM0();
+            __syncthreads();                          // block blk has landed; stage^1 is free again
+            if (blk + 1 < nblocks) issue(blk + 1, stage ^ 1);
+            const unsigned char *ks = lds + stage * G::KSTAGE;
+            const unsigned char *vs = lds + 2 * G::KSTAGE + stage * G::VSTAGE;
+
+            // causal: a 32-key tile entirely above this wave's 32 queries is skipped, and only
+            // blocks that straddle the diagonal pay for the mask (all wave-uniform decisions)
+            const int64_t kb0 = blk * SD_BKV, wq_lo = q0 + wave * 32;
+            const bool tile_on[2] = {!CAUSAL || kb0 <= wq_lo + 31, !CAUSAL || kb0 + 32 <= wq_lo + 31};
+            const bool need_mask = CAUSAL && kb0 + SD_BKV - 1 > wq_lo;
+            const int qrel = (int)(qg - kb0);         // keys of this block with index > qrel are masked
+
+            // ---- scores of 64 keys ----
+            v16f acc_s[2];
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+            for (int kt = 0; kt < 2; kt++) {
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int key = kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3);
-                const float *vrow = reinterpret_cast<const float *>(vs + G::v_addr(key));
+                for (int v = 0; v < 16; v++) acc_s[kt][v] = 0.0f;
+                if (!tile_on[kt]) continue;
+                const int r = kt * 32 + frow;
+                const unsigned char *krow = ks + r * G::ROWB;
 #pragma unroll
-                for (int d = 0; d < DT; d++)
-                    acc_o[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[d * 32 + frow], acc_s[kt][v], acc_o[d], 0, 0, 0);
+                for (int kb = 0; kb < KB; kb++) {
+                    const v4f kf = *reinterpret_cast<const v4f *>(krow + (((kb * 2 + fhalf) ^ G::swz(r)) << 4));
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        acc_s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[kb][e], acc_s[kt], 0, 0, 0);
+                }
             }
-    }
 
-    // ---- normalise and write: lane owns query qg, dk columns 32*d + 8*g + 4*fhalf .. +3 ----
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-    const float inv = 1.0f / l_tot;
-    float *orow = O + (head * S + qg) * DK;
+            // ---- online softmax ----
+            float m_blk = -INFINITY;
 #pragma unroll
-    for (int d = 0; d < DT; d++)
+            for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            v4f r;
+                for (int v = 0; v < 16; v++) {
+                    float s = acc_s[kt][v] * scale_log2e;
+                    if (!tile_on[kt] || (need_mask && kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3) > qrel)) s = -INFINITY;
+                    acc_s[kt][v] = s;
+                    m_blk = fmaxf(m_blk, s);
+                }
+            m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
+            const float m_new = fmaxf(m_run, m_blk);      // finite: key 0 is visible to every query
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            float l_blk = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 4; e++) r[e] = acc_o[d][4 * g + e] * inv;
-            *reinterpret_cast<v4f *>(orow + d * 32 + 8 * g + 4 * fhalf) = r;
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const float p = __builtin_amdgcn_exp2f(acc_s[kt][v] - m_new);
+                    acc_s[kt][v] = p;
+                    l_blk += p;
+                }
+            l_run = l_run * alpha + l_blk;
+            m_run = m_new;
+#pragma unroll
+            for (int d = 0; d < DT; d++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc_o[d][v] *= alpha;
+
+            // ---- O^T += V^T P^T ----
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++) {
+                if (!tile_on[kt]) continue;
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int key = kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3);
+                    const float *vrow = reinterpret_cast<const float *>(vs + G::v_addr(key));
+#pragma unroll
+                    for (int d = 0; d < DT; d++)
+                        acc_o[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[d * 32 + frow], acc_s[kt][v], acc_o[d], 0, 0, 0);
+                }
+            }
         }
-    if (L && fhalf == 0) L[head * S + qg] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+
+        // ---- normalise and write: lane owns query qg, dk columns 32*d + 8*g + 4*fhalf .. +3 ----
+        const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+        const float inv = 1.0f / l_tot;
+        float *orow = O + (head * S + qg) * DK;
+#pragma unroll
+        for (int d = 0; d < DT; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                v4f r;
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = acc_o[d][4 * g + e] * inv;
+                *reinterpret_cast<v4f *>(orow + d * 32 + 8 * g + 4 * fhalf) = r;
+            }
+        if (L && fhalf == 0) L[head * S + qg] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+    }
 }
 
 template <int DK>
@@ -234,9 +255,10 @@ int launch_sdpa(const float *Q, const float *K, const float *V, float *O, float 
         attr_set = true;
     }
     const float sl2 = scale * 1.4426950408889634f;
-    dim3 grid((unsigned)(S / SD_BQ), (unsigned)BH);
-    if (causal) hipLaunchKernelGGL((k_sdpa<DK, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, S, sl2);
-    else hipLaunchKernelGGL((k_sdpa<DK, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, S, sl2);
+    const int64_t nq = S / SD_BQ;
+    dim3 grid((unsigned)((causal ? (nq + 1) / 2 : nq) * BH));
+    if (causal) hipLaunchKernelGGL((k_sdpa<DK, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
+    else hipLaunchKernelGGL((k_sdpa<DK, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
     return check_launch("sdpa_fwd");
 }
 
@@ -312,7 +334,7 @@ extern "C" int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, fl
     if (BH < 0 || S < 0 || dk <= 0) return fail(AXHIP_ERR_SHAPE, "sdpa_fwd: bad extent");
     if (BH == 0 || S == 0) return AXHIP_OK;
     const bool aligned = ((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O) & 15) == 0);
-    if ((dk == 32 || dk == 64 || dk == 128) && S % SD_BQ == 0 && aligned && BH <= 65535 && S / SD_BQ <= 0x7fffffff) {
+    if ((dk == 32 || dk == 64 || dk == 128) && S % SD_BQ == 0 && aligned && S / SD_BQ * BH <= 0x7fffffff) {
         int rc;
         if (dk == 32) {
             rc = launch_sdpa<32>(Q, K, V, O, L, BH, S, scale, causal);
