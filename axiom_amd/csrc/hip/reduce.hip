@@ -1,6 +1,7 @@
-// Sum reductions behind the .sum vtable slot: out[o, i] = sum_a in[o, a, i] for a contiguous
-// fp32 tensor viewed as [outer, axis_len, inner] (the reference's reduction_dims,
-// cuda/ops_reduce.cu:246-251).  HBM-bound: one pass over the input.
+// Reductions behind the .sum/.mean/.max_op/.min_op vtable slots, row softmax and layer
+// normalisation.  out[o, i] = reduce_a in[o, a, i] for a contiguous fp32 tensor viewed as
+// [outer, axis_len, inner] (the reference's reduction_dims, cuda/ops_reduce.cu:246-251).
+// HBM-bound: one pass over the input.  Sums:
 //
 //   inner > 1  (column sums; axis 0 of [rows, cols] is the dense layer's bias gradient):
 //              the skinny-M GEMM with a row of ones as the activations, out = 1^T * in.  A
@@ -9,49 +10,180 @@
 //   inner == 1 (row sums): one wave per row, lanes stride over the row, then a fixed-order
 //              cross-lane tree.
 //   axis == -1 (everything): row sums over equal chunks, then one row sum over the partials.
-// All orders are fixed, so results are bit-identical run to run.
+// All orders are fixed, so results are bit-identical run to run.  Maxima and minima start from
+// -FLT_MAX / +FLT_MAX and take a value only when it compares strictly beyond the running one
+// (cpu_naive.c:395-433, 441-479), so NaNs are passed over and the result does not depend on order.
+#include <float.h>
+
 #include "common.h"
 
 namespace {
 using namespace axhip;
 
-// Row r covers in[r*stride, r*stride + min(len, total - r*stride)).
-template <bool VEC>
+template <int OP> __device__ __forceinline__ float red_init() {
+    return OP == AXHIP_RED_MAX ? -FLT_MAX : OP == AXHIP_RED_MIN ? FLT_MAX : 0.0f;
+}
+template <int OP> __device__ __forceinline__ float red_join(float acc, float v) {
+    if (OP == AXHIP_RED_MAX) return v > acc ? v : acc;
+    if (OP == AXHIP_RED_MIN) return v < acc ? v : acc;
+    return acc + v;
+}
+
+// One wave per segment.  Segment R = (row r, part p) with r = R / parts covers
+// in[r*row_stride + p*part_len, ... + min(part_len, row_len - p*part_len)).
+template <int OP, bool VEC>
 __global__ void __launch_bounds__(256)
-k_rowsum(const float *__restrict__ in, int64_t rows, int64_t stride, int64_t len, int64_t total,
-         float *__restrict__ out) {
+k_reduce_rows(const float *__restrict__ in, int64_t segments, int64_t parts, int64_t row_stride,
+              int64_t part_len, int64_t row_len, float *__restrict__ out) {
     const int lane = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= rows) return;
-    const int64_t begin = r * stride;
-    int64_t n = total - begin;
-    if (n > len) n = len;
-    const float *p = in + begin;
-    float s = 0.0f;
+    const int64_t seg = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (seg >= segments) return;
+    const int64_t r = seg / parts, part = seg - r * parts;
+    int64_t n = row_len - part * part_len;
+    if (n > part_len) n = part_len;
+    const float *p = in + r * row_stride + part * part_len;
+    float s = red_init<OP>();
     if (VEC) {
         int64_t c = (int64_t)lane * 4;
         for (; c + 4 <= n; c += 256) {
             const v4f v = *reinterpret_cast<const v4f *>(p + c);
-            s += (v.x + v.y) + (v.z + v.w);
+            if (OP == AXHIP_RED_SUM) {
+                s += (v.x + v.y) + (v.z + v.w);
+            } else {                              // the running value must stay on the left: it is never NaN
+#pragma unroll
+                for (int e = 0; e < 4; e++) s = red_join<OP>(s, v[e]);
+            }
         }
-        for (; c < n; c++) s += p[c];          // at most one lane holds the ragged tail
+        for (; c < n; c++) s = red_join<OP>(s, p[c]);          // at most one lane holds the ragged tail
     } else {
-        for (int64_t c = lane; c < n; c += 64) s += p[c];
+        for (int64_t c = lane; c < n; c += 64) s = red_join<OP>(s, p[c]);
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off, 64);
-    if (lane == 0) out[r] = s;
+    for (int off = 32; off > 0; off >>= 1) s = red_join<OP>(s, __shfl_down(s, off, 64));
+    if (lane == 0) out[seg] = s;
 }
 
-int launch_rowsum(const float *in, int64_t rows, int64_t stride, int64_t len, int64_t total, float *out) {
-    const int64_t blocks = (rows + 3) / 4;
-    if (blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "sum: too many rows");
-    const bool vec = ((uintptr_t)in % 16 == 0) && (stride % 4 == 0);
+template <int OP>
+int launch_rows(const float *in, int64_t rows, int64_t parts, int64_t row_stride, int64_t part_len,
+                int64_t row_len, float *out) {
+    const int64_t segments = rows * parts, blocks = (segments + 3) / 4;
+    if (blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "reduce: too many rows");
+    const bool vec = ((uintptr_t)in % 16 == 0) && (row_stride % 4 == 0) && (part_len % 4 == 0 || parts == 1);
     if (vec)
-        hipLaunchKernelGGL(k_rowsum<true>, dim3((unsigned)blocks), dim3(256), 0, kStream, in, rows, stride, len, total, out);
+        hipLaunchKernelGGL((k_reduce_rows<OP, true>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, segments,
+                           parts, row_stride, part_len, row_len, out);
     else
-        hipLaunchKernelGGL(k_rowsum<false>, dim3((unsigned)blocks), dim3(256), 0, kStream, in, rows, stride, len, total, out);
-    return check_launch("sum_rows");
+        hipLaunchKernelGGL((k_reduce_rows<OP, false>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, segments,
+                           parts, row_stride, part_len, row_len, out);
+    return check_launch("reduce_rows");
+}
+
+// Row reductions of [rows, len]: few long rows are cut into parts first so that the whole chip
+// streams, then the parts of each row are reduced.
+template <int OP>
+int reduce_rows(const float *in, int64_t rows, int64_t len, float *out) {
+    int64_t parts = 1;
+    if (rows < 2048 && len > 8192) {
+        parts = 4096 / rows;
+        const int64_t most = (len + 4095) / 4096;
+        if (parts > most) parts = most;
+        if (parts < 1) parts = 1;
+    }
+    if (parts == 1) return launch_rows<OP>(in, rows, 1, len, len, len, out);
+    int64_t part_len = (len + parts - 1) / parts;
+    part_len = (part_len + 3) / 4 * 4;
+    parts = (len + part_len - 1) / part_len;
+    float *partial = static_cast<float *>(workspace((size_t)(rows * parts) * sizeof(float)));
+    if (!partial) return AXHIP_ERR_ALLOC;
+    if (int rc = launch_rows<OP>(in, rows, parts, len, part_len, len, partial)) return rc;
+    return launch_rows<OP>(partial, rows, 1, parts, parts, parts, out);
+}
+
+// Column reductions of [outer, axis_len, inner], inner > 1.  A workgroup is TY axis positions
+// by TX column groups of VW columns; it walks a slice of the axis TY positions at a time and
+// joins its TY partial rows through LDS.  Slice s of `splits` writes out[(o*splits + s), :].
+template <int OP, int VW>
+__global__ void __launch_bounds__(256)
+k_reduce_cols(const float *__restrict__ in, int64_t axis_len, int64_t inner, int tx_log2, int64_t col_blocks,
+              int64_t splits, int64_t slice, float *__restrict__ out) {
+    __shared__ float join[256 * VW];
+    const int tx = threadIdx.x & ((1 << tx_log2) - 1), ty = threadIdx.x >> tx_log2, TY = 256 >> tx_log2;
+    int64_t b = blockIdx.x;
+    const int64_t cb = b % col_blocks;
+    b /= col_blocks;
+    const int64_t s = b % splits, o = b / splits;
+    const int64_t col = (cb << tx_log2) * VW + (int64_t)tx * VW;
+    float acc[VW];
+#pragma unroll
+    for (int e = 0; e < VW; e++) acc[e] = red_init<OP>();
+    int64_t a1 = (s + 1) * slice;
+    if (a1 > axis_len) a1 = axis_len;
+    if (col < inner) {
+        const float *base = in + o * axis_len * inner + col;
+        for (int64_t a = s * slice + ty; a < a1; a += TY) {
+            if (VW == 4) {
+                const v4f v = *reinterpret_cast<const v4f *>(base + a * inner);
+#pragma unroll
+                for (int e = 0; e < VW; e++) acc[e] = red_join<OP>(acc[e], v[e]);
+            } else {
+                acc[0] = red_join<OP>(acc[0], base[a * inner]);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VW; e++) join[e * 256 + threadIdx.x] = acc[e];
+    __syncthreads();
+    if (ty == 0 && col < inner) {
+        for (int y = 1; y < TY; y++)
+#pragma unroll
+            for (int e = 0; e < VW; e++) acc[e] = red_join<OP>(acc[e], join[e * 256 + (y << tx_log2) + tx]);
+        float *dst = out + (o * splits + s) * inner + col;
+#pragma unroll
+        for (int e = 0; e < VW; e++) dst[e] = acc[e];
+    }
+}
+
+template <int OP>
+int launch_cols(const float *in, int64_t outer, int64_t axis_len, int64_t inner, int64_t splits, float *out) {
+    const bool vec = ((uintptr_t)in % 16 == 0) && inner % 4 == 0;
+    const int64_t groups = vec ? inner / 4 : inner;
+    int tx_log2 = 0;
+    while (tx_log2 < 8 && (int64_t(1) << tx_log2) < groups) tx_log2++;
+    const int64_t col_blocks = (groups + (int64_t(1) << tx_log2) - 1) >> tx_log2;
+    const int64_t slice = (axis_len + splits - 1) / splits;
+    const int64_t blocks = col_blocks * splits * outer;
+    if (blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "reduce: too many column blocks");
+    if (vec)
+        hipLaunchKernelGGL((k_reduce_cols<OP, 4>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, axis_len, inner,
+                           tx_log2, col_blocks, splits, slice, out);
+    else
+        hipLaunchKernelGGL((k_reduce_cols<OP, 1>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, axis_len, inner,
+                           tx_log2, col_blocks, splits, slice, out);
+    return check_launch("reduce_cols");
+}
+
+template <int OP>
+int reduce_cols(const float *in, int64_t outer, int64_t axis_len, int64_t inner, float *out) {
+    // enough workgroups to stream from every CU: cut the axis when outer x column blocks is small
+    const int64_t groups = (inner + 3) / 4, col_blocks = (groups + 255) / 256;
+    int64_t splits = 1;
+    if (outer * col_blocks < 1024) {
+        splits = 1024 / (outer * col_blocks);
+        const int64_t most = axis_len / 64;
+        if (splits > most) splits = most;
+        if (splits < 1) splits = 1;
+    }
+    if (splits == 1) return launch_cols<OP>(in, outer, axis_len, inner, 1, out);
+    float *partial = static_cast<float *>(workspace((size_t)(outer * splits * inner) * sizeof(float)));
+    if (!partial) return AXHIP_ERR_ALLOC;
+    if (int rc = launch_cols<OP>(in, outer, axis_len, inner, splits, partial)) return rc;
+    return launch_cols<OP>(partial, outer, splits, inner, 1, out);
+}
+
+template <int OP>
+int reduce_axis(const float *in, int64_t outer, int64_t axis_len, int64_t inner, float *out) {
+    if (inner == 1) return reduce_rows<OP>(in, outer, axis_len, out);
+    return reduce_cols<OP>(in, outer, axis_len, inner, out);
 }
 
 __global__ void __launch_bounds__(256)
@@ -61,7 +193,107 @@ k_axpy(const float *__restrict__ x, float alpha, float *__restrict__ y, int64_t 
         y[i] = __builtin_fmaf(alpha, x[i], y[i]);
 }
 
+// first index of the largest value along the axis (cpu_opt.c:7236-7247)
+__global__ void __launch_bounds__(256)
+k_argmax(const float *__restrict__ in, int64_t outer, int64_t axis_len, int64_t inner, int64_t *__restrict__ out) {
+    const int64_t stride = (int64_t)gridDim.x * 256, total = outer * inner;
+    for (int64_t oi = (int64_t)blockIdx.x * 256 + threadIdx.x; oi < total; oi += stride) {
+        const int64_t o = oi / inner, i = oi - o * inner;
+        const float *base = in + o * axis_len * inner + i;
+        int64_t best = 0;
+        float bestv = base[0];
+        for (int64_t a = 1; a < axis_len; a++) {
+            const float v = base[a * inner];
+            if (v > bestv) {
+                bestv = v;
+                best = a;
+            }
+        }
+        out[oi] = best;
+    }
+}
+
+// one wave per row, for rows along the contiguous axis
+__global__ void __launch_bounds__(256)
+k_argmax_rows(const float *__restrict__ in, int64_t rows, int64_t len, int64_t *__restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const float *p = in + r * len;
+    // lanes scan interleaved positions in ascending order, so each keeps its first maximum;
+    // a lane without elements, or with NaNs only ahead of row element 0's rule, defers below
+    float bestv = p[0];
+    int64_t best = 0;
+    for (int64_t c = lane; c < len; c += 64) {
+        const float v = p[c];
+        if (v > bestv || (v == bestv && c < best)) {
+            bestv = v;
+            best = c;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_down(bestv, off, 64);
+        const int64_t oi = __shfl_down(best, off, 64);
+        if (ov > bestv || (ov == bestv && oi < best)) {
+            bestv = ov;
+            best = oi;
+        }
+    }
+    if (lane == 0) out[r] = best;
+}
+
 }  // namespace
+
+extern "C" int axhip_reduce_axis(int op, const float *in, int64_t outer, int64_t axis_len, int64_t inner,
+                                 float *out) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!in || !out) return fail(AXHIP_ERR_NULL_ARG, "reduce: NULL");
+    if (outer < 0 || axis_len < 0 || inner < 0) return fail(AXHIP_ERR_SHAPE, "reduce: negative extent");
+    if (outer == 0 || inner == 0) return AXHIP_OK;
+    switch (op) {
+        case AXHIP_RED_SUM: return axhip_sum_axis(in, outer, axis_len, inner, out);
+        case AXHIP_RED_MEAN: {
+            if (axis_len == 0) return fail(AXHIP_ERR_SHAPE, "mean: empty axis");
+            if (int rc = axhip_sum_axis(in, outer, axis_len, inner, out)) return rc;
+            return axhip_unary(AXHIP_UN_MUL_SCALAR, out, out, outer * inner, 1.0f / (float)axis_len);
+        }
+        case AXHIP_RED_MAX:
+            if (axis_len == 0) return axhip_fill_f32(out, -FLT_MAX, outer * inner);
+            return reduce_axis<AXHIP_RED_MAX>(in, outer, axis_len, inner, out);
+        case AXHIP_RED_MIN:
+            if (axis_len == 0) return axhip_fill_f32(out, FLT_MAX, outer * inner);
+            return reduce_axis<AXHIP_RED_MIN>(in, outer, axis_len, inner, out);
+        default: return fail(AXHIP_ERR_SHAPE, "reduce: unknown op %d", op);
+    }
+}
+
+extern "C" int axhip_reduce_all(int op, const float *in, int64_t n, float *out) {
+    if (op == AXHIP_RED_SUM) return axhip_sum_all(in, n, out);
+    if (op == AXHIP_RED_MEAN) {
+        if (n <= 0) return fail(AXHIP_ERR_SHAPE, "mean: empty tensor");
+        if (int rc = axhip_sum_all(in, n, out)) return rc;
+        return axhip_unary(AXHIP_UN_MUL_SCALAR, out, out, 1, 1.0f / (float)n);
+    }
+    return axhip_reduce_axis(op, in, 1, n, 1, out);
+}
+
+extern "C" int axhip_argmax_axis(const float *in, int64_t outer, int64_t axis_len, int64_t inner, int64_t *out) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!in || !out) return fail(AXHIP_ERR_NULL_ARG, "argmax: NULL");
+    if (outer < 0 || axis_len <= 0 || inner < 0) return fail(AXHIP_ERR_SHAPE, "argmax: bad extent");
+    if (outer == 0 || inner == 0) return AXHIP_OK;
+    if (inner == 1 && axis_len >= 64) {
+        const int64_t blocks = (outer + 3) / 4;
+        if (blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "argmax: too many rows");
+        hipLaunchKernelGGL(k_argmax_rows, dim3((unsigned)blocks), dim3(256), 0, kStream, in, outer, axis_len, out);
+        return check_launch("argmax_rows");
+    }
+    int64_t blocks = (outer * inner + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(k_argmax, dim3((unsigned)blocks), dim3(256), 0, kStream, in, outer, axis_len, inner, out);
+    return check_launch("argmax");
+}
 
 extern "C" int axhip_sum_axis(const float *in, int64_t outer, int64_t axis_len, int64_t inner, float *out) {
     if (int rc = axhip::ensure_ready()) return rc;
@@ -69,7 +301,8 @@ extern "C" int axhip_sum_axis(const float *in, int64_t outer, int64_t axis_len, 
     if (outer < 0 || axis_len < 0 || inner < 0) return fail(AXHIP_ERR_SHAPE, "sum: negative extent");
     if (outer == 0 || inner == 0) return AXHIP_OK;
     if (axis_len == 0) return axhip_fill_f32(out, 0.0f, outer * inner);
-    if (inner == 1) return launch_rowsum(in, outer, axis_len, axis_len, outer * axis_len, out);
+    if (inner == 1) return reduce_rows<AXHIP_RED_SUM>(in, outer, axis_len, out);
+    if (outer > 4 || inner < 64) return reduce_cols<AXHIP_RED_SUM>(in, outer, axis_len, inner, out);
     float *ones = axhip::ones_vector((size_t)axis_len);
     if (!ones) return AXHIP_ERR_ALLOC;
     for (int64_t o = 0; o < outer; o++) {
@@ -86,16 +319,7 @@ extern "C" int axhip_sum_all(const float *in, int64_t n, float *out) {
     if (!in || !out) return fail(AXHIP_ERR_NULL_ARG, "sum: NULL");
     if (n < 0) return fail(AXHIP_ERR_SHAPE, "sum: negative extent");
     if (n == 0) return axhip_fill_f32(out, 0.0f, 1);
-    if (n <= 4096) return launch_rowsum(in, 1, n, n, n, out);
-    int64_t parts = (n + 4095) / 4096;
-    if (parts > 1024) parts = 1024;
-    int64_t len = (n + parts - 1) / parts;
-    len = (len + 3) / 4 * 4;
-    parts = (n + len - 1) / len;
-    float *partial = static_cast<float *>(axhip::workspace((size_t)parts * sizeof(float)));
-    if (!partial) return AXHIP_ERR_ALLOC;
-    if (int rc = launch_rowsum(in, parts, len, len, n, partial)) return rc;
-    return launch_rowsum(partial, 1, parts, parts, parts, out);
+    return reduce_rows<AXHIP_RED_SUM>(in, 1, n, out);
 }
 
 extern "C" int axhip_axpy(const float *x, float alpha, float *y, int64_t n) {

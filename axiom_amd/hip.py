@@ -39,6 +39,15 @@ SIGNATURES = {
     "axhip_sum_axis": (C.c_int, [vp, i64, i64, i64, vp]),
     "axhip_sum_all": (C.c_int, [vp, i64, vp]),
     "axhip_axpy": (C.c_int, [vp, C.c_float, vp, i64]),
+    "axhip_binary": (C.c_int, [C.c_int, vp, vp, vp, C.c_int, C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)]),
+    "axhip_unary": (C.c_int, [C.c_int, vp, vp, i64, C.c_float]),
+    "axhip_reduce_axis": (C.c_int, [C.c_int, vp, i64, i64, i64, vp]),
+    "axhip_reduce_all": (C.c_int, [C.c_int, vp, i64, vp]),
+    "axhip_argmax_axis": (C.c_int, [vp, i64, i64, i64, vp]),
+    "axhip_softmax_rows": (C.c_int, [vp, vp, i64, i64]),
+    "axhip_layernorm_fwd": (C.c_int, [vp, vp, vp, vp, vp, vp, i64, i64, C.c_float]),
+    "axhip_adam_update": (C.c_int, [vp, vp, vp, vp, i64] + [C.c_float] * 7 + [C.c_int]),
+    "axhip_sgd_update": (C.c_int, [vp, vp, vp, i64, C.c_float, C.c_float, C.c_float, C.c_int]),
     "axhip_relu": (C.c_int, [vp, vp, i64]),
     "axhip_gelu": (C.c_int, [vp, vp, i64]),
     "axhip_fill_f32": (C.c_int, [vp, C.c_float, i64]),

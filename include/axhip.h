@@ -130,14 +130,70 @@ int axhip_sum_all(const float *in, int64_t n, float *out);
  * cpu_opt.c:7287-7307). */
 int axhip_axpy(const float *x, float alpha, float *y, int64_t n);
 
+/* ---- the remaining elementwise, reduction and optimizer vtable slots ------------------- */
+/* Broadcasting binary ops (.add .sub .mul .div_op .equal .greater .add_relu): out is contiguous
+ * with shape out_shape[ndim] (ndim <= 8); a_strides / b_strides are the operands' element
+ * strides per OUTPUT dimension, 0 where the operand is broadcast along it — the mapping of
+ * bcast_offset (cuda/ops_elementwise.cu:20-35) / broadcast_index (cpu_naive.c:48-62) resolved by
+ * the caller.  equal/greater write 1.0f / 0.0f (cuda/ops_elementwise.cu:64-65); add_relu is
+ * max(a + b, 0) (cuda/ops_fused.cu:13-21).  out may alias an operand that is not broadcast. */
+enum {
+    AXHIP_BIN_ADD = 0, AXHIP_BIN_SUB, AXHIP_BIN_MUL, AXHIP_BIN_DIV, AXHIP_BIN_EQUAL, AXHIP_BIN_GREATER,
+    AXHIP_BIN_ADD_RELU
+};
+int axhip_binary(int op, const float *a, const float *b, float *out, int ndim, const int64_t *out_shape,
+                 const int64_t *a_strides, const int64_t *b_strides);
+
+/* Unary and scalar ops over n contiguous elements; in/out may alias.  Definitions:
+ * cuda/ops_elementwise.cu:147-155 (neg, abs, exp, log: v > 0 ? logf(v) : -FLT_MAX, sqrt:
+ * v >= 0 ? sqrtf(v) : 0, square, sigmoid, tanh), :195-208 (add_scalar, mul_scalar with the
+ * scalar in `param`), cuda/ops_activations.cu:23-52 (swish = v / (1 + exp(-v)), leaky_relu and
+ * elu with alpha in `param`). */
+enum {
+    AXHIP_UN_NEG = 0, AXHIP_UN_ABS, AXHIP_UN_EXP, AXHIP_UN_LOG, AXHIP_UN_SQRT, AXHIP_UN_SQUARE,
+    AXHIP_UN_SIGMOID, AXHIP_UN_TANH, AXHIP_UN_LEAKY_RELU, AXHIP_UN_ELU, AXHIP_UN_SWISH,
+    AXHIP_UN_ADD_SCALAR, AXHIP_UN_MUL_SCALAR
+};
+int axhip_unary(int op, const float *in, float *out, int64_t n, float param);
+
+/* .sum .mean .max_op .min_op over one axis of [outer, axis_len, inner], or over everything
+ * (cuda/ops_reduce.cu:262-378; cpu_naive.c:311-479).  mean = sum * (1 / count); max / min start
+ * from -FLT_MAX / FLT_MAX and pass over NaNs, as the reference's compare-and-replace loops do. */
+enum { AXHIP_RED_SUM = 0, AXHIP_RED_MEAN, AXHIP_RED_MAX, AXHIP_RED_MIN };
+int axhip_reduce_axis(int op, const float *in, int64_t outer, int64_t axis_len, int64_t inner, float *out);
+int axhip_reduce_all(int op, const float *in, int64_t n, float *out);
+/* .argmax: index (int64) of the first largest element along the axis (opt_argmax,
+ * cpu_opt.c:7202-7249). */
+int axhip_argmax_axis(const float *in, int64_t outer, int64_t axis_len, int64_t inner, int64_t *out);
+
+/* .softmax_rowwise over contiguous [rows, cols]: exp(x - rowmax) / sum (cuda/ops_fused.cu:44-91,
+ * cpu_naive.c:235-270); in/out may alias. */
+int axhip_softmax_rows(const float *in, float *out, int64_t rows, int64_t cols);
+
+/* Layer normalisation forward over the last axis of contiguous [rows, cols]
+ * (layernorm_forward, src/core/norm.c:1338-1399): mean and E[x^2] in one pass, var clamped at 0,
+ * inv_std = 1 / sqrt(var + eps), out = gamma * x_hat + beta.  x_hat [rows, cols] and inv_std
+ * [rows] are the tensors the reference saves for its backward pass; either may be NULL. */
+int axhip_layernorm_fwd(const float *x, const float *gamma, const float *beta, float *out, float *x_hat,
+                        float *inv_std, int64_t rows, int64_t cols, float eps);
+
+/* .adam_update / .sgd_update: one fused pass per parameter tensor, w (and m, v / the momentum
+ * buffer) updated in place (cuda_adam_update / cuda_sgd_update, cuda/ops_optim.cu:17-110, which
+ * follow adam_step / sgd_step of src/core/optim.c).  bc1 = 1 - beta1^t, bc2 = 1 - beta2^t;
+ * momentum_buf may be NULL. */
+int axhip_adam_update(float *w, const float *g, float *m, float *v, int64_t n, float lr, float beta1,
+                      float beta2, float eps, float weight_decay, float bc1, float bc2, int decoupled);
+int axhip_sgd_update(float *w, const float *g, float *momentum_buf, int64_t n, float lr, float momentum,
+                     float weight_decay, int nesterov);
+
 /* ---- scaled dot-product attention forward --------------------------------------------- */
 /* O[h] = softmax(scale * Q[h] K[h]^T) V[h] for BH heads; Q, K, V, O are [BH, S, dk] row-major
  * fp32 in device memory, L is [BH, S] (log-sum-exp of each score row, natural log) or NULL;
  * causal != 0: query i sees keys j <= i.  Replaces ax_cuda_sdpa_fwd
  * (cuda/ops_attention.cu:299-392) and the device form of ax_fused_attention_fwd /
  * ax_fused_attention_fwd_causal (include/axiom/attention.h:273-283,
- * src/core/fused_attention.c:559-573).  dk = 64 with S a multiple of 128 runs fused (no score
- * matrix in memory); other shapes go through batched GEMMs and a row softmax. */
+ * src/core/fused_attention.c:559-573).  dk of 32, 64 or 128 with S a multiple of 128 runs fused (no
+ * score matrix in memory); other shapes go through batched GEMMs and a row softmax. */
 int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L,
                    int64_t BH, int64_t S, int64_t dk, float scale, int causal);
 

@@ -7,6 +7,7 @@
  */
 #include "ax_oracle.h"
 
+#include <float.h>
 #include <immintrin.h>
 #include <math.h>
 #include <stdlib.h>
@@ -539,5 +540,167 @@ void axo_sdpa_fwd_f64(const float *Q, const float *K, const float *V, double *O,
             if (L) L[h * S + i] = mx + log(sum);
         }
         free(scores);
+    }
+}
+
+/* ---- remaining elementwise / reduction / optimizer slots -------------------------------- */
+static int64_t bcast_offset(const int64_t *t_shape, int t_ndim, const int64_t *out_shape, int out_ndim,
+                            int64_t out_flat) {
+    int64_t t_strides[8], st = 1;
+    for (int d = t_ndim - 1; d >= 0; d--) {
+        t_strides[d] = st;
+        st *= t_shape[d];
+    }
+    int64_t remaining = out_flat, off = 0;
+    for (int d = out_ndim - 1; d >= 0; d--) {
+        const int64_t idx = remaining % out_shape[d];
+        remaining /= out_shape[d];
+        const int td = d - (out_ndim - t_ndim);
+        if (td >= 0 && t_shape[td] > 1) off += idx * t_strides[td];
+    }
+    return off;
+}
+
+void axo_binary(int op, const float *a, const int64_t *a_shape, int a_ndim, const float *b,
+                const int64_t *b_shape, int b_ndim, float *out, const int64_t *out_shape, int out_ndim) {
+    int64_t n = 1;
+    for (int d = 0; d < out_ndim; d++) n *= out_shape[d];
+    for (int64_t i = 0; i < n; i++) {
+        const float va = a[bcast_offset(a_shape, a_ndim, out_shape, out_ndim, i)];
+        const float vb = b[bcast_offset(b_shape, b_ndim, out_shape, out_ndim, i)];
+        float r;
+        switch (op) {
+            case 0: r = va + vb; break;
+            case 1: r = va - vb; break;
+            case 2: r = va * vb; break;
+            case 3: r = va / vb; break;
+            case 4: r = (va == vb) ? 1.0f : 0.0f; break;
+            case 5: r = (va > vb) ? 1.0f : 0.0f; break;
+            default: r = va + vb; r = r > 0.0f ? r : 0.0f; break;
+        }
+        out[i] = r;
+    }
+}
+
+void axo_unary(int op, const float *in, float *out, int64_t n, float p) {
+    for (int64_t i = 0; i < n; i++) {
+        const float v = in[i];
+        float r;
+        switch (op) {
+            case 0: r = -v; break;
+            case 1: r = fabsf(v); break;
+            case 2: r = expf(v); break;
+            case 3: r = v > 0.0f ? logf(v) : -FLT_MAX; break;
+            case 4: r = v >= 0.0f ? sqrtf(v) : 0.0f; break;
+            case 5: r = v * v; break;
+            case 6: r = 1.0f / (1.0f + expf(-v)); break;
+            case 7: r = tanhf(v); break;
+            case 8: r = v > 0.0f ? v : p * v; break;
+            case 9: r = v > 0.0f ? v : p * (expf(v) - 1.0f); break;
+            case 10: r = v / (1.0f + expf(-v)); break;
+            case 11: r = v + p; break;
+            default: r = v * p; break;
+        }
+        out[i] = r;
+    }
+}
+
+void axo_reduce_axis(int op, const float *in, int64_t outer, int64_t axis_len, int64_t inner, float *out) {
+    for (int64_t o = 0; o < outer; o++)
+        for (int64_t i = 0; i < inner; i++) {
+            float acc = op == 2 ? -FLT_MAX : op == 3 ? FLT_MAX : 0.0f;
+            for (int64_t a = 0; a < axis_len; a++) {
+                const float v = in[(o * axis_len + a) * inner + i];
+                if (op == 2) { if (v > acc) acc = v; }
+                else if (op == 3) { if (v < acc) acc = v; }
+                else acc += v;
+            }
+            if (op == 1) acc *= 1.0f / (float)axis_len;
+            out[o * inner + i] = acc;
+        }
+}
+
+void axo_argmax_axis(const float *in, int64_t outer, int64_t axis_len, int64_t inner, int64_t *out) {
+    for (int64_t oi = 0; oi < outer * inner; oi++) {
+        const int64_t o = oi / inner, i = oi - o * inner;
+        const float *base = in + o * axis_len * inner + i;
+        int64_t best = 0;
+        float bestv = base[0];
+        for (int64_t a = 1; a < axis_len; a++) {
+            const float v = base[a * inner];
+            if (v > bestv) { bestv = v; best = a; }
+        }
+        out[oi] = best;
+    }
+}
+
+void axo_softmax_rows(const float *in, float *out, int64_t rows, int64_t cols) {
+    for (int64_t r = 0; r < rows; r++) {
+        const float *x = in + r * cols;
+        float *y = out + r * cols;
+        float mx = x[0];
+        for (int64_t c = 1; c < cols; c++) if (x[c] > mx) mx = x[c];
+        float sum = 0.0f;
+        for (int64_t c = 0; c < cols; c++) {
+            const float e = expf(x[c] - mx);
+            y[c] = e;
+            sum += e;
+        }
+        const float inv = 1.0f / sum;
+        for (int64_t c = 0; c < cols; c++) y[c] *= inv;
+    }
+}
+
+void axo_layernorm_fwd(const float *x, const float *gamma, const float *beta, float *out, float *x_hat,
+                       float *inv_std_out, int64_t rows, int64_t cols, float eps) {
+    for (int64_t r = 0; r < rows; r++) {
+        const float *ip = x + r * cols;
+        float sum = 0.0f, sum2 = 0.0f;
+        for (int64_t f = 0; f < cols; f++) {
+            sum += ip[f];
+            sum2 += ip[f] * ip[f];
+        }
+        const float mean = sum / (float)cols;
+        float var = sum2 / (float)cols - mean * mean;
+        if (var < 0.0f) var = 0.0f;
+        const float inv_std = 1.0f / sqrtf(var + eps);
+        if (inv_std_out) inv_std_out[r] = inv_std;
+        for (int64_t f = 0; f < cols; f++) {
+            const float xh = (ip[f] - mean) * inv_std;
+            out[r * cols + f] = gamma[f] * xh + beta[f];
+            if (x_hat) x_hat[r * cols + f] = xh;
+        }
+    }
+}
+
+void axo_adam_update(float *w, const float *g, float *m, float *v, int64_t n, float lr, float beta1,
+                     float beta2, float eps, float weight_decay, float bc1, float bc2, int decoupled) {
+    float decay_scale = decoupled ? (1.0f - lr * weight_decay) : 1.0f;
+    if (decay_scale < 0.0f) decay_scale = 0.0f;
+    const float wd_grad = (!decoupled && weight_decay > 0.0f) ? weight_decay : 0.0f;
+    for (int64_t i = 0; i < n; i++) {
+        const float wi = w[i] * decay_scale;
+        const float gi = g[i] + wd_grad * wi;
+        const float mi = beta1 * m[i] + (1.0f - beta1) * gi;
+        const float vi = beta2 * v[i] + (1.0f - beta2) * gi * gi;
+        const float mh = mi / bc1, vh = vi / bc2;
+        w[i] = wi - lr * mh / (sqrtf(vh) + eps);
+        m[i] = mi;
+        v[i] = vi;
+    }
+}
+
+void axo_sgd_update(float *w, const float *g, float *mom, int64_t n, float lr, float momentum,
+                    float weight_decay, int nesterov) {
+    for (int64_t i = 0; i < n; i++) {
+        float gi = g[i];
+        if (weight_decay > 0.0f) gi += weight_decay * w[i];
+        if (mom && momentum > 0.0f) {
+            const float vi = momentum * mom[i] + gi;
+            mom[i] = vi;
+            w[i] -= nesterov ? lr * (gi + momentum * vi) : lr * vi;
+        } else {
+            w[i] -= lr * gi;
+        }
     }
 }

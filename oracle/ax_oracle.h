@@ -83,6 +83,35 @@ float axo_gelu_tanh(float x);
 void  axo_gelu(float *x, int64_t n);
 double axo_gelu_f64(double x);
 
+/* ---- remaining elementwise / reduction / optimizer slots ----------------------------------
+ * Pinned in tests/test_oracle.py against oracle/_ref through the golden vectors (the reference's
+ * naive and optimised CPU backends, its activation functions, its layer-norm layer and its
+ * optimizers) and against numpy closed forms. */
+/* Broadcasting binary op, element by element as cpu_naive.c:48-62,70-97,482-507: trailing
+ * dimensions are aligned, an operand dimension of extent 1 is broadcast.  op: 0 add, 1 sub,
+ * 2 mul, 3 div, 4 equal, 5 greater, 6 add_relu (cpu_naive.c:192-216).  Operands are contiguous. */
+void axo_binary(int op, const float *a, const int64_t *a_shape, int a_ndim, const float *b,
+                const int64_t *b_shape, int b_ndim, float *out, const int64_t *out_shape, int out_ndim);
+/* cpu_naive.c:112-147,552-576 and the parametrised activations of src/core/activations.c
+ * (leaky_relu :79-93, elu :141-155, swish :363-376): op numbering of axhip_unary. */
+void axo_unary(int op, const float *in, float *out, int64_t n, float param);
+/* cpu_naive.c:311-479: op 0 sum, 1 mean (sum * (1/count)), 2 max, 3 min over [outer, axis, inner];
+ * sums add in ascending axis order. */
+void axo_reduce_axis(int op, const float *in, int64_t outer, int64_t axis_len, int64_t inner, float *out);
+/* cpu_opt.c:7236-7247 */
+void axo_argmax_axis(const float *in, int64_t outer, int64_t axis_len, int64_t inner, int64_t *out);
+/* cpu_naive.c:235-270 */
+void axo_softmax_rows(const float *in, float *out, int64_t rows, int64_t cols);
+/* src/core/norm.c:1338-1399, scalar form; x_hat / inv_std may be NULL. */
+void axo_layernorm_fwd(const float *x, const float *gamma, const float *beta, float *out, float *x_hat,
+                       float *inv_std, int64_t rows, int64_t cols, float eps);
+/* cuda/ops_optim.cu:17-35,66-77 (the per-element form of adam_step, src/core/optim.c:262-330) */
+void axo_adam_update(float *w, const float *g, float *m, float *v, int64_t n, float lr, float beta1,
+                     float beta2, float eps, float weight_decay, float bc1, float bc2, int decoupled);
+/* cuda/ops_optim.cu:40-62 (sgd_step, src/core/optim.c:100-205); mom may be NULL */
+void axo_sgd_update(float *w, const float *g, float *mom, int64_t n, float lr, float momentum,
+                    float weight_decay, int nesterov);
+
 /* ---- int8 --------------------------------------------------------------- */
 /* quantize.c:21-57: per-row absmax/127, zero row -> 1, lrintf, clamp +-127. */
 void axo_quantize_rows(const float *w, int64_t N, int64_t K, int8_t *q, float *scales);

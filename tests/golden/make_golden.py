@@ -143,6 +143,60 @@ for (BH, S, dk, causal) in ((6, 24, 16, 0), (2, 16, 8, 1), (3, 128, 64, 0), (3, 
     o, l = r.sdpa(q, k, v, float(np.float32(1.0) / np.sqrt(np.float32(dk))), bool(causal))
     G[f"sdpa_{BH}x{S}x{dk}_c{causal}_O"], G[f"sdpa_{BH}x{S}x{dk}_c{causal}_L"] = o, l
 
+# ---- remaining elementwise / reduction / optimizer slots --------------------------------
+# inputs come from ax_rng_seed + ax_rng_uniform so that the tests can regenerate them; the
+# shapes follow tests/test_compute.c (broadcast [2,3]+[3], [2,1]+[1,3]) and tests/test_cuda.c
+BCAST = (((5, 7), (5, 7)), ((2, 3), (3,)), ((2, 1), (1, 3)), ((4, 1, 6), (3, 1)), ((2, 3, 4), (1,)),
+         ((3, 8, 16), (8, 1)))
+for case, (sa, sb) in enumerate(BCAST):
+    L.ax_rng_seed(7000 + case)
+    # values on a coarse grid so that equal / greater see ties
+    a = np.round(ref_uniform(int(np.prod(sa)), -2.0, 2.0) * 4) / 4
+    b = np.round(ref_uniform(int(np.prod(sb)), -2.0, 2.0) * 4) / 4
+    a, b = a.reshape(sa).astype(np.float32), b.reshape(sb).astype(np.float32)
+    for name in ("add", "sub", "mul", "div", "equal", "greater"):
+        G[f"bin_{name}_{case}"] = r.binary(name, a, b, backend=0)
+        assert np.array_equal(G[f"bin_{name}_{case}"], r.binary(name, a, b, backend=1), equal_nan=True)
+    if sa == sb:
+        G[f"bin_add_relu_{case}"] = r.binary("add_relu", a, b, backend=0)
+L.ax_rng_seed(7100)
+ux = np.concatenate([ref_uniform(200, -4.0, 4.0), np.array([0.0, -0.0, 1.0, -1.0, 30.0, -30.0, 1e-20], np.float32)])
+for name in ("neg", "abs", "exp", "log", "sqrt", "square", "sigmoid", "tanh"):
+    G[f"un_{name}"] = r.unary(name, ux, backend=0)
+G["un_add_scalar"] = r.unary("add_scalar", ux, backend=0, scalar=0.37)
+G["un_mul_scalar"] = r.unary("mul_scalar", ux, backend=0, scalar=-1.7)
+G["un_leaky_relu"] = r.activation("leaky_relu", ux, 0.1)
+G["un_elu"] = r.activation("elu", ux, 0.7)
+G["un_swish"] = r.activation("swish", ux)
+L.ax_rng_seed(7200)
+for name_shape in (((6, 10),), ((4, 5, 6),), ((3, 200),)):
+    shp = name_shape[0]
+    arr = ref_uniform(int(np.prod(shp)), -1.0, 1.0).reshape(shp)
+    tag = "x".join(map(str, shp))
+    for axis in range(-1, len(shp)):
+        for name in ("mean", "max", "min"):
+            G[f"red_{name}_{tag}_axis{axis}"] = r.reduce(name, arr, axis, backend=1)
+            G[f"red_{name}_{tag}_axis{axis}_naive"] = r.reduce(name, arr, axis, backend=0)
+        G[f"red_argmax_{tag}_axis{axis}"] = r.reduce("argmax", arr, axis, backend=1)
+L.ax_rng_seed(7300)
+for (rows, cols) in ((5, 7), (3, 300), (2, 1000), (4, 64)):
+    arr = ref_uniform(rows * cols, -6.0, 6.0).reshape(rows, cols)
+    G[f"softmax_{rows}x{cols}"] = r.unary("softmax_rowwise", arr, backend=1)
+    G[f"softmax_{rows}x{cols}_naive"] = r.unary("softmax_rowwise", arr, backend=0)
+L.ax_rng_seed(7400)
+for shp in ((6, 16), (2, 5, 100), (3, 768)):
+    arr = ref_uniform(int(np.prod(shp)), -3.0, 5.0).reshape(shp)
+    gamma, beta = ref_uniform(shp[-1], 0.5, 1.5), ref_uniform(shp[-1], -1.0, 1.0)
+    G["layernorm_" + "x".join(map(str, shp))] = r.layernorm(arr, gamma, beta, 1e-5)
+L.ax_rng_seed(7500)
+w0 = ref_uniform(300, -1.0, 1.0)
+grads = [ref_uniform(300, -1.0, 1.0) for _ in range(3)]
+G["opt_adam"] = np.stack(r.optimizer_steps("adam", w0, grads, lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01))
+G["opt_adamw"] = np.stack(r.optimizer_steps("adamw", w0, grads, lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01))
+G["opt_sgd_plain"] = np.stack(r.optimizer_steps("sgd", w0, grads, lr=5e-2, momentum=0.0, wd=0.0, nesterov=False))
+G["opt_sgd_momentum"] = np.stack(r.optimizer_steps("sgd", w0, grads, lr=5e-2, momentum=0.9, wd=0.01, nesterov=False))
+G["opt_sgd_nesterov"] = np.stack(r.optimizer_steps("sgd", w0, grads, lr=5e-2, momentum=0.9, wd=0.01, nesterov=True))
+
 np.savez_compressed(os.path.join(HERE, "golden.npz"), **G)
 print("wrote", len(G), "arrays,", os.path.getsize(os.path.join(HERE, "golden.npz")), "bytes")
 

@@ -67,6 +67,15 @@ class Oracle:
         L.axo_qgemm_w8a32.argtypes = [f32p, i8p, f32p, f32p, i64, i64, i64]
         L.axo_qgemm_w8a8_acc.argtypes = [i8p, i8p, i32p, i64, i64, i64]
         L.axo_w8a8_epilogue.argtypes = [i32p, C.c_float, f32p, C.c_void_p, C.c_int, f32p, i64, i64]
+        i64p = np.ctypeslib.ndpointer(np.int64, flags="C_CONTIGUOUS")
+        L.axo_binary.argtypes = [C.c_int, f32p, i64p, C.c_int, f32p, i64p, C.c_int, f32p, i64p, C.c_int]
+        L.axo_unary.argtypes = [C.c_int, f32p, f32p, i64, C.c_float]
+        L.axo_reduce_axis.argtypes = [C.c_int, f32p, i64, i64, i64, f32p]
+        L.axo_argmax_axis.argtypes = [f32p, i64, i64, i64, i64p]
+        L.axo_softmax_rows.argtypes = [f32p, f32p, i64, i64]
+        L.axo_layernorm_fwd.argtypes = [f32p, f32p, f32p, f32p, C.c_void_p, C.c_void_p, i64, i64, C.c_float]
+        L.axo_adam_update.argtypes = [f32p, f32p, f32p, f32p, i64] + [C.c_float] * 7 + [C.c_int]
+        L.axo_sgd_update.argtypes = [f32p, f32p, C.c_void_p, i64, C.c_float, C.c_float, C.c_float, C.c_int]
 
     # ---- RNG -------------------------------------------------------------
     def seed(self, s, drop_spare=True):
@@ -173,6 +182,74 @@ class Oracle:
         o, l = np.empty(BH * S * dk, dt), np.empty(BH * S, dt)
         (self.L.axo_sdpa_fwd_f64 if f64 else self.L.axo_sdpa_fwd)(q, k, v, o, l, BH, S, dk, scale, int(causal))
         return o.reshape(BH, S, dk), l.reshape(BH, S)
+
+    BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3, "equal": 4, "greater": 5, "add_relu": 6}
+    UNARY = {"neg": 0, "abs": 1, "exp": 2, "log": 3, "sqrt": 4, "square": 5, "sigmoid": 6, "tanh": 7,
+             "leaky_relu": 8, "elu": 9, "swish": 10, "add_scalar": 11, "mul_scalar": 12}
+    REDUCE = {"sum": 0, "mean": 1, "max": 2, "min": 3}
+
+    def binary(self, name, a, b):
+        a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)
+        shape = np.broadcast_shapes(a.shape, b.shape)
+        out = np.empty(shape, np.float32)
+        sh = lambda t: np.array(t.shape if t.ndim else (1,), np.int64)
+        self.L.axo_binary(self.BINARY[name], a.reshape(-1), sh(a), max(a.ndim, 1), b.reshape(-1), sh(b),
+                          max(b.ndim, 1), out.reshape(-1), np.array(shape, np.int64), len(shape))
+        return out
+
+    def unary(self, name, x, param=0.0):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty_like(x)
+        self.L.axo_unary(self.UNARY[name], x.reshape(-1), out.reshape(-1), x.size, param)
+        return out
+
+    def reduce(self, name, x, axis):
+        """axis -1 reduces everything (to shape (1,))."""
+        x = np.ascontiguousarray(x, np.float32)
+        if axis == -1:
+            out = np.empty(1, np.float32)
+            self.L.axo_reduce_axis(self.REDUCE[name], x.reshape(-1), 1, x.size, 1, out)
+            return out
+        outer, inner = int(np.prod(x.shape[:axis])), int(np.prod(x.shape[axis + 1:]))
+        out = np.empty(outer * inner, np.float32)
+        self.L.axo_reduce_axis(self.REDUCE[name], x.reshape(-1), outer, x.shape[axis], inner, out)
+        return out.reshape(x.shape[:axis] + x.shape[axis + 1:])
+
+    def argmax(self, x, axis):
+        x = np.ascontiguousarray(x, np.float32)
+        if axis == -1:
+            out = np.empty(1, np.int64)
+            self.L.axo_argmax_axis(x.reshape(-1), 1, x.size, 1, out)
+            return out
+        outer, inner = int(np.prod(x.shape[:axis])), int(np.prod(x.shape[axis + 1:]))
+        out = np.empty(outer * inner, np.int64)
+        self.L.axo_argmax_axis(x.reshape(-1), outer, x.shape[axis], inner, out)
+        return out.reshape(x.shape[:axis] + x.shape[axis + 1:])
+
+    def softmax_rows(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty_like(x)
+        self.L.axo_softmax_rows(x.reshape(-1), out.reshape(-1), x.shape[0], x.shape[1])
+        return out
+
+    def layernorm(self, x, gamma, beta, eps):
+        """(out, x_hat, inv_std) over the last axis."""
+        x = np.ascontiguousarray(x, np.float32)
+        rows, cols = int(np.prod(x.shape[:-1])), x.shape[-1]
+        out, xh, inv = np.empty_like(x), np.empty_like(x), np.empty(rows, np.float32)
+        self.L.axo_layernorm_fwd(x.reshape(-1), np.ascontiguousarray(gamma, np.float32),
+                                 np.ascontiguousarray(beta, np.float32), out.reshape(-1), xh.ctypes.data,
+                                 inv.ctypes.data, rows, cols, eps)
+        return out, xh, inv
+
+    def adam_update(self, w, g, m, v, lr, beta1, beta2, eps, wd, bc1, bc2, decoupled):
+        """Updates w, m, v (float32 arrays) in place."""
+        self.L.axo_adam_update(w.reshape(-1), np.ascontiguousarray(g, np.float32).reshape(-1), m.reshape(-1),
+                               v.reshape(-1), w.size, lr, beta1, beta2, eps, wd, bc1, bc2, int(decoupled))
+
+    def sgd_update(self, w, g, mom, lr, momentum, wd, nesterov):
+        self.L.axo_sgd_update(w.reshape(-1), np.ascontiguousarray(g, np.float32).reshape(-1),
+                              mom.ctypes.data if mom is not None else None, w.size, lr, momentum, wd, int(nesterov))
 
     def gelu(self, x):
         x = np.ascontiguousarray(x, np.float32).copy()
@@ -318,6 +395,34 @@ class RefLib:
         L.ax_layer_destroy.argtypes = [C.c_void_p]
         L.ax_layer_get_params.restype = C.c_int
         L.ax_layer_get_params.argtypes = [C.c_void_p, C.POINTER(TP), C.c_int]
+        for name in ("add", "sub", "mul", "div", "equal", "greater", "add_relu"):
+            getattr(L, "ax_compute_" + name).argtypes = [TP, TP, TP]
+            getattr(L, "ax_compute_" + name).restype = C.c_int
+        for name in ("neg", "abs", "exp", "log", "sqrt", "square", "sigmoid", "tanh", "relu", "softmax_rowwise"):
+            getattr(L, "ax_compute_" + name).argtypes = [TP, TP]
+            getattr(L, "ax_compute_" + name).restype = C.c_int
+        for name in ("add_scalar", "mul_scalar"):
+            getattr(L, "ax_compute_" + name).argtypes = [TP, C.c_double, TP]
+            getattr(L, "ax_compute_" + name).restype = C.c_int
+        for name in ("sum", "mean", "max", "min", "argmax"):
+            getattr(L, "ax_compute_" + name).argtypes = [TP, C.c_int, TP]
+            getattr(L, "ax_compute_" + name).restype = C.c_int
+        for name in ("ax_leaky_relu", "ax_elu"):
+            getattr(L, name).argtypes = [TP, C.c_float]
+            getattr(L, name).restype = TP
+        L.ax_swish.argtypes = [TP]
+        L.ax_swish.restype = TP
+        L.ax_layernorm_create.restype = C.c_void_p
+        L.ax_layernorm_create.argtypes = [i64, C.c_float]
+        PP = C.POINTER(TP)
+        L.ax_adam_create.restype = C.c_void_p
+        L.ax_adam_create.argtypes = [PP, C.c_int] + [C.c_float] * 5
+        L.ax_adamw_create.restype = C.c_void_p
+        L.ax_adamw_create.argtypes = [PP, C.c_int] + [C.c_float] * 5
+        L.ax_sgd_create.restype = C.c_void_p
+        L.ax_sgd_create.argtypes = [PP, C.c_int, C.c_float, C.c_float, C.c_float, C.c_bool]
+        L.ax_optimizer_step.argtypes = [C.c_void_p]
+        L.ax_optimizer_destroy.argtypes = [C.c_void_p]
         L.ax_compute_init()
         L.ax_no_grad()
 
@@ -440,3 +545,91 @@ class RefLib:
                                    a.shape[0])
         assert st == 0
         return out
+
+    # ---- the remaining elementwise / reduction / optimizer slots ----------------------------
+    def empty_dtype(self, shape, dtype):
+        sh = (i64 * len(shape))(*shape)
+        return self.L.ax_tensor_zeros(sh, len(shape), dtype)
+
+    def binary(self, name, a, b, backend=1):
+        self.backend(backend)
+        a, b = np.asarray(a, np.float32), np.asarray(b, np.float32)
+        ta, tb = self.tensor(a), self.tensor(b)
+        to = self.empty(*np.broadcast_shapes(a.shape, b.shape))
+        st = getattr(self.L, "ax_compute_" + name)(ta, tb, to)
+        assert st == 0, (name, st)
+        out = self.numpy(to)
+        self.free(ta, tb, to)
+        return out
+
+    def unary(self, name, x, backend=1, scalar=None):
+        self.backend(backend)
+        t, to = self.tensor(x), self.empty(*np.shape(x))
+        fn = getattr(self.L, "ax_compute_" + name)
+        st = fn(t, to) if scalar is None else fn(t, scalar, to)
+        assert st == 0, (name, st)
+        out = self.numpy(to)
+        self.free(t, to)
+        return out
+
+    def reduce(self, name, x, axis, backend=1):
+        self.backend(backend)
+        x = np.ascontiguousarray(x, np.float32)
+        shape = (1,) if axis == -1 else x.shape[:axis] + x.shape[axis + 1:]
+        t = self.tensor(x)
+        to = self.empty_dtype(shape, 3) if name == "argmax" else self.empty(*shape)
+        st = getattr(self.L, "ax_compute_" + name)(t, axis, to)
+        assert st == 0, (name, st)
+        if name == "argmax":
+            n = int(np.prod(shape))
+            buf = (C.c_int64 * n).from_address(to.contents.storage.contents.data)
+            out = np.frombuffer(buf, np.int64).reshape(shape).copy()
+        else:
+            out = self.numpy(to)
+        self.free(t, to)
+        return out
+
+    def activation(self, name, x, alpha=None):
+        """ax_leaky_relu / ax_elu / ax_swish (src/core/activations.c) on host tensors."""
+        t = self.tensor(x)
+        fn = getattr(self.L, "ax_" + name)
+        o = fn(t) if alpha is None else fn(t, alpha)
+        out = self.numpy(o)
+        self.free(t, o)
+        return out
+
+    def layernorm(self, x, gamma, beta, eps):
+        ln = self.L.ax_layernorm_create(x.shape[-1], eps)
+        params = (C.POINTER(RefTensor) * 4)()
+        assert self.L.ax_layer_get_params(ln, params, 4) == 2
+        for prm, val in zip(params, (gamma, beta)):
+            val = np.ascontiguousarray(val, np.float32)
+            C.memmove(prm.contents.storage.contents.data, val.ctypes.data, val.nbytes)
+        t = self.tensor(x)
+        o = self.L.ax_layer_forward(ln, t)
+        out = self.numpy(o)
+        self.free(t, o)
+        self.L.ax_layer_destroy(ln)
+        return out
+
+    def optimizer_steps(self, kind, w0, grads, **kw):
+        """Runs one reference optimizer step per gradient in `grads` on a single parameter
+        tensor; returns the weights after each step.  kind: adam, adamw, sgd."""
+        tw = self.tensor(w0)
+        params = (C.POINTER(RefTensor) * 1)(tw)
+        if kind == "sgd":
+            opt = self.L.ax_sgd_create(params, 1, kw["lr"], kw["momentum"], kw["wd"], kw["nesterov"])
+        else:
+            make = self.L.ax_adam_create if kind == "adam" else self.L.ax_adamw_create
+            opt = make(params, 1, kw["lr"], kw["beta1"], kw["beta2"], kw["eps"], kw["wd"])
+        outs = []
+        for g in grads:
+            tg = self.tensor(g)
+            tw.contents.grad = tg
+            self.L.ax_optimizer_step(opt)
+            tw.contents.grad = None
+            self.free(tg)
+            outs.append(self.numpy(tw))
+        self.L.ax_optimizer_destroy(opt)
+        self.free(tw)
+        return outs

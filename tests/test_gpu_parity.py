@@ -561,3 +561,238 @@ def test_error_paths(hip):
     assert "activation" in hip.last_error()
     assert L.axhip_sgemm(0, 0, 0, 8, 8, 1.0, a.ptr, 8, a.ptr, 8, 0.0, a.ptr, 8, None, 0) == 0   # empty
     hip.sync()
+
+
+# ---------------------------------------------------------------- elementwise / reduction / optimizer slots
+import ctypes as C  # noqa: E402
+
+import slot_cases as sc  # noqa: E402
+from oracle_bind import Oracle as _O  # noqa: E402
+
+
+def bcast_strides(shape, out_shape):
+    """Element strides of a contiguous operand per output dimension, 0 where it is broadcast:
+    the mapping of cpu_naive.c:48-62 resolved on the host."""
+    shape = (1,) * (len(out_shape) - len(shape)) + tuple(shape)
+    strides, st = [], 1
+    for n in reversed(shape):
+        strides.append(st if n > 1 else 0)
+        st *= n
+    return list(reversed(strides))
+
+
+def run_binary(hip, name, a, b):
+    out_shape = np.broadcast_shapes(a.shape, b.shape)
+    nd = len(out_shape)
+    arr = lambda v: (C.c_int64 * max(nd, 1))(*v)
+    da, db, out = hip.array(a), hip.array(b), hip.empty(out_shape)
+    hip.check(hip.L.axhip_binary(_O.BINARY[name], da.ptr, db.ptr, out.ptr, nd, arr(out_shape),
+                                 arr(bcast_strides(a.shape, out_shape)), arr(bcast_strides(b.shape, out_shape))))
+    return out.numpy()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", range(len(sc.BCAST)))
+def test_binary_broadcast_golden(hip, oracle, golden, case):
+    """Single IEEE operations: bit-exact with the reference vectors."""
+    say("binary golden", case)
+    a, b = sc.binary_inputs(oracle, case)
+    for name in sc.BINARY:
+        assert np.array_equal(run_binary(hip, name, a, b), golden[f"bin_{name}_{case}"], equal_nan=True), name
+    if a.shape == b.shape:
+        assert np.array_equal(run_binary(hip, "add_relu", a, b), golden[f"bin_add_relu_{case}"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sa,sb", [((1024, 4096), (4096,)), ((1024, 4096), (1024, 1)), ((64, 33, 17), (33, 1)),
+                                   ((7, 1, 5, 1, 3), (2, 1, 4, 3)), ((1,), (3, 5)), ((2048, 2048), (2048, 2048)),
+                                   ((3, 1000003), (1,)), ((5, 6), (5, 6))])
+def test_binary_broadcast_shapes(hip, oracle, sa, sb):
+    say("binary", sa, sb)
+    oracle.seed(sum(sa) + 7 * sum(sb))
+    a, b = oracle.uniform(sa, -2, 2), oracle.uniform(sb, 0.5, 2)
+    with np.errstate(all="ignore"):
+        want = {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b, "greater": (a > b).astype(np.float32)}
+    for name, w in want.items():
+        assert np.array_equal(run_binary(hip, name, a, b), w), name
+    if np.prod(np.broadcast_shapes(sa, sb)) <= 4096:           # the element-by-element restatement is slow
+        assert np.array_equal(run_binary(hip, "mul", a, b), oracle.binary("mul", a, b))
+
+
+# exp/log/tanh come from the device math library, not the host's: a few ulp apart
+# (relative for large results, absolute below 1, where elu's exp(v) - 1 cancels)
+UNARY_TOL = {"exp": 4e-7, "log": 4e-7, "sigmoid": 4e-7, "tanh": 1e-6, "elu": 4e-7, "swish": 4e-7}
+
+
+def run_unary(hip, name, x, param=0.0):
+    dx, out = hip.array(x), hip.empty(x.shape)
+    hip.check(hip.L.axhip_unary(_O.UNARY[name], dx.ptr, out.ptr, x.size, param))
+    return out.numpy()
+
+
+@pytest.mark.gpu
+def test_unary_golden_and_large(hip, oracle, golden):
+    say("unary")
+    params = {"leaky_relu": 0.1, "elu": 0.7, "add_scalar": 0.37, "mul_scalar": -1.7}
+    x = sc.unary_input(oracle)
+    oracle.seed(99)
+    big = oracle.uniform((1 << 20) + 3, -4, 4)
+    for name in _O.UNARY:
+        p = params.get(name, 0.0)
+        got, ref = run_unary(hip, name, x, p), golden[f"un_{name}"]
+        tol = UNARY_TOL.get(name)
+        if tol is None:
+            assert np.array_equal(got, ref, equal_nan=True), name
+        else:
+            assert (np.abs(got - ref) <= tol * np.maximum(np.abs(ref), 1)).all(), name
+        got, ref = run_unary(hip, name, big, p), oracle.unary(name, big, p)
+        if tol is None:
+            assert np.array_equal(got, ref), name
+        else:
+            assert (np.abs(got - ref) <= tol * np.maximum(np.abs(ref), 1)).all(), name
+
+
+def run_reduce(hip, name, x, axis):
+    dx = hip.array(x)
+    if axis == -1:
+        out = hip.empty((1,))
+        hip.check(hip.L.axhip_reduce_all(_O.REDUCE[name], dx.ptr, x.size, out.ptr))
+        return out.numpy()
+    outer, inner = int(np.prod(x.shape[:axis])), int(np.prod(x.shape[axis + 1:]))
+    out = hip.empty((outer * inner,))
+    hip.check(hip.L.axhip_reduce_axis(_O.REDUCE[name], dx.ptr, outer, x.shape[axis], inner, out.ptr))
+    return out.numpy().reshape(x.shape[:axis] + x.shape[axis + 1:])
+
+
+def run_argmax(hip, x, axis):
+    dx = hip.array(x)
+    if axis == -1:
+        outer, n, inner, shape = 1, x.size, 1, (1,)
+    else:
+        outer, n, inner = int(np.prod(x.shape[:axis])), x.shape[axis], int(np.prod(x.shape[axis + 1:]))
+        shape = x.shape[:axis] + x.shape[axis + 1:]
+    out = hip.empty((outer * inner,), np.int64)
+    hip.check(hip.L.axhip_argmax_axis(dx.ptr, outer, n, inner, out.ptr))
+    return out.numpy().reshape(shape)
+
+
+@pytest.mark.gpu
+def test_reductions_golden(hip, oracle, golden):
+    say("reductions golden")
+    for shp, arr in zip(sc.REDUCE_SHAPES, sc.reduce_inputs(oracle)):
+        tag = "x".join(map(str, shp))
+        for axis in range(-1, len(shp)):
+            for name in ("max", "min"):                        # order-independent: bit-exact
+                assert np.array_equal(run_reduce(hip, name, arr, axis), golden[f"red_{name}_{tag}_axis{axis}_naive"])
+            assert np.abs(run_reduce(hip, "mean", arr, axis) - golden[f"red_mean_{tag}_axis{axis}_naive"]).max() < 2e-6
+            assert np.array_equal(run_argmax(hip, arr, axis), golden[f"red_argmax_{tag}_axis{axis}"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,axis", [((4096, 4096), 0), ((4096, 4096), 1), ((3, 100000, 5), 1), ((64, 7, 64), 1),
+                                        ((2, 3000001), 1), ((1 << 22,), 0), ((5, 4, 3, 130), 2), ((33, 1000), 0),
+                                        ((1000, 33), 1), ((100000, 8), 0), ((17, 1), 0)])
+def test_reductions_shapes(hip, oracle, shape, axis):
+    say("reduce", shape, axis)
+    oracle.seed(sum(shape) + axis)
+    x = oracle.uniform(shape, -1, 1)
+    x.reshape(-1)[::97] = np.nan                               # passed over by max / min
+    assert np.array_equal(run_reduce(hip, "max", x, axis), np.nanmax(x, axis=axis))
+    assert np.array_equal(run_reduce(hip, "min", x, axis), np.nanmin(x, axis=axis))
+    x = np.nan_to_num(x, nan=0.25)
+    x64 = x.astype(np.float64)
+    bound = SUM_BOUND * np.abs(x64).sum(axis=axis) + 1e-30
+    assert (np.abs(run_reduce(hip, "sum", x, axis) - x64.sum(axis=axis)) <= bound).all()
+    assert (np.abs(run_reduce(hip, "mean", x, axis) - x64.mean(axis=axis)) <= bound / shape[axis] + 1e-7).all()
+    x.reshape(-1)[::5] = 0.75                                  # ties: the first index wins
+    assert np.array_equal(run_argmax(hip, x, axis), np.argmax(x, axis=axis))
+    # everything at once
+    assert run_reduce(hip, "max", x, -1)[0] == x.max() and run_reduce(hip, "min", x, -1)[0] == x.min()
+    assert run_argmax(hip, x, -1)[0] == int(np.argmax(x))
+    got = float(run_reduce(hip, "mean", x, -1)[0])
+    assert abs(got - x.astype(np.float64).mean()) <= SUM_BOUND * np.abs(x).astype(np.float64).mean() + 1e-7
+
+
+@pytest.mark.gpu
+def test_reduce_starting_values(hip):
+    """cpu_naive.c:395-433: a row of NaN / -inf leaves the starting value -FLT_MAX."""
+    x = np.array([[np.nan, -np.inf, np.nan], [1.0, np.nan, 2.0]], np.float32)
+    assert np.array_equal(run_reduce(hip, "max", x, 1), np.array([-np.finfo(np.float32).max, 2.0], np.float32))
+    assert np.array_equal(run_reduce(hip, "min", -x, 1), np.array([np.finfo(np.float32).max, -2.0], np.float32))
+
+
+def run_softmax(hip, x):
+    dx, out = hip.array(x), hip.empty(x.shape)
+    hip.check(hip.L.axhip_softmax_rows(dx.ptr, out.ptr, x.shape[0], x.shape[1]))
+    return out.numpy()
+
+
+@pytest.mark.gpu
+def test_softmax_rows(hip, oracle, golden):
+    say("softmax")
+    for (rows, cols), arr in zip(sc.SOFTMAX_SHAPES, sc.softmax_inputs(oracle)):
+        assert np.abs(run_softmax(hip, arr) - golden[f"softmax_{rows}x{cols}_naive"]).max() < 1e-6
+    for (rows, cols) in [(1, 1), (7, 129), (1000, 512), (33, 513), (64, 1024), (5, 4096), (3, 4097), (2, 100000),
+                         (8192, 512), (4097, 64)]:
+        oracle.seed(rows + cols)
+        x = oracle.uniform((rows, cols), -8, 8)
+        got = run_softmax(hip, x)
+        e = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
+        want = e / e.sum(axis=1, keepdims=True)
+        assert (np.abs(got - want) <= 2e-6 * want + 1e-12).all(), (rows, cols)
+        if rows * cols <= 1 << 20:
+            assert np.abs(got - oracle.softmax_rows(x)).max() < 1e-6
+
+
+def run_layernorm(hip, x, gamma, beta, eps, save=True):
+    rows, cols = int(np.prod(x.shape[:-1])), x.shape[-1]
+    dx, dg, db = hip.array(x), hip.array(gamma), hip.array(beta)
+    out, xh, inv = hip.empty(x.shape), hip.empty(x.shape), hip.empty((rows,))
+    hip.check(hip.L.axhip_layernorm_fwd(dx.ptr, dg.ptr, db.ptr, out.ptr, xh.ptr if save else None,
+                                        inv.ptr if save else None, rows, cols, eps))
+    return out.numpy(), xh.numpy(), inv.numpy()
+
+
+@pytest.mark.gpu
+def test_layernorm_forward(hip, oracle, golden):
+    say("layernorm")
+    for shp, (x, gamma, beta) in zip(sc.LAYERNORM_SHAPES, sc.layernorm_inputs(oracle)):
+        out, xh, inv = run_layernorm(hip, x, gamma, beta, 1e-5)
+        assert np.abs(out - golden["layernorm_" + "x".join(map(str, shp))]).max() < 5e-6
+        o_out, o_xh, o_inv = oracle.layernorm(x, gamma, beta, 1e-5)
+        assert np.abs(out - o_out).max() < 5e-6 and np.abs(xh - o_xh).max() < 5e-6
+        assert np.allclose(inv, o_inv, rtol=2e-6)
+    for shp in [(4096, 1024), (2048, 768), (100, 4096), (3, 5000), (9, 1), (4097, 96)]:
+        oracle.seed(sum(shp))
+        x, gamma, beta = oracle.uniform(shp, -3, 5), oracle.uniform((shp[-1],), 0.5, 1.5), oracle.uniform((shp[-1],), -1, 1)
+        out, xh, inv = run_layernorm(hip, x, gamma, beta, 1e-5)
+        x64 = x.astype(np.float64)
+        want_xh = (x64 - x64.mean(axis=-1, keepdims=True)) / np.sqrt(x64.var(axis=-1, keepdims=True) + 1e-5)
+        assert np.abs(xh - want_xh).max() < 2e-5 and np.abs(out - (gamma * want_xh + beta)).max() < 2e-5, shp
+        out2, _, _ = run_layernorm(hip, x, gamma, beta, 1e-5, save=False)
+        assert np.array_equal(out, out2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("key", list(sc.OPTIMIZERS))
+def test_optimizer_updates(hip, oracle, golden, key):
+    say("optimizer", key)
+    kind, kw = sc.OPTIMIZERS[key]
+    w0, grads = sc.optimizer_inputs(oracle)
+    dw, dm, dv = hip.array(w0), hip.array(np.zeros_like(w0)), hip.array(np.zeros_like(w0))
+    w, m, v = w0.copy(), np.zeros_like(w0), np.zeros_like(w0)
+    for step, g in enumerate(grads, 1):
+        dg = hip.array(g)
+        if kind == "sgd":
+            use_m = kw["momentum"] > 0
+            hip.check(hip.L.axhip_sgd_update(dw.ptr, dg.ptr, dm.ptr if use_m else None, w0.size, kw["lr"], kw["momentum"],
+                                             kw["wd"], int(kw["nesterov"])))
+            oracle.sgd_update(w, g, m if use_m else None, kw["lr"], kw["momentum"], kw["wd"], kw["nesterov"])
+        else:
+            bc1, bc2 = sc.bias_corrections(kw["beta1"], kw["beta2"], step)
+            hip.check(hip.L.axhip_adam_update(dw.ptr, dg.ptr, dm.ptr, dv.ptr, w0.size, kw["lr"], kw["beta1"], kw["beta2"],
+                                              kw["eps"], kw["wd"], bc1, bc2, int(kind == "adamw")))
+            oracle.adam_update(w, g, m, v, kw["lr"], kw["beta1"], kw["beta2"], kw["eps"], kw["wd"], bc1, bc2, kind == "adamw")
+        got = dw.numpy()
+        assert np.abs(got - golden[key][step - 1]).max() < 2e-6, step        # the reference's CPU optimizer
+        assert np.abs(got - w).max() < 5e-7, step                            # same formula; fma contraction apart

@@ -312,3 +312,132 @@ def test_oracle_equals_compiled_reference(oracle, reflib):
     x, wq = oracle.int8((3, 4096)), oracle.int8((32, 4096))
     via_ref = reflib.qgemm_w8a32(x.astype(np.float32), wq, np.ones(32, np.float32))
     assert np.array_equal(oracle.qgemm_w8a8_acc(x, wq).astype(np.float64), via_ref.astype(np.float64))
+
+
+# ---------------------------------------------------------------- elementwise / reduction / optimizer slots
+import slot_cases as sc  # noqa: E402
+
+
+@pytest.mark.parametrize("case", range(len(sc.BCAST)))
+def test_binary_broadcast_against_reference_vectors(oracle, golden, case):
+    """Bit-exact against both reference CPU backends (they agree, checked when the vectors were
+    written), and against numpy's broadcasting, which fixes the index mapping independently."""
+    a, b = sc.binary_inputs(oracle, case)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        want = {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b,
+                "equal": (a == b).astype(np.float32), "greater": (a > b).astype(np.float32)}
+    for name in sc.BINARY:
+        got = oracle.binary(name, a, b)
+        assert np.array_equal(got, golden[f"bin_{name}_{case}"], equal_nan=True), name
+        assert np.array_equal(got, want[name], equal_nan=True), name
+    assert np.array_equal(oracle.binary("equal", a, a), np.ones_like(a)) and not oracle.binary("greater", a, a).any()
+    if a.shape == b.shape:
+        got = oracle.binary("add_relu", a, b)
+        assert np.array_equal(got, golden[f"bin_add_relu_{case}"]) and np.array_equal(got, np.maximum(a + b, 0))
+
+
+def test_unary_against_reference_vectors(oracle, golden):
+    """Bit-exact with the reference's naive backend and activation functions (same libm here);
+    numpy float64 closed forms bound the values themselves."""
+    x = sc.unary_input(oracle)
+    x64 = x.astype(np.float64)
+    with np.errstate(all="ignore"):
+        closed = {"neg": -x64, "abs": np.abs(x64), "exp": np.exp(x64),
+                  "log": np.where(x64 > 0, np.log(np.where(x64 > 0, x64, 1)), -np.finfo(np.float32).max),
+                  "sqrt": np.where(x64 >= 0, np.sqrt(np.abs(x64)), 0.0), "square": x64 * x64,
+                  "sigmoid": 1 / (1 + np.exp(-x64)), "tanh": np.tanh(x64),
+                  "leaky_relu": np.where(x64 > 0, x64, np.float32(0.1) * x64),
+                  "elu": np.where(x64 > 0, x64, np.float32(0.7) * np.expm1(x64)),
+                  "swish": x64 / (1 + np.exp(-x64)),
+                  "add_scalar": x64 + np.float32(0.37), "mul_scalar": x64 * np.float32(-1.7)}
+    params = {"leaky_relu": 0.1, "elu": 0.7, "add_scalar": 0.37, "mul_scalar": -1.7}
+    for name, want in closed.items():
+        got = oracle.unary(name, x, params.get(name, 0.0))
+        assert np.array_equal(got, golden[f"un_{name}"], equal_nan=True), name
+        assert np.allclose(got, want, rtol=2e-6, atol=1e-6), name
+
+
+def test_reductions_against_reference_vectors(oracle, golden):
+    for shp, arr in zip(sc.REDUCE_SHAPES, sc.reduce_inputs(oracle)):
+        tag = "x".join(map(str, shp))
+        for axis in range(-1, len(shp)):
+            np_axis = None if axis == -1 else axis
+            for name, fn in (("mean", np.mean), ("max", np.max), ("min", np.min)):
+                got = oracle.reduce(name, arr, axis)
+                # the naive backend adds in the same order; the optimised one in lanes
+                assert np.array_equal(got, golden[f"red_{name}_{tag}_axis{axis}_naive"]), (name, tag, axis)
+                assert np.allclose(got, golden[f"red_{name}_{tag}_axis{axis}"], rtol=0, atol=2e-6)
+                assert np.allclose(got.reshape(-1), np.asarray(fn(arr.astype(np.float64), axis=np_axis)).reshape(-1),
+                                   rtol=0, atol=2e-6)
+            got = oracle.argmax(arr, axis)
+            assert np.array_equal(got, golden[f"red_argmax_{tag}_axis{axis}"])
+            assert np.array_equal(got.reshape(-1), np.asarray(np.argmax(arr, axis=np_axis)).reshape(-1))
+    # ties take the first index; values that fail every comparison leave the starting value
+    assert oracle.argmax(np.array([[1, 3, 3, 2]], np.float32), 1)[0] == 1
+    assert oracle.reduce("max", np.array([[np.nan, -np.inf]], np.float32), 1)[0] == -np.finfo(np.float32).max
+
+
+def test_softmax_rows_against_reference_vectors(oracle, golden):
+    for (rows, cols), arr in zip(sc.SOFTMAX_SHAPES, sc.softmax_inputs(oracle)):
+        got = oracle.softmax_rows(arr)
+        assert np.array_equal(got, golden[f"softmax_{rows}x{cols}_naive"])
+        assert np.abs(got - golden[f"softmax_{rows}x{cols}"]).max() < 2e-6      # polynomial exp there
+        e = np.exp(arr.astype(np.float64) - arr.max(axis=1, keepdims=True))
+        assert np.abs(got - e / e.sum(axis=1, keepdims=True)).max() < 1e-6
+        assert np.abs(got.sum(axis=1) - 1).max() < 1e-5
+    # shift invariance and the uniform row
+    x = sc.softmax_inputs(oracle)[0]
+    assert np.abs(oracle.softmax_rows(x + 3.0) - oracle.softmax_rows(x)).max() < 1e-6
+    assert np.allclose(oracle.softmax_rows(np.full((2, 8), 5.0, np.float32)), 0.125)
+
+
+def test_layernorm_against_reference_vectors(oracle, golden):
+    for shp, (x, gamma, beta) in zip(sc.LAYERNORM_SHAPES, sc.layernorm_inputs(oracle)):
+        out, xh, inv = oracle.layernorm(x, gamma, beta, 1e-5)
+        ref = golden["layernorm_" + "x".join(map(str, shp))]
+        assert np.abs(out - ref).max() < 5e-6
+        x64 = x.astype(np.float64)
+        mu, var = x64.mean(axis=-1, keepdims=True), x64.var(axis=-1, keepdims=True)
+        want_xh = (x64 - mu) / np.sqrt(var + 1e-5)
+        assert np.abs(xh - want_xh).max() < 5e-6 and np.abs(ref - (gamma * want_xh + beta)).max() < 5e-6
+        assert np.abs(out - (gamma * want_xh + beta)).max() < 5e-6
+        assert np.allclose(inv, 1 / np.sqrt(var.reshape(-1) + 1e-5), rtol=2e-6)
+    # a constant row has zero variance: x_hat = 0 and the output is beta
+    out, xh, inv = oracle.layernorm(np.full((1, 12), 3.0, np.float32), np.ones(12, np.float32),
+                                    np.arange(12, dtype=np.float32), 1e-5)
+    assert np.array_equal(xh, np.zeros((1, 12), np.float32)) and np.array_equal(out[0], np.arange(12, dtype=np.float32))
+
+
+@pytest.mark.parametrize("key", list(sc.OPTIMIZERS))
+def test_optimizer_updates_against_reference_vectors(oracle, golden, key):
+    """The per-element update formulas against what the reference's CPU optimizers produced
+    over three steps (its Adam folds the bias corrections into the step size, hence a tolerance),
+    and against a float64 evaluation of the textbook recurrences."""
+    kind, kw = sc.OPTIMIZERS[key]
+    w0, grads = sc.optimizer_inputs(oracle)
+    w, m, v = w0.copy(), np.zeros_like(w0), np.zeros_like(w0)
+    w64, m64, v64 = w0.astype(np.float64), np.zeros(300), np.zeros(300)
+    for step, g in enumerate(grads, 1):
+        g64 = g.astype(np.float64)
+        if kind == "sgd":
+            oracle.sgd_update(w, g, m if kw["momentum"] > 0 else None, kw["lr"], kw["momentum"], kw["wd"], kw["nesterov"])
+            gi = g64 + kw["wd"] * w64
+            if kw["momentum"] > 0:
+                m64 = kw["momentum"] * m64 + gi
+                w64 = w64 - kw["lr"] * ((gi + kw["momentum"] * m64) if kw["nesterov"] else m64)
+            else:
+                w64 = w64 - kw["lr"] * gi
+        else:
+            bc1, bc2 = sc.bias_corrections(kw["beta1"], kw["beta2"], step)
+            oracle.adam_update(w, g, m, v, kw["lr"], kw["beta1"], kw["beta2"], kw["eps"], kw["wd"], bc1, bc2,
+                               kind == "adamw")
+            if kind == "adamw":
+                w64 = w64 * (1 - kw["lr"] * kw["wd"])
+                gi = g64
+            else:
+                gi = g64 + kw["wd"] * w64
+            m64 = kw["beta1"] * m64 + (1 - kw["beta1"]) * gi
+            v64 = kw["beta2"] * v64 + (1 - kw["beta2"]) * gi * gi
+            w64 = w64 - kw["lr"] * (m64 / (1 - kw["beta1"] ** step)) / (np.sqrt(v64 / (1 - kw["beta2"] ** step)) + kw["eps"])
+        assert np.abs(w - golden[key][step - 1]).max() < 2e-6, step
+        assert np.abs(w - w64).max() < 2e-6, step
