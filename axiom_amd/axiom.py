@@ -57,6 +57,17 @@ SIGNATURES = {
     "ax_hip_sdpa_fwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, i64, i64, i64,
                                  C.c_float, C.c_bool, C.c_void_p]),
     "ax_compute_sum": (C.c_int, [TP, C.c_int, TP]), "ax_compute_axpy": (C.c_int, [TP, C.c_float, TP]),
+    **{"ax_compute_" + n: (C.c_int, [TP, TP, TP]) for n in ("add", "sub", "mul", "div", "equal", "greater", "add_relu")},
+    **{"ax_compute_" + n: (C.c_int, [TP, TP]) for n in ("neg", "abs", "exp", "log", "sqrt", "square", "sigmoid", "tanh",
+                                                        "swish", "softmax_rowwise")},
+    **{"ax_compute_" + n: (C.c_int, [TP, C.c_double, TP]) for n in ("add_scalar", "mul_scalar")},
+    **{"ax_compute_" + n: (C.c_int, [TP, C.c_float, TP]) for n in ("leaky_relu", "elu")},
+    **{"ax_compute_" + n: (C.c_int, [TP, C.c_int, TP]) for n in ("mean", "max", "min", "argmax")},
+    "ax_compute_adam_update": (C.c_int, [TP, TP, TP, TP] + [C.c_float] * 7 + [C.c_bool]),
+    "ax_compute_sgd_update": (C.c_int, [TP, TP, TP, C.c_float, C.c_float, C.c_float, C.c_bool]),
+    "ax_compute_has_adam_update": (C.c_int, []), "ax_compute_has_sgd_update": (C.c_int, []),
+    "ax_compute_layernorm": (C.c_int, [TP, TP, TP, C.c_float, TP, TP, TP]),
+    "ax_layernorm_create": (C.c_void_p, [C.c_int64, C.c_float]),
     "ax_compute_gemm_bias_act": (C.c_int, [TP, TP, TP, C.c_int, TP]),
     "ax_compute_has_gemm_relu": (C.c_int, []), "ax_compute_has_gemm_nt": (C.c_int, []),
     "ax_compute_has_gemm_tn": (C.c_int, []), "ax_compute_has_gemm_ex": (C.c_int, []),

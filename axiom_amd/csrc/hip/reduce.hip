@@ -120,7 +120,26 @@ k_reduce_cols(const float *__restrict__ in, int64_t axis_len, int64_t inner, int
     if (a1 > axis_len) a1 = axis_len;
     if (col < inner) {
         const float *base = in + o * axis_len * inner + col;
-        for (int64_t a = s * slice + ty; a < a1; a += TY) {
+        int64_t a = s * slice + ty;
+        // eight rows in flight per thread, then joined in ascending order
+        for (; a + 7 * TY < a1; a += 8 * TY) {
+            float v[8][VW];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                if (VW == 4) {
+                    const v4f t = *reinterpret_cast<const v4f *>(base + (a + u * TY) * inner);
+#pragma unroll
+                    for (int e = 0; e < VW; e++) v[u][e] = t[e];
+                } else {
+                    v[u][0] = base[(a + u * TY) * inner];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+#pragma unroll
+                for (int e = 0; e < VW; e++) acc[e] = red_join<OP>(acc[e], v[u][e]);
+        }
+        for (; a < a1; a += TY) {
             if (VW == 4) {
                 const v4f v = *reinterpret_cast<const v4f *>(base + a * inner);
 #pragma unroll

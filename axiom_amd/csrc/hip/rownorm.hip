@@ -1,7 +1,7 @@
 // Row softmax (the .softmax_rowwise vtable slot; cpu_naive.c:235-270, cuda/ops_fused.cu:44-91)
 // and layer normalisation forward (src/core/norm.c:1278-1399) over contiguous [rows, cols] fp32.
 // HBM-bound.  A row of up to TPR*VPT columns is read once into registers (one wave per row up to
-// 512 columns, one workgroup per row up to 4096), reduced, and written once; longer rows are
+// 1024 columns, one workgroup per row up to 4096), reduced, and written once; longer rows are
 // re-read from memory by one workgroup per row.
 #include <float.h>
 
@@ -26,6 +26,25 @@ __device__ __forceinline__ float row_join(float v, float *lds, int wave) {
     return MAX ? fmaxf(fmaxf(a, b), fmaxf(c, d)) : (a + b) + (c + d);
 }
 
+// two sums at once (layer norm's sum and sum of squares): one LDS round instead of two
+template <int TPR>
+__device__ __forceinline__ void row_join2(float &a, float &b, float *lds, int wave) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        a += __shfl_xor(a, off, 64);
+        b += __shfl_xor(b, off, 64);
+    }
+    if (TPR == 64) return;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) {
+        lds[wave] = a;
+        lds[4 + wave] = b;
+    }
+    __syncthreads();
+    a = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+    b = (lds[4] + lds[5]) + (lds[6] + lds[7]);
+}
+
 struct LnArgs {
     const float *gamma, *beta;
     float *x_hat, *inv_std;
@@ -36,7 +55,7 @@ struct LnArgs {
 template <int TPR, int VPT, int KIND>
 __global__ void __launch_bounds__(256)
 k_rows_cached(const float *__restrict__ in, float *__restrict__ out, int64_t rows, int cols, LnArgs ln) {
-    __shared__ float lds[4];
+    __shared__ float lds[8];
     constexpr int RPB = 256 / TPR;
     const int t = threadIdx.x % TPR, wave = threadIdx.x >> 6;
     const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
@@ -68,8 +87,7 @@ k_rows_cached(const float *__restrict__ in, float *__restrict__ out, int64_t row
             s += v[i];
             s2 = __builtin_fmaf(v[i], v[i], s2);
         }
-        s = row_join<TPR, false>(s, lds, wave);
-        s2 = row_join<TPR, false>(s2, lds, wave);
+        row_join2<TPR>(s, s2, lds, wave);
         const float mean = s / (float)cols;
         float var = s2 / (float)cols - mean * mean;
         if (var < 0.0f) var = 0.0f;
@@ -91,7 +109,7 @@ k_rows_cached(const float *__restrict__ in, float *__restrict__ out, int64_t row
 template <int KIND>
 __global__ void __launch_bounds__(256)
 k_rows_streamed(const float *__restrict__ in, float *__restrict__ out, int64_t cols, LnArgs ln) {
-    __shared__ float lds[4];
+    __shared__ float lds[8];
     const int t = threadIdx.x, wave = t >> 6;
     const int64_t row = blockIdx.x;
     const float *x = in + row * cols;
@@ -116,8 +134,7 @@ k_rows_streamed(const float *__restrict__ in, float *__restrict__ out, int64_t c
             s += v;
             s2 = __builtin_fmaf(v, v, s2);
         }
-        s = row_join<256, false>(s, lds, wave);
-        s2 = row_join<256, false>(s2, lds, wave);
+        row_join2<256>(s, s2, lds, wave);
         const float mean = s / (float)cols;
         float var = s2 / (float)cols - mean * mean;
         if (var < 0.0f) var = 0.0f;
@@ -133,18 +150,18 @@ k_rows_streamed(const float *__restrict__ in, float *__restrict__ out, int64_t c
 
 template <int KIND>
 int launch_rows(const float *in, float *out, int64_t rows, int64_t cols, const LnArgs &ln, const char *what) {
-    if (cols <= 512) {
+    if (cols <= 1024) {
         const int64_t blocks = (rows + 3) / 4;
         if (blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "%s: too many rows", what);
         if (cols <= 128)
             hipLaunchKernelGGL((k_rows_cached<64, 2, KIND>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
-        else
+        else if (cols <= 512)
             hipLaunchKernelGGL((k_rows_cached<64, 8, KIND>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
+        else
+            hipLaunchKernelGGL((k_rows_cached<64, 16, KIND>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
     } else {
         if (rows > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "%s: too many rows", what);
-        if (cols <= 1024)
-            hipLaunchKernelGGL((k_rows_cached<256, 4, KIND>), dim3((unsigned)rows), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
-        else if (cols <= 4096)
+        if (cols <= 4096)
             hipLaunchKernelGGL((k_rows_cached<256, 16, KIND>), dim3((unsigned)rows), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
         else
             hipLaunchKernelGGL((k_rows_streamed<KIND>), dim3((unsigned)rows), dim3(256), 0, kStream, in, out, cols, ln);

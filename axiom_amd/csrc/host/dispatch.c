@@ -143,9 +143,50 @@ ax_status_t ax_compute_fill(ax_tensor_t *t, double value) { AX_DISPATCH(fill, t,
 ax_status_t ax_compute_copy(const ax_tensor_t *src, ax_tensor_t *dst) { AX_DISPATCH(copy, dst, copy(src, dst)); }
 ax_status_t ax_compute_sum(const ax_tensor_t *in, int axis, ax_tensor_t *out) { AX_DISPATCH(sum, out, sum(in, axis, out)); }
 ax_status_t ax_compute_axpy(const ax_tensor_t *x, float alpha, ax_tensor_t *y) { AX_DISPATCH(axpy, y, axpy(x, alpha, y)); }
+/* the remaining wrappers of src/compute/dispatch.c:385-412, 657-721, 762-841 */
+ax_status_t ax_compute_add(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { AX_DISPATCH(add, out, add(a, b, out)); }
+ax_status_t ax_compute_sub(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { AX_DISPATCH(sub, out, sub(a, b, out)); }
+ax_status_t ax_compute_mul(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { AX_DISPATCH(mul, out, mul(a, b, out)); }
+ax_status_t ax_compute_div(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { AX_DISPATCH(div_op, out, div_op(a, b, out)); }
+ax_status_t ax_compute_equal(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { AX_DISPATCH(equal, out, equal(a, b, out)); }
+ax_status_t ax_compute_greater(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { AX_DISPATCH(greater, out, greater(a, b, out)); }
+ax_status_t ax_compute_add_relu(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { AX_DISPATCH(add_relu, out, add_relu(a, b, out)); }
+ax_status_t ax_compute_neg(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(neg, out, neg(in, out)); }
+ax_status_t ax_compute_abs(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(abs_op, out, abs_op(in, out)); }
+ax_status_t ax_compute_exp(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(exp_op, out, exp_op(in, out)); }
+ax_status_t ax_compute_log(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(log_op, out, log_op(in, out)); }
+ax_status_t ax_compute_sqrt(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(sqrt_op, out, sqrt_op(in, out)); }
+ax_status_t ax_compute_square(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(square, out, square(in, out)); }
+ax_status_t ax_compute_sigmoid(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(sigmoid, out, sigmoid(in, out)); }
+ax_status_t ax_compute_tanh(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(tanh_op, out, tanh_op(in, out)); }
+ax_status_t ax_compute_add_scalar(const ax_tensor_t *in, double scalar, ax_tensor_t *out) { AX_DISPATCH(add_scalar, out, add_scalar(in, scalar, out)); }
+ax_status_t ax_compute_mul_scalar(const ax_tensor_t *in, double scalar, ax_tensor_t *out) { AX_DISPATCH(mul_scalar, out, mul_scalar(in, scalar, out)); }
+ax_status_t ax_compute_softmax_rowwise(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(softmax_rowwise, out, softmax_rowwise(in, out)); }
+ax_status_t ax_compute_mean(const ax_tensor_t *in, int axis, ax_tensor_t *out) { AX_DISPATCH(mean, out, mean(in, axis, out)); }
+ax_status_t ax_compute_max(const ax_tensor_t *in, int axis, ax_tensor_t *out) { AX_DISPATCH(max_op, out, max_op(in, axis, out)); }
+ax_status_t ax_compute_min(const ax_tensor_t *in, int axis, ax_tensor_t *out) { AX_DISPATCH(min_op, out, min_op(in, axis, out)); }
+ax_status_t ax_compute_argmax(const ax_tensor_t *in, int axis, ax_tensor_t *out) { AX_DISPATCH(argmax, out, argmax(in, axis, out)); }
+ax_status_t ax_compute_adam_update(ax_tensor_t *weight, ax_tensor_t *grad, ax_tensor_t *m, ax_tensor_t *v, float lr,
+                                   float beta1, float beta2, float eps, float weight_decay, float bc1, float bc2,
+                                   bool decoupled) {
+    AX_DISPATCH(adam_update, weight, adam_update(weight, grad, m, v, lr, beta1, beta2, eps, weight_decay, bc1, bc2, decoupled));
+}
+ax_status_t ax_compute_sgd_update(ax_tensor_t *weight, ax_tensor_t *grad, ax_tensor_t *momentum_buf, float lr,
+                                  float momentum, float weight_decay, bool nesterov) {
+    AX_DISPATCH(sgd_update, weight, sgd_update(weight, grad, momentum_buf, lr, momentum, weight_decay, nesterov));
+}
+/* the three activation slots the reference's dispatch layer has no wrapper for */
+ax_status_t ax_compute_leaky_relu(const ax_tensor_t *in, float alpha, ax_tensor_t *out) { AX_DISPATCH(leaky_relu, out, leaky_relu(in, alpha, out)); }
+ax_status_t ax_compute_elu(const ax_tensor_t *in, float alpha, ax_tensor_t *out) { AX_DISPATCH(elu_op, out, elu_op(in, alpha, out)); }
+ax_status_t ax_compute_swish(const ax_tensor_t *in, ax_tensor_t *out) { AX_DISPATCH(swish_op, out, swish_op(in, out)); }
 ax_status_t ax_compute_gemm_bias_act(const ax_tensor_t *a, const ax_tensor_t *b, const ax_tensor_t *bias,
                                      ax_activation_t act, ax_tensor_t *out) {
     AX_DISPATCH(gemm_bias_act, out, gemm_bias_act(a, b, bias, (int)act, out));
+}
+
+ax_status_t ax_compute_layernorm(const ax_tensor_t *x, const ax_tensor_t *gamma, const ax_tensor_t *beta, float eps,
+                                 ax_tensor_t *out, ax_tensor_t *x_hat, ax_tensor_t *inv_std) {
+    AX_DISPATCH(layernorm_fwd, out, layernorm_fwd(x, gamma, beta, eps, out, x_hat, inv_std));
 }
 
 #define AX_HAS(slot) (ensure_init(), (g_active && g_active->slot) ? 1 : 0)
@@ -155,3 +196,5 @@ int ax_compute_has_gemm_tn(void) { return AX_HAS(gemm_tn); }
 int ax_compute_has_gemm_ex(void) { return AX_HAS(gemm_ex); }
 int ax_compute_has_bias_add(void) { return AX_HAS(bias_add); }
 int ax_compute_has_gemm_bias_act(void) { return AX_HAS(gemm_bias_act); }
+int ax_compute_has_adam_update(void) { return AX_HAS(adam_update); }
+int ax_compute_has_sgd_update(void) { return AX_HAS(sgd_update); }

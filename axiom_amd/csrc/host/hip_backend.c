@@ -2,8 +2,9 @@
  *
  * Plain C: it unpacks ax_tensor_t (shape, strides, offset, device) into pointers and sizes and
  * calls the C ABI of libaxhip.so; no HIP header is included here.  It takes the place of
- * ax_cuda_ops (src/compute/backends/cuda/backend.cu:140-192) for the GEMM family, bias_add,
- * relu, gelu_op, fill, copy and the ten device-owner hooks; every other slot stays NULL.
+ * ax_cuda_ops (src/compute/backends/cuda/backend.cu:140-192): every slot that object fills
+ * except conv_gemm, plus gemm_relu and argmax, and the ten device-owner hooks; the attention
+ * training slots and the convolution slots stay NULL.
  * Operands are borrowed, never retained.  Errors follow the reference's backend convention
  * (cuda/ops_gemm.cu:16-23): dtype != f32 -> AX_ERR_DTYPE_MISMATCH, rank/shape -> AX_ERR_SHAPE_MISMATCH,
  * plus AX_ERR_BACKEND for a tensor that does not live on this backend's device. */
@@ -253,6 +254,232 @@ static ax_status_t hip_axpy(const ax_tensor_t *x, float alpha, ax_tensor_t *y) {
     return lift(axhip_axpy(xp, alpha, yp, nx), "hip axpy");
 }
 
+/* ---- broadcasting binary slots ---------------------------------------------------------
+ * Operands may be any strided views; the output is contiguous.  Each operand's stride per
+ * OUTPUT dimension follows broadcast_index (cpu_naive.c:48-62): trailing dimensions aligned,
+ * an operand extent of 1 contributes stride 0. */
+static ax_status_t on_device_f32(const ax_tensor_t *t, const char *who) {
+    if (!t || !t->storage) {
+        ax_err_set(AX_ERR_NULL_ARG, "%s: NULL tensor", who);
+        return AX_ERR_NULL_ARG;
+    }
+    if (t->dtype != AX_FLOAT32) {
+        ax_err_set(AX_ERR_DTYPE_MISMATCH, "%s only supports float32", who);
+        return AX_ERR_DTYPE_MISMATCH;
+    }
+    if (t->storage->device != g_my_device) {
+        ax_err_set(AX_ERR_BACKEND, "%s: tensor is not on the hip device", who);
+        return AX_ERR_BACKEND;
+    }
+    return AX_OK;
+}
+
+static ax_status_t operand_strides(const ax_tensor_t *t, const ax_tensor_t *out, const char *who, int64_t *st) {
+    for (int d = 0; d < out->ndim; d++) {
+        const int td = d - (out->ndim - t->ndim);
+        st[d] = 0;
+        if (td < 0 || t->shape[td] == 1) continue;
+        if (t->shape[td] != out->shape[d]) {
+            ax_err_set(AX_ERR_SHAPE_MISMATCH, "%s: extent %lld does not broadcast to %lld", who,
+                       (long long)t->shape[td], (long long)out->shape[d]);
+            return AX_ERR_SHAPE_MISMATCH;
+        }
+        st[d] = t->strides[td];
+    }
+    return AX_OK;
+}
+
+static ax_status_t run_binary(const char *who, int op, const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) {
+    ax_status_t st;
+    float *op_;
+    int64_t no, sa[AX_MAX_DIMS], sb[AX_MAX_DIMS];
+    if ((st = on_device_f32(a, who)) || (st = on_device_f32(b, who)) || (st = as_flat(out, who, &op_, &no))) return st;
+    if (a->ndim > out->ndim || b->ndim > out->ndim) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "%s: operand has more dimensions than the output", who);
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    if ((st = operand_strides(a, out, who, sa)) || (st = operand_strides(b, out, who, sb))) return st;
+    return lift(axhip_binary(op, (const float *)a->storage->data + a->offset, (const float *)b->storage->data + b->offset,
+                             op_, out->ndim, out->shape, sa, sb), who);
+}
+
+static ax_status_t hip_add(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { return run_binary("hip add", AXHIP_BIN_ADD, a, b, out); }
+static ax_status_t hip_sub(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { return run_binary("hip sub", AXHIP_BIN_SUB, a, b, out); }
+static ax_status_t hip_mul(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { return run_binary("hip mul", AXHIP_BIN_MUL, a, b, out); }
+static ax_status_t hip_div(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { return run_binary("hip div", AXHIP_BIN_DIV, a, b, out); }
+static ax_status_t hip_equal(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { return run_binary("hip equal", AXHIP_BIN_EQUAL, a, b, out); }
+static ax_status_t hip_greater(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) { return run_binary("hip greater", AXHIP_BIN_GREATER, a, b, out); }
+
+/* same element counts only, as cuda_add_relu (cuda/ops_fused.cu:168-190) */
+static ax_status_t hip_add_relu(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out) {
+    float *ap, *bp, *op;
+    int64_t na, nb, no;
+    ax_status_t st;
+    if ((st = as_flat(a, "hip add_relu", &ap, &na)) || (st = as_flat(b, "hip add_relu", &bp, &nb)) ||
+        (st = as_flat(out, "hip add_relu", &op, &no)))
+        return st;
+    if (na != no || nb != no) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "hip add_relu requires matching shapes");
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    const int64_t one = 1;
+    return lift(axhip_binary(AXHIP_BIN_ADD_RELU, ap, bp, op, 1, &no, &one, &one), "hip add_relu");
+}
+
+/* ---- unary, scalar and activation slots (contiguous, element count of the output) ---- */
+static ax_status_t run_unary(const char *who, int op, const ax_tensor_t *in, float param, ax_tensor_t *out) {
+    float *ip, *op_;
+    int64_t n, no;
+    ax_status_t st;
+    if ((st = as_flat(in, who, &ip, &n)) || (st = as_flat(out, who, &op_, &no))) return st;
+    if (n != no) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "%s: in/out element counts differ", who);
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    return lift(axhip_unary(op, ip, op_, n, param), who);
+}
+
+static ax_status_t hip_neg(const ax_tensor_t *in, ax_tensor_t *out) { return run_unary("hip neg", AXHIP_UN_NEG, in, 0.0f, out); }
+static ax_status_t hip_abs(const ax_tensor_t *in, ax_tensor_t *out) { return run_unary("hip abs", AXHIP_UN_ABS, in, 0.0f, out); }
+static ax_status_t hip_exp(const ax_tensor_t *in, ax_tensor_t *out) { return run_unary("hip exp", AXHIP_UN_EXP, in, 0.0f, out); }
+static ax_status_t hip_log(const ax_tensor_t *in, ax_tensor_t *out) { return run_unary("hip log", AXHIP_UN_LOG, in, 0.0f, out); }
+static ax_status_t hip_sqrt(const ax_tensor_t *in, ax_tensor_t *out) { return run_unary("hip sqrt", AXHIP_UN_SQRT, in, 0.0f, out); }
+static ax_status_t hip_square(const ax_tensor_t *in, ax_tensor_t *out) { return run_unary("hip square", AXHIP_UN_SQUARE, in, 0.0f, out); }
+static ax_status_t hip_sigmoid(const ax_tensor_t *in, ax_tensor_t *out) { return run_unary("hip sigmoid", AXHIP_UN_SIGMOID, in, 0.0f, out); }
+static ax_status_t hip_tanh(const ax_tensor_t *in, ax_tensor_t *out) { return run_unary("hip tanh", AXHIP_UN_TANH, in, 0.0f, out); }
+static ax_status_t hip_swish(const ax_tensor_t *in, ax_tensor_t *out) { return run_unary("hip swish", AXHIP_UN_SWISH, in, 0.0f, out); }
+static ax_status_t hip_leaky_relu(const ax_tensor_t *in, float alpha, ax_tensor_t *out) { return run_unary("hip leaky_relu", AXHIP_UN_LEAKY_RELU, in, alpha, out); }
+static ax_status_t hip_elu(const ax_tensor_t *in, float alpha, ax_tensor_t *out) { return run_unary("hip elu", AXHIP_UN_ELU, in, alpha, out); }
+static ax_status_t hip_add_scalar(const ax_tensor_t *in, double s, ax_tensor_t *out) { return run_unary("hip add_scalar", AXHIP_UN_ADD_SCALAR, in, (float)s, out); }
+static ax_status_t hip_mul_scalar(const ax_tensor_t *in, double s, ax_tensor_t *out) { return run_unary("hip mul_scalar", AXHIP_UN_MUL_SCALAR, in, (float)s, out); }
+
+/* ---- mean / max / min / argmax: the shape rules of hip_sum ---- */
+static ax_status_t reduction_extents(const char *who, const ax_tensor_t *in, int axis, int64_t n_out, int64_t *outer,
+                                     int64_t *axis_len, int64_t *inner) {
+    if (axis == -1) {
+        *outer = 1;
+        *inner = 1;
+        *axis_len = ax_tensor_numel(in);
+    } else {
+        if (axis < 0 || axis >= in->ndim) {
+            ax_err_set(AX_ERR_INVALID_AXIS, "axis %d out of range", axis);
+            return AX_ERR_INVALID_AXIS;
+        }
+        *outer = *inner = 1;
+        for (int d = 0; d < axis; d++) *outer *= in->shape[d];
+        for (int d = axis + 1; d < in->ndim; d++) *inner *= in->shape[d];
+        *axis_len = in->shape[axis];
+    }
+    if (n_out != *outer * *inner) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "%s: output holds %lld elements, expected %lld", who, (long long)n_out,
+                   (long long)(*outer * *inner));
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    return AX_OK;
+}
+
+static ax_status_t run_reduce(const char *who, int op, const ax_tensor_t *in, int axis, ax_tensor_t *out) {
+    float *ip, *op_;
+    int64_t n, no, outer, axis_len, inner;
+    ax_status_t st;
+    if (!in || !out) return AX_ERR_NULL_ARG;
+    if ((st = as_flat(in, who, &ip, &n)) || (st = as_flat(out, who, &op_, &no)) ||
+        (st = reduction_extents(who, in, axis, no, &outer, &axis_len, &inner)))
+        return st;
+    if (axis == -1) return lift(axhip_reduce_all(op, ip, n, op_), who);
+    return lift(axhip_reduce_axis(op, ip, outer, axis_len, inner, op_), who);
+}
+
+static ax_status_t hip_mean(const ax_tensor_t *in, int axis, ax_tensor_t *out) { return run_reduce("hip mean", AXHIP_RED_MEAN, in, axis, out); }
+static ax_status_t hip_max(const ax_tensor_t *in, int axis, ax_tensor_t *out) { return run_reduce("hip max", AXHIP_RED_MAX, in, axis, out); }
+static ax_status_t hip_min(const ax_tensor_t *in, int axis, ax_tensor_t *out) { return run_reduce("hip min", AXHIP_RED_MIN, in, axis, out); }
+
+/* int64 output (opt_argmax, cpu_opt.c:7202-7249) */
+static ax_status_t hip_argmax(const ax_tensor_t *in, int axis, ax_tensor_t *out) {
+    float *ip;
+    int64_t n, outer, axis_len, inner;
+    ax_status_t st;
+    if (!in || !out) return AX_ERR_NULL_ARG;
+    if ((st = as_flat(in, "hip argmax", &ip, &n))) return st;
+    if (out->dtype != AX_INT64) return AX_ERR_DTYPE_MISMATCH;
+    if (!out->storage || !out->storage->data || out->storage->device != g_my_device || !ax_tensor_is_contiguous(out))
+        return AX_ERR_BACKEND;
+    if ((st = reduction_extents("hip argmax", in, axis, ax_tensor_numel(out), &outer, &axis_len, &inner))) return st;
+    return lift(axhip_argmax_axis(ip, outer, axis_len, inner, (int64_t *)out->storage->data + out->offset), "hip argmax");
+}
+
+/* 2-D, matching shapes (cuda_softmax_rowwise, cuda/ops_fused.cu:213-229) */
+static ax_status_t hip_softmax_rowwise(const ax_tensor_t *in, ax_tensor_t *out) {
+    float *ip, *op;
+    int64_t n, no;
+    ax_status_t st;
+    if ((st = as_flat(in, "hip softmax_rowwise", &ip, &n)) || (st = as_flat(out, "hip softmax_rowwise", &op, &no))) return st;
+    if (in->ndim != 2 || out->ndim != 2 || in->shape[0] != out->shape[0] || in->shape[1] != out->shape[1]) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "hip softmax_rowwise shape mismatch");
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    return lift(axhip_softmax_rows(ip, op, in->shape[0], in->shape[1]), "hip softmax_rowwise");
+}
+
+/* ---- optimizer slots (cuda_adam_update / cuda_sgd_update, cuda/ops_optim.cu:66-110) ---- */
+static ax_status_t hip_adam_update(ax_tensor_t *weight, ax_tensor_t *grad, ax_tensor_t *m, ax_tensor_t *v, float lr,
+                                   float beta1, float beta2, float eps, float weight_decay, float bc1, float bc2,
+                                   bool decoupled) {
+    float *wp, *gp, *mp, *vp;
+    int64_t n, ng, nm, nv;
+    ax_status_t st;
+    if (!weight || !grad || !m || !v) return AX_ERR_NULL_ARG;
+    if ((st = as_flat(weight, "hip adam_update", &wp, &n)) || (st = as_flat(grad, "hip adam_update", &gp, &ng)) ||
+        (st = as_flat(m, "hip adam_update", &mp, &nm)) || (st = as_flat(v, "hip adam_update", &vp, &nv)))
+        return st;
+    if (ng != n || nm != n || nv != n) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "hip adam_update: element counts differ");
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    return lift(axhip_adam_update(wp, gp, mp, vp, n, lr, beta1, beta2, eps, weight_decay, bc1, bc2, decoupled ? 1 : 0),
+                "hip adam_update");
+}
+
+static ax_status_t hip_sgd_update(ax_tensor_t *weight, ax_tensor_t *grad, ax_tensor_t *momentum_buf, float lr,
+                                  float momentum, float weight_decay, bool nesterov) {
+    float *wp, *gp, *mp = NULL;
+    int64_t n, ng, nm = 0;
+    ax_status_t st;
+    if (!weight || !grad) return AX_ERR_NULL_ARG;
+    if ((st = as_flat(weight, "hip sgd_update", &wp, &n)) || (st = as_flat(grad, "hip sgd_update", &gp, &ng))) return st;
+    if (momentum_buf && (st = as_flat(momentum_buf, "hip sgd_update", &mp, &nm))) return st;
+    if (ng != n || (momentum_buf && nm != n)) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "hip sgd_update: element counts differ");
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    return lift(axhip_sgd_update(wp, gp, mp, n, lr, momentum, weight_decay, nesterov ? 1 : 0), "hip sgd_update");
+}
+
+/* x is [rows..., D] contiguous; gamma, beta are [D] */
+static ax_status_t hip_layernorm_fwd(const ax_tensor_t *x, const ax_tensor_t *gamma, const ax_tensor_t *beta, float eps,
+                                     ax_tensor_t *out, ax_tensor_t *x_hat, ax_tensor_t *inv_std) {
+    float *xp, *op, *gp, *bp, *hp = NULL, *sp = NULL;
+    int64_t n, no, ng, nb, nh = 0, ns = 0;
+    ax_status_t st;
+    if (!x || !gamma || !beta || !out) return AX_ERR_NULL_ARG;
+    if ((st = as_flat(x, "hip layernorm", &xp, &n)) || (st = as_flat(out, "hip layernorm", &op, &no)) ||
+        (st = as_flat(gamma, "hip layernorm", &gp, &ng)) || (st = as_flat(beta, "hip layernorm", &bp, &nb)))
+        return st;
+    if (x_hat && (st = as_flat(x_hat, "hip layernorm", &hp, &nh))) return st;
+    if (inv_std && (st = as_flat(inv_std, "hip layernorm", &sp, &ns))) return st;
+    if (x->ndim < 1 || x->shape[x->ndim - 1] < 1) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "hip layernorm: input needs a non-empty feature axis");
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    const int64_t cols = x->shape[x->ndim - 1], rows = n / cols;
+    if (no != n || ng != cols || nb != cols || (x_hat && nh != n) || (inv_std && ns != rows)) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "hip layernorm: operand sizes do not match [%lld, %lld]", (long long)rows,
+                   (long long)cols);
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    return lift(axhip_layernorm_fwd(xp, gp, bp, op, hp, sp, rows, cols, eps), "hip layernorm");
+}
+
 /* ---- device-owner hooks ---- */
 static ax_status_t hook_init(void) { return lift(axhip_init(), "hip init"); }
 static void hook_shutdown(void) { axhip_shutdown(); }
@@ -270,7 +497,16 @@ static ax_status_t hook_d2d(void *d, const void *s, size_t n) { return lift(axhi
 
 #define AX_HIP_OPS_INIT(dev)                                                                    \
     {                                                                                           \
-        .name = "hip", .gemm = hip_gemm, .gemm_nt = hip_gemm_nt, .gemm_tn = hip_gemm_tn,        \
+        .name = "hip", .add = hip_add, .sub = hip_sub, .mul = hip_mul, .div_op = hip_div,       \
+        .neg = hip_neg, .abs_op = hip_abs, .exp_op = hip_exp, .log_op = hip_log,                \
+        .sqrt_op = hip_sqrt, .square = hip_square, .add_scalar = hip_add_scalar,                \
+        .mul_scalar = hip_mul_scalar, .add_relu = hip_add_relu,                                 \
+        .softmax_rowwise = hip_softmax_rowwise, .mean = hip_mean, .max_op = hip_max,            \
+        .min_op = hip_min, .argmax = hip_argmax, .equal = hip_equal, .greater = hip_greater,    \
+        .sigmoid = hip_sigmoid, .tanh_op = hip_tanh, .leaky_relu = hip_leaky_relu,              \
+        .elu_op = hip_elu, .swish_op = hip_swish, .adam_update = hip_adam_update,               \
+        .sgd_update = hip_sgd_update,                                                           \
+        .gemm = hip_gemm, .gemm_nt = hip_gemm_nt, .gemm_tn = hip_gemm_tn,                       \
         .gemm_relu = hip_gemm_relu, .gemm_ex = hip_gemm_ex, .bias_add = hip_bias_add,           \
         .fill = hip_fill, .copy = hip_copy, .relu = hip_relu, .gelu_op = hip_gelu,              \
         .sum = hip_sum, .axpy = hip_axpy,                                                       \
@@ -278,6 +514,7 @@ static ax_status_t hook_d2d(void *d, const void *s, size_t n) { return lift(axhi
         .synchronize = hook_synchronize, .device_count = hook_device_count,                     \
         .storage_alloc = hook_alloc, .storage_free = hook_free, .memcpy_h2d = hook_h2d,         \
         .memcpy_d2h = hook_d2h, .memcpy_d2d = hook_d2d, .gemm_bias_act = hip_gemm_bias_act,     \
+        .layernorm_fwd = hip_layernorm_fwd,                                                     \
     }
 
 const ax_backend_ops_t ax_hip_ops = AX_HIP_OPS_INIT(AX_DEVICE_HIP);

@@ -1,6 +1,8 @@
-/* Dense / ReLU / GELU / Sequential, forward only (Axiom's src/core/layer.c:48-103, 181-300). */
+/* Dense / ReLU / GELU / LayerNorm / Sequential, forward only (Axiom's src/core/layer.c:48-103,
+ * 181-300; src/core/norm.c:1278-1455). */
 #include <stdlib.h>
 
+#include "axiom/compute.h"
 #include "axiom/init.h"
 #include "axiom/layer.h"
 #include "axiom/ops.h"
@@ -80,6 +82,65 @@ static ax_layer_t *activation_layer(ax_layer_type_t type, ax_tensor_t *(*fwd)(ax
 
 ax_layer_t *ax_relu_layer_create(void) { return activation_layer(AX_LAYER_RELU, relu_forward); }
 ax_layer_t *ax_gelu_layer_create(void) { return activation_layer(AX_LAYER_GELU, gelu_forward); }
+
+/* normalises the last axis of a 2-D or 3-D input (norm.c:1281-1298); inference: nothing saved */
+static ax_tensor_t *layernorm_forward(ax_layer_t *self, ax_tensor_t *x) {
+    ax_layernorm_t *ln = (ax_layernorm_t *)self;
+    if (!x || (x->ndim != 2 && x->ndim != 3)) return NULL;
+    if (x->shape[x->ndim - 1] != ln->num_features) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "layernorm: last axis is %lld, layer has %lld features",
+                   (long long)x->shape[x->ndim - 1], (long long)ln->num_features);
+        return NULL;
+    }
+    ax_device_t prev = ax_get_default_device();
+    ax_set_default_device(x->storage->device);
+    ax_tensor_t *out = ax_tensor_create(x->shape, x->ndim, x->dtype);
+    ax_set_default_device(prev);
+    if (!out) return NULL;
+    if (ax_compute_layernorm(x, ln->gamma, ln->beta, ln->eps, out, NULL, NULL) != AX_OK) {
+        ax_tensor_destroy(out);
+        return NULL;
+    }
+    return out;
+}
+
+static void layernorm_destroy(ax_layer_t *self) {
+    ax_layernorm_t *ln = (ax_layernorm_t *)self;
+    ax_tensor_destroy(ln->gamma);
+    ax_tensor_destroy(ln->beta);
+    free(ln);
+}
+
+ax_layer_t *ax_layernorm_create(int64_t num_features, float eps) {
+    if (num_features <= 0) {
+        ax_err_set(AX_ERR_INVALID_SHAPE, "ax_layernorm_create: features must be positive");
+        return NULL;
+    }
+    ax_layernorm_t *ln = calloc(1, sizeof *ln);
+    if (!ln) {
+        ax_err_set(AX_ERR_ALLOC, "ax_layernorm_create: out of memory");
+        return NULL;
+    }
+    ln->base.ops.forward = layernorm_forward;
+    ln->base.ops.destroy = layernorm_destroy;
+    ln->base.type = AX_LAYER_LAYERNORM;
+    ln->base.training = true;
+    ln->num_features = num_features;
+    ln->eps = eps > 0 ? eps : 1e-5f;
+    ln->gamma = ax_tensor_zeros(&num_features, 1, AX_FLOAT32);
+    ln->beta = ax_tensor_zeros(&num_features, 1, AX_FLOAT32);
+    if (!ln->gamma || !ln->beta || ax_compute_fill(ln->gamma, 1.0) != AX_OK) {
+        layernorm_destroy(&ln->base);
+        return NULL;
+    }
+    ln->gamma->requires_grad = true;
+    ln->beta->requires_grad = true;
+    ln->base.params[0] = ln->gamma;
+    ln->base.params[1] = ln->beta;
+    ln->base.n_params = 2;
+    ln->base.input_features = ln->base.output_features = num_features;
+    return &ln->base;
+}
 
 static ax_tensor_t *sequential_forward(ax_layer_t *self, ax_tensor_t *input) {
     ax_sequential_t *seq = (ax_sequential_t *)self;

@@ -229,6 +229,44 @@ def secondary(hip):
                                        "frac_of_fp32_mfma_peak": 4 * Bn * S * S * D / ms / 1e9 / PEAK_FP32_TFLOPS,
                                        "kernel": hip.last_kernel(),
                                        "unfused_us": res["fp32_batched_qkt"]["us"] + res["fp32_batched_pv"]["us"]}
+    _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sdpa_fwd(q.ptr, k.ptr, v.ptr, o.ptr, l.ptr, Bn, S, D,
+                                                                  0.125, 1)))
+    res["fp32_sdpa_fwd_causal_512x512x64"] = {"us": ms * 1e3, "useful_TFLOP/s": 2 * Bn * S * S * D / ms / 1e9,
+                                              "kernel": hip.last_kernel()}
+    del q, k, v, s, o, l
+
+    # the HBM-bound slots around the FFN (an encoder block's residual add, layer norm, softmax) and
+    # the optimizer pass: algorithmic bytes = every operand read once + every result written once
+    stream = {}
+    R, Dm = 16384, 4096                                     # 268 MB per [R, Dm] tensor
+    xa, xb = hip.array(rng.normal(0, 1, (R, Dm)).astype(np.float32)), hip.array(rng.normal(0, 1, (R, Dm)).astype(np.float32))
+    xo, vec = hip.empty((R, Dm)), hip.array(rng.normal(1, 0.1, (Dm,)).astype(np.float32))
+    rowv, colv = hip.empty((R,)), hip.empty((Dm,))
+    full = 4 * R * Dm
+    shape2 = (C.c_int64 * 2)(R, Dm)
+    dense2, bcast2 = (C.c_int64 * 2)(Dm, 1), (C.c_int64 * 2)(0, 1)
+
+    def rate(name, nbytes, fn):
+        _, ms = time_calls(hip, fn)
+        stream[name] = {"us": ms * 1e3, "GB/s": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+
+    rate("add_same_shape", 3 * full, lambda: hip.check(hip.L.axhip_binary(0, xa.ptr, xb.ptr, xo.ptr, 2, shape2, dense2, dense2)))
+    rate("add_row_vector", 2 * full, lambda: hip.check(hip.L.axhip_binary(0, xa.ptr, vec.ptr, xo.ptr, 2, shape2, dense2, bcast2)))
+    rate("tanh", 2 * full, lambda: hip.check(hip.L.axhip_unary(7, xa.ptr, xo.ptr, R * Dm, 0.0)))
+    rate("max_axis0", full, lambda: hip.check(hip.L.axhip_reduce_axis(2, xa.ptr, 1, R, Dm, colv.ptr)))
+    rate("max_axis1", full, lambda: hip.check(hip.L.axhip_reduce_axis(2, xa.ptr, R, Dm, 1, rowv.ptr)))
+    rate("sum_axis0", full, lambda: hip.check(hip.L.axhip_reduce_axis(0, xa.ptr, 1, R, Dm, colv.ptr)))
+    rate("softmax_rows_4096", 2 * full, lambda: hip.check(hip.L.axhip_softmax_rows(xa.ptr, xo.ptr, R, Dm)))
+    rate("softmax_rows_512", 2 * full, lambda: hip.check(hip.L.axhip_softmax_rows(xa.ptr, xo.ptr, R * 8, Dm // 8)))
+    rate("layernorm_4096", 2 * full, lambda: hip.check(hip.L.axhip_layernorm_fwd(xa.ptr, vec.ptr, vec.ptr, xo.ptr, None, None,
+                                                                                 R, Dm, 1e-5)))
+    rate("layernorm_1024", 2 * full, lambda: hip.check(hip.L.axhip_layernorm_fwd(xa.ptr, vec.ptr, vec.ptr, xo.ptr, None, None,
+                                                                                 R * 4, Dm // 4, 1e-5)))
+    hip.check(hip.L.axhip_fill_f32(xo.ptr, 0.0, R * Dm))
+    m2 = hip.array(np.zeros((R, Dm), np.float32))
+    rate("adam_update", 7 * full, lambda: hip.check(hip.L.axhip_adam_update(xa.ptr, xb.ptr, xo.ptr, m2.ptr, R * Dm, 1e-3, 0.9,
+                                                                            0.999, 1e-8, 0.01, 0.1, 0.001, 1)))
+    res["streaming_slots_16384x4096"] = stream
     return res
 
 

@@ -57,6 +57,39 @@ ax_status_t ax_compute_copy(const ax_tensor_t *src, ax_tensor_t *dst);
  * dBias = sum(dY, 0), and axpy to add into a gradient that already exists. */
 ax_status_t ax_compute_sum(const ax_tensor_t *in, int axis, ax_tensor_t *out);
 ax_status_t ax_compute_axpy(const ax_tensor_t *x, float alpha, ax_tensor_t *y);
+/* The remaining elementwise, reduction and optimizer wrappers (src/compute/dispatch.c:385-412,
+ * 657-721, 762-841; include/axiom/compute.h of the reference).  Binary ops broadcast (trailing
+ * dimensions aligned, extent 1 repeats); reductions take axis -1 for "everything" and want the
+ * output to hold numel(in) / shape[axis] elements; argmax writes int64. */
+ax_status_t ax_compute_add(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_sub(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_mul(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_div(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_equal(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_greater(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_add_relu(const ax_tensor_t *a, const ax_tensor_t *b, ax_tensor_t *out);
+ax_status_t ax_compute_neg(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_abs(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_exp(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_log(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_sqrt(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_square(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_sigmoid(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_tanh(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_add_scalar(const ax_tensor_t *in, double scalar, ax_tensor_t *out);
+ax_status_t ax_compute_mul_scalar(const ax_tensor_t *in, double scalar, ax_tensor_t *out);
+ax_status_t ax_compute_softmax_rowwise(const ax_tensor_t *in, ax_tensor_t *out);
+ax_status_t ax_compute_mean(const ax_tensor_t *in, int axis, ax_tensor_t *out);
+ax_status_t ax_compute_max(const ax_tensor_t *in, int axis, ax_tensor_t *out);
+ax_status_t ax_compute_min(const ax_tensor_t *in, int axis, ax_tensor_t *out);
+ax_status_t ax_compute_argmax(const ax_tensor_t *in, int axis, ax_tensor_t *out);
+ax_status_t ax_compute_adam_update(ax_tensor_t *weight, ax_tensor_t *grad, ax_tensor_t *m, ax_tensor_t *v, float lr,
+                                   float beta1, float beta2, float eps, float weight_decay, float bc1, float bc2,
+                                   bool decoupled);
+ax_status_t ax_compute_sgd_update(ax_tensor_t *weight, ax_tensor_t *grad, ax_tensor_t *momentum_buf, float lr,
+                                  float momentum, float weight_decay, bool nesterov);
+int ax_compute_has_adam_update(void);
+int ax_compute_has_sgd_update(void);
 int ax_compute_has_gemm_relu(void);
 int ax_compute_has_gemm_nt(void);
 int ax_compute_has_gemm_tn(void);
@@ -70,6 +103,16 @@ ax_status_t ax_compute_gelu(const ax_tensor_t *in, ax_tensor_t *out);
 ax_status_t ax_compute_gemm_bias_act(const ax_tensor_t *a, const ax_tensor_t *b, const ax_tensor_t *bias,
                                      ax_activation_t act, ax_tensor_t *out);
 int ax_compute_has_gemm_bias_act(void);
+/* The reference's vtable has leaky_relu / elu_op / swish_op slots (filled by its GPU backend,
+ * cuda/ops_activations.cu) but no dispatch wrapper: ax_leaky_relu, ax_elu, ax_swish
+ * (src/core/activations.c:79,141,363) loop over host pointers. */
+ax_status_t ax_compute_leaky_relu(const ax_tensor_t *in, float alpha, ax_tensor_t *out);
+ax_status_t ax_compute_elu(const ax_tensor_t *in, float alpha, ax_tensor_t *out);
+ax_status_t ax_compute_swish(const ax_tensor_t *in, ax_tensor_t *out);
+/* Layer normalisation over the last axis, the device form of the loop in layernorm_forward
+ * (src/core/norm.c:1338-1399); x_hat and inv_std (saved for backward) may be NULL. */
+ax_status_t ax_compute_layernorm(const ax_tensor_t *x, const ax_tensor_t *gamma, const ax_tensor_t *beta, float eps,
+                                 ax_tensor_t *out, ax_tensor_t *x_hat, ax_tensor_t *inv_std);
 
 #ifdef __cplusplus
 }

@@ -7,8 +7,8 @@
  * reference's offsets and tests/test_host_core.py compares them with this header.
  * Any slot may be NULL; dispatch answers AX_ERR_NOT_IMPLEMENTED for those.
  *
- * One slot is appended after the reference's last member (gemm_bias_act); the reference
- * never reads that far, this repository's dispatch layer does. */
+ * Two slots are appended after the reference's last member (gemm_bias_act, layernorm_fwd); the
+ * reference never reads that far, this repository's dispatch layer does. */
 #ifndef AX_INTERNAL_BACKEND_OPS_H
 #define AX_INTERNAL_BACKEND_OPS_H
 
@@ -26,7 +26,7 @@ typedef ax_tensor_t *ax_tout_t;          /* borrowed output, pre-allocated by th
 struct ax_backend_ops {
     const char *name;
 
-    /* broadcasting binary, unary and scalar elementwise slots — not provided by ax_hip_ops */
+    /* broadcasting binary, unary and scalar elementwise slots */
     ax_status_t (*add)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
     ax_status_t (*sub)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
     ax_status_t (*mul)(ax_tin_t a, ax_tin_t b, ax_tout_t out);
@@ -109,6 +109,11 @@ struct ax_backend_ops {
     /* ---- appended by this repository (absent from the reference's struct) ---- */
     /* out = act(a x b + bias[n]); bias may be NULL; act is an ax_activation_t */
     ax_status_t (*gemm_bias_act)(ax_tin_t a, ax_tin_t b, ax_tin_t bias, int act, ax_tout_t out);
+    /* layer normalisation over the last axis (the loop of layernorm_forward, src/core/norm.c:1338-1399,
+     * which the reference runs on host pointers): out = gamma * x_hat + beta; x_hat (shape of x) and
+     * inv_std (one value per row) are the tensors its backward pass keeps, either may be NULL */
+    ax_status_t (*layernorm_fwd)(ax_tin_t x, ax_tin_t gamma, ax_tin_t beta, float eps, ax_tout_t out,
+                                 ax_tout_t x_hat, ax_tout_t inv_std);
 };
 
 /* The MI355X backend.  `device` is AX_DEVICE_HIP. */

@@ -1,5 +1,5 @@
-/* axiom/layer.h — Dense, ReLU, GELU and Sequential, forward only (include/axiom/layer.h:30-187,
- * src/core/layer.c).  Struct layouts and enum values follow the reference.  Sequential fuses
+/* axiom/layer.h — Dense, ReLU, GELU, LayerNorm and Sequential, forward only
+ * (include/axiom/layer.h:30-187, src/core/layer.c; include/axiom/norm.h:33-44, src/core/norm.c).  Struct layouts and enum values follow the reference.  Sequential fuses
  * Dense+ReLU as the reference does (layer.c:188-230) and additionally Dense+GELU; in both
  * cases intermediates are released as soon as the next layer has consumed them. */
 #ifndef AX_LAYER_H
@@ -52,6 +52,16 @@ typedef struct {
     int n_layers;
 } ax_sequential_t;
 
+/* include/axiom/norm.h:36-42: gamma ones, beta zeros at creation; eps <= 0 means 1e-5 */
+typedef struct {
+    ax_layer_t base;
+    int64_t num_features;
+    float eps;
+    ax_tensor_t *gamma;
+    ax_tensor_t *beta;
+} ax_layernorm_t;
+
+ax_layer_t  *ax_layernorm_create(int64_t num_features, float eps);   /* input [N, D] or [B, S, D] */
 ax_layer_t  *ax_dense_create(int64_t in_features, int64_t out_features, bool use_bias);
 ax_layer_t  *ax_relu_layer_create(void);
 ax_layer_t  *ax_gelu_layer_create(void);

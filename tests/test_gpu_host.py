@@ -285,3 +285,116 @@ def test_backend_dropped_into_the_unmodified_reference(oracle):
     say(r.stdout[-3000:], r.stderr[-3000:])
     assert r.returncode == 0
     assert "DROPIN OK" in r.stdout
+
+
+def test_elementwise_reduction_optimizer_slots(ax, oracle, golden):
+    """The remaining vtable slots through the ax_compute_* wrappers on device tensors, against the
+    reference vectors (inputs regenerated from their seeds) and the CPU restatement."""
+    import slot_cases as sc
+    L = ax.L
+    # broadcasting binaries: bit-exact
+    for case in range(len(sc.BCAST)):
+        a, b = sc.binary_inputs(oracle, case)
+        ta, tb = ax.from_numpy(a), ax.from_numpy(b)
+        out = ax.empty(np.broadcast_shapes(a.shape, b.shape))
+        for name in sc.BINARY:
+            assert getattr(L, "ax_compute_" + name)(ta, tb, out) == 0, ax.err()
+            assert np.array_equal(ax.to_numpy(out), golden[f"bin_{name}_{case}"], equal_nan=True), (name, case)
+        if a.shape == b.shape:
+            assert L.ax_compute_add_relu(ta, tb, out) == 0
+            assert np.array_equal(ax.to_numpy(out), golden[f"bin_add_relu_{case}"])
+        ax.free(ta, tb, out)
+    # a strided operand: the transpose view [K, M] of an [M, K] tensor, added to a contiguous [K, M]
+    oracle.seed(77)
+    m = oracle.uniform((6, 10), -1, 1)
+    tm, tn = ax.from_numpy(m), ax.from_numpy(np.ascontiguousarray(m.T) * 2)
+    view = ax.from_numpy(m)
+    v = view.contents
+    v.shape[0], v.shape[1], v.strides[0], v.strides[1] = 10, 6, 1, 10
+    out = ax.empty((10, 6))
+    assert L.ax_compute_add(view, tn, out) == 0 and np.array_equal(ax.to_numpy(out), m.T + 2 * m.T)
+    bad = ax.empty((7, 6))
+    assert L.ax_compute_add(tm, tn, bad) == 3                      # [6,10] does not broadcast to [7,6]
+    v.shape[0], v.shape[1], v.strides[0], v.strides[1] = 6, 10, 10, 1
+    ax.free(tm, tn, view, out, bad)
+    # unary / scalar / activation slots
+    x = sc.unary_input(oracle)
+    tx, out = ax.from_numpy(x), ax.empty(x.shape)
+    calls = {"neg": (L.ax_compute_neg,), "abs": (L.ax_compute_abs,), "exp": (L.ax_compute_exp,),
+             "log": (L.ax_compute_log,), "sqrt": (L.ax_compute_sqrt,), "square": (L.ax_compute_square,),
+             "sigmoid": (L.ax_compute_sigmoid,), "tanh": (L.ax_compute_tanh,), "swish": (L.ax_compute_swish,),
+             "leaky_relu": (L.ax_compute_leaky_relu, 0.1), "elu": (L.ax_compute_elu, 0.7),
+             "add_scalar": (L.ax_compute_add_scalar, 0.37), "mul_scalar": (L.ax_compute_mul_scalar, -1.7)}
+    for name, call in calls.items():
+        st = call[0](tx, out) if len(call) == 1 else call[0](tx, call[1], out)
+        assert st == 0, (name, ax.err())
+        ref = golden[f"un_{name}"]
+        assert (np.abs(ax.to_numpy(out) - ref) <= 1e-6 * np.maximum(np.abs(ref), 1)).all(), name
+    assert ax.to_numpy(out).shape == x.shape
+    ax.free(tx, out)
+    # reductions (int64 argmax through a tensor of that dtype)
+    for shp, arr in zip(sc.REDUCE_SHAPES, sc.reduce_inputs(oracle)):
+        tag = "x".join(map(str, shp))
+        t = ax.from_numpy(arr)
+        for axis in range(-1, len(shp)):
+            oshape = (1,) if axis == -1 else shp[:axis] + shp[axis + 1:]
+            out = ax.empty(oshape)
+            for name in ("mean", "max", "min"):
+                assert getattr(L, "ax_compute_" + name)(t, axis, out) == 0, ax.err()
+                assert np.abs(ax.to_numpy(out) - golden[f"red_{name}_{tag}_axis{axis}_naive"]).max() < 2e-6
+            sh, nd = ax.shape_arg(oshape)
+            L.ax_set_default_device(2)
+            idx = L.ax_tensor_create(sh, nd, 3)                    # AX_INT64
+            assert L.ax_compute_argmax(t, axis, idx) == 0, ax.err()
+            got = np.empty(oshape, np.int64)
+            assert L.ax_tensor_read(idx, got.ctypes.data, got.nbytes) == 0
+            assert np.array_equal(got, golden[f"red_argmax_{tag}_axis{axis}"])
+            assert L.ax_compute_argmax(t, axis, out) == 4          # AX_ERR_DTYPE_MISMATCH: float output
+            ax.free(out, idx)
+        assert L.ax_compute_max(t, len(shp), t) == 5               # AX_ERR_INVALID_AXIS
+        ax.free(t)
+    # softmax_rowwise and its shape rule
+    for (rows, cols), arr in zip(sc.SOFTMAX_SHAPES, sc.softmax_inputs(oracle)):
+        t, out = ax.from_numpy(arr), ax.empty((rows, cols))
+        assert L.ax_compute_softmax_rowwise(t, out) == 0
+        assert np.abs(ax.to_numpy(out) - golden[f"softmax_{rows}x{cols}_naive"]).max() < 1e-6
+        ax.free(t, out)
+    t3, o3 = ax.from_numpy(np.zeros((2, 3, 4), np.float32)), ax.empty((2, 3, 4))
+    assert L.ax_compute_softmax_rowwise(t3, o3) == 3
+    ax.free(t3, o3)
+    # the LayerNorm layer: gamma ones / beta zeros at creation, then the reference's vectors
+    for shp, (xv, gamma, beta) in zip(sc.LAYERNORM_SHAPES, sc.layernorm_inputs(oracle)):
+        ln = L.ax_layernorm_create(shp[-1], 1e-5)
+        from axiom_amd.axiom import TP
+        params = (TP * 4)()
+        assert L.ax_layer_get_params(ln, params, 4) == 2
+        assert np.array_equal(ax.to_numpy(params[0]), np.ones(shp[-1], np.float32))
+        assert np.array_equal(ax.to_numpy(params[1]), np.zeros(shp[-1], np.float32))
+        for prm, val in zip(params, (gamma, beta)):
+            tv_ = ax.from_numpy(val)
+            assert L.ax_compute_copy(tv_, prm) == 0
+            ax.free(tv_)
+        t = ax.from_numpy(xv)
+        y = L.ax_layer_forward(ln, t)
+        assert y, ax.err()
+        assert np.abs(ax.to_numpy(y) - golden["layernorm_" + "x".join(map(str, shp))]).max() < 5e-6
+        ax.free(t, y)
+        L.ax_layer_destroy(ln)
+    # optimizer slots over three steps
+    assert L.ax_compute_has_adam_update() == 1 and L.ax_compute_has_sgd_update() == 1
+    w0, grads = sc.optimizer_inputs(oracle)
+    for key, (kind, kw) in sc.OPTIMIZERS.items():
+        tw, tm_, tv = ax.from_numpy(w0), ax.from_numpy(np.zeros_like(w0)), ax.from_numpy(np.zeros_like(w0))
+        for step, g in enumerate(grads, 1):
+            tg = ax.from_numpy(g)
+            if kind == "sgd":
+                st = L.ax_compute_sgd_update(tw, tg, tm_ if kw["momentum"] > 0 else None, kw["lr"], kw["momentum"],
+                                             kw["wd"], kw["nesterov"])
+            else:
+                bc1, bc2 = sc.bias_corrections(kw["beta1"], kw["beta2"], step)
+                st = L.ax_compute_adam_update(tw, tg, tm_, tv, kw["lr"], kw["beta1"], kw["beta2"], kw["eps"], kw["wd"],
+                                              bc1, bc2, kind == "adamw")
+            assert st == 0, ax.err()
+            assert np.abs(ax.to_numpy(tw) - golden[key][step - 1]).max() < 2e-6, (key, step)
+            ax.free(tg)
+        ax.free(tw, tm_, tv)
