@@ -68,6 +68,17 @@ SIGNATURES = {
     "ax_compute_has_adam_update": (C.c_int, []), "ax_compute_has_sgd_update": (C.c_int, []),
     "ax_compute_layernorm": (C.c_int, [TP, TP, TP, C.c_float, TP, TP, TP]),
     "ax_layernorm_create": (C.c_void_p, [C.c_int64, C.c_float]),
+    "ax_sigmoid_layer_create": (C.c_void_p, []), "ax_tanh_layer_create": (C.c_void_p, []),
+    "ax_swish_layer_create": (C.c_void_p, []), "ax_leaky_relu_layer_create": (C.c_void_p, [C.c_float]),
+    "ax_elu_layer_create": (C.c_void_p, [C.c_float]), "ax_softmax_layer_create": (C.c_void_p, [C.c_int]),
+    "ax_sigmoid": (TP, [TP]), "ax_tanh_op": (TP, [TP]), "ax_swish": (TP, [TP]),
+    "ax_leaky_relu": (TP, [TP, C.c_float]), "ax_elu": (TP, [TP, C.c_float]), "ax_softmax": (TP, [TP, C.c_int]),
+    "ax_tensor_write": (C.c_int, [TP, C.c_void_p, C.c_size_t]),
+    "ax_model_create": (C.c_void_p, [C.c_void_p]), "ax_model_predict": (TP, [C.c_void_p, TP]),
+    "ax_model_destroy": (None, [C.c_void_p]),
+    "ax_model_save": (C.c_int, [C.c_void_p, C.c_char_p]), "ax_model_load": (C.c_void_p, [C.c_char_p]),
+    "ax_tensor_save": (C.c_int, [TP, C.c_char_p]), "ax_tensor_load": (TP, [C.c_char_p]),
+    "ax_qweight_save": (C.c_int, [QP, C.c_char_p]), "ax_qweight_load": (QP, [C.c_char_p]),
     "ax_compute_gemm_bias_act": (C.c_int, [TP, TP, TP, C.c_int, TP]),
     "ax_compute_has_gemm_relu": (C.c_int, []), "ax_compute_has_gemm_nt": (C.c_int, []),
     "ax_compute_has_gemm_tn": (C.c_int, []), "ax_compute_has_gemm_ex": (C.c_int, []),

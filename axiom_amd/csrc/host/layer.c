@@ -65,23 +65,52 @@ ax_layer_t *ax_dense_create(int64_t in_features, int64_t out_features, bool use_
 
 static ax_tensor_t *relu_forward(ax_layer_t *self, ax_tensor_t *x) { (void)self; return ax_relu(x); }
 static ax_tensor_t *gelu_forward(ax_layer_t *self, ax_tensor_t *x) { (void)self; return ax_gelu(x); }
+static ax_tensor_t *sigmoid_forward(ax_layer_t *self, ax_tensor_t *x) { (void)self; return ax_sigmoid(x); }
+static ax_tensor_t *tanh_forward(ax_layer_t *self, ax_tensor_t *x) { (void)self; return ax_tanh_op(x); }
+static ax_tensor_t *swish_forward(ax_layer_t *self, ax_tensor_t *x) { (void)self; return ax_swish(x); }
+static ax_tensor_t *leaky_relu_forward(ax_layer_t *self, ax_tensor_t *x) {
+    return ax_leaky_relu(x, ((ax_activation_layer_t *)self)->alpha);
+}
+static ax_tensor_t *elu_forward(ax_layer_t *self, ax_tensor_t *x) { return ax_elu(x, ((ax_activation_layer_t *)self)->alpha); }
+static ax_tensor_t *softmax_forward(ax_layer_t *self, ax_tensor_t *x) {
+    return ax_softmax(x, ((ax_activation_layer_t *)self)->axis);
+}
 static void plain_destroy(ax_layer_t *self) { free(self); }
 
+/* layer.c:136-174 */
 static ax_layer_t *activation_layer(ax_layer_type_t type, ax_tensor_t *(*fwd)(ax_layer_t *, ax_tensor_t *)) {
-    ax_layer_t *l = calloc(1, sizeof *l);
+    ax_activation_layer_t *l = calloc(1, sizeof *l);
     if (!l) {
         ax_err_set(AX_ERR_ALLOC, "activation layer: out of memory");
         return NULL;
     }
-    l->ops.forward = fwd;
-    l->ops.destroy = plain_destroy;
-    l->type = type;
-    l->training = true;
-    return l;
+    l->base.ops.forward = fwd;
+    l->base.ops.destroy = plain_destroy;
+    l->base.type = type;
+    l->base.training = true;
+    return &l->base;
 }
 
 ax_layer_t *ax_relu_layer_create(void) { return activation_layer(AX_LAYER_RELU, relu_forward); }
 ax_layer_t *ax_gelu_layer_create(void) { return activation_layer(AX_LAYER_GELU, gelu_forward); }
+ax_layer_t *ax_sigmoid_layer_create(void) { return activation_layer(AX_LAYER_SIGMOID, sigmoid_forward); }
+ax_layer_t *ax_tanh_layer_create(void) { return activation_layer(AX_LAYER_TANH, tanh_forward); }
+ax_layer_t *ax_swish_layer_create(void) { return activation_layer(AX_LAYER_SWISH, swish_forward); }
+ax_layer_t *ax_leaky_relu_layer_create(float alpha) {
+    ax_layer_t *l = activation_layer(AX_LAYER_LEAKY_RELU, leaky_relu_forward);
+    if (l) ((ax_activation_layer_t *)l)->alpha = alpha;
+    return l;
+}
+ax_layer_t *ax_elu_layer_create(float alpha) {
+    ax_layer_t *l = activation_layer(AX_LAYER_ELU, elu_forward);
+    if (l) ((ax_activation_layer_t *)l)->alpha = alpha;
+    return l;
+}
+ax_layer_t *ax_softmax_layer_create(int axis) {
+    ax_layer_t *l = activation_layer(AX_LAYER_SOFTMAX, softmax_forward);
+    if (l) ((ax_activation_layer_t *)l)->axis = axis;
+    return l;
+}
 
 /* normalises the last axis of a 2-D or 3-D input (norm.c:1281-1298); inference: nothing saved */
 static ax_tensor_t *layernorm_forward(ax_layer_t *self, ax_tensor_t *x) {
@@ -129,7 +158,13 @@ ax_layer_t *ax_layernorm_create(int64_t num_features, float eps) {
     ln->eps = eps > 0 ? eps : 1e-5f;
     ln->gamma = ax_tensor_zeros(&num_features, 1, AX_FLOAT32);
     ln->beta = ax_tensor_zeros(&num_features, 1, AX_FLOAT32);
-    if (!ln->gamma || !ln->beta || ax_compute_fill(ln->gamma, 1.0) != AX_OK) {
+    bool ok = ln->gamma && ln->beta;
+    if (ok && ln->gamma->storage->device == AX_DEVICE_CPU) {
+        for (int64_t i = 0; i < num_features; i++) ((float *)ln->gamma->storage->data)[i] = 1.0f;
+    } else if (ok) {
+        ok = ax_compute_fill(ln->gamma, 1.0) == AX_OK;
+    }
+    if (!ok) {
         layernorm_destroy(&ln->base);
         return NULL;
     }

@@ -97,3 +97,54 @@ static ax_tensor_t *unary(ax_tensor_t *a, ax_status_t (*op)(const ax_tensor_t *,
 
 ax_tensor_t *ax_relu(ax_tensor_t *a) { return unary(a, ax_compute_relu, "relu"); }
 ax_tensor_t *ax_gelu(ax_tensor_t *a) { return unary(a, ax_compute_gelu, "gelu"); }
+ax_tensor_t *ax_sigmoid(ax_tensor_t *a) { return unary(a, ax_compute_sigmoid, "sigmoid"); }
+ax_tensor_t *ax_tanh_op(ax_tensor_t *a) { return unary(a, ax_compute_tanh, "tanh"); }
+ax_tensor_t *ax_swish(ax_tensor_t *a) { return unary(a, ax_compute_swish, "swish"); }
+
+static ax_tensor_t *unary_alpha(ax_tensor_t *a, float alpha,
+                                ax_status_t (*op)(const ax_tensor_t *, float, ax_tensor_t *), const char *who) {
+    if (!a) {
+        ax_err_set(AX_ERR_NULL_ARG, "%s: NULL tensor", who);
+        return NULL;
+    }
+    if (a->dtype != AX_FLOAT32) {
+        ax_err_set(AX_ERR_DTYPE_MISMATCH, "%s only supports float32", who);
+        return NULL;
+    }
+    ax_tensor_t *out = alloc_like_device(a, a->shape, a->ndim);
+    if (!out) return NULL;
+    if (op(a, alpha, out) != AX_OK) {
+        ax_tensor_destroy(out);
+        return NULL;
+    }
+    return out;
+}
+
+ax_tensor_t *ax_leaky_relu(ax_tensor_t *a, float alpha) { return unary_alpha(a, alpha, ax_compute_leaky_relu, "leaky_relu"); }
+ax_tensor_t *ax_elu(ax_tensor_t *a, float alpha) { return unary_alpha(a, alpha, ax_compute_elu, "elu"); }
+
+/* softmax over the last axis: the rows of the tensor viewed as [numel / last, last] */
+ax_tensor_t *ax_softmax(ax_tensor_t *a, int axis) {
+    if (!a || a->dtype != AX_FLOAT32 || a->ndim < 1) {
+        ax_err_set(AX_ERR_NULL_ARG, "softmax: needs a float32 tensor");
+        return NULL;
+    }
+    if (axis == -1) axis = a->ndim - 1;
+    if (axis != a->ndim - 1) {
+        ax_err_set(AX_ERR_NOT_IMPLEMENTED, "softmax: only the last axis is supported");
+        return NULL;
+    }
+    const int64_t cols = a->shape[a->ndim - 1];
+    int64_t flat[2] = {cols ? ax_tensor_numel(a) / cols : 0, cols};
+    ax_tensor_t *a2 = ax_tensor_reshape(a, flat, 2);
+    ax_tensor_t *out = a2 ? alloc_like_device(a, flat, 2) : NULL;
+    ax_status_t st = out ? ax_compute_softmax_rowwise(a2, out) : AX_ERR_ALLOC;
+    if (a2) ax_tensor_destroy(a2);
+    if (st != AX_OK) {
+        ax_tensor_destroy(out);
+        return NULL;
+    }
+    ax_tensor_t *view = ax_tensor_reshape(out, a->shape, a->ndim);
+    ax_tensor_destroy(out);
+    return view;
+}

@@ -212,6 +212,20 @@ ax_tensor_t *ax_tensor_reshape(ax_tensor_t *t, const int64_t *new_shape, int new
     return v;
 }
 
+ax_status_t ax_tensor_write(ax_tensor_t *t, const void *host_src, size_t bytes) {
+    if (!t || !t->storage || !host_src) {
+        ax_err_set(AX_ERR_NULL_ARG, "tensor_write: NULL");
+        return AX_ERR_NULL_ARG;
+    }
+    if (!ax_tensor_is_contiguous(t) || bytes > (size_t)ax_tensor_numel(t) * ax_dtype_size(t->dtype)) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "tensor_write: non-contiguous tensor or too many bytes");
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    ax_status_t st = write_from_host(t, host_src, bytes);
+    if (st == AX_OK) t->storage->generation++;
+    return st;
+}
+
 ax_status_t ax_tensor_read(const ax_tensor_t *t, void *host_dst, size_t bytes) {
     if (!t || !host_dst) {
         ax_err_set(AX_ERR_NULL_ARG, "tensor_read: NULL");

@@ -1,4 +1,5 @@
-/* axiom/axiom.h — master include of the GEMM-path subset of the Axiom C API. */
+/* axiom/axiom.h — master include of the GEMM-path subset of the Axiom C API (plus layers, model
+ * container and model files around it). */
 #ifndef AXIOM_H
 #define AXIOM_H
 #include "compute.h"
@@ -6,9 +7,11 @@
 #include "error.h"
 #include "init.h"
 #include "layer.h"
+#include "model.h"
 #include "ops.h"
 #include "quantize.h"
 #include "rng.h"
+#include "serialize.h"
 #include "tensor.h"
 #include "types.h"
 #ifdef __cplusplus

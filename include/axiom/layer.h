@@ -63,8 +63,22 @@ typedef struct {
 
 ax_layer_t  *ax_layernorm_create(int64_t num_features, float eps);   /* input [N, D] or [B, S, D] */
 ax_layer_t  *ax_dense_create(int64_t in_features, int64_t out_features, bool use_bias);
+/* include/axiom/layer.h:120-141: stateless activation layers; the struct is public so that the
+ * model file code can reach alpha / axis */
+typedef struct {
+    ax_layer_t base;
+    float alpha;             /* leaky relu, elu */
+    int axis;                /* softmax */
+} ax_activation_layer_t;
+
 ax_layer_t  *ax_relu_layer_create(void);
+ax_layer_t  *ax_sigmoid_layer_create(void);
+ax_layer_t  *ax_tanh_layer_create(void);
+ax_layer_t  *ax_leaky_relu_layer_create(float alpha);
+ax_layer_t  *ax_elu_layer_create(float alpha);
 ax_layer_t  *ax_gelu_layer_create(void);
+ax_layer_t  *ax_swish_layer_create(void);
+ax_layer_t  *ax_softmax_layer_create(int axis);
 ax_layer_t  *ax_sequential_create(void);
 ax_layer_t  *ax_sequential_add(ax_layer_t *seq, ax_layer_t *layer);   /* NULL when full */
 ax_tensor_t *ax_layer_forward(ax_layer_t *layer, ax_tensor_t *input);

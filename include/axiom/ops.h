@@ -1,4 +1,4 @@
-/* axiom/ops.h — tensor-level matmul family and the two activations of the path
+/* axiom/ops.h — tensor-level matmul family and the activations
  * (include/axiom/ops.h, src/core/ops.c:285-440; activations.c).  Each returns a new tensor on
  * the inputs' device (NULL + ax_err on failure).  Inference only: no grad_fn is attached.
  *
@@ -17,6 +17,13 @@ ax_tensor_t *ax_matmul_bias_relu(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bi
 ax_tensor_t *ax_matmul_bias_gelu(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bias); /* not in the reference */
 ax_tensor_t *ax_relu(ax_tensor_t *a);
 ax_tensor_t *ax_gelu(ax_tensor_t *a);                                                /* tanh form */
+/* src/core/ops.c:509-537, src/core/activations.c:79,141,363,598 — on the tensor's device */
+ax_tensor_t *ax_sigmoid(ax_tensor_t *a);
+ax_tensor_t *ax_tanh_op(ax_tensor_t *a);
+ax_tensor_t *ax_leaky_relu(ax_tensor_t *a, float alpha);
+ax_tensor_t *ax_elu(ax_tensor_t *a, float alpha);
+ax_tensor_t *ax_swish(ax_tensor_t *a);
+ax_tensor_t *ax_softmax(ax_tensor_t *a, int axis);   /* last axis only (-1 or ndim-1), as the reference */
 #ifdef __cplusplus
 }
 #endif

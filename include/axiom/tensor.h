@@ -64,6 +64,9 @@ ax_tensor_t *ax_tensor_to_device(ax_tensor_t *t, ax_device_t dev);   /* contiguo
 ax_tensor_t *ax_tensor_to_cpu(ax_tensor_t *t);
 /* copy a contiguous tensor's elements to host memory, whatever device holds them */
 ax_status_t  ax_tensor_read(const ax_tensor_t *t, void *host_dst, size_t bytes);
+/* the reverse: fill a contiguous tensor from host memory (what the model loader uses to place
+ * parameters on a device; the reference's loader memcpy()s into host storage, serialize.c:690) */
+ax_status_t  ax_tensor_write(ax_tensor_t *t, const void *host_src, size_t bytes);
 
 #ifdef __cplusplus
 }

@@ -197,6 +197,75 @@ G["opt_sgd_plain"] = np.stack(r.optimizer_steps("sgd", w0, grads, lr=5e-2, momen
 G["opt_sgd_momentum"] = np.stack(r.optimizer_steps("sgd", w0, grads, lr=5e-2, momentum=0.9, wd=0.01, nesterov=False))
 G["opt_sgd_nesterov"] = np.stack(r.optimizer_steps("sgd", w0, grads, lr=5e-2, momentum=0.9, wd=0.01, nesterov=True))
 
+# ---- model files written by the reference (src/core/serialize.c) ------------------------------
+import ctypes as C  # noqa: E402
+
+for name in ("ax_relu_layer_create", "ax_sigmoid_layer_create", "ax_tanh_layer_create", "ax_gelu_layer_create",
+             "ax_swish_layer_create", "ax_flatten_create"):
+    getattr(L, name).restype = C.c_void_p
+    getattr(L, name).argtypes = []
+for name in ("ax_leaky_relu_layer_create", "ax_elu_layer_create"):
+    getattr(L, name).restype = C.c_void_p
+    getattr(L, name).argtypes = [C.c_float]
+L.ax_softmax_layer_create.restype = C.c_void_p
+L.ax_softmax_layer_create.argtypes = [C.c_int]
+L.ax_model_create.restype = C.c_void_p
+L.ax_model_create.argtypes = [C.c_void_p]
+L.ax_model_save.argtypes = [C.c_void_p, C.c_char_p]
+L.ax_model_destroy.argtypes = [C.c_void_p]
+L.ax_tensor_save.argtypes = [C.POINTER(type(r.empty(1).contents)), C.c_char_p]
+
+
+def ref_model(tag, layers, in_shape, seed):
+    """Builds a Sequential in the reference, perturbs every parameter, saves it and records the
+    reference's CPU forward of a seeded input."""
+    L.ax_set_seed(seed)
+    seq = L.ax_sequential_create()
+    for make in layers:
+        assert L.ax_sequential_add(seq, make())
+    params = (C.POINTER(type(r.empty(1).contents)) * 64)()
+    n = L.ax_layer_get_params(seq, params, 64)
+    L.ax_rng_seed(seed + 1)
+    for i in range(n):                                   # biases / gamma / beta away from 0 and 1
+        t = params[i].contents
+        cnt = int(np.prod([t.shape[d] for d in range(t.ndim)]))
+        buf = (C.c_float * cnt).from_address(t.storage.contents.data)
+        if t.ndim == 1:
+            buf[:] = list(np.frombuffer(buf, np.float32) + ref_uniform(cnt, -0.5, 0.5))
+    x = ref_uniform(int(np.prod(in_shape)), -1.0, 1.0).reshape(in_shape)
+    r.backend(1)
+    tx = r.tensor(x)
+    y = L.ax_layer_forward(seq, tx)
+    G[f"axm_{tag}_out"] = r.numpy(y)
+    r.free(tx, y)
+    model = L.ax_model_create(seq)
+    assert L.ax_model_save(model, os.path.join(HERE, f"ref_{tag}.axm").encode()) == 0
+    L.ax_model_destroy(model)
+
+
+ref_model("mlp", [lambda: L.ax_dense_create(12, 20, True), L.ax_relu_layer_create,
+                  lambda: L.ax_layernorm_create(20, 1e-5), lambda: L.ax_dense_create(20, 6, False),
+                  lambda: L.ax_leaky_relu_layer_create(0.1), lambda: L.ax_softmax_layer_create(1)], (5, 12), 8100)
+# a Dense that is not followed by ReLU carries no bias here: the reference's unfused path hands its
+# bias to bias_add with axis 0 (src/core/ops.c:357), which rejects it or adds it down the rows, so
+# its outputs for such layers are not the layer's definition
+ref_model("ffn", [lambda: L.ax_layernorm_create(64, 1e-5), lambda: L.ax_dense_create(64, 256, False),
+                  L.ax_gelu_layer_create, lambda: L.ax_dense_create(256, 64, False)], (2, 7, 64), 8200)
+ref_model("acts", [lambda: L.ax_dense_create(9, 9, False), L.ax_sigmoid_layer_create, L.ax_tanh_layer_create,
+                   lambda: L.ax_elu_layer_create(0.7), L.ax_swish_layer_create], (4, 9), 8300)
+# a file whose first layer has no forward pass in the port: it must be refused, not misread
+L.ax_set_seed(8400)
+seq = L.ax_sequential_create()
+L.ax_sequential_add(seq, L.ax_flatten_create())
+L.ax_sequential_add(seq, L.ax_dense_create(4, 3, True))
+model = L.ax_model_create(seq)
+assert L.ax_model_save(model, os.path.join(HERE, "ref_flatten.axm").encode()) == 0
+L.ax_model_destroy(model)
+L.ax_rng_seed(8500)
+tt = r.tensor(ref_uniform(3 * 4 * 5, -1.0, 1.0).reshape(3, 4, 5))
+assert L.ax_tensor_save(tt, os.path.join(HERE, "ref_tensor.axt").encode()) == 0
+r.free(tt)
+
 np.savez_compressed(os.path.join(HERE, "golden.npz"), **G)
 print("wrote", len(G), "arrays,", os.path.getsize(os.path.join(HERE, "golden.npz")), "bytes")
 

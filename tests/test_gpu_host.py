@@ -398,3 +398,39 @@ def test_elementwise_reduction_optimizer_slots(ax, oracle, golden):
             assert np.abs(ax.to_numpy(tw) - golden[key][step - 1]).max() < 2e-6, (key, step)
             ax.free(tg)
         ax.free(tw, tm_, tv)
+
+
+@pytest.mark.parametrize("tag,in_shape,seed", [("mlp", (5, 12), 8100), ("ffn", (2, 7, 64), 8200), ("acts", (4, 9), 8300)])
+def test_reference_model_file_runs_on_device(ax, oracle, golden, tag, in_shape, seed, tmp_path):
+    """A model the reference built, initialised and saved (tests/golden/ref_*.axm) is loaded onto
+    the GPU, reproduces the reference's CPU forward of the same input, and is written back from
+    device memory byte for byte."""
+    L = ax.L
+    path = os.path.join(ROOT, "tests", "golden", f"ref_{tag}.axm")
+    L.ax_set_default_device(2)
+    model = L.ax_model_load(path.encode())
+    assert model, ax.err()
+    from axiom_amd.axiom import TP
+    params = (TP * 64)()
+    net = C.cast(model, C.POINTER(C.c_void_p))[0]
+    n = L.ax_layer_get_params(net, params, 64)
+    assert n > 0 and all(params[i].contents.storage.contents.device == 2 for i in range(n))
+    # the input the generator drew: parameters' perturbations first, then x, from seed + 1
+    oracle.seed(seed + 1)
+    for i in range(n):
+        t = params[i].contents
+        if t.ndim == 1:
+            oracle.uniform((t.shape[0],), -0.5, 0.5)
+    x = oracle.uniform(in_shape, -1.0, 1.0)
+    tx = ax.from_numpy(x)
+    y = L.ax_model_predict(model, tx)
+    assert y, ax.err()
+    want = golden[f"axm_{tag}_out"]
+    got = ax.to_numpy(y)
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max()), np.abs(got - want).max()
+    out = tmp_path / "from_device.axm"
+    assert L.ax_model_save(model, str(out).encode()) == 0, ax.err()
+    assert out.read_bytes() == open(path, "rb").read()
+    ax.free(tx, y)
+    L.ax_model_destroy(model)
