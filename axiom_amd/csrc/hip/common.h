@@ -62,6 +62,23 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     tn = in_band / rows;
 }
 
+// The same for a batched launch with grid (tiles, batch): the hardware numbers workgroups x
+// fastest, so workgroup lin = x + tiles * y lands on XCD lin % 8.  Eight batch entries form a
+// group; inside a group workgroup r works on entry r % 8 and tile r / 8, so every tile of one
+// batch entry runs on the same XCD, back to back, and that entry's operands are fetched into one
+// L2 only (a partial last group of `left` entries uses r % left, r / left).
+__device__ __forceinline__ void tile_of_batched_block(int tiles_m, int tiles_n, int &tm, int &tn, int64_t &batch) {
+    const int64_t tiles = (int64_t)tiles_m * tiles_n, entries = gridDim.y;
+    const int64_t lin = blockIdx.x + tiles * blockIdx.y;
+    const int64_t group = lin / (8 * tiles), r = lin - group * 8 * tiles;
+    const int64_t left = entries - group * 8, per = left < 8 ? left : 8;
+    batch = group * 8 + r % per;
+    const int tile = (int)(r / per);
+    // consecutive workgroups walk along a tile row: their write-backs fill whole output rows
+    tm = tile / tiles_n;
+    tn = tile - tm * tiles_n;
+}
+
 // Write-back of one 32x32 MFMA result tile held in the layout "lane l owns row (l & 31), and
 // for g = 0..3 the four consecutive columns 8*g + 4*(l >> 5) + e": the wave turns the tile
 // through 4 KiB of LDS private to it so that each store instruction writes 8 rows of 128

@@ -125,9 +125,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm(SgemmArgs g) {
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int tiles_m = (int)((g.M + BM - 1) / BM), tiles_n = (int)((g.N + BN - 1) / BN);
     int tm, tn;
-    tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    int64_t batch = 0;
+    if (gridDim.y == 1) tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    else tile_of_batched_block(tiles_m, tiles_n, tm, tn, batch);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
-    const int64_t batch = blockIdx.y;
     const float *A = static_cast<const float *>(g.A) + batch * g.stride_a;
     const BSRC *B = static_cast<const BSRC *>(g.B) + batch * g.stride_b;
     float *C = g.C + batch * g.stride_c;
@@ -359,9 +360,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     const int wk = wave / (WAVES_M * WAVES_N), wmn = wave % (WAVES_M * WAVES_N);
     const int wm = wmn / WAVES_N, wn = wmn % WAVES_N;
     int tm, tn;
-    tile_of_block(blockIdx.x, (int)(g.M / BM), (int)(g.N / BN), tm, tn);
+    int64_t batch = 0;
+    if (gridDim.y == 1) tile_of_block(blockIdx.x, (int)(g.M / BM), (int)(g.N / BN), tm, tn);
+    else tile_of_batched_block((int)(g.M / BM), (int)(g.N / BN), tm, tn, batch);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
-    const int64_t batch = blockIdx.y;
     const float *A = static_cast<const float *>(g.A) + batch * g.stride_a;
     const float *B = static_cast<const float *>(g.B) + batch * g.stride_b;
     float *C = g.C + batch * g.stride_c;

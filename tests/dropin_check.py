@@ -165,5 +165,66 @@ for (M, K, N) in [(48, 40, 24), (256, 512, 384)]:
         assert np.abs(g - r_).max() <= 1e-4 * np.abs(r_).max(), (name, M, K, N)
     print("dense backward", M, K, N, "ok", flush=True)
 
+# 4. the reference's tensor-level ops (src/core/ops.c:107-283, 444-537) on device tensors: each
+#    allocates its result through our storage hooks and dispatches to our elementwise / reduction slots
+for name in ("ax_add", "ax_sub", "ax_mul", "ax_div"):
+    getattr(L, name).restype = TP
+    getattr(L, name).argtypes = [TP, TP]
+for name in ("ax_neg", "ax_exp", "ax_square", "ax_sigmoid", "ax_tanh_op", "ax_relu"):
+    getattr(L, name).restype = TP
+    getattr(L, name).argtypes = [TP]
+for name in ("ax_sum", "ax_mean", "ax_max", "ax_min"):
+    getattr(L, name).restype = TP
+    getattr(L, name).argtypes = [TP, C.c_int]
+
+
+def run_ops(a, b):
+    ta, tb = (L.ax_tensor_from_array(v.ctypes.data, (i64 * v.ndim)(*v.shape), v.ndim, 0) for v in (a, b))
+    outs = {}
+    for name in ("ax_add", "ax_sub", "ax_mul", "ax_div"):
+        outs[name] = getattr(L, name)(ta, tb)
+    for name in ("ax_neg", "ax_exp", "ax_square", "ax_sigmoid", "ax_tanh_op", "ax_relu"):
+        outs[name] = getattr(L, name)(ta)
+    for name in ("ax_sum", "ax_mean", "ax_max", "ax_min"):
+        for axis in (-1, 0, 1, 2):
+            outs[f"{name}{axis}"] = getattr(L, name)(ta, axis)
+    res = {}
+    for k, t in outs.items():
+        assert t, (k, L.ax_err_last_message())
+        res[k] = fetch(t) if t.contents.storage.contents.device != 0 else ref.numpy(t)
+        ref.free(t)
+    ref.free(ta, tb)
+    return res
+
+
+a = rng.uniform(-2, 2, (6, 5, 32)).astype(np.float32)
+b = rng.uniform(0.5, 2, (5, 1)).astype(np.float32)
+L.ax_no_grad()
+on_cpu()
+want = run_ops(a, b)
+on_gpu()
+got = run_ops(a, b)
+for k in want:
+    assert got[k].shape == want[k].shape, k
+    assert np.abs(got[k] - want[k]).max() <= 2e-5 * max(1.0, np.abs(want[k]).max()), k
+print("tensor ops ok:", len(want), flush=True)
+
+# 5. the reference's optimizers (src/core/optim.c): with a parameter on the device, sgd_step and
+#    adam_step hand each update to the backend's sgd_update / adam_update slot (optim.c:78-110, 243-266)
+on_cpu()
+w0 = rng.uniform(-1, 1, 500).astype(np.float32)
+grads = [rng.uniform(-1, 1, 500).astype(np.float32) for _ in range(3)]
+for kind, kw in (("adam", dict(lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01)),
+                 ("adamw", dict(lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01)),
+                 ("sgd", dict(lr=5e-2, momentum=0.9, wd=0.01, nesterov=True)),
+                 ("sgd", dict(lr=5e-2, momentum=0.0, wd=0.0, nesterov=False))):
+    on_cpu()
+    want = ref.optimizer_steps(kind, w0, grads, **kw)
+    on_gpu()
+    got = ref.optimizer_steps(kind, w0, grads, fetch=fetch, **kw)
+    for step, (g_, w_) in enumerate(zip(got, want)):
+        assert np.abs(g_ - w_).max() <= 2e-6, (kind, step)
+    print("optimizer", kind, "ok", flush=True)
+
 on_cpu()
 print("DROPIN OK", flush=True)

@@ -612,10 +612,17 @@ class RefLib:
         self.L.ax_layer_destroy(ln)
         return out
 
-    def optimizer_steps(self, kind, w0, grads, **kw):
+    def optimizer_steps(self, kind, w0, grads, fetch=None, **kw):
         """Runs one reference optimizer step per gradient in `grads` on a single parameter
-        tensor; returns the weights after each step.  kind: adam, adamw, sgd."""
-        tw = self.tensor(w0)
+        tensor; returns the weights after each step.  kind: adam, adamw, sgd.  Tensors are made
+        with ax_tensor_from_array on the reference's default device; `fetch` reads one back when
+        that device is not the CPU."""
+        def from_host(arr):
+            arr = np.ascontiguousarray(arr, np.float32)
+            return self.L.ax_tensor_from_array(arr.ctypes.data, (i64 * arr.ndim)(*arr.shape), arr.ndim, 0)
+        self.L.ax_tensor_from_array.restype = C.POINTER(RefTensor)
+        self.L.ax_tensor_from_array.argtypes = [C.c_void_p, C.POINTER(i64), C.c_int, C.c_int]
+        tw = from_host(w0)
         params = (C.POINTER(RefTensor) * 1)(tw)
         if kind == "sgd":
             opt = self.L.ax_sgd_create(params, 1, kw["lr"], kw["momentum"], kw["wd"], kw["nesterov"])
@@ -624,12 +631,12 @@ class RefLib:
             opt = make(params, 1, kw["lr"], kw["beta1"], kw["beta2"], kw["eps"], kw["wd"])
         outs = []
         for g in grads:
-            tg = self.tensor(g)
+            tg = from_host(g)
             tw.contents.grad = tg
             self.L.ax_optimizer_step(opt)
             tw.contents.grad = None
             self.free(tg)
-            outs.append(self.numpy(tw))
+            outs.append(fetch(tw) if fetch else self.numpy(tw))
         self.L.ax_optimizer_destroy(opt)
         self.free(tw)
         return outs
