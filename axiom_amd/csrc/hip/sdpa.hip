@@ -33,6 +33,8 @@ using namespace axhip;
                  "v"(voff), "s"(base)                                                          \
                  : "memory")
 #define AXS_VM0() __builtin_amdgcn_s_waitcnt(0 | (0 << 14) | (7 << 4) | (15 << 8))
+// at most n (a constant below 64) vector-memory loads still in flight
+#define AXS_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 
 constexpr int SD_BQ = 128, SD_BKV = 64;
 
@@ -108,36 +110,42 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
     for (int pass = 0; pass < passes; pass++) {
         const int64_t q0 = (CAUSAL && pass == 0 ? nq - 1 - unit : unit) * SD_BQ;
         if (pass) __syncthreads();                   // the first tile's last key block has been read
-        // ---- Q tile (128 rows) through the two K stages, then into registers ----
+        // ---- Q tile (128 rows) through the V area, then into registers; the first key block's
+        // K rows stream into their own stage at the same time, so a workgroup pays one load
+        // latency, not two, before its first MFMA.  Its V rows follow once Q has left the V area.
+        const int64_t nblocks = CAUSAL ? (q0 + SD_BQ) / SD_BKV : S / SD_BKV;
+        constexpr unsigned Q_BASE = 2 * G::KSTAGE;   // 2 * KSTAGE bytes of Q fit the two V stages
+        static_assert(2 * G::KSTAGE <= 2 * G::VSTAGE, "Q staging area");
+        auto issue_k = [&](int64_t blk, int stage) {
+            const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * DK);
+#pragma unroll
+            for (int i = 0; i < G::IPW; i++) AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
+        };
+        auto issue_v = [&](int64_t blk, int stage) {
+            const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * DK);
+#pragma unroll
+            for (int i = 0; i < G::IPW; i++)
+                AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff[i], vg);
+        };
 #pragma unroll
         for (int i = 0; i < G::IPW; i++) {
-            AXS_LOAD_LDS(lds0 + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * DK));
-            AXS_LOAD_LDS(lds0 + G::KSTAGE + (4 * i + wave) * 1024, koff[i],
+            AXS_LOAD_LDS(lds0 + Q_BASE + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * DK));
+            AXS_LOAD_LDS(lds0 + Q_BASE + G::KSTAGE + (4 * i + wave) * 1024, koff[i],
                          reinterpret_cast<const char *>(Qh + (q0 + 64) * DK));
         }
+        issue_k(0, 0);
         AXS_VM0();
         __syncthreads();
         v4f qf[KB];                                  // k-block kb: dk 8*kb + 4*fhalf .. +3 of this lane's query
         {
-            const int r = wave * 32 + frow;          // rows 64..127 sit in the second stage, same swizzle
-            const unsigned char *qrow = lds + (r >> 6) * G::KSTAGE + (r & 63) * G::ROWB;
+            const int r = wave * 32 + frow;          // rows 64..127 sit KSTAGE bytes further on, same swizzle
+            const unsigned char *qrow = lds + Q_BASE + (r >> 6) * G::KSTAGE + (r & 63) * G::ROWB;
 #pragma unroll
-            for (int kb = 0; kb < KB; kb++)
-                qf[kb] = *reinterpret_cast<const v4f *>(qrow + (((kb * 2 + fhalf) ^ G::swz(r & 63)) << 4));
+            for (int kb = 0; kb < KB; kb++)      // scale * log2(e) goes into Q once: scores come out in log2 units
+                qf[kb] = *reinterpret_cast<const v4f *>(qrow + (((kb * 2 + fhalf) ^ G::swz(r & 63)) << 4)) * scale_log2e;
         }
         __syncthreads();
-
-        const int64_t nblocks = CAUSAL ? (q0 + SD_BQ) / SD_BKV : S / SD_BKV;
-        auto issue = [&](int64_t blk, int stage) {
-            const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * DK);
-            const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * DK);
-#pragma unroll
-            for (int i = 0; i < G::IPW; i++) {
-                AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
-                AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff[i], vg);
-            }
-        };
-        issue(0, 0);
+        issue_v(0, 0);
 
         v16f acc_o[DT];
 #pragma unroll
@@ -149,9 +157,14 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
 
         for (int64_t blk = 0; blk < nblocks; blk++) {
             const int stage = (int)(blk & 1);
-            AXS_VM0();
-            __syncthreads();                          // block blk has landed; stage^1 is free again
-            if (blk + 1 < nblocks) issue(blk + 1, stage ^ 1);
+            if (blk > 0) {
+                AXS_VM0();
+                __syncthreads();                      // block blk has landed; stage^1 is free again
+            }
+            if (blk + 1 < nblocks) {
+                issue_k(blk + 1, stage ^ 1);
+                issue_v(blk + 1, stage ^ 1);
+            }
             const unsigned char *ks = lds + stage * G::KSTAGE;
             const unsigned char *vs = lds + 2 * G::KSTAGE + stage * G::VSTAGE;
 
@@ -164,6 +177,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
 
             // ---- scores of 64 keys ----
             v16f acc_s[2];
+            __builtin_amdgcn_s_setprio(1);      // MFMA phases go ahead of the co-resident wave's VALU work
 #pragma unroll
             for (int kt = 0; kt < 2; kt++) {
 #pragma unroll
@@ -180,37 +194,54 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
                 }
             }
 
+            __builtin_amdgcn_s_setprio(0);
             // ---- online softmax ----
+            // Scores arrive in log2 units (Q was scaled once, above).  The reference point m_run
+            // of the exponentials only moves when some query's block maximum exceeds it by more
+            // than 2^8: until then p = 2^(s - m_run) <= 256 is safe in fp32 and exact in the
+            // quotient O = sum(p v) / sum(p), and the accumulator needs no rescaling pass (which
+            // costs as many vector instructions as the exponentials themselves; the fp32 MFMAs
+            // run on the same lanes as vector instructions, so every one saved is MFMA time).
             float m_blk = -INFINITY;
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
-                    float s = acc_s[kt][v] * scale_log2e;
-                    if (!tile_on[kt] || (need_mask && kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3) > qrel)) s = -INFINITY;
+                    float s = acc_s[kt][v];
+                    if (CAUSAL && (!tile_on[kt] || (need_mask && kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3) > qrel)))
+                        s = -INFINITY;
                     acc_s[kt][v] = s;
                     m_blk = fmaxf(m_blk, s);
                 }
             m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
-            const float m_new = fmaxf(m_run, m_blk);      // finite: key 0 is visible to every query
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            if (__builtin_amdgcn_ballot_w64(m_blk > m_run + 8.0f)) {      // wave-uniform; always taken for block 0
+                const float m_new = fmaxf(m_run, m_blk);  // finite: key 0 is visible to every query
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                l_run *= alpha;
+                m_run = m_new;
+#pragma unroll
+                for (int d = 0; d < DT; d++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) acc_o[d][v] *= alpha;
+            }
             float l_blk = 0.0f;
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
-                    const float p = __builtin_amdgcn_exp2f(acc_s[kt][v] - m_new);
+                    const float p = __builtin_amdgcn_exp2f(acc_s[kt][v] - m_run);
                     acc_s[kt][v] = p;
                     l_blk += p;
                 }
-            l_run = l_run * alpha + l_blk;
-            m_run = m_new;
-#pragma unroll
-            for (int d = 0; d < DT; d++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) acc_o[d][v] *= alpha;
+            l_run += l_blk;
 
+            if (blk == 0) {                           // the first block's V rows were issued last
+                if (nblocks > 1) AXS_VM(2 * G::IPW);      // loads return in order: all but block 1's
+                else AXS_VM0();
+                __syncthreads();
+            }
             // ---- O^T += V^T P^T ----
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int kt = 0; kt < 2; kt++) {
                 if (!tile_on[kt]) continue;
@@ -223,6 +254,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
                         acc_o[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[d * 32 + frow], acc_s[kt][v], acc_o[d], 0, 0, 0);
                 }
             }
+            __builtin_amdgcn_s_setprio(0);
         }
 
         // ---- normalise and write: lane owns query qg, dk columns 32*d + 8*g + 4*fhalf .. +3 ----
