@@ -68,6 +68,10 @@ SIGNATURES = {
     "ax_compute_has_adam_update": (C.c_int, []), "ax_compute_has_sgd_update": (C.c_int, []),
     "ax_compute_layernorm": (C.c_int, [TP, TP, TP, C.c_float, TP, TP, TP]),
     "ax_layernorm_create": (C.c_void_p, [C.c_int64, C.c_float]),
+    "ax_mha_create": (C.c_void_p, [C.c_int64, C.c_int, C.c_bool, C.c_bool]),
+    "ax_init_xavier_uniform": (None, [TP, C.c_int64, C.c_int64]),
+    "ax_compute_register_cuda_extension": (C.c_int, [C.c_void_p]),
+    "ax_compute_get_cuda_extension": (C.c_void_p, []),
     "ax_sigmoid_layer_create": (C.c_void_p, []), "ax_tanh_layer_create": (C.c_void_p, []),
     "ax_swish_layer_create": (C.c_void_p, []), "ax_leaky_relu_layer_create": (C.c_void_p, [C.c_float]),
     "ax_elu_layer_create": (C.c_void_p, [C.c_float]), "ax_softmax_layer_create": (C.c_void_p, [C.c_int]),
@@ -123,7 +127,7 @@ SIGNATURES = {
     "ax_qgemm_w8a8_dev": (C.c_int, [C.c_void_p, C.c_float, QP, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, i64]),
     "ax_hip_ops_for_device": (C.c_void_p, [C.c_int]),
 }
-DATA_SYMBOLS = ["ax_hip_ops"]
+DATA_SYMBOLS = ["ax_hip_ops", "ax_hip_extension"]
 
 
 class Axiom:

@@ -33,10 +33,16 @@ typedef int   v16i __attribute__((ext_vector_type(16)));
 typedef float v4f  __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
+// 0.5 x (1 + tanh(u)) with u = sqrt(2/pi) (x + 0.044715 x^3), evaluated as x / (1 + e^(-2u)):
+// the same function (0.5 (1 + tanh u) is the logistic of 2u; the reference's vector path also
+// goes through 2*sigmoid(2x) - 1, src/compute/backends/simd_defs.h:308-321) in one hardware
+// exponential and one reciprocal instead of a library tanh.  In a fused GEMM write-back every
+// vector instruction is time taken from the fp32 MFMAs, which run on the same lanes.
 __device__ __forceinline__ float gelu_tanh(float x) {
     const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    float inner = k0 * (x + k1 * x * x * x);
-    return 0.5f * x * (1.0f + tanhf(inner));
+    const float u = k0 * (x + k1 * x * x * x);
+    const float t = __builtin_amdgcn_exp2f(u * -2.8853900817779268f);      // e^(-2u); inf for u << 0
+    return x * __builtin_amdgcn_rcpf(1.0f + t);
 }
 
 __device__ __forceinline__ float apply_act(float v, int act) {

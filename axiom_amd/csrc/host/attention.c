@@ -1,0 +1,170 @@
+/* Multi-head self-attention layer, forward pass (Axiom's src/core/attention.c:121-430 for a tensor
+ * on a GPU device): fused QKV projection as one GEMM, head split (+ bias) through the extension
+ * table, attention forward through its sdpa_fwd member, head merge, output projection with the
+ * column bias.  Every step runs on the device that holds the input. */
+#include <math.h>
+#include <stdlib.h>
+
+#include "axiom/attention.h"
+#include "axiom/compute.h"
+#include "axiom/error.h"
+#include "axiom/init.h"
+#include "axiom/internal/cuda_extension.h"
+
+static float *dev_ptr(const ax_tensor_t *t) { return (float *)t->storage->data + t->offset; }
+
+static ax_tensor_t *on_device_of(const ax_tensor_t *like, const int64_t *shape, int ndim) {
+    ax_device_t prev = ax_get_default_device();
+    ax_set_default_device(like->storage->device);
+    ax_tensor_t *t = ax_tensor_create(shape, ndim, AX_FLOAT32);
+    ax_set_default_device(prev);
+    return t;
+}
+
+/* src/core/attention/cache.c:24-85 */
+static ax_status_t refresh_fused_qkv(ax_mha_t *m, const ax_cuda_extension_t *ext) {
+    const int64_t D = m->d_model;
+    const uint64_t gq = m->Wq->storage->generation, gk = m->Wk->storage->generation, gv = m->Wv->storage->generation;
+    if (!m->Wqkv_cache || gq != m->Wq_gen || gk != m->Wk_gen || gv != m->Wv_gen) {
+        if (!m->Wqkv_cache) {
+            int64_t sh[2] = {D, 3 * D};
+            if (!(m->Wqkv_cache = on_device_of(m->Wq, sh, 2))) return AX_ERR_ALLOC;
+        }
+        ax_status_t st = ext->qkv_cache_build(dev_ptr(m->Wqkv_cache), dev_ptr(m->Wq), dev_ptr(m->Wk), dev_ptr(m->Wv), D);
+        if (st != AX_OK) return st;
+        m->Wqkv_cache->storage->generation++;
+        m->Wq_gen = gq;
+        m->Wk_gen = gk;
+        m->Wv_gen = gv;
+    }
+    if (m->use_bias) {
+        if (!m->bqkv_cache) {
+            int64_t sh[1] = {3 * D};
+            if (!(m->bqkv_cache = on_device_of(m->Wq, sh, 1))) return AX_ERR_ALLOC;
+        }
+        ax_status_t st = ext->bias_cache_build(dev_ptr(m->bqkv_cache), dev_ptr(m->bq), dev_ptr(m->bk), dev_ptr(m->bv), D);
+        if (st != AX_OK) return st;
+        m->bqkv_cache->storage->generation++;
+    }
+    return AX_OK;
+}
+
+static ax_tensor_t *mha_forward(ax_layer_t *self, ax_tensor_t *x) {
+    ax_mha_t *m = (ax_mha_t *)self;
+    if (!x || x->ndim != 3 || x->dtype != AX_FLOAT32 || x->shape[2] != m->d_model) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "mha: input must be float32 [B, S, %lld]", (long long)m->d_model);
+        return NULL;
+    }
+    const ax_cuda_extension_t *ext = ax_compute_get_cuda_extension();
+    if (x->storage->device == AX_DEVICE_CPU || !ext || !ext->sdpa_fwd || !ext->head_interleave_qkv_split ||
+        !ext->head_interleave_qkv_split_bias || !ext->head_deinterleave || !ext->qkv_cache_build || !ext->bias_cache_build) {
+        ax_err_set(AX_ERR_NOT_IMPLEMENTED, "mha: needs a device tensor and a registered GPU extension table");
+        return NULL;
+    }
+    if (!ax_tensor_is_contiguous(x) || m->Wq->storage->device != x->storage->device) {
+        ax_err_set(AX_ERR_BACKEND, "mha: input must be contiguous and on the device that holds the weights");
+        return NULL;
+    }
+    const int64_t B = x->shape[0], S = x->shape[1], D = m->d_model, H = m->n_heads, dk = m->d_k, rows = B * S;
+    ax_tensor_t *x_flat = NULL, *qkv = NULL, *Qh = NULL, *Kh = NULL, *Vh = NULL, *Oh = NULL, *attn = NULL, *out_flat = NULL,
+                *out = NULL;
+    int64_t flat_sh[2] = {rows, D}, qkv_sh[2] = {rows, 3 * D}, head_sh[3] = {B * H, S, dk};
+    ax_status_t st = refresh_fused_qkv(m, ext);
+    if (st == AX_OK && (!(x_flat = ax_tensor_reshape(x, flat_sh, 2)) || !(qkv = on_device_of(x, qkv_sh, 2)) ||
+                        !(Qh = on_device_of(x, head_sh, 3)) || !(Kh = on_device_of(x, head_sh, 3)) ||
+                        !(Vh = on_device_of(x, head_sh, 3)) || !(Oh = on_device_of(x, head_sh, 3)) ||
+                        !(attn = on_device_of(x, flat_sh, 2)) || !(out_flat = on_device_of(x, flat_sh, 2))))
+        st = AX_ERR_ALLOC;
+    if (st == AX_OK) st = ax_compute_gemm(x_flat, m->Wqkv_cache, qkv);
+    if (st == AX_OK) {
+        ax_err_clear();
+        if (m->use_bias)
+            ext->head_interleave_qkv_split_bias(dev_ptr(qkv), dev_ptr(m->bqkv_cache), dev_ptr(Qh), dev_ptr(Kh), dev_ptr(Vh),
+                                                B, S, H, dk, D);
+        else
+            ext->head_interleave_qkv_split(dev_ptr(qkv), dev_ptr(Qh), dev_ptr(Kh), dev_ptr(Vh), B, S, H, dk, D);
+        st = ax_err_last_status();
+    }
+    if (st == AX_OK)
+        st = ext->sdpa_fwd(dev_ptr(Qh), dev_ptr(Kh), dev_ptr(Vh), dev_ptr(Oh), NULL, B * H, S, dk, 1.0f / sqrtf((float)dk),
+                           m->causal, NULL);
+    if (st == AX_OK) {
+        ext->head_deinterleave(dev_ptr(Oh), dev_ptr(attn), B, S, H, dk);
+        st = ax_err_last_status();
+    }
+    if (st == AX_OK) {                                       /* attention.c:402-417: gemm, then bias along axis 1 */
+        if (m->use_bias && ax_compute_has_gemm_bias_act()) st = ax_compute_gemm_bias_act(attn, m->Wo, m->bo, AX_ACT_NONE, out_flat);
+        else {
+            st = ax_compute_gemm(attn, m->Wo, out_flat);
+            if (st == AX_OK && m->use_bias) st = ax_compute_bias_add(out_flat, m->bo, 1, out_flat);
+        }
+    }
+    if (st == AX_OK) out = ax_tensor_reshape(out_flat, x->shape, 3);
+    ax_tensor_destroy(x_flat);
+    ax_tensor_destroy(qkv);
+    ax_tensor_destroy(Qh);
+    ax_tensor_destroy(Kh);
+    ax_tensor_destroy(Vh);
+    ax_tensor_destroy(Oh);
+    ax_tensor_destroy(attn);
+    ax_tensor_destroy(out_flat);
+    return out;
+}
+
+static void mha_destroy(ax_layer_t *self) {
+    ax_mha_t *m = (ax_mha_t *)self;
+    ax_tensor_t *all[10] = {m->Wq, m->Wk, m->Wv, m->Wo, m->bq, m->bk, m->bv, m->bo, m->Wqkv_cache, m->bqkv_cache};
+    for (int i = 0; i < 10; i++) ax_tensor_destroy(all[i]);
+    free(m);
+}
+
+ax_layer_t *ax_mha_create(int64_t d_model, int n_heads, bool use_bias, bool causal) {
+    if (d_model <= 0 || n_heads <= 0) return NULL;
+    if (d_model % n_heads != 0) {
+        ax_err_set(AX_ERR_INVALID_SHAPE, "ax_mha_create: d_model=%lld must be divisible by n_heads=%d", (long long)d_model,
+                   n_heads);
+        return NULL;
+    }
+    ax_mha_t *m = calloc(1, sizeof *m);
+    if (!m) {
+        ax_err_set(AX_ERR_ALLOC, "ax_mha_create: out of memory");
+        return NULL;
+    }
+    m->base.ops.forward = mha_forward;
+    m->base.ops.destroy = mha_destroy;
+    m->base.type = AX_LAYER_MHA;
+    m->base.training = true;
+    m->base.input_features = m->base.output_features = d_model;
+    m->d_model = d_model;
+    m->n_heads = n_heads;
+    m->d_k = d_model / n_heads;
+    m->use_bias = use_bias;
+    m->causal = causal;
+    int64_t ws[2] = {d_model, d_model};
+    ax_tensor_t **w[4] = {&m->Wq, &m->Wk, &m->Wv, &m->Wo};
+    for (int i = 0; i < 4; i++) {                            /* drawn in this order: attention.c:980-992 */
+        if (!(*w[i] = ax_tensor_create(ws, 2, AX_FLOAT32))) {
+            mha_destroy(&m->base);
+            return NULL;
+        }
+    }
+    for (int i = 0; i < 4; i++) {
+        ax_init_xavier_uniform(*w[i], d_model, d_model);
+        (*w[i])->requires_grad = true;
+        m->base.params[i] = *w[i];
+    }
+    m->base.n_params = 4;
+    if (use_bias) {
+        ax_tensor_t **b[4] = {&m->bq, &m->bk, &m->bv, &m->bo};
+        for (int i = 0; i < 4; i++) {
+            if (!(*b[i] = ax_tensor_zeros(&d_model, 1, AX_FLOAT32))) {
+                mha_destroy(&m->base);
+                return NULL;
+            }
+            (*b[i])->requires_grad = true;
+            m->base.params[4 + i] = *b[i];
+        }
+        m->base.n_params = 8;
+    }
+    return &m->base;
+}

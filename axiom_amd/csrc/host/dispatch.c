@@ -5,6 +5,7 @@
  * returns AX_ERR_BACKEND — there is no CPU compute path to fall back to. */
 #include "axiom/axiom.h"
 #include "axiom/internal/backend_ops.h"
+#include "axiom/internal/cuda_extension.h"
 
 static const ax_backend_ops_t *g_backends[AX_BACKEND_COUNT];
 static const ax_backend_ops_t *g_device_owner[AX_DEVICE_COUNT];
@@ -27,6 +28,16 @@ const ax_backend_ops_t *ax_backend_for_device(ax_device_t device) {
     return g_device_owner[device];
 }
 
+/* the GPU extension table (src/compute/dispatch.c:286-300) */
+static const ax_cuda_extension_t *g_extension;
+
+ax_status_t ax_compute_register_cuda_extension(const ax_cuda_extension_t *ext) {
+    g_extension = ext;
+    return AX_OK;
+}
+
+const ax_cuda_extension_t *ax_compute_get_cuda_extension(void) { return g_extension; }
+
 ax_status_t ax_compute_init(void) {
     if (g_initialised) {
         if (g_active) return AX_OK;
@@ -36,6 +47,7 @@ ax_status_t ax_compute_init(void) {
     g_initialised = 1;
     g_backends[AX_BACKEND_HIP] = &ax_hip_ops;
     claim_device(&ax_hip_ops);
+    g_extension = &ax_hip_extension;
     if (ax_hip_ops.device_count && ax_hip_ops.device_count() > 0) {
         g_active_id = AX_BACKEND_HIP;
         g_active = &ax_hip_ops;
@@ -58,6 +70,7 @@ void ax_compute_shutdown(void) {
         g_device_inited[d] = 0;
     }
     g_active = NULL;
+    g_extension = NULL;
     g_initialised = 0;
 }
 

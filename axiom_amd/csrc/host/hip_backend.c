@@ -13,6 +13,7 @@
 #include "axhip.h"
 #include "axiom/error.h"
 #include "axiom/internal/backend_ops.h"
+#include "axiom/internal/cuda_extension.h"
 
 static ax_device_t g_my_device = AX_DEVICE_HIP;
 
@@ -531,6 +532,34 @@ ax_status_t ax_hip_sdpa_fwd(const float *Q, const float *K, const float *V, floa
     }
     return lift(axhip_sdpa_fwd(Q, K, V, out, L, BH, S, dk, scale, causal ? 1 : 0), "hip sdpa_fwd");
 }
+
+/* ---- the extension table (include/axiom/internal/cuda_extension.h).  The layout members return
+ * nothing in the reference's table; a failure is left for ax_err_last_message(). ---- */
+static void ext_split(const float *src, float *q, float *k, float *v, int64_t B, int64_t S, int64_t H, int64_t dk, int64_t D) {
+    (void)lift(axhip_head_split_qkv(src, NULL, q, k, v, B, S, H, dk, D), "hip head_interleave_qkv_split");
+}
+static void ext_split_bias(const float *src, const float *bqkv, float *q, float *k, float *v, int64_t B, int64_t S,
+                           int64_t H, int64_t dk, int64_t D) {
+    (void)lift(axhip_head_split_qkv(src, bqkv, q, k, v, B, S, H, dk, D), "hip head_interleave_qkv_split_bias");
+}
+static void ext_interleave(const float *src, float *dst, int64_t B, int64_t S, int64_t H, int64_t dk) {
+    (void)lift(axhip_head_interleave(src, dst, B, S, H, dk), "hip head_interleave");
+}
+static void ext_deinterleave(const float *src, float *dst, int64_t B, int64_t S, int64_t H, int64_t dk) {
+    (void)lift(axhip_head_deinterleave(src, dst, B, S, H, dk), "hip head_deinterleave");
+}
+static ax_status_t ext_qkv_cache(float *dst, const float *wq, const float *wk, const float *wv, int64_t D) {
+    return lift(axhip_concat3_rows(dst, wq, wk, wv, D, D), "hip qkv_cache_build");
+}
+static ax_status_t ext_bias_cache(float *dst, const float *bq, const float *bk, const float *bv, int64_t D) {
+    return lift(axhip_concat3_rows(dst, bq, bk, bv, 1, D), "hip bias_cache_build");
+}
+
+const ax_cuda_extension_t ax_hip_extension = {
+    .head_interleave_qkv_split = ext_split, .head_interleave_qkv_split_bias = ext_split_bias,
+    .head_interleave = ext_interleave, .head_deinterleave = ext_deinterleave,
+    .qkv_cache_build = ext_qkv_cache, .bias_cache_build = ext_bias_cache, .sdpa_fwd = ax_hip_sdpa_fwd,
+};
 
 const ax_backend_ops_t *ax_hip_ops_for_device(ax_device_t as_device) {
     static ax_backend_ops_t alias = AX_HIP_OPS_INIT(AX_DEVICE_HIP);

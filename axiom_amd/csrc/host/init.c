@@ -31,5 +31,10 @@ void ax_init_kaiming_uniform(ax_tensor_t *t, int64_t fan_in) {
     fill_with(t, ax_rng_uniform, -limit, limit);
 }
 
+void ax_init_xavier_uniform(ax_tensor_t *t, int64_t fan_in, int64_t fan_out) {
+    const float limit = sqrtf(6.0f / (float)(fan_in + fan_out));
+    fill_with(t, ax_rng_uniform, -limit, limit);
+}
+
 void ax_init_uniform(ax_tensor_t *t, float low, float high) { fill_with(t, ax_rng_uniform, low, high); }
 void ax_init_normal(ax_tensor_t *t, float mean, float std) { fill_with(t, ax_rng_normal_params, mean, std); }

@@ -8,6 +8,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include "axiom/attention.h"
 #include "axiom/error.h"
 #include "axiom/serialize.h"
 
@@ -197,7 +198,7 @@ ax_status_t ax_model_save(ax_model_t *model, const char *path) {
         switch (seq->layers[i]->type) {
             case AX_LAYER_DENSE: case AX_LAYER_RELU: case AX_LAYER_SIGMOID: case AX_LAYER_TANH:
             case AX_LAYER_LEAKY_RELU: case AX_LAYER_ELU: case AX_LAYER_GELU: case AX_LAYER_SWISH:
-            case AX_LAYER_SOFTMAX: case AX_LAYER_LAYERNORM: break;
+            case AX_LAYER_SOFTMAX: case AX_LAYER_LAYERNORM: case AX_LAYER_MHA: break;
             default: return refuse_layer(seq->layers[i]->type, i);
         }
     }
@@ -230,6 +231,14 @@ ax_status_t ax_model_save(ax_model_t *model, const char *path) {
             case AX_LAYER_SOFTMAX:
                 put_u32(&s, 1);                               /* the reference writes a constant 1 here */
                 break;
+            case AX_LAYER_MHA: {
+                const ax_mha_t *mh = (const ax_mha_t *)l;
+                put_i64(&s, mh->d_model);
+                put_u32(&s, (uint32_t)mh->n_heads);
+                put_u8(&s, mh->use_bias ? 1 : 0);
+                put_u8(&s, mh->causal ? 1 : 0);
+                break;
+            }
             default: break;
         }
     }
@@ -280,6 +289,18 @@ static ax_layer_t *read_layer(stream_t *s, uint32_t type, uint32_t index) {
             uint32_t axis;
             if (!get_u32(s, &axis)) return NULL;
             return ax_softmax_layer_create((int)axis);
+        }
+        case AX_LAYER_MHA: {
+            int64_t d_model;
+            uint32_t n_heads;
+            uint8_t use_bias, causal;
+            if (!get_i64(s, &d_model) || !get_u32(s, &n_heads) || !get_u8(s, &use_bias) || !get_u8(s, &causal)) return NULL;
+            if (d_model <= 0 || n_heads == 0 || n_heads > (uint32_t)INT_MAX || d_model % (int64_t)n_heads != 0 ||
+                (uint64_t)d_model * (uint64_t)d_model * 4 > MAX_TENSOR_BYTES) {
+                ax_err_set(AX_ERR_INVALID_SHAPE, "layer %u: attention with d_model %" PRId64 " and %u heads", index, d_model, n_heads);
+                return NULL;
+            }
+            return ax_mha_create(d_model, (int)n_heads, use_bias & 1, causal & 1);
         }
         case AX_LAYER_RELU: return ax_relu_layer_create();
         case AX_LAYER_SIGMOID: return ax_sigmoid_layer_create();

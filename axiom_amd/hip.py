@@ -48,6 +48,10 @@ SIGNATURES = {
     "axhip_layernorm_fwd": (C.c_int, [vp, vp, vp, vp, vp, vp, i64, i64, C.c_float]),
     "axhip_adam_update": (C.c_int, [vp, vp, vp, vp, i64] + [C.c_float] * 7 + [C.c_int]),
     "axhip_sgd_update": (C.c_int, [vp, vp, vp, i64, C.c_float, C.c_float, C.c_float, C.c_int]),
+    "axhip_head_split_qkv": (C.c_int, [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64]),
+    "axhip_head_interleave": (C.c_int, [vp, vp, i64, i64, i64, i64]),
+    "axhip_head_deinterleave": (C.c_int, [vp, vp, i64, i64, i64, i64]),
+    "axhip_concat3_rows": (C.c_int, [vp, vp, vp, vp, i64, i64]),
     "axhip_relu": (C.c_int, [vp, vp, i64]),
     "axhip_gelu": (C.c_int, [vp, vp, i64]),
     "axhip_fill_f32": (C.c_int, [vp, C.c_float, i64]),

@@ -197,6 +197,20 @@ int axhip_sgd_update(float *w, const float *g, float *momentum_buf, int64_t n, f
 int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L,
                    int64_t BH, int64_t S, int64_t dk, float scale, int causal);
 
+/* ---- layout transforms around attention (the layout members of the reference's GPU extension
+ * table, include/axiom/internal/cuda_extension.h:45-84) ------------------------------------- */
+/* qkv [B*S, 3D] (row = [q | k | v], D = H*dk) -> q, k, v each [B*H, S, dk]; bqkv [3D] is added
+ * when not NULL (ax_attn_head_interleave_qkv_split[_bias], src/core/attention/layout.c:215-262). */
+int axhip_head_split_qkv(const float *qkv, const float *bqkv, float *q, float *k, float *v, int64_t B, int64_t S,
+                         int64_t H, int64_t dk, int64_t D);
+/* [B, S, H, dk] -> [B*H, S, dk] and back (ax_attn_head_interleave / ax_attn_head_deinterleave,
+ * src/core/attention/layout.c:84-152). */
+int axhip_head_interleave(const float *src, float *dst, int64_t B, int64_t S, int64_t H, int64_t dk);
+int axhip_head_deinterleave(const float *src, float *dst, int64_t B, int64_t S, int64_t H, int64_t dk);
+/* dst [rows, 3*cols]: row i = [a[i,:] | b[i,:] | c[i,:]] — the fused projection weight [D, 3D] from
+ * Wq, Wk, Wv, and with rows = 1 the fused bias (src/core/attention/cache.c:49-57, 79-81). */
+int axhip_concat3_rows(float *dst, const float *a, const float *b, const float *c, int64_t rows, int64_t cols);
+
 /* ---- timing on the library's stream (for benchmarks) -------------------------------- */
 void *axhip_event_create(void);
 void  axhip_event_destroy(void *ev);

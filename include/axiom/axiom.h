@@ -2,6 +2,7 @@
  * container and model files around it). */
 #ifndef AXIOM_H
 #define AXIOM_H
+#include "attention.h"
 #include "compute.h"
 #include "device.h"
 #include "error.h"

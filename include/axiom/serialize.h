@@ -10,7 +10,7 @@
  * ax_model_load builds the layers on the thread's default device and copies each parameter
  * there, so a model trained and saved by the reference runs on the GPU as loaded; ax_model_save
  * reads parameters back from whatever device holds them.  Layer types with a forward pass in
- * this library are accepted (Dense, the activation layers, LayerNorm); a file that names any
+ * this library are accepted (Dense, the activation layers, LayerNorm, MHA); a file that names any
  * other type is refused with AX_ERR_NOT_IMPLEMENTED.  Every count and extent read from a file is
  * validated before it is used (serialize.c:189-260, 560-585).
  *

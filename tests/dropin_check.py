@@ -226,5 +226,85 @@ for kind, kw in (("adam", dict(lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.0
         assert np.abs(g_ - w_).max() <= 2e-6, (kind, step)
     print("optimizer", kind, "ok", flush=True)
 
+# 6. the extension table through the reference's own registry (src/compute/dispatch.c:286-300).  The
+#    reference's attention layer rebuilds its fused projection cache through the table
+#    (ax_attn_refresh_fused_qkv, src/core/attention/cache.c:24-85); its forward pass itself cannot be
+#    driven on any GPU device: it wraps the input in a stack view labelled AX_DEVICE_CPU
+#    (src/core/attention.c:71-89,176-179) and then decides `on_cuda` from that label (:211), so it
+#    walks device pointers with host memcpy.  What runs here: registration, the cache rebuild by the
+#    reference's code, and every forward member of the table on the reference's device tensors.
+class RefLayer(C.Structure):                 # include/axiom/layer.h:72-85
+    _fields_ = [("forward", C.c_void_p), ("destroy", C.c_void_p), ("type", C.c_int), ("training", C.c_bool),
+                ("params", TP * 8), ("n_params", C.c_int), ("buffers", TP * 4), ("n_buffers", C.c_int),
+                ("input_features", i64), ("output_features", i64)]
+
+
+class RefMHA(C.Structure):                   # include/axiom/attention.h:59-89
+    _fields_ = [("base", RefLayer), ("d_model", i64), ("n_heads", C.c_int), ("d_k", i64), ("use_bias", C.c_bool),
+                ("causal", C.c_bool), ("Wq", TP), ("Wk", TP), ("Wv", TP), ("Wo", TP), ("bq", TP), ("bk", TP), ("bv", TP),
+                ("bo", TP), ("Wqkv_cache", TP), ("bqkv_cache", TP)]
+
+
+EXT_FIELDS = [("split", C.CFUNCTYPE(None, *([C.c_void_p] * 4 + [i64] * 5))),
+              ("split_bias", C.CFUNCTYPE(None, *([C.c_void_p] * 5 + [i64] * 5))),
+              ("interleave", C.CFUNCTYPE(None, C.c_void_p, C.c_void_p, i64, i64, i64, i64)),
+              ("deinterleave", C.CFUNCTYPE(None, C.c_void_p, C.c_void_p, i64, i64, i64, i64)),
+              ("merge", C.c_void_p), ("qkv_cache_build", C.c_void_p), ("bias_cache_build", C.c_void_p),
+              ("sdpa_fwd", C.CFUNCTYPE(C.c_int, *([C.c_void_p] * 5 + [i64] * 3 + [C.c_float, C.c_bool, C.c_void_p])))]
+
+
+class RefExtension(C.Structure):             # include/axiom/internal/cuda_extension.h:41-140, leading members
+    _fields_ = EXT_FIELDS
+
+
+ext_addr = C.addressof(C.c_char.in_dll(plugin, "ax_hip_extension"))
+L.ax_compute_register_cuda_extension.argtypes = [C.c_void_p]
+L.ax_compute_register_cuda_extension.restype = C.c_int
+L.ax_compute_get_cuda_extension.restype = C.c_void_p
+assert L.ax_compute_register_cuda_extension(ext_addr) == 0
+assert L.ax_compute_get_cuda_extension() == ext_addr
+L.ax_mha_create.restype = C.c_void_p
+L.ax_mha_create.argtypes = [C.c_int64, C.c_int, C.c_bool, C.c_bool]
+L.ax_attn_refresh_fused_qkv.argtypes = [C.c_void_p]
+on_gpu()
+L.ax_set_seed(4242)
+D, H = 96, 6
+layer = L.ax_mha_create(D, H, True, False)
+assert layer, L.ax_err_last_message()
+mha = C.cast(layer, C.POINTER(RefMHA)).contents
+assert mha.d_model == D and mha.n_heads == H and mha.Wq.contents.storage.contents.device == REF_DEVICE_GPU
+L.ax_attn_refresh_fused_qkv(layer)
+assert mha.Wqkv_cache and mha.Wqkv_cache.contents.storage.contents.device == REF_DEVICE_GPU
+wq, wk, wv = fetch(mha.Wq), fetch(mha.Wk), fetch(mha.Wv)
+assert np.array_equal(fetch(mha.Wqkv_cache), np.concatenate([wq, wk, wv], axis=1))
+assert np.array_equal(fetch(mha.bqkv_cache), np.concatenate([fetch(mha.bq), fetch(mha.bk), fetch(mha.bv)]))
+# the forward members, called through the registered table on the reference's device tensors
+ext = C.cast(L.ax_compute_get_cuda_extension(), C.POINTER(RefExtension)).contents
+B, S, dk = 2, 40, D // H
+x = rng.uniform(-1, 1, (B * S, D)).astype(np.float32)
+tx = dev_tensor(x)
+qkv = L.ax_tensor_zeros((i64 * 2)(B * S, 3 * D), 2, 0)
+assert L.ax_compute_gemm(tx, mha.Wqkv_cache, qkv) == 0, L.ax_err_last_message()
+heads = [L.ax_tensor_zeros((i64 * 3)(B * H, S, dk), 3, 0) for _ in range(4)]
+attn = L.ax_tensor_zeros((i64 * 2)(B * S, D), 2, 0)
+ptr = lambda t: t.contents.storage.contents.data
+ext.split_bias(ptr(qkv), ptr(mha.bqkv_cache), ptr(heads[0]), ptr(heads[1]), ptr(heads[2]), B, S, H, dk, D)
+assert ext.sdpa_fwd(ptr(heads[0]), ptr(heads[1]), ptr(heads[2]), ptr(heads[3]), None, B * H, S, dk,
+                    1.0 / np.sqrt(dk), False, None) == 0, L.ax_err_last_message()
+ext.deinterleave(ptr(heads[3]), ptr(attn), B, S, H, dk)
+got = fetch(attn)
+on_cpu()
+full = ref.gemm(x, np.concatenate([wq, wk, wv], axis=1)) + fetch(mha.bqkv_cache)
+hq, hk, hv = (np.ascontiguousarray(full[:, i * D:(i + 1) * D].reshape(B, S, H, dk).transpose(0, 2, 1, 3)).reshape(B * H, S, dk)
+              for i in range(3))
+o, _ = ref.sdpa(hq, hk, hv, float(1.0 / np.sqrt(dk)))
+want = o.reshape(B, H, S, dk).transpose(0, 2, 1, 3).reshape(B * S, D)
+assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max()), np.abs(got - want).max()
+on_gpu()
+ref.free(tx, qkv, attn, *heads)
+L.ax_layer_destroy(layer)
+L.ax_compute_register_cuda_extension(None)
+print("extension table ok", flush=True)
+
 on_cpu()
 print("DROPIN OK", flush=True)

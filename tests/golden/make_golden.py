@@ -253,6 +253,14 @@ ref_model("ffn", [lambda: L.ax_layernorm_create(64, 1e-5), lambda: L.ax_dense_cr
                   L.ax_gelu_layer_create, lambda: L.ax_dense_create(256, 64, False)], (2, 7, 64), 8200)
 ref_model("acts", [lambda: L.ax_dense_create(9, 9, False), L.ax_sigmoid_layer_create, L.ax_tanh_layer_create,
                    lambda: L.ax_elu_layer_create(0.7), L.ax_swish_layer_create], (4, 9), 8300)
+L.ax_mha_create.restype = C.c_void_p
+L.ax_mha_create.argtypes = [C.c_int64, C.c_int, C.c_bool, C.c_bool]
+# the encoder block of benchmarks/bench_transformer.c:33-44 (LN, MHA, LN, Dense, GELU, Dense) and a
+# causal attention layer whose head size takes the fused kernel
+ref_model("encoder", [lambda: L.ax_layernorm_create(64, 1e-5), lambda: L.ax_mha_create(64, 4, True, False),
+                      lambda: L.ax_layernorm_create(64, 1e-5), lambda: L.ax_dense_create(64, 128, False),
+                      L.ax_gelu_layer_create, lambda: L.ax_dense_create(128, 64, False)], (2, 24, 64), 8600)
+ref_model("mha_causal", [lambda: L.ax_mha_create(128, 2, True, True)], (2, 128, 128), 8700)
 # a file whose first layer has no forward pass in the port: it must be refused, not misread
 L.ax_set_seed(8400)
 seq = L.ax_sequential_create()

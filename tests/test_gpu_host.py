@@ -400,7 +400,8 @@ def test_elementwise_reduction_optimizer_slots(ax, oracle, golden):
         ax.free(tw, tm_, tv)
 
 
-@pytest.mark.parametrize("tag,in_shape,seed", [("mlp", (5, 12), 8100), ("ffn", (2, 7, 64), 8200), ("acts", (4, 9), 8300)])
+@pytest.mark.parametrize("tag,in_shape,seed", [("mlp", (5, 12), 8100), ("ffn", (2, 7, 64), 8200), ("acts", (4, 9), 8300),
+                                               ("encoder", (2, 24, 64), 8600), ("mha_causal", (2, 128, 128), 8700)])
 def test_reference_model_file_runs_on_device(ax, oracle, golden, tag, in_shape, seed, tmp_path):
     """A model the reference built, initialised and saved (tests/golden/ref_*.axm) is loaded onto
     the GPU, reproduces the reference's CPU forward of the same input, and is written back from
@@ -434,3 +435,52 @@ def test_reference_model_file_runs_on_device(ax, oracle, golden, tag, in_shape, 
     assert out.read_bytes() == open(path, "rb").read()
     ax.free(tx, y)
     L.ax_model_destroy(model)
+
+
+@pytest.mark.parametrize("B,S,D,H,bias,causal", [(2, 128, 128, 2, True, True), (1, 256, 256, 4, False, False),
+                                                 (3, 40, 96, 6, True, False), (2, 77, 64, 2, True, True)])
+def test_attention_layer_forward(ax, oracle, B, S, D, H, bias, causal):
+    """ax_mha_create + forward on the device against the layer restated from the oracle's pieces
+    (pinned to the reference's own layer output in test_oracle.py)."""
+    import attn_cases as ac
+    from axiom_amd.axiom import TP
+    L = ax.L
+    L.ax_set_default_device(2)
+    L.ax_set_seed(1234)
+    layer = L.ax_mha_create(D, H, bias, causal)
+    assert layer, ax.err()
+    params = (TP * 8)()
+    n = L.ax_layer_get_params(layer, params, 8)
+    assert n == (8 if bias else 4)
+    oracle.seed(B + S + D)
+    w = [ax.to_numpy(params[i]) for i in range(4)]
+    limit = np.sqrt(np.float32(6.0) / np.float32(2 * D))
+    assert all(np.abs(m).max() <= limit and m.std() > 0.4 * limit for m in w)       # Xavier-uniform
+    if bias:
+        for i in range(4, 8):
+            b = oracle.uniform((D,), -0.5, 0.5)
+            tb = ax.from_numpy(b)
+            assert L.ax_compute_copy(tb, params[i]) == 0
+            ax.free(tb)
+            w.append(b)
+    x = oracle.uniform((B, S, D), -1, 1)
+    tx = ax.from_numpy(x)
+    y = L.ax_layer_forward(layer, tx)
+    assert y, ax.err()
+    want = ac.mha_forward(oracle, x, w, H, causal)
+    got = ax.to_numpy(y)
+    assert got.shape == (B, S, D)
+    assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max()), np.abs(got - want).max()
+    # a second call reuses the fused projection cache; a changed weight invalidates it
+    y2 = L.ax_layer_forward(layer, tx)
+    assert np.array_equal(ax.to_numpy(y2), got)
+    w[0] = w[0] * 0.5
+    tw = ax.from_numpy(w[0])
+    assert L.ax_compute_copy(tw, params[0]) == 0
+    y3 = L.ax_layer_forward(layer, tx)
+    want3 = ac.mha_forward(oracle, x, w, H, causal)
+    assert np.abs(ax.to_numpy(y3) - want3).max() <= 2e-5 * max(1.0, np.abs(want3).max())
+    bad = ax.from_numpy(np.zeros((2, D), np.float32))
+    assert not L.ax_layer_forward(layer, bad)
+    ax.free(tx, y, y2, y3, tw, bad)
+    L.ax_layer_destroy(layer)

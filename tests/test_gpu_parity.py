@@ -796,3 +796,37 @@ def test_optimizer_updates(hip, oracle, golden, key):
         got = dw.numpy()
         assert np.abs(got - golden[key][step - 1]).max() < 2e-6, step        # the reference's CPU optimizer
         assert np.abs(got - w).max() < 5e-7, step                            # same formula; fma contraction apart
+
+
+# ---------------------------------------------------------------- attention layout transforms
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,S,H,dk", [(2, 3, 4, 5), (1, 1, 1, 1), (3, 7, 2, 8), (2, 128, 8, 64), (4, 33, 3, 20), (8, 512, 16, 64)])
+def test_attention_layout_transforms(hip, oracle, B, S, H, dk):
+    """Pure copies: bit-exact against numpy reshapes / transposes (the reference's index maps,
+    src/core/attention/layout.c:134-148, 237-253)."""
+    import attn_cases as ac
+    say("attn layout", B, S, H, dk)
+    D = H * dk
+    oracle.seed(B * 1000 + S * 10 + H + dk)
+    qkv, bias = oracle.uniform((B * S, 3 * D), -1, 1), oracle.uniform((3 * D,), -1, 1)
+    dqkv, dbias = hip.array(qkv), hip.array(bias)
+    q, k, v = (hip.empty((B * H, S, dk)) for _ in range(3))
+    for use_bias in (False, True):
+        hip.check(hip.L.axhip_head_split_qkv(dqkv.ptr, dbias.ptr if use_bias else None, q.ptr, k.ptr, v.ptr, B, S, H, dk, D))
+        src = qkv + bias if use_bias else qkv
+        for i, got in enumerate((q, k, v)):
+            want = ac.split_heads(np.ascontiguousarray(src[:, i * D:(i + 1) * D]), B, S, H, dk)
+            assert np.array_equal(got.numpy(), want), (use_bias, i)
+    heads = oracle.uniform((B * H, S, dk), -1, 1)
+    dh, merged, back = hip.array(heads), hip.empty((B * S, D)), hip.empty((B * H, S, dk))
+    hip.check(hip.L.axhip_head_deinterleave(dh.ptr, merged.ptr, B, S, H, dk))
+    assert np.array_equal(merged.numpy(), ac.merge_heads(heads, B, S, H, dk))
+    hip.check(hip.L.axhip_head_interleave(merged.ptr, back.ptr, B, S, H, dk))
+    assert np.array_equal(back.numpy(), heads)
+    # fused projection panel [D, 3D] and bias [3D]
+    wq, wk, wv = (oracle.uniform((D, D), -1, 1) for _ in range(3))
+    dq, dk_, dv, panel = hip.array(wq), hip.array(wk), hip.array(wv), hip.empty((D, 3 * D))
+    hip.check(hip.L.axhip_concat3_rows(panel.ptr, dq.ptr, dk_.ptr, dv.ptr, D, D))
+    assert np.array_equal(panel.numpy(), np.concatenate([wq, wk, wv], axis=1))
+    hip.check(hip.L.axhip_concat3_rows(panel.ptr, dq.ptr, dk_.ptr, dv.ptr, 1, D))
+    assert np.array_equal(panel.numpy().reshape(-1)[:3 * D], np.concatenate([wq[0], wk[0], wv[0]]))

@@ -441,3 +441,28 @@ def test_optimizer_updates_against_reference_vectors(oracle, golden, key):
             w64 = w64 - kw["lr"] * (m64 / (1 - kw["beta1"] ** step)) / (np.sqrt(v64 / (1 - kw["beta2"] ** step)) + kw["eps"])
         assert np.abs(w - golden[key][step - 1]).max() < 2e-6, step
         assert np.abs(w - w64).max() < 2e-6, step
+
+
+# ---------------------------------------------------------------- attention layer
+def test_mha_layer_restatement_against_reference_vectors(oracle, golden):
+    """GEMM + head split + attention + head merge + GEMM, assembled from the oracle's pieces,
+    against what the reference's own layer produced (its CPU path fuses these differently)."""
+    import attn_cases as ac
+    _, w = ac.fixture_model("mha_causal")
+    x = ac.fixture_input(oracle, w, (2, 128, 128), 8700)
+    got = ac.mha_forward(oracle, x, w, 2, True)
+    want = golden["axm_mha_causal_out"]
+    assert np.abs(got - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
+    # numpy float64 evaluation of the definition
+    B, S, D, H, dk = 2, 128, 128, 2, 64
+    x64 = x.astype(np.float64).reshape(B * S, D)
+    q, k, v = ((x64 @ w[i] + w[4 + i]).reshape(B, S, H, dk).transpose(0, 2, 1, 3) for i in range(3))
+    s = q @ k.transpose(0, 1, 3, 2) / np.sqrt(dk)
+    s = np.where(np.tril(np.ones((S, S), bool)), s, -np.inf)
+    p = np.exp(s - s.max(axis=-1, keepdims=True))
+    o = (p / p.sum(axis=-1, keepdims=True)) @ v
+    ref = o.transpose(0, 2, 1, 3).reshape(B * S, D) @ w[3] + w[7]
+    assert np.abs(want.reshape(B * S, D) - ref).max() <= 1e-5 * max(1.0, np.abs(ref).max())
+    # the two layout maps are inverses of numpy's own transposes
+    t = np.arange(2 * 3 * 4 * 5, dtype=np.float32).reshape(6, 20)
+    assert np.array_equal(ac.merge_heads(ac.split_heads(t, 2, 3, 4, 5), 2, 3, 4, 5), t)
