@@ -830,3 +830,36 @@ def test_attention_layout_transforms(hip, oracle, B, S, H, dk):
     assert np.array_equal(panel.numpy(), np.concatenate([wq, wk, wv], axis=1))
     hip.check(hip.L.axhip_concat3_rows(panel.ptr, dq.ptr, dk_.ptr, dv.ptr, 1, D))
     assert np.array_equal(panel.numpy().reshape(-1)[:3 * D], np.concatenate([wq[0], wk[0], wv[0]]))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,M", [(65537, 32771), (262147, 32772)])
+def test_binary_and_reductions_beyond_2_31_elements(hip, oracle, N, M):
+    """An outer sum a[N,1] + b[1,M] whose work-item count passes 2^31 takes the 64-bit index path of
+    the broadcasting kernel (one element per item for the odd M, four for the other: 8.6 and 34 GB
+    of output).  The result is checked on the device: max and min are exact functions of the
+    operands, the total is M*sum(a) + N*sum(b), and a window around flat index 2^31 is read back."""
+    say("binary beyond 2^31", N, M)
+    assert N * M // (4 if M % 4 == 0 else 1) > 2 ** 31
+    oracle.seed(77)
+    a, b = oracle.uniform((N, 1), -1, 1), oracle.uniform((1, M), -1, 1)
+    out_shape = (C.c_int64 * 2)(N, M)
+    da, db, out = hip.array(a), hip.array(b), hip.empty((N, M))
+    hip.check(hip.L.axhip_binary(0, da.ptr, db.ptr, out.ptr, 2, out_shape, (C.c_int64 * 2)(1, 0), (C.c_int64 * 2)(0, 1)))
+    one = hip.empty((1,))
+    hip.check(hip.L.axhip_reduce_all(2, out.ptr, N * M, one.ptr))
+    assert one.numpy()[0] == np.float32(a.max() + b.max())
+    hip.check(hip.L.axhip_reduce_all(3, out.ptr, N * M, one.ptr))
+    assert one.numpy()[0] == np.float32(a.min() + b.min())
+    hip.check(hip.L.axhip_reduce_all(0, out.ptr, N * M, one.ptr))
+    want = M * a.astype(np.float64).sum() + N * b.astype(np.float64).sum()
+    bound = SUM_BOUND * (M * np.abs(a).astype(np.float64).sum() + N * np.abs(b).astype(np.float64).sum())
+    assert abs(float(one.numpy()[0]) - want) <= bound
+    rows = hip.empty((N,))
+    hip.check(hip.L.axhip_reduce_axis(2, out.ptr, N, M, 1, rows.ptr))
+    assert np.array_equal(rows.numpy(), (a + b.max()).reshape(-1))
+    # rows around flat index 2^31
+    r0 = 2 ** 31 // M - 1
+    window = np.empty((3, M), np.float32)
+    hip.check(hip.L.axhip_memcpy_d2h(window.ctypes.data, out.ptr + r0 * M * 4, window.nbytes))
+    assert np.array_equal(window, a[r0:r0 + 3] + b)
