@@ -23,6 +23,10 @@ void *workspace(size_t bytes);
 // `n` zero-initialised device ints owned by the runtime.  Kernels that use them as arrival counters
 // leave them at zero when they finish.
 int *strip_counters(size_t n);
+// The allocation pool behind axhip_malloc / axhip_free: the size class of a request, and the call
+// that hands every cached block back to the driver.
+size_t pool_class(size_t bytes);
+void pool_release_all();
 // At least `n` device floats, all 1.0f, owned by the runtime (grown on demand).
 float *ones_vector(size_t n);
 

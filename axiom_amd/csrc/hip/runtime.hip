@@ -3,6 +3,10 @@
 #include <cstdio>
 #include <cstring>
 
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
 #include "common.h"
 
 namespace {
@@ -18,6 +22,14 @@ int *g_ctr = nullptr;
 size_t g_ctr_n = 0;
 float *g_ones = nullptr;
 size_t g_ones_n = 0;
+
+// allocation pool: block -> rounded size for everything handed out, and the free blocks per size
+std::mutex g_pool_mutex;
+std::unordered_map<void *, size_t> g_pool_size;
+std::unordered_map<size_t, std::vector<void *>> g_pool_free;
+size_t g_pool_cached = 0;
+constexpr size_t kPoolMaxBlock = size_t(1) << 30;        // larger blocks go straight back to the driver
+constexpr size_t kPoolMaxCached = size_t(16) << 30;      // bytes the pool may hold back
 }  // namespace
 
 namespace axhip {
@@ -31,6 +43,33 @@ int fail(int code, const char *fmt, ...) {
 }
 
 int cu_count() { return g_cu_count; }
+
+// sizes are rounded so that blocks get reused: powers of two up to 1 MiB, then multiples of 1 MiB
+size_t pool_class(size_t bytes) {
+    if (bytes <= (size_t(1) << 20)) {
+        size_t c = 256;
+        while (c < bytes) c <<= 1;
+        return c;
+    }
+    const size_t mib = size_t(1) << 20;
+    return (bytes + mib - 1) / mib * mib;
+}
+
+// returns every cached block to the driver (out of memory, shutdown)
+void pool_release_all() {
+    std::vector<void *> blocks;
+    {
+        std::lock_guard<std::mutex> lock(g_pool_mutex);
+        for (auto &kv : g_pool_free)
+            for (void *p : kv.second) {
+                blocks.push_back(p);
+                g_pool_size.erase(p);
+            }
+        g_pool_free.clear();
+        g_pool_cached = 0;
+    }
+    for (void *p : blocks) (void)hipFree(p);
+}
 
 void note_kernel(const char *name) { t_kernel = name; }
 
@@ -139,6 +178,7 @@ int axhip_init(void) {
 void axhip_shutdown(void) {
     if (!g_ready) return;
     (void)hipDeviceSynchronize();
+    axhip::pool_release_all();
     if (g_ws) (void)hipFree(g_ws);
     if (g_ctr) (void)hipFree(g_ctr);
     if (g_ones) (void)hipFree(g_ones);
@@ -161,16 +201,49 @@ const char *axhip_last_error(void) { return t_err; }
 const char *axhip_device_name(void) { return g_name; }
 const char *axhip_last_kernel(void) { return t_kernel; }
 
-void *axhip_malloc(size_t bytes) {
+// Device allocations go through a pool: a freed block is kept, keyed by its rounded size, and
+// handed out again without a trip to the driver.  hipMalloc costs tens of microseconds and
+// hipFree waits for the whole device, which is several times the run time of the bs=1 kernels
+// whose outputs the host core allocates and releases on every call.  Reuse is safe because all
+// work runs in issue order on one stream: whatever still reads a released block was enqueued
+// before whatever writes its next owner.  Blocks above 1 GiB are returned to the driver at once;
+// when the driver is out of memory the pool is emptied and the request retried.
+static void *pool_take(size_t bytes) {
     if (axhip::ensure_ready()) return nullptr;
-    void *p = nullptr;
     if (bytes == 0) bytes = 4;
-    if (hipMalloc(&p, bytes) != hipSuccess) {
-        fail(AXHIP_ERR_ALLOC, "hipMalloc(%zu) failed", bytes);
-        return nullptr;
+    const size_t size = axhip::pool_class(bytes);
+    void *p = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_pool_mutex);
+        auto it = g_pool_free.find(size);
+        if (it != g_pool_free.end() && !it->second.empty()) {
+            p = it->second.back();
+            it->second.pop_back();
+            g_pool_cached -= size;
+        }
     }
-    if (hipMemsetAsync(p, 0, bytes, axhip::kStream) != hipSuccess) {
-        (void)hipFree(p);
+    if (!p) {
+        if (hipMalloc(&p, size) != hipSuccess) {
+            (void)hipGetLastError();
+            axhip::pool_release_all();
+            if (hipMalloc(&p, size) != hipSuccess) {
+                (void)hipGetLastError();
+                fail(AXHIP_ERR_ALLOC, "hipMalloc(%zu) failed", size);
+                return nullptr;
+            }
+        }
+        std::lock_guard<std::mutex> lock(g_pool_mutex);
+        g_pool_size[p] = size;
+    }
+    return p;
+}
+
+void *axhip_malloc_uninit(size_t bytes) { return pool_take(bytes); }
+
+void *axhip_malloc(size_t bytes) {
+    void *p = pool_take(bytes);
+    if (p && bytes && hipMemsetAsync(p, 0, bytes, axhip::kStream) != hipSuccess) {
+        axhip_free(p);
         fail(AXHIP_ERR_BACKEND, "zero-fill of %zu bytes failed", bytes);
         return nullptr;
     }
@@ -178,7 +251,21 @@ void *axhip_malloc(size_t bytes) {
 }
 
 void axhip_free(void *p) {
-    if (p) (void)hipFree(p);
+    if (!p) return;
+    size_t size = 0;
+    {
+        std::lock_guard<std::mutex> lock(g_pool_mutex);
+        auto it = g_pool_size.find(p);
+        if (it == g_pool_size.end()) return;             // not ours (or freed twice): leave it alone
+        size = it->second;
+        if (size <= kPoolMaxBlock && g_pool_cached + size <= kPoolMaxCached) {
+            g_pool_free[size].push_back(p);
+            g_pool_cached += size;
+            return;
+        }
+        g_pool_size.erase(it);
+    }
+    (void)hipFree(p);
 }
 
 int axhip_memset(void *p, int v, size_t bytes) {

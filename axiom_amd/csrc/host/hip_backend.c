@@ -491,6 +491,11 @@ static void *hook_alloc(size_t bytes) {
     if (!p) ax_err_set(AX_ERR_ALLOC, "hip storage_alloc(%zu): %s", bytes, axhip_last_error());
     return p;
 }
+static void *hook_alloc_uninit(size_t bytes) {
+    void *p = axhip_malloc_uninit(bytes);
+    if (!p) ax_err_set(AX_ERR_ALLOC, "hip storage_alloc(%zu): %s", bytes, axhip_last_error());
+    return p;
+}
 static void hook_free(void *p) { axhip_free(p); }
 static ax_status_t hook_h2d(void *d, const void *s, size_t n) { return lift(axhip_memcpy_h2d(d, s, n), "hip memcpy_h2d"); }
 static ax_status_t hook_d2h(void *d, const void *s, size_t n) { return lift(axhip_memcpy_d2h(d, s, n), "hip memcpy_d2h"); }
@@ -515,7 +520,7 @@ static ax_status_t hook_d2d(void *d, const void *s, size_t n) { return lift(axhi
         .synchronize = hook_synchronize, .device_count = hook_device_count,                     \
         .storage_alloc = hook_alloc, .storage_free = hook_free, .memcpy_h2d = hook_h2d,         \
         .memcpy_d2h = hook_d2h, .memcpy_d2d = hook_d2d, .gemm_bias_act = hip_gemm_bias_act,     \
-        .layernorm_fwd = hip_layernorm_fwd,                                                     \
+        .layernorm_fwd = hip_layernorm_fwd, .storage_alloc_uninit = hook_alloc_uninit,          \
     }
 
 const ax_backend_ops_t ax_hip_ops = AX_HIP_OPS_INIT(AX_DEVICE_HIP);

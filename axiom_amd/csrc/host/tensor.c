@@ -15,7 +15,8 @@ void ax_set_default_device(ax_device_t dev) { tl_default_device = dev; }
 ax_device_t ax_get_default_device(void) { return tl_default_device; }
 void ax_set_seed(unsigned int seed) { ax_rng_seed((uint64_t)seed); }
 
-ax_storage_t *ax_storage_create(size_t size_bytes, ax_device_t device) {
+/* zeroed = false: the caller overwrites everything (host memory is never cleared here either way) */
+static ax_storage_t *storage_create(size_t size_bytes, ax_device_t device, bool zeroed) {
     ax_storage_t *s = calloc(1, sizeof *s);
     if (!s) {
         ax_err_set(AX_ERR_ALLOC, "ax_storage_create: out of memory");
@@ -32,7 +33,9 @@ ax_storage_t *ax_storage_create(size_t size_bytes, ax_device_t device) {
             free(s);
             return NULL;
         }
-        s->data = ops->storage_alloc(size_bytes);   /* the hook reports its own failure */
+        /* the hooks report their own failures */
+        s->data = (!zeroed && ops->storage_alloc_uninit) ? ops->storage_alloc_uninit(size_bytes)
+                                                         : ops->storage_alloc(size_bytes);
     }
     if (!s->data) {
         free(s);
@@ -45,6 +48,8 @@ ax_storage_t *ax_storage_create(size_t size_bytes, ax_device_t device) {
     s->generation = 1;
     return s;
 }
+
+ax_storage_t *ax_storage_create(size_t size_bytes, ax_device_t device) { return storage_create(size_bytes, device, true); }
 
 void ax_storage_retain(ax_storage_t *s) {
     if (s) atomic_fetch_add(&s->refcount, 1);
@@ -82,7 +87,7 @@ static void set_contiguous(ax_tensor_t *t, const int64_t *shape, int ndim) {
     }
 }
 
-ax_tensor_t *ax_tensor_create(const int64_t *shape, int ndim, ax_dtype_t dtype) {
+static ax_tensor_t *tensor_create(const int64_t *shape, int ndim, ax_dtype_t dtype, bool zeroed) {
     if (!shape || ndim < 0 || ndim > AX_MAX_DIMS) {
         ax_err_set(AX_ERR_INVALID_SHAPE, "tensor_create: bad shape (ndim=%d)", ndim);
         return NULL;
@@ -98,7 +103,7 @@ ax_tensor_t *ax_tensor_create(const int64_t *shape, int ndim, ax_dtype_t dtype) 
         ax_err_set(AX_ERR_ALLOC, "tensor_create: out of memory");
         return NULL;
     }
-    t->storage = ax_storage_create((size_t)n * esz, tl_default_device);
+    t->storage = storage_create((size_t)n * esz, tl_default_device, zeroed);
     if (!t->storage) {
         free(t);
         return NULL;
@@ -106,6 +111,10 @@ ax_tensor_t *ax_tensor_create(const int64_t *shape, int ndim, ax_dtype_t dtype) 
     t->dtype = dtype;
     set_contiguous(t, shape, ndim);
     return t;
+}
+
+ax_tensor_t *ax_tensor_create(const int64_t *shape, int ndim, ax_dtype_t dtype) {
+    return tensor_create(shape, ndim, dtype, false);
 }
 
 static ax_status_t write_from_host(ax_tensor_t *t, const void *src, size_t bytes) {
@@ -124,7 +133,7 @@ static ax_status_t write_from_host(ax_tensor_t *t, const void *src, size_t bytes
 }
 
 ax_tensor_t *ax_tensor_zeros(const int64_t *shape, int ndim, ax_dtype_t dtype) {
-    ax_tensor_t *t = ax_tensor_create(shape, ndim, dtype);
+    ax_tensor_t *t = tensor_create(shape, ndim, dtype, true);
     if (!t) return NULL;
     /* device allocations arrive zero-filled from storage_alloc; host memory is cleared here */
     if (t->storage->device == AX_DEVICE_CPU) memset(t->storage->data, 0, t->storage->size_bytes);

@@ -21,6 +21,7 @@ SIGNATURES = {
     "axhip_last_error": (C.c_char_p, []),
     "axhip_device_name": (C.c_char_p, []),
     "axhip_malloc": (vp, [C.c_size_t]),
+    "axhip_malloc_uninit": (vp, [C.c_size_t]),
     "axhip_free": (None, [vp]),
     "axhip_memset": (C.c_int, [vp, C.c_int, C.c_size_t]),
     "axhip_memcpy_h2d": (C.c_int, [vp, vp, C.c_size_t]),

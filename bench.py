@@ -267,6 +267,43 @@ def secondary(hip):
     rate("adam_update", 7 * full, lambda: hip.check(hip.L.axhip_adam_update(xa.ptr, xb.ptr, xo.ptr, m2.ptr, R * Dm, 1e-3, 0.9,
                                                                             0.999, 1e-8, 0.01, 0.1, 0.001, 1)))
     res["streaming_slots_16384x4096"] = stream
+    del xa, xb, xo, vec, rowv, colv, m2
+
+    # config 1 again, end to end through the public API the reference's users call: ax_layer_forward of a
+    # Sequential (Dense 784-4096-4096-10 with ReLU) on a device tensor, output tensor created and destroyed
+    # every call — so this figure includes the host code and the device allocator, not only the kernels
+    from axiom_amd.axiom import Axiom
+    ax = Axiom()
+    L = ax.L
+    if L.ax_init() == 0:
+        L.ax_set_default_device(2)
+        L.ax_set_seed(1)
+        seq = L.ax_sequential_create()
+        for (i, o, relu) in ((784, 4096, True), (4096, 4096, True), (4096, 10, False)):
+            L.ax_sequential_add(seq, L.ax_dense_create(i, o, True))
+            if relu:
+                L.ax_sequential_add(seq, L.ax_relu_layer_create())
+        api = {}
+        for M in (1, 8):
+            tx = ax.from_numpy(rng.uniform(0, 1, (M, 784)).astype(np.float32))
+
+            def forward():
+                y = L.ax_layer_forward(seq, tx)
+                L.ax_tensor_destroy(y)
+
+            for _ in range(50):
+                forward()
+            hip.sync()
+            n = 2000
+            t0 = time.perf_counter()
+            for _ in range(n):
+                forward()
+            hip.sync()
+            api[f"M{M}_us_per_forward"] = (time.perf_counter() - t0) * 1e6 / n
+            ax.free(tx)
+        L.ax_layer_destroy(seq)
+        L.ax_set_default_device(0)
+        res["mlp3_through_ax_layer_forward"] = api
     return res
 
 

@@ -49,8 +49,11 @@ const char *axhip_device_name(void);          /* gcnArchName of device 0, "" wit
 
 /* ---- memory: .storage_alloc/.storage_free/.memcpy_* hooks
  *      (src/compute/backends/cuda/memory.cu:78-140).  axhip_malloc returns zero-filled
- *      memory like the reference's allocator (memory.cu:90), or NULL. ---------------- */
+ *      memory like the reference's allocator (memory.cu:90), or NULL.  Blocks are pooled: axhip_free
+ *      keeps a block (up to 1 GiB each, 16 GiB in all) for the next request of its size class, and
+ *      neither call waits for the device; axhip_shutdown returns everything to the driver. ------ */
 void *axhip_malloc(size_t bytes);
+void *axhip_malloc_uninit(size_t bytes);   /* contents undefined: for results that are fully overwritten */
 void  axhip_free(void *device_ptr);
 int   axhip_memset(void *device_ptr, int byte_value, size_t bytes);
 int   axhip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes);

@@ -7,8 +7,8 @@
  * reference's offsets and tests/test_host_core.py compares them with this header.
  * Any slot may be NULL; dispatch answers AX_ERR_NOT_IMPLEMENTED for those.
  *
- * Two slots are appended after the reference's last member (gemm_bias_act, layernorm_fwd); the
- * reference never reads that far, this repository's dispatch layer does. */
+ * Three slots are appended after the reference's last member (gemm_bias_act, layernorm_fwd,
+ * storage_alloc_uninit); the reference never reads that far, this repository's host core does. */
 #ifndef AX_INTERNAL_BACKEND_OPS_H
 #define AX_INTERNAL_BACKEND_OPS_H
 
@@ -114,6 +114,10 @@ struct ax_backend_ops {
      * inv_std (one value per row) are the tensors its backward pass keeps, either may be NULL */
     ax_status_t (*layernorm_fwd)(ax_tin_t x, ax_tin_t gamma, ax_tin_t beta, float eps, ax_tout_t out,
                                  ax_tout_t x_hat, ax_tout_t inv_std);
+    /* storage_alloc without the zero fill, for ax_tensor_create, whose contents are undefined by
+     * contract (include/axiom/tensor.h of the reference): an operator's result is overwritten in
+     * full, and a fill launch per result is a sizeable share of a bs=1 layer's time */
+    void *(*storage_alloc_uninit)(size_t size_bytes);
 };
 
 /* The MI355X backend.  `device` is AX_DEVICE_HIP. */

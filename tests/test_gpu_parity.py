@@ -863,3 +863,34 @@ def test_binary_and_reductions_beyond_2_31_elements(hip, oracle, N, M):
     window = np.empty((3, M), np.float32)
     hip.check(hip.L.axhip_memcpy_d2h(window.ctypes.data, out.ptr + r0 * M * 4, window.nbytes))
     assert np.array_equal(window, a[r0:r0 + 3] + b)
+
+
+@pytest.mark.gpu
+def test_allocation_pool(hip):
+    """Freed blocks come back for the next request of their size class, zero-filled, with earlier
+    work on them finished first (one stream); foreign pointers and double frees are ignored."""
+    say("allocation pool")
+    a = hip.empty((1000,))
+    p = a.ptr
+    hip.check(hip.L.axhip_fill_f32(p, 3.0, 1000))
+    del a                                                      # DeviceArray.__del__ -> axhip_free
+    b = hip.empty((1024,))                                     # same 4 KiB class
+    assert b.ptr == p and not b.numpy().any()
+    c = hip.empty((1024,))
+    assert c.ptr != p
+    hip.L.axhip_free(p + 16)                                   # not a block of ours
+    hip.L.axhip_free(None)
+    big = [hip.empty((1 << 28,)) for _ in range(3)]            # 1 GiB each: still pooled
+    ptrs = {x.ptr for x in big}
+    del big
+    again = [hip.empty((1 << 28,)) for _ in range(3)]
+    assert {x.ptr for x in again} == ptrs
+    assert not again[0].numpy()[::4097].any()
+    del again
+    huge = hip.empty(((1 << 28) + (1 << 20),))                 # above 1 GiB: not kept
+    hp = huge.ptr
+    hip.check(hip.L.axhip_fill_f32(hp, 1.0, 16))
+    del huge
+    out = hip.empty((16,))
+    hip.check(hip.L.axhip_fill_f32(out.ptr, 2.0, 16))
+    assert np.array_equal(out.numpy(), np.full(16, 2.0, np.float32))
