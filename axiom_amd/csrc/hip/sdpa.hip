@@ -20,7 +20,7 @@
 // pitch (or, for dk = 32, a row order) that puts the two lane halves of a fragment read (keys 4
 // apart) on different banks.
 //
-// Every other shape: scores through a workspace, one batched NT GEMM, a row softmax kernel and
+// Every other head size: scores through a workspace, one batched NT GEMM, a row softmax kernel and
 // one batched NN GEMM over as many heads at a time as fit 256 MiB (the structure of
 // ax_cuda_sdpa_fwd, cuda/ops_attention.cu:299-392).
 #include "common.h"
@@ -69,7 +69,10 @@ struct SdGeom {
     }
 };
 
-template <int DK, bool CAUSAL>
+// RAG: S is not a multiple of 128.  Rows past the end of a head are never loaded (the load of such
+// a row is redirected to the head's last row, which keeps V finite), keys past the end are masked
+// like causal ones, and queries past the end are computed but not stored.
+template <int DK, bool CAUSAL, bool RAG>
 __global__ void __launch_bounds__(256)
 k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__restrict__ V,
        float *__restrict__ O, float *__restrict__ L, int64_t BH, int64_t S, float scale_log2e) {
@@ -80,7 +83,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int frow = lane & 31, fhalf = lane >> 5;
-    const int64_t nq = S / SD_BQ;
+    const int64_t nq = (S + SD_BQ - 1) / SD_BQ;
     // Workgroups are handed to the 8 XCDs round-robin by linear index, and inside an XCD to its
     // CUs in a fixed rotation, so every workgroup has to carry the same amount of work.  Eight
     // heads form a group: workgroup r of a group works on head r % 8 (every query tile of a
@@ -106,6 +109,18 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
         const int vrow = G::RPI * (4 * i + wave) + G::v_row_of_slot(slot);
         voff[i] = (unsigned)(vrow * G::ROWB + (c << 4));
     }
+    // the same offsets for a 64-row block of which only the first `valid` (1..63) rows exist: the
+    // LDS slot (and so the swizzle) stays that of the nominal row, the source row is the last one
+    auto koff_clamped = [&](int i, int valid) {
+        const int slot = lane / G::CH, c = lane % G::CH;
+        const int krow = G::RPI * (4 * i + wave) + slot;
+        return (unsigned)((krow < valid ? krow : valid - 1) * G::ROWB + ((c ^ G::swz(krow)) << 4));
+    };
+    auto voff_clamped = [&](int i, int valid) {
+        const int slot = lane / G::CH, c = lane % G::CH;
+        const int vrow = G::RPI * (4 * i + wave) + G::v_row_of_slot(slot);
+        return (unsigned)((vrow < valid ? vrow : valid - 1) * G::ROWB + (c << 4));
+    };
 
     for (int pass = 0; pass < passes; pass++) {
         const int64_t q0 = (CAUSAL && pass == 0 ? nq - 1 - unit : unit) * SD_BQ;
@@ -113,25 +128,53 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
         // ---- Q tile (128 rows) through the V area, then into registers; the first key block's
         // K rows stream into their own stage at the same time, so a workgroup pays one load
         // latency, not two, before its first MFMA.  Its V rows follow once Q has left the V area.
-        const int64_t nblocks = CAUSAL ? (q0 + SD_BQ) / SD_BKV : S / SD_BKV;
+        const int64_t all_blocks = (S + SD_BKV - 1) / SD_BKV;
+        const int64_t nblocks = CAUSAL && (q0 + SD_BQ) / SD_BKV < all_blocks ? (q0 + SD_BQ) / SD_BKV : all_blocks;
         constexpr unsigned Q_BASE = 2 * G::KSTAGE;   // 2 * KSTAGE bytes of Q fit the two V stages
         static_assert(2 * G::KSTAGE <= 2 * G::VSTAGE, "Q staging area");
         auto issue_k = [&](int64_t blk, int stage) {
             const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * DK);
+            const int64_t valid = S - blk * SD_BKV;
+            if (RAG && valid < SD_BKV) {
 #pragma unroll
-            for (int i = 0; i < G::IPW; i++) AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
+                for (int i = 0; i < G::IPW; i++)
+                    AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff_clamped(i, (int)valid), kg);
+            } else {
+#pragma unroll
+                for (int i = 0; i < G::IPW; i++) AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
+            }
         };
         auto issue_v = [&](int64_t blk, int stage) {
             const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * DK);
+            const int64_t valid = S - blk * SD_BKV;
+            if (RAG && valid < SD_BKV) {
 #pragma unroll
-            for (int i = 0; i < G::IPW; i++)
-                AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff[i], vg);
+                for (int i = 0; i < G::IPW; i++)
+                    AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff_clamped(i, (int)valid), vg);
+            } else {
+#pragma unroll
+                for (int i = 0; i < G::IPW; i++)
+                    AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff[i], vg);
+            }
         };
+        if (RAG && q0 + SD_BQ > S) {
+            // a half with no row inside the head re-reads the first half (its queries are never stored)
+            const int64_t valid0 = S - q0 < 64 ? S - q0 : 64, left1 = S - q0 - 64;
+            const int64_t base1 = left1 > 0 ? q0 + 64 : q0, valid1 = left1 > 0 ? (left1 < 64 ? left1 : 64) : valid0;
 #pragma unroll
-        for (int i = 0; i < G::IPW; i++) {
-            AXS_LOAD_LDS(lds0 + Q_BASE + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * DK));
-            AXS_LOAD_LDS(lds0 + Q_BASE + G::KSTAGE + (4 * i + wave) * 1024, koff[i],
-                         reinterpret_cast<const char *>(Qh + (q0 + 64) * DK));
+            for (int i = 0; i < G::IPW; i++) {
+                AXS_LOAD_LDS(lds0 + Q_BASE + (4 * i + wave) * 1024, koff_clamped(i, (int)valid0),
+                             reinterpret_cast<const char *>(Qh + q0 * DK));
+                AXS_LOAD_LDS(lds0 + Q_BASE + G::KSTAGE + (4 * i + wave) * 1024, koff_clamped(i, (int)valid1),
+                             reinterpret_cast<const char *>(Qh + base1 * DK));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < G::IPW; i++) {
+                AXS_LOAD_LDS(lds0 + Q_BASE + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * DK));
+                AXS_LOAD_LDS(lds0 + Q_BASE + G::KSTAGE + (4 * i + wave) * 1024, koff[i],
+                             reinterpret_cast<const char *>(Qh + (q0 + 64) * DK));
+            }
         }
         issue_k(0, 0);
         AXS_VM0();
@@ -171,9 +214,12 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
             // causal: a 32-key tile entirely above this wave's 32 queries is skipped, and only
             // blocks that straddle the diagonal pay for the mask (all wave-uniform decisions)
             const int64_t kb0 = blk * SD_BKV, wq_lo = q0 + wave * 32;
-            const bool tile_on[2] = {!CAUSAL || kb0 <= wq_lo + 31, !CAUSAL || kb0 + 32 <= wq_lo + 31};
-            const bool need_mask = CAUSAL && kb0 + SD_BKV - 1 > wq_lo;
-            const int qrel = (int)(qg - kb0);         // keys of this block with index > qrel are masked
+            const bool tile_on[2] = {!CAUSAL || kb0 <= wq_lo + 31,
+                                     (!CAUSAL || kb0 + 32 <= wq_lo + 31) && (!RAG || kb0 + 32 < S)};
+            const bool need_mask = (CAUSAL && kb0 + SD_BKV - 1 > wq_lo) || (RAG && !CAUSAL && kb0 + SD_BKV > S);
+            // keys of this block with index > qrel are masked: those after the query (causal; such a
+            // query lies inside the head, so they cover the keys past its end too) or past the end
+            const int qrel = (int)((CAUSAL ? qg : S - 1) - kb0);
 
             // ---- scores of 64 keys ----
             v16f acc_s[2];
@@ -208,7 +254,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     float s = acc_s[kt][v];
-                    if (CAUSAL && (!tile_on[kt] || (need_mask && kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3) > qrel)))
+                    if ((CAUSAL || RAG) && (!tile_on[kt] || (need_mask && kt * 32 + 8 * (v >> 2) + 4 * fhalf + (v & 3) > qrel)))
                         s = -INFINITY;
                     acc_s[kt][v] = s;
                     m_blk = fmaxf(m_blk, s);
@@ -261,16 +307,18 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
         const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
         const float inv = 1.0f / l_tot;
         float *orow = O + (head * S + qg) * DK;
+        if (!RAG || qg < S) {
 #pragma unroll
-        for (int d = 0; d < DT; d++)
+            for (int d = 0; d < DT; d++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                v4f r;
+                for (int g = 0; g < 4; g++) {
+                    v4f r;
 #pragma unroll
-                for (int e = 0; e < 4; e++) r[e] = acc_o[d][4 * g + e] * inv;
-                *reinterpret_cast<v4f *>(orow + d * 32 + 8 * g + 4 * fhalf) = r;
-            }
-        if (L && fhalf == 0) L[head * S + qg] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+                    for (int e = 0; e < 4; e++) r[e] = acc_o[d][4 * g + e] * inv;
+                    *reinterpret_cast<v4f *>(orow + d * 32 + 8 * g + 4 * fhalf) = r;
+                }
+            if (L && fhalf == 0) L[head * S + qg] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+        }
     }
 }
 
@@ -279,18 +327,23 @@ int launch_sdpa(const float *Q, const float *K, const float *V, float *O, float 
                 float scale, int causal) {
     using G = SdGeom<DK>;
     static bool attr_set = false;
+    const void *kernels[4] = {reinterpret_cast<const void *>(k_sdpa<DK, false, false>),
+                              reinterpret_cast<const void *>(k_sdpa<DK, true, false>),
+                              reinterpret_cast<const void *>(k_sdpa<DK, false, true>),
+                              reinterpret_cast<const void *>(k_sdpa<DK, true, true>)};
     if (!attr_set) {
-        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sdpa<DK, false>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, G::SMEM), "hipFuncSetAttribute");
-        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sdpa<DK, true>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, G::SMEM), "hipFuncSetAttribute");
+        for (const void *k : kernels)
+            AXHIP_HIP_TRY(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, G::SMEM), "hipFuncSetAttribute");
         attr_set = true;
     }
     const float sl2 = scale * 1.4426950408889634f;
-    const int64_t nq = S / SD_BQ;
+    const int64_t nq = (S + SD_BQ - 1) / SD_BQ;
     dim3 grid((unsigned)((causal ? (nq + 1) / 2 : nq) * BH));
-    if (causal) hipLaunchKernelGGL((k_sdpa<DK, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
-    else hipLaunchKernelGGL((k_sdpa<DK, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
+    const bool rag = S % SD_BQ != 0;
+    if (causal && rag) hipLaunchKernelGGL((k_sdpa<DK, true, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
+    else if (causal) hipLaunchKernelGGL((k_sdpa<DK, true, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
+    else if (rag) hipLaunchKernelGGL((k_sdpa<DK, false, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
+    else hipLaunchKernelGGL((k_sdpa<DK, false, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
     return check_launch("sdpa_fwd");
 }
 
@@ -366,7 +419,7 @@ extern "C" int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, fl
     if (BH < 0 || S < 0 || dk <= 0) return fail(AXHIP_ERR_SHAPE, "sdpa_fwd: bad extent");
     if (BH == 0 || S == 0) return AXHIP_OK;
     const bool aligned = ((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O) & 15) == 0);
-    if ((dk == 32 || dk == 64 || dk == 128) && S % SD_BQ == 0 && aligned && S / SD_BQ * BH <= 0x7fffffff) {
+    if ((dk == 32 || dk == 64 || dk == 128) && aligned && (S + SD_BQ - 1) / SD_BQ * BH <= 0x7fffffff) {
         int rc;
         if (dk == 32) {
             rc = launch_sdpa<32>(Q, K, V, O, L, BH, S, scale, causal);

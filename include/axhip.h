@@ -195,8 +195,8 @@ int axhip_sgd_update(float *w, const float *g, float *momentum_buf, int64_t n, f
  * causal != 0: query i sees keys j <= i.  Replaces ax_cuda_sdpa_fwd
  * (cuda/ops_attention.cu:299-392) and the device form of ax_fused_attention_fwd /
  * ax_fused_attention_fwd_causal (include/axiom/attention.h:273-283,
- * src/core/fused_attention.c:559-573).  dk of 32, 64 or 128 with S a multiple of 128 runs fused (no
- * score matrix in memory); other shapes go through batched GEMMs and a row softmax. */
+ * src/core/fused_attention.c:559-573).  dk of 32, 64 or 128 (16-byte aligned tensors, any S) runs
+ * fused, with no score matrix in memory; other head sizes go through batched GEMMs and a row softmax. */
 int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L,
                    int64_t BH, int64_t S, int64_t dk, float scale, int causal);
 

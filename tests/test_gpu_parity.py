@@ -502,7 +502,9 @@ def run_sdpa(hip, q, k, v, scale, causal, want_l=True):
                                             (1, 129, 64, 1), (3, 384, 64, 1), (2, 77, 128, 0), (4, 512, 64, 0),
                                             (3, 128, 32, 0), (2, 256, 32, 1), (3, 128, 128, 0), (2, 256, 128, 1),
                                             (2, 384, 128, 0), (11, 640, 64, 1), (19, 256, 32, 0), (9, 512, 128, 1),
-                                            (17, 128, 64, 1)])
+                                            (17, 128, 64, 1), (3, 200, 64, 0), (2, 1000, 64, 1), (5, 63, 32, 0),
+                                            (2, 191, 128, 1), (9, 65, 64, 0), (2, 64, 64, 1), (3, 127, 32, 1),
+                                            (1, 897, 128, 0)])
 def test_sdpa_forward(hip, oracle, golden, BH, S, dk, causal):
     say("sdpa", BH, S, dk, causal)
     oracle.seed(5000 + BH * 100 + S + dk + causal)
