@@ -1,7 +1,7 @@
 // Scaled dot-product attention forward: O = softmax(scale * Q K^T [+ causal mask]) V per head,
 // Q, K, V, O [BH, S, dk] row-major fp32, L [BH, S] = log-sum-exp of each score row (or NULL).
 //
-// Fused kernel (dk = 32, 64 or 128, S a multiple of 128): the score matrix never leaves the chip.  A
+// Fused kernel (dk = 32, 64 or 128, any S): the score matrix never leaves the chip.  A
 // workgroup of 4 waves owns 128 query rows of one head, a wave 32 of them; keys and values
 // stream through LDS in blocks of 64 (direct-to-LDS loads, two stages).  Both products run on
 // v_mfma_f32_32x32x2_f32 with the query index on the MFMA's column side, so lane l of a wave
