@@ -644,6 +644,112 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
     return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
 }
 
+// ---- split-K for shapes with few output tiles -----------------------------------------
+// A GEMM with a handful of 64x64 tiles and a long K (M of 9..128 against a wide weight) would
+// occupy a handful of CUs.  It is run instead as a batched GEMM over `splits` equal K ranges —
+// the ranges are sub-matrices reached by pointer offsets, so the batched kernels above serve
+// unchanged — into a workspace of partial products, and one finishing pass adds the partials in
+// split order and applies alpha, beta, the column scale's sibling terms, bias and activation.
+// The order is fixed, so results do not vary from run to run.
+// One workgroup covers 256 / LANES neighbouring items (four columns each when VEC); lane l adds
+// the splits [l * per, (l + 1) * per) in order, with all its loads in flight together, and the
+// lanes' sums are then joined in lane order by lane 0.
+template <bool VEC, int LANES>
+__global__ void __launch_bounds__(256)
+k_splitk_finish(const float *__restrict__ part, int splits, int64_t M, int64_t N, float alpha, float beta,
+                const float *__restrict__ bias, int act, float *__restrict__ C, int64_t ldc) {
+    constexpr int ITEMS = 256 / LANES, W = VEC ? 4 : 1;
+    typedef float vw __attribute__((ext_vector_type(W)));
+    __shared__ vw sums[LANES][ITEMS];
+    const int lane = threadIdx.x / ITEMS, it = threadIdx.x % ITEMS;
+    const int64_t per_row = N / W, items = M * per_row;
+    const int64_t t = (int64_t)blockIdx.x * ITEMS + it;
+    const bool live = t < items;
+    const int64_t m = live ? t / per_row : 0, n = live ? (t - m * per_row) * W : 0;
+    const int per = (splits + LANES - 1) / LANES;
+    const int k0 = lane * per, k1 = min(splits, k0 + per);
+    vw s = 0.0f;
+    if (live) {
+        const float *p = part + m * N + n + (int64_t)k0 * M * N;
+        int k = k0;
+        for (; k + 4 <= k1; k += 4, p += 4 * M * N) {
+            const vw x0 = *reinterpret_cast<const vw *>(p), x1 = *reinterpret_cast<const vw *>(p + M * N),
+                     x2 = *reinterpret_cast<const vw *>(p + 2 * M * N), x3 = *reinterpret_cast<const vw *>(p + 3 * M * N);
+            s = (((s + x0) + x1) + x2) + x3;
+        }
+        for (; k < k1; k++, p += M * N) s += *reinterpret_cast<const vw *>(p);
+    }
+    sums[lane][it] = s;
+    __syncthreads();
+    if (lane != 0 || !live) return;
+#pragma unroll
+    for (int l = 1; l < LANES; l++) s += sums[l][it];
+    vw *dst = reinterpret_cast<vw *>(C + m * ldc + n);
+    vw r = s * alpha;
+    if (beta != 0.0f) r += *dst * beta;
+    if (bias) r += *reinterpret_cast<const vw *>(bias + n);
+#pragma unroll
+    for (int e = 0; e < W; e++) r[e] = apply_act(r[e], act);
+    *dst = r;
+}
+
+int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch);
+
+// how many K ranges to use (1: none).  Every range must be a whole number of 32-wide slabs.
+int64_t split_count(int64_t M, int64_t N, int64_t K) {
+    const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
+    const int64_t cus = cu_count();
+    if (tiles * 2 > cus || K < 256 || K % 32 != 0) return 1;
+    // One workgroup per CU measured best (32x768x768: 10.5 us against 27 unsplit; 64x1024x4096:
+    // 12 against 70; 128x4096x1024: 16.5 against 20); more ranges only add partial sums to move.
+    int64_t want = (cus + tiles - 1) / tiles;
+    if (want > K / 64) want = K / 64;                      // ranges of at least 64
+    for (int64_t s = want; s >= 2; s--)
+        if (K % (s * 32) == 0) return s;
+    return 1;
+}
+
+// returns -1 when the shape is left to the ordinary path
+template <typename BSRC>
+int try_split_k(const SgemmArgs &g, int transa, int transb, const char *name, const char *const i8_names[3]) {
+    const int64_t splits = split_count(g.M, g.N, g.K);
+    if (splits < 2 || splits > 65535) return -1;
+    const int64_t kr = g.K / splits;
+    float *part = static_cast<float *>(workspace((size_t)splits * g.M * g.N * sizeof(float)));
+    if (!part) return AXHIP_ERR_ALLOC;
+    SgemmArgs p = g;
+    p.K = kr;
+    p.C = part;
+    p.ldc = g.N;
+    p.stride_a = transa ? kr * g.lda : kr;                 // op(A) = [M, K]: the K index runs along rows of A^T
+    p.stride_b = transb ? kr : kr * g.ldb;
+    p.stride_c = g.M * g.N;
+    p.alpha = 1.0f;
+    p.beta = 0.0f;
+    p.bias = nullptr;
+    p.act = AXHIP_ACT_NONE;
+    int rc;
+    if (std::is_same<BSRC, float>::value) rc = dispatch_f32(p, transa, transb, splits);
+    else rc = pick_tile<true, true, int8_t>(i8_names, p, splits);
+    if (rc) return rc;
+    const bool vec = g.N % 4 == 0 && g.ldc % 4 == 0 && (((uintptr_t)g.C | (uintptr_t)g.bias) & 15) == 0;
+    const int64_t items = g.M * (vec ? g.N / 4 : g.N);
+    // enough workgroups for the chip: 16 split lanes over 16 items when the result is small
+    const bool wide = items >= 64 * 512 || splits < 8;
+    const int64_t blocks = (items + (wide ? 63 : 15)) / (wide ? 64 : 16);
+    if (blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "sgemm split-k: result too large");
+#define AX_FINISH(V, L)                                                                                     \
+    hipLaunchKernelGGL((k_splitk_finish<V, L>), dim3((unsigned)blocks), dim3(256), 0, kStream, part, (int)splits, \
+                       g.M, g.N, g.alpha, g.beta, g.bias, g.act, g.C, g.ldc)
+    if (vec && wide) AX_FINISH(true, 4);
+    else if (vec) AX_FINISH(true, 16);
+    else if (wide) AX_FINISH(false, 4);
+    else AX_FINISH(false, 16);
+#undef AX_FINISH
+    note_kernel(name);
+    return check_launch("sgemm split-k finish");
+}
+
 int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     static const char *const nn[3] = {"sgemm_nn_128x128", "sgemm_nn_64x64", "sgemm_nn_64x64_guarded"};
     static const char *const nt[3] = {"sgemm_nt_128x128", "sgemm_nt_64x64", "sgemm_nt_64x64_guarded"};
@@ -671,6 +777,8 @@ int sgemm_i8w(int64_t M, int64_t N, int64_t K, const float *a, const int8_t *w,
     static const char *const names[3] = {"qgemm_w8a32_mfma_128x128", "qgemm_w8a32_mfma_64x64",
                                          "qgemm_w8a32_mfma_64x64_guarded"};
     SgemmArgs g{a, w, out, M, N, K, K, K, N, 0, 0, 0, 1.0f, 0.0f, w_scales, nullptr, AXHIP_ACT_NONE};
+    const int rc = try_split_k<int8_t>(g, 0, 1, "qgemm_w8a32_mfma_splitk", names);
+    if (rc >= 0) return rc;
     return pick_tile<true, true, int8_t>(names, g, 1);
 }
 }  // namespace axhip
@@ -684,6 +792,10 @@ extern "C" int axhip_sgemm(int transa, int transb, int64_t M, int64_t N, int64_t
     if (M <= 8 && !transa && !transb && alpha == 1.0f && beta == 0.0f)
         return axhip_sgemm_skinny(M, N, K, A, lda, B, ldb, C, ldc, bias, act);
     SgemmArgs g{A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, alpha, beta, nullptr, bias, act};
+    if (!(transa && transb)) {
+        const int rc = try_split_k<float>(g, transa, transb, "sgemm_splitk", nullptr);
+        if (rc >= 0) return rc;
+    }
     return dispatch_f32(g, transa, transb, 1);
 }
 

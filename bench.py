@@ -269,6 +269,26 @@ def secondary(hip):
     res["streaming_slots_16384x4096"] = stream
     del xa, xb, xo, vec, rowv, colv, m2
 
+    # the seven shapes of the reference's benchmarks/bench_qgemm.c:76-82 (fp32 GEMM against W8A32 on the
+    # same weights), on device-resident operands, plus W8A8 with the activations quantized per tensor
+    qshapes = {}
+    for (M, N, K) in ((1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024),
+                      (64, 1024, 4096), (1, 4096, 4096)):
+        a = hip.array(rng.uniform(-1, 1, (M, K)).astype(np.float32))
+        wt = hip.array(rng.uniform(-1, 1, (K, N)).astype(np.float32))          # [K, N] for the fp32 GEMM
+        wq = hip.array(rand_i8(rng, (N, K)))
+        ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+        xq = hip.array(rand_i8(rng, (M, K)))
+        out = hip.empty((M, N))
+        _, t_fp = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm(0, 0, M, N, K, 1.0, a.ptr, K, wt.ptr, N, 0.0, out.ptr, N,
+                                                                      None, 0)))
+        _, t_q = time_calls(hip, lambda: hip.check(hip.L.axhip_qgemm_w8a32(a.ptr, wq.ptr, ws.ptr, out.ptr, M, N, K)))
+        _, t_8 = time_calls(hip, lambda: hip.check(hip.L.axhip_qgemm_w8a8(xq.ptr, 0.02, wq.ptr, ws.ptr, None, 0, out.ptr, None,
+                                                                         M, N, K)))
+        qshapes[f"{M}x{N}x{K}"] = {"fp32_us": t_fp * 1e3, "w8a32_us": t_q * 1e3, "w8a8_us": t_8 * 1e3,
+                                   "w8a32_speedup_over_fp32": t_fp / t_q, "w8a8_kernel": hip.last_kernel()}
+    res["bench_qgemm_shapes"] = qshapes
+
     # config 1 again, end to end through the public API the reference's users call: ax_layer_forward of a
     # Sequential (Dense 784-4096-4096-10 with ReLU) on a device tensor, output tensor created and destroyed
     # every call — so this figure includes the host code and the device allocator, not only the kernels

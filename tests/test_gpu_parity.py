@@ -110,7 +110,9 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               (128, 128, 64), (130, 260, 700), (256, 384, 512), (33, 40, 100), (96, 96, 96),
               (2048, 1024, 256),
               # shapes that take the 128x256 tile, and ones just short of it in N or in tile count
-              (2048, 4096, 64), (4096, 2176, 64), (4096, 1088, 32), (128, 64, 4096)]
+              (2048, 4096, 64), (4096, 2176, 64), (4096, 1088, 32), (128, 64, 4096),
+              # few output tiles and a long K: the split-K route (bench_qgemm.c shapes among them)
+              (32, 768, 768), (64, 1024, 4096), (128, 4096, 1024), (9, 100, 512), (16, 16, 8192), (70, 130, 1536)]
 
 
 @pytest.mark.parametrize("M,N,K", F32_SHAPES)
@@ -212,7 +214,7 @@ def test_sgemm_config0_1024_cube(hip, oracle, golden):
         assert np.array_equal(hip.sgemm(da, db).numpy(), c)
 
 
-@pytest.mark.parametrize("M,N,K", [(130, 200, 96), (256, 320, 96), (2048, 4096, 32)])
+@pytest.mark.parametrize("M,N,K", [(130, 200, 96), (256, 320, 96), (2048, 4096, 32), (64, 128, 2048), (33, 70, 512)])
 def test_sgemm_alpha_beta_bias_act(hip, oracle, M, N, K):
     say("sgemm epilogue", M, N, K)
     oracle.seed(21)
