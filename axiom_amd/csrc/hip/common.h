@@ -89,6 +89,41 @@ __device__ __forceinline__ void tile_of_batched_block(int tiles_m, int tiles_n, 
     tn = tile - tm * tiles_n;
 }
 
+// Sums NV per-lane values over the 64 lanes of a wave, all NV at once.  A butterfly per value
+// would cost 6 cross-lane moves each; here every step also halves the number of values a lane
+// carries (lane bit `off` decides which half it keeps, the other half goes to its partner), so NV
+// values cost about NV moves in total and end up spread over the lanes: afterwards v[0] of lane l
+// holds the wave-wide sum of value number l / (64 / NV).  The first two steps exchange 32- and
+// 16-lane rows with the swap instructions of this chip; later ones go through the cross-lane
+// network.  The association order is a fixed tree, the same for every value.
+template <int NV, typename T>
+__device__ __forceinline__ void wave_sum_spread(T (&v)[NV], int lane) {
+    static_assert(NV >= 1 && NV <= 64 && (NV & (NV - 1)) == 0 && sizeof(T) == 4, "power of two 32-bit values");
+    int n = NV;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        if (n > 1) {
+            const int half = n / 2;
+#pragma unroll
+            for (int i = 0; i < half; i++) {
+                if (off >= 16) {
+                    const unsigned a = __builtin_bit_cast(unsigned, v[i]), b = __builtin_bit_cast(unsigned, v[i + half]);
+                    const auto r = off == 32 ? __builtin_amdgcn_permlane32_swap(a, b, false, false)
+                                             : __builtin_amdgcn_permlane16_swap(a, b, false, false);
+                    v[i] = __builtin_bit_cast(T, (unsigned)r[0]) + __builtin_bit_cast(T, (unsigned)r[1]);
+                } else {
+                    const bool up = (lane & off) != 0;
+                    const T keep = up ? v[i + half] : v[i], send = up ? v[i] : v[i + half];
+                    v[i] = keep + __shfl_xor(send, off, 64);
+                }
+            }
+            n = half;
+        } else {
+            v[0] += __shfl_xor(v[0], off, 64);
+        }
+    }
+}
+
 // Write-back of one 32x32 MFMA result tile held in the layout "lane l owns row (l & 31), and
 // for g = 0..3 the four consecutive columns 8*g + 4*(l >> 5) + e": the wave turns the tile
 // through 4 KiB of LDS private to it so that each store instruction writes 8 rows of 128

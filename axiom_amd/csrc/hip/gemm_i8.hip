@@ -761,6 +761,67 @@ int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_s
     return check_launch("qgemm_w8a8_256x256_dma");
 }
 
+// ---- M <= 8: bandwidth-bound, no matrix cores ---------------------------------------------
+// One wave owns 4 weight rows.  Lanes walk K in 16-byte steps (a wave-wide load covers 1 KiB of a
+// row), keep the activation bytes of their k positions in registers across the 4 rows, and feed
+// four-byte integer dot products; the per-lane int32 sums are added over the wave, all 4 * M at
+// once, and end up one per lane for the write-back.  Integer
+// addition is exact in any order, so the accumulators equal the matrix-core kernels' bit for bit,
+// and the write-back applies the same expression to them.
+constexpr int GEMV_ROWS = 4;
+
+template <int MR>
+__global__ void __launch_bounds__(64)
+k_w8a8_gemv(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t N, int64_t K, float x_scale,
+            const float *__restrict__ w_scales, const float *__restrict__ bias, int act,
+            float *__restrict__ out, int32_t *__restrict__ acc_out) {
+    const int lane = threadIdx.x;
+    const int64_t n0 = (int64_t)blockIdx.x * GEMV_ROWS;
+    int acc[GEMV_ROWS][MR];
+#pragma unroll
+    for (int r = 0; r < GEMV_ROWS; r++)
+#pragma unroll
+        for (int m = 0; m < MR; m++) acc[r][m] = 0;
+    for (int64_t k = (int64_t)lane * 16; k < K; k += 64 * 16) {
+        v4i xa[MR];
+#pragma unroll
+        for (int m = 0; m < MR; m++) xa[m] = *reinterpret_cast<const v4i *>(X + m * K + k);
+#pragma unroll
+        for (int r = 0; r < GEMV_ROWS; r++) {
+            const int64_t n = n0 + r < N ? n0 + r : N - 1;   // the last wave re-reads a row it does not store
+            const v4i wv = __builtin_nontemporal_load(reinterpret_cast<const v4i *>(W + n * K + k));
+#pragma unroll
+            for (int m = 0; m < MR; m++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) acc[r][m] = __builtin_amdgcn_sdot4(xa[m][q], wv[q], acc[r][m], false);
+        }
+    }
+    constexpr int NV = GEMV_ROWS * MR <= 4 ? 4 : GEMV_ROWS * MR <= 8 ? 8 : GEMV_ROWS * MR <= 16 ? 16 : 32;
+    int v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) v[i] = i < GEMV_ROWS * MR ? acc[i / MR][i % MR] : 0;
+    wave_sum_spread(v, lane);
+    const int idx = lane / (64 / NV), r = idx / MR, m = idx % MR;
+    const int64_t n = n0 + r;
+    if (lane % (64 / NV) != 0 || idx >= GEMV_ROWS * MR || n >= N) return;
+    const int a = v[0];
+    if (acc_out) acc_out[m * N + n] = a;
+    if (out) {
+        const float f = (float)a, scale = x_scale * w_scales[n];
+        const float o = bias ? __builtin_fmaf(f, scale, bias[n]) : f * scale;
+        out[m * N + n] = apply_act(o, act);
+    }
+}
+
+template <int MR>
+int launch_gemv(const int8_t *x, float x_scale, const int8_t *w, const float *w_scales, const float *bias,
+                int act, float *out, int32_t *acc_out, int64_t N, int64_t K) {
+    note_kernel("qgemm_w8a8_gemv");
+    hipLaunchKernelGGL(k_w8a8_gemv<MR>, dim3((unsigned)((N + GEMV_ROWS - 1) / GEMV_ROWS)), dim3(64), 0, kStream, x, w,
+                       N, K, x_scale, w_scales, bias, act, out, acc_out);
+    return check_launch("qgemm_w8a8_gemv");
+}
+
 }  // namespace
 
 extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
@@ -774,6 +835,19 @@ extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
     if (act < AXHIP_ACT_NONE || act > AXHIP_ACT_GELU)
         return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: unknown activation %d", act);
     if (M == 0 || N == 0) return AXHIP_OK;
+    if (M <= 8 && K % 16 == 0 && K > 0 && ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) &&
+        (N + GEMV_ROWS - 1) / GEMV_ROWS <= 0x7fffffff) {
+        switch (M) {
+            case 1: return launch_gemv<1>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
+            case 2: return launch_gemv<2>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
+            case 3: return launch_gemv<3>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
+            case 4: return launch_gemv<4>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
+            case 5: return launch_gemv<5>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
+            case 6: return launch_gemv<6>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
+            case 7: return launch_gemv<7>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
+            default: return launch_gemv<8>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
+        }
+    }
     const bool aligned = ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) && (K % BK == 0) && K > 0;
     const bool vec_out = (!out || (((uintptr_t)out | (uintptr_t)w_scales | (uintptr_t)bias) & 15) == 0) &&
                          (((uintptr_t)acc_out & 15) == 0);

@@ -3,7 +3,7 @@
 // M <= 8 (the bandwidth-bound inference case): one wave owns 4 weight rows.  Lanes walk K in
 // 16-byte steps (a wave-wide load covers 1 KiB of one row), each lane keeps the activations of
 // its k positions in registers across the 4 rows, and the 4*M partial sums are reduced over
-// the wave with DPP-free xor shuffles in a fixed order.  Larger M goes through the fp32
+// the wave together, in a fixed tree order, ending one per lane for the write-back.  Larger M goes through the fp32
 // matrix-core GEMM with the int8 operand converted while it is staged in LDS.
 #include "common.h"
 
@@ -16,12 +16,6 @@ namespace {
 using namespace axhip;
 
 constexpr int ROWS = 4;   // weight rows per wave
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
 
 template <int MR, bool VEC>
 __global__ void __launch_bounds__(64)
@@ -76,16 +70,14 @@ k_w8a32_gemv(const float *__restrict__ a, const int8_t *__restrict__ w,
                 for (int e = 0; e < 16; e++) acc[r][m] = __builtin_fmaf(xa[m][e], wf[e], acc[r][m]);
         }
     }
+    constexpr int NV = ROWS * MR <= 4 ? 4 : ROWS * MR <= 8 ? 8 : ROWS * MR <= 16 ? 16 : 32;
+    float v[NV];
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-        const int64_t n = n0 + r;
-        if (n >= N) break;
-#pragma unroll
-        for (int m = 0; m < MR; m++) {
-            float s = wave_sum(acc[r][m]);
-            if (lane == 0) out[m * N + n] = s * w_scales[n];
-        }
-    }
+    for (int i = 0; i < NV; i++) v[i] = i < ROWS * MR ? acc[i / MR][i % MR] : 0.0f;
+    wave_sum_spread(v, lane);
+    const int idx = lane / (64 / NV), r = idx / MR, m = idx % MR;
+    if (lane % (64 / NV) != 0 || idx >= ROWS * MR || n0 + r >= N) return;
+    out[m * N + n0 + r] = v[0] * w_scales[n0 + r];
 }
 
 template <int MR>
