@@ -75,7 +75,8 @@ struct SdGeom {
 template <int DK, bool CAUSAL, bool RAG>
 __global__ void __launch_bounds__(256)
 k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__restrict__ V,
-       float *__restrict__ O, float *__restrict__ L, int64_t BH, int64_t S, float scale_log2e) {
+       float *__restrict__ O, float *__restrict__ L, int64_t BH, int64_t S, float scale_log2e,
+       int64_t H, int64_t ld, int64_t ldo) {
     using G = SdGeom<DK>;
     constexpr int KB = DK / 8;                   // 8-wide k-blocks of the score product
     constexpr int DT = DK / 32;                  // 32-wide column tiles of the output
@@ -95,7 +96,13 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
     const int64_t r = lin - group * 8 * units, hpg = left < 8 ? left : 8;
     const int64_t head = group * 8 + r % hpg, unit = r / hpg;
     const int passes = (CAUSAL && unit != nq - 1 - unit) ? 2 : 1;
-    const float *Qh = Q + head * S * DK, *Kh = K + head * S * DK, *Vh = V + head * S * DK;
+    // head b * H + h starts at row b * S, column h * DK of matrices with row pitch ld (Q, K, V)
+    // and ldo (O): H = 1, ld = DK is one matrix per head; H heads side by side in rows of
+    // ld >= H * DK floats is the layout a fused projection writes and the output projection reads
+    const int64_t hb = head / H, hh = head - hb * H;
+    const int64_t in0 = hb * S * ld + hh * DK;
+    const float *Qh = Q + in0, *Kh = K + in0, *Vh = V + in0;
+    const unsigned rowb = (unsigned)ld * 4;      // bytes between rows in global memory
     const unsigned lds0 = (unsigned)(uintptr_t)lds;
 
     // per-lane byte offsets of the direct-to-LDS loads: instruction i of this wave is number
@@ -105,21 +112,21 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
     for (int i = 0; i < G::IPW; i++) {
         const int slot = lane / G::CH, c = lane % G::CH;
         const int krow = G::RPI * (4 * i + wave) + slot;
-        koff[i] = (unsigned)(krow * G::ROWB + ((c ^ G::swz(krow)) << 4));
+        koff[i] = (unsigned)(krow * rowb + ((c ^ G::swz(krow)) << 4));
         const int vrow = G::RPI * (4 * i + wave) + G::v_row_of_slot(slot);
-        voff[i] = (unsigned)(vrow * G::ROWB + (c << 4));
+        voff[i] = (unsigned)(vrow * rowb + (c << 4));
     }
     // the same offsets for a 64-row block of which only the first `valid` (1..63) rows exist: the
     // LDS slot (and so the swizzle) stays that of the nominal row, the source row is the last one
     auto koff_clamped = [&](int i, int valid) {
         const int slot = lane / G::CH, c = lane % G::CH;
         const int krow = G::RPI * (4 * i + wave) + slot;
-        return (unsigned)((krow < valid ? krow : valid - 1) * G::ROWB + ((c ^ G::swz(krow)) << 4));
+        return (unsigned)((krow < valid ? krow : valid - 1) * rowb + ((c ^ G::swz(krow)) << 4));
     };
     auto voff_clamped = [&](int i, int valid) {
         const int slot = lane / G::CH, c = lane % G::CH;
         const int vrow = G::RPI * (4 * i + wave) + G::v_row_of_slot(slot);
-        return (unsigned)((vrow < valid ? vrow : valid - 1) * G::ROWB + (c << 4));
+        return (unsigned)((vrow < valid ? vrow : valid - 1) * rowb + (c << 4));
     };
 
     for (int pass = 0; pass < passes; pass++) {
@@ -133,7 +140,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
         constexpr unsigned Q_BASE = 2 * G::KSTAGE;   // 2 * KSTAGE bytes of Q fit the two V stages
         static_assert(2 * G::KSTAGE <= 2 * G::VSTAGE, "Q staging area");
         auto issue_k = [&](int64_t blk, int stage) {
-            const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * DK);
+            const char *kg = reinterpret_cast<const char *>(Kh + blk * SD_BKV * ld);
             const int64_t valid = S - blk * SD_BKV;
             if (RAG && valid < SD_BKV) {
 #pragma unroll
@@ -145,7 +152,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
             }
         };
         auto issue_v = [&](int64_t blk, int stage) {
-            const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * DK);
+            const char *vg = reinterpret_cast<const char *>(Vh + blk * SD_BKV * ld);
             const int64_t valid = S - blk * SD_BKV;
             if (RAG && valid < SD_BKV) {
 #pragma unroll
@@ -164,16 +171,16 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
 #pragma unroll
             for (int i = 0; i < G::IPW; i++) {
                 AXS_LOAD_LDS(lds0 + Q_BASE + (4 * i + wave) * 1024, koff_clamped(i, (int)valid0),
-                             reinterpret_cast<const char *>(Qh + q0 * DK));
+                             reinterpret_cast<const char *>(Qh + q0 * ld));
                 AXS_LOAD_LDS(lds0 + Q_BASE + G::KSTAGE + (4 * i + wave) * 1024, koff_clamped(i, (int)valid1),
-                             reinterpret_cast<const char *>(Qh + base1 * DK));
+                             reinterpret_cast<const char *>(Qh + base1 * ld));
             }
         } else {
 #pragma unroll
             for (int i = 0; i < G::IPW; i++) {
-                AXS_LOAD_LDS(lds0 + Q_BASE + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * DK));
+                AXS_LOAD_LDS(lds0 + Q_BASE + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * ld));
                 AXS_LOAD_LDS(lds0 + Q_BASE + G::KSTAGE + (4 * i + wave) * 1024, koff[i],
-                             reinterpret_cast<const char *>(Qh + (q0 + 64) * DK));
+                             reinterpret_cast<const char *>(Qh + (q0 + 64) * ld));
             }
         }
         issue_k(0, 0);
@@ -306,7 +313,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
         // ---- normalise and write: lane owns query qg, dk columns 32*d + 8*g + 4*fhalf .. +3 ----
         const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
         const float inv = 1.0f / l_tot;
-        float *orow = O + (head * S + qg) * DK;
+        float *orow = O + (hb * S + qg) * ldo + hh * DK;
         if (!RAG || qg < S) {
 #pragma unroll
             for (int d = 0; d < DT; d++)
@@ -324,7 +331,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
 
 template <int DK>
 int launch_sdpa(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH, int64_t S,
-                float scale, int causal) {
+                float scale, int causal, int64_t H, int64_t ld, int64_t ldo) {
     using G = SdGeom<DK>;
     static bool attr_set = false;
     const void *kernels[4] = {reinterpret_cast<const void *>(k_sdpa<DK, false, false>),
@@ -340,10 +347,10 @@ int launch_sdpa(const float *Q, const float *K, const float *V, float *O, float 
     const int64_t nq = (S + SD_BQ - 1) / SD_BQ;
     dim3 grid((unsigned)((causal ? (nq + 1) / 2 : nq) * BH));
     const bool rag = S % SD_BQ != 0;
-    if (causal && rag) hipLaunchKernelGGL((k_sdpa<DK, true, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
-    else if (causal) hipLaunchKernelGGL((k_sdpa<DK, true, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
-    else if (rag) hipLaunchKernelGGL((k_sdpa<DK, false, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
-    else hipLaunchKernelGGL((k_sdpa<DK, false, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2);
+    if (causal && rag) hipLaunchKernelGGL((k_sdpa<DK, true, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, ldo);
+    else if (causal) hipLaunchKernelGGL((k_sdpa<DK, true, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, ldo);
+    else if (rag) hipLaunchKernelGGL((k_sdpa<DK, false, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, ldo);
+    else hipLaunchKernelGGL((k_sdpa<DK, false, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, ldo);
     return check_launch("sdpa_fwd");
 }
 
@@ -412,6 +419,23 @@ int sdpa_unfused(const float *Q, const float *K, const float *V, float *O, float
 
 }  // namespace
 
+// shared by both entry points: H heads side by side in rows of ld (Q, K, V) / ldo (O) floats
+static int sdpa_fused(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH, int64_t S,
+                      int64_t dk, float scale, int causal, int64_t H, int64_t ld, int64_t ldo) {
+    int rc;
+    if (dk == 32) {
+        rc = launch_sdpa<32>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo);
+        axhip::note_kernel(causal ? "sdpa_fused_dk32_causal" : "sdpa_fused_dk32");
+    } else if (dk == 64) {
+        rc = launch_sdpa<64>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo);
+        axhip::note_kernel(causal ? "sdpa_fused_dk64_causal" : "sdpa_fused_dk64");
+    } else {
+        rc = launch_sdpa<128>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo);
+        axhip::note_kernel(causal ? "sdpa_fused_dk128_causal" : "sdpa_fused_dk128");
+    }
+    return rc;
+}
+
 extern "C" int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH,
                               int64_t S, int64_t dk, float scale, int causal) {
     if (int rc = axhip::ensure_ready()) return rc;
@@ -419,19 +443,24 @@ extern "C" int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, fl
     if (BH < 0 || S < 0 || dk <= 0) return fail(AXHIP_ERR_SHAPE, "sdpa_fwd: bad extent");
     if (BH == 0 || S == 0) return AXHIP_OK;
     const bool aligned = ((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O) & 15) == 0);
-    if ((dk == 32 || dk == 64 || dk == 128) && aligned && (S + SD_BQ - 1) / SD_BQ * BH <= 0x7fffffff) {
-        int rc;
-        if (dk == 32) {
-            rc = launch_sdpa<32>(Q, K, V, O, L, BH, S, scale, causal);
-            axhip::note_kernel(causal ? "sdpa_fused_dk32_causal" : "sdpa_fused_dk32");
-        } else if (dk == 64) {
-            rc = launch_sdpa<64>(Q, K, V, O, L, BH, S, scale, causal);
-            axhip::note_kernel(causal ? "sdpa_fused_dk64_causal" : "sdpa_fused_dk64");
-        } else {
-            rc = launch_sdpa<128>(Q, K, V, O, L, BH, S, scale, causal);
-            axhip::note_kernel(causal ? "sdpa_fused_dk128_causal" : "sdpa_fused_dk128");
-        }
-        return rc;
-    }
+    if ((dk == 32 || dk == 64 || dk == 128) && aligned && (S + SD_BQ - 1) / SD_BQ * BH <= 0x7fffffff)
+        return sdpa_fused(Q, K, V, O, L, BH, S, dk, scale, causal, 1, dk, dk);
     return sdpa_unfused(Q, K, V, O, L, BH, S, dk, scale, causal);
+}
+
+extern "C" int axhip_sdpa_fwd_rows(const float *Q, const float *K, const float *V, int64_t ld, float *O, int64_t ldo,
+                                   float *L, int64_t B, int64_t H, int64_t S, int64_t dk, float scale, int causal) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!Q || !K || !V || !O) return fail(AXHIP_ERR_NULL_ARG, "sdpa_fwd_rows: NULL tensor");
+    if (B < 0 || H <= 0 || S < 0) return fail(AXHIP_ERR_SHAPE, "sdpa_fwd_rows: bad extent");
+    if (dk != 32 && dk != 64 && dk != 128)
+        return fail(AXHIP_ERR_NOT_IMPLEMENTED, "sdpa_fwd_rows: head size %lld (32, 64 or 128 only)", (long long)dk);
+    if (ld < H * dk || ldo < H * dk || ld % 4 != 0 || ldo % 4 != 0 || ld > (1 << 22))
+        return fail(AXHIP_ERR_SHAPE, "sdpa_fwd_rows: row pitch must hold H * dk floats and be a multiple of 4");
+    if ((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O) & 15) != 0)
+        return fail(AXHIP_ERR_SHAPE, "sdpa_fwd_rows: tensors must be 16-byte aligned");
+    if (B == 0 || S == 0) return AXHIP_OK;
+    if (B > 0x7fffffff / H || (S + SD_BQ - 1) / SD_BQ * (B * H) > 0x7fffffff)
+        return fail(AXHIP_ERR_SHAPE, "sdpa_fwd_rows: too many tiles");
+    return sdpa_fused(Q, K, V, O, L, B * H, S, dk, scale, causal, H, ld, ldo);
 }

@@ -38,13 +38,21 @@ static ax_status_t refresh_fused_qkv(ax_mha_t *m, const ax_cuda_extension_t *ext
         m->Wv_gen = gv;
     }
     if (m->use_bias) {
-        if (!m->bqkv_cache) {
-            int64_t sh[1] = {3 * D};
-            if (!(m->bqkv_cache = on_device_of(m->Wq, sh, 1))) return AX_ERR_ALLOC;
+        /* the reference rebuilds the bias on every call (cache.c:67-84: "cheap"); here that is a
+         * kernel launch, so it follows the generations like the weights */
+        const uint64_t bq = m->bq->storage->generation, bk = m->bk->storage->generation, bv = m->bv->storage->generation;
+        if (!m->bqkv_cache || bq != m->bq_gen || bk != m->bk_gen || bv != m->bv_gen) {
+            if (!m->bqkv_cache) {
+                int64_t sh[1] = {3 * D};
+                if (!(m->bqkv_cache = on_device_of(m->Wq, sh, 1))) return AX_ERR_ALLOC;
+            }
+            ax_status_t st = ext->bias_cache_build(dev_ptr(m->bqkv_cache), dev_ptr(m->bq), dev_ptr(m->bk), dev_ptr(m->bv), D);
+            if (st != AX_OK) return st;
+            m->bqkv_cache->storage->generation++;
+            m->bq_gen = bq;
+            m->bk_gen = bk;
+            m->bv_gen = bv;
         }
-        ax_status_t st = ext->bias_cache_build(dev_ptr(m->bqkv_cache), dev_ptr(m->bq), dev_ptr(m->bk), dev_ptr(m->bv), D);
-        if (st != AX_OK) return st;
-        m->bqkv_cache->storage->generation++;
     }
     return AX_OK;
 }
@@ -70,6 +78,24 @@ static ax_tensor_t *mha_forward(ax_layer_t *self, ax_tensor_t *x) {
                 *out = NULL;
     int64_t flat_sh[2] = {rows, D}, qkv_sh[2] = {rows, 3 * D}, head_sh[3] = {B * H, S, dk};
     ax_status_t st = refresh_fused_qkv(m, ext);
+    /* Head sizes the fused kernel covers: attention reads the heads where the projection wrote
+     * them (columns h*dk.. of the q, k and v thirds of qkv) and writes them where the output
+     * projection reads them, so the three layout passes of attention.c:211-262, 391-400 and their
+     * four [B*H, S, dk] temporaries fall away; the projection bias moves into the GEMM write-back. */
+    const bool direct = ext->sdpa_fwd_rows && (dk == 32 || dk == 64 || dk == 128) &&
+                        (!m->use_bias || ax_compute_has_gemm_bias_act());
+    if (direct) {
+        if (st == AX_OK && (!(x_flat = ax_tensor_reshape(x, flat_sh, 2)) || !(qkv = on_device_of(x, qkv_sh, 2)) ||
+                            !(attn = on_device_of(x, flat_sh, 2)) || !(out_flat = on_device_of(x, flat_sh, 2))))
+            st = AX_ERR_ALLOC;
+        if (st == AX_OK)
+            st = m->use_bias ? ax_compute_gemm_bias_act(x_flat, m->Wqkv_cache, m->bqkv_cache, AX_ACT_NONE, qkv)
+                             : ax_compute_gemm(x_flat, m->Wqkv_cache, qkv);
+        if (st == AX_OK)
+            st = ext->sdpa_fwd_rows(dev_ptr(qkv), dev_ptr(qkv) + D, dev_ptr(qkv) + 2 * D, 3 * D, dev_ptr(attn), D, NULL, B, H, S,
+                                    dk, 1.0f / sqrtf((float)dk), m->causal);
+        goto project;
+    }
     if (st == AX_OK && (!(x_flat = ax_tensor_reshape(x, flat_sh, 2)) || !(qkv = on_device_of(x, qkv_sh, 2)) ||
                         !(Qh = on_device_of(x, head_sh, 3)) || !(Kh = on_device_of(x, head_sh, 3)) ||
                         !(Vh = on_device_of(x, head_sh, 3)) || !(Oh = on_device_of(x, head_sh, 3)) ||
@@ -92,6 +118,7 @@ static ax_tensor_t *mha_forward(ax_layer_t *self, ax_tensor_t *x) {
         ext->head_deinterleave(dev_ptr(Oh), dev_ptr(attn), B, S, H, dk);
         st = ax_err_last_status();
     }
+project:
     if (st == AX_OK) {                                       /* attention.c:402-417: gemm, then bias along axis 1 */
         if (m->use_bias && ax_compute_has_gemm_bias_act()) st = ax_compute_gemm_bias_act(attn, m->Wo, m->bo, AX_ACT_NONE, out_flat);
         else {

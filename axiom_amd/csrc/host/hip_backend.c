@@ -538,6 +538,11 @@ ax_status_t ax_hip_sdpa_fwd(const float *Q, const float *K, const float *V, floa
     return lift(axhip_sdpa_fwd(Q, K, V, out, L, BH, S, dk, scale, causal ? 1 : 0), "hip sdpa_fwd");
 }
 
+static ax_status_t ext_sdpa_fwd_rows(const float *Q, const float *K, const float *V, int64_t ld, float *out, int64_t ldo,
+                                     float *L, int64_t B, int64_t H, int64_t S, int64_t dk, float scale, bool causal) {
+    return lift(axhip_sdpa_fwd_rows(Q, K, V, ld, out, ldo, L, B, H, S, dk, scale, causal ? 1 : 0), "hip sdpa_fwd_rows");
+}
+
 /* ---- the extension table (include/axiom/internal/cuda_extension.h).  The layout members return
  * nothing in the reference's table; a failure is left for ax_err_last_message(). ---- */
 static void ext_split(const float *src, float *q, float *k, float *v, int64_t B, int64_t S, int64_t H, int64_t dk, int64_t D) {
@@ -564,6 +569,7 @@ const ax_cuda_extension_t ax_hip_extension = {
     .head_interleave_qkv_split = ext_split, .head_interleave_qkv_split_bias = ext_split_bias,
     .head_interleave = ext_interleave, .head_deinterleave = ext_deinterleave,
     .qkv_cache_build = ext_qkv_cache, .bias_cache_build = ext_bias_cache, .sdpa_fwd = ax_hip_sdpa_fwd,
+    .sdpa_fwd_rows = ext_sdpa_fwd_rows,
 };
 
 const ax_backend_ops_t *ax_hip_ops_for_device(ax_device_t as_device) {

@@ -37,6 +37,7 @@ SIGNATURES = {
     "axhip_quantize_rows": (C.c_int, [vp, i64, i64, vp, vp]),
     "axhip_bias_add": (C.c_int, [vp, vp, i64, i64, i64, vp]),
     "axhip_sdpa_fwd": (C.c_int, [vp, vp, vp, vp, vp, i64, i64, i64, C.c_float, C.c_int]),
+    "axhip_sdpa_fwd_rows": (C.c_int, [vp, vp, vp, i64, vp, i64, vp, i64, i64, i64, i64, C.c_float, C.c_int]),
     "axhip_sum_axis": (C.c_int, [vp, i64, i64, i64, vp]),
     "axhip_sum_all": (C.c_int, [vp, i64, vp]),
     "axhip_axpy": (C.c_int, [vp, C.c_float, vp, i64]),

@@ -322,8 +322,42 @@ def secondary(hip):
             api[f"M{M}_us_per_forward"] = (time.perf_counter() - t0) * 1e6 / n
             ax.free(tx)
         L.ax_layer_destroy(seq)
-        L.ax_set_default_device(0)
         res["mlp3_through_ax_layer_forward"] = api
+
+        # the encoder of the reference's bench_transformer.c (:20-53): 6 x [LayerNorm, MHA(4 heads),
+        # LayerNorm, Dense 256-1024, GELU, Dense 1024-256], LayerNorm, Dense 256-1024 on [8,128,256];
+        # forward only, every layer on the device (LayerNorm, fused attention, GEMM epilogues)
+        enc = L.ax_sequential_create()
+        for _ in range(6):
+            L.ax_sequential_add(enc, L.ax_layernorm_create(256, 1e-5))
+            L.ax_sequential_add(enc, L.ax_mha_create(256, 4, True, False))
+            L.ax_sequential_add(enc, L.ax_layernorm_create(256, 1e-5))
+            L.ax_sequential_add(enc, L.ax_dense_create(256, 1024, True))
+            L.ax_sequential_add(enc, L.ax_gelu_layer_create())
+            L.ax_sequential_add(enc, L.ax_dense_create(1024, 256, True))
+        L.ax_sequential_add(enc, L.ax_layernorm_create(256, 1e-5))
+        L.ax_sequential_add(enc, L.ax_dense_create(256, 1024, True))
+        tx = ax.from_numpy(rng.uniform(-0.1, 0.1, (8, 128, 256)).astype(np.float32))
+
+        def enc_forward():
+            y = L.ax_layer_forward(enc, tx)
+            if not y:
+                raise RuntimeError("encoder forward failed: %s" % (ax.err(),))
+            L.ax_tensor_destroy(y)
+
+        for _ in range(20):
+            enc_forward()
+        hip.sync()
+        n = 300
+        t0 = time.perf_counter()
+        for _ in range(n):
+            enc_forward()
+        hip.sync()
+        res["encoder6_forward_8x128x256"] = {"us_per_forward": (time.perf_counter() - t0) * 1e6 / n,
+                                             "layers": 38}
+        ax.free(tx)
+        L.ax_layer_destroy(enc)
+        L.ax_set_default_device(0)
     return res
 
 

@@ -199,6 +199,17 @@ int axhip_sgd_update(float *w, const float *g, float *momentum_buf, int64_t n, f
  * fused, with no score matrix in memory; other head sizes go through batched GEMMs and a row softmax. */
 int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L,
                    int64_t BH, int64_t S, int64_t dk, float scale, int causal);
+/* The same attention on heads that lie side by side in the rows of wider matrices: head (b, h)
+ * reads rows b*S .. b*S+S-1, columns h*dk .. h*dk+dk-1 of Q, K and V (row pitch ld floats) and
+ * writes the same block of O (row pitch ldo); L is [B*H, S] or NULL.  With Q = qkv, K = qkv + D,
+ * V = qkv + 2D, ld = 3D, ldo = D this consumes the fused projection [B*S, 3D] and produces the
+ * [B*S, D] input of the output projection directly, i.e. it stands for the sequence
+ * head_interleave_qkv_split -> sdpa_fwd -> head_deinterleave of the reference's MHA forward
+ * (src/core/attention.c:211-262, 391-400) without the three layout passes.  dk must be 32, 64 or
+ * 128, pitches multiples of 4 floats, tensors 16-byte aligned (AXHIP_ERR_NOT_IMPLEMENTED /
+ * AXHIP_ERR_SHAPE otherwise). */
+int axhip_sdpa_fwd_rows(const float *Q, const float *K, const float *V, int64_t ld, float *O, int64_t ldo,
+                        float *L, int64_t B, int64_t H, int64_t S, int64_t dk, float scale, int causal);
 
 /* ---- layout transforms around attention (the layout members of the reference's GPU extension
  * table, include/axiom/internal/cuda_extension.h:45-84) ------------------------------------- */

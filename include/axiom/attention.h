@@ -22,6 +22,9 @@ typedef struct {
      * storage generation has moved (src/core/attention/cache.c:24-85) */
     ax_tensor_t *Wqkv_cache, *bqkv_cache;
     uint64_t Wq_gen, Wk_gen, Wv_gen;
+    /* appended after the reference's last member: the generations the fused bias was built from
+     * (the reference rebuilds it on every forward, which on a device is a kernel launch) */
+    uint64_t bq_gen, bk_gen, bv_gen;
 } ax_mha_t;
 
 ax_layer_t *ax_mha_create(int64_t d_model, int n_heads, bool use_bias, bool causal);

@@ -43,6 +43,15 @@ typedef struct {
     ax_status_t (*conv_winograd_f23)(const ax_tensor_t *weight, const float *in_dev, int64_t N,
                                      const ax_conv_params_t *single, ax_tensor_t *out);
     bool (*winograd_f23_prefer)(int64_t C_in, int64_t C_out, int64_t H, int64_t W);
+    /* Appended after the reference's last member (only tables built against this header carry it):
+     * attention straight on the fused projection.  Head (b, h) is the block of rows b*S.., columns
+     * h*dk.. of Q, K, V (row pitch ld floats) and of out (pitch ldo), so qkv [B*S, 3D] goes in as
+     * (qkv, qkv + D, qkv + 2D, ld = 3D) and out [B*S, D] comes back ready for the output
+     * projection, with no split / interleave pass.  AX_ERR_NOT_IMPLEMENTED for a head size it
+     * does not cover: the caller then takes the split path. */
+    ax_status_t (*sdpa_fwd_rows)(const float *Q, const float *K, const float *V, int64_t ld, float *out,
+                                 int64_t ldo, float *L, int64_t B, int64_t H, int64_t S, int64_t dk, float scale,
+                                 bool causal);
 } ax_cuda_extension_t;
 
 /* The MI355X table: the layout transforms, both cache builders and sdpa_fwd are filled. */

@@ -533,6 +533,43 @@ def test_sdpa_forward(hip, oracle, golden, BH, S, dk, causal):
     assert none is None and np.array_equal(o2, o)
 
 
+@pytest.mark.parametrize("B,H,S,dk,causal,pad_in,pad_out", [(2, 4, 128, 64, 0, 0, 0), (2, 4, 128, 64, 1, 0, 0),
+                                                            (3, 2, 77, 32, 1, 8, 4), (1, 3, 200, 128, 0, 4, 12),
+                                                            (2, 5, 256, 32, 0, 0, 8), (1, 2, 1, 64, 0, 0, 0),
+                                                            (9, 4, 128, 64, 0, 0, 0), (2, 3, 321, 64, 1, 16, 0)])
+def test_sdpa_on_the_fused_projection_layout(hip, oracle, B, H, S, dk, causal, pad_in, pad_out):
+    """Heads side by side in the rows of qkv [B*S, 3D (+ padding)]: the same numbers as the same
+    heads handed over one matrix each, bit for bit, written into [B*S, D (+ padding)] with the
+    padding columns untouched."""
+    say("sdpa rows", B, H, S, dk, causal, pad_in, pad_out)
+    D = H * dk
+    ld, ldo = 3 * D + pad_in, D + pad_out
+    oracle.seed(9000 + B * 1000 + H * 100 + S + dk + causal)
+    qkv = oracle.uniform((B * S, ld), -0.5, 0.5)
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(dk)))
+    heads = lambda third: np.ascontiguousarray(                       # noqa: E731  [B*H, S, dk]
+        qkv[:, third * D:(third + 1) * D].reshape(B, S, H, dk).transpose(0, 2, 1, 3).reshape(B * H, S, dk))
+    q, k, v = heads(0), heads(1), heads(2)
+    want_o, want_l = run_sdpa(hip, q, k, v, scale, causal)
+    o64, _ = oracle.sdpa(q, k, v, scale, causal, f64=True)
+    assert np.abs(want_o - o64).max() <= SDPA_TOL
+    dqkv = hip.array(qkv)
+    out = hip.array(np.full((B * S, ldo), 7.0, np.float32))
+    l = hip.empty((B * H, S))
+    base = dqkv.ptr
+    hip.check(hip.L.axhip_sdpa_fwd_rows(base, base + 4 * D, base + 8 * D, ld, out.ptr, ldo, l.ptr, B, H, S, dk,
+                                        scale, int(causal)))
+    got = out.numpy()
+    assert (got[:, D:] == 7.0).all()
+    got_heads = got[:, :D].reshape(B, S, H, dk).transpose(0, 2, 1, 3).reshape(B * H, S, dk)
+    assert np.array_equal(got_heads, want_o)
+    assert np.array_equal(l.numpy(), want_l)
+    # refusals: a head size without a fused kernel, a pitch shorter than the heads, a pitch off the 16-byte grid
+    assert hip.L.axhip_sdpa_fwd_rows(base, base, base, ld, out.ptr, ldo, None, B, H, S, 48, scale, 0) == 10
+    assert hip.L.axhip_sdpa_fwd_rows(base, base, base, D - 4, out.ptr, ldo, None, B, H, S, dk, scale, 0) == 3
+    assert hip.L.axhip_sdpa_fwd_rows(base, base, base, ld + 2, out.ptr, ldo, None, B, H, S, dk, scale, 0) == 3
+
+
 def test_sdpa_large_scores_and_full_size(hip, oracle):
     """Scores far from zero (the running maximum must absorb them), and the attention shape of
     the benchmark (512 heads of [512, 64]) checked on sampled heads."""
