@@ -30,7 +30,8 @@ INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300
                (128, 128, 256), (128, 256, 128), (256, 512, 384), (384, 128, 4096),
                (2048, 4096, 512), (256, 4096, 4096),
                # M <= 8 with whole 16-byte steps of K: the wave-per-rows dot-product route
-               (1, 768, 3072), (1, 4096, 4096), (8, 768, 768), (3, 5, 16), (7, 1001, 1040), (2, 3, 4112)]
+               (1, 768, 3072), (1, 4096, 4096), (8, 768, 768), (3, 5, 16), (7, 1001, 1040), (2, 3, 4112),
+               (4, 33, 64), (5, 9, 48), (6, 130, 256)]
 
 
 @pytest.mark.parametrize("M,N,K", INT8_SHAPES)
@@ -346,7 +347,8 @@ def test_config4b_attention_shapes_full_size(hip, oracle):
 # ------------------------------------------------------------------ W8A32
 W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 1024), (3, 17, 45),
                 (1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024),
-                (64, 1024, 4096), (1, 4096, 4096), (5, 33, 100)]
+                (64, 1024, 4096), (1, 4096, 4096), (5, 33, 100),
+                (2, 130, 256), (6, 67, 1040), (7, 5, 2064)]       # every row count of the wave-per-rows form
 
 
 @pytest.mark.parametrize("M,N,K", W8A32_SHAPES)
