@@ -267,7 +267,10 @@ def test_config3_ffn_block(hip, oracle):
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_skinny_against_oracle(hip, oracle, M):
     oracle.seed(100 + M)
-    for (K, N) in [(784, 4096), (4096, 4096), (4096, 10), (1, 5), (130, 67), (16, 64), (3000, 1000)]:
+    # (100, 3076) and (5000, 3072): a ragged last strip with K below one batch of rows, and splits longer
+    # than the first staging pass of the activations
+    for (K, N) in [(784, 4096), (4096, 4096), (4096, 10), (1, 5), (130, 67), (16, 64), (3000, 1000), (100, 3076),
+                   (5000, 3072)]:
         say("skinny", M, K, N)
         a, b = oracle.uniform((M, K), 0, 1), oracle.kaiming((K, N), K)
         bias = oracle.normal((N,), 0, 0.1)
@@ -280,6 +283,26 @@ def test_skinny_against_oracle(hip, oracle, M):
         assert hip.last_kernel().startswith("sgemm_skinny")
         assert np.array_equal(via, fused)
         assert np.array_equal(hip.sgemm_skinny(da, db).numpy(), got)  # deterministic
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 1030, 4096), (3, 2048, 3104), (8, 777, 4100)])
+def test_skinny_padded_leading_dimensions(hip, oracle, M, K, N):
+    """Sub-matrices of wider buffers (lda > K, ldb > N, ldc > N): the padding is neither read into
+    the result nor written."""
+    oracle.seed(300 + M + K + N)
+    lda, ldb, ldc = K + 5, N + 8, N + 3
+    abuf, bbuf = oracle.uniform((M, lda), 0, 1), oracle.kaiming((K, ldb), K)
+    bias = oracle.normal((N,), 0, 0.1)
+    a, b = np.ascontiguousarray(abuf[:, :K]), np.ascontiguousarray(bbuf[:, :N])
+    da, db, dbias = hip.array(abuf), hip.array(bbuf), hip.array(bias)
+    dc = hip.array(np.full((M, ldc), -3.0, np.float32))
+    hip.check(hip.L.axhip_sgemm_skinny(M, N, K, da.ptr, lda, db.ptr, ldb, dc.ptr, ldc, dbias.ptr, 1))
+    say("  kernel", hip.last_kernel())
+    got = dc.numpy()
+    assert (got[:, N:] == -3.0).all()
+    want = np.maximum(hip.sgemm_skinny(hip.array(a), hip.array(b)).numpy() + bias[None, :], 0)
+    assert np.array_equal(got[:, :N], want)
+    check_fp32(oracle, hip.sgemm_skinny(hip.array(a), hip.array(b)).numpy(), a, b)
 
 
 @pytest.mark.parametrize("M", [1, 2, 4, 8])
