@@ -5,6 +5,7 @@
 
 #include <mutex>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "common.h"
@@ -27,6 +28,9 @@ size_t g_ones_n = 0;
 std::mutex g_pool_mutex;
 std::unordered_map<void *, size_t> g_pool_size;
 std::unordered_map<size_t, std::vector<void *>> g_pool_free;
+std::unordered_set<void *> g_pool_idle;                  // blocks sitting in g_pool_free: a second free of one is ignored
+// what callers asked for and gave back (ax_cuda_alloc_stats, cuda/memory.cu:13-29), and how often the driver was needed
+int64_t g_stat_allocs = 0, g_stat_frees = 0, g_stat_bytes_alloc = 0, g_stat_bytes_free = 0, g_stat_driver_allocs = 0;
 size_t g_pool_cached = 0;
 constexpr size_t kPoolMaxBlock = size_t(1) << 30;        // larger blocks go straight back to the driver
 constexpr size_t kPoolMaxCached = size_t(16) << 30;      // bytes the pool may hold back
@@ -66,6 +70,7 @@ void pool_release_all() {
                 g_pool_size.erase(p);
             }
         g_pool_free.clear();
+        g_pool_idle.clear();
         g_pool_cached = 0;
     }
     for (void *p : blocks) (void)hipFree(p);
@@ -220,6 +225,9 @@ static void *pool_take(size_t bytes) {
             p = it->second.back();
             it->second.pop_back();
             g_pool_cached -= size;
+            g_pool_idle.erase(p);
+            g_stat_allocs++;
+            g_stat_bytes_alloc += (int64_t)size;
         }
     }
     if (!p) {
@@ -234,6 +242,9 @@ static void *pool_take(size_t bytes) {
         }
         std::lock_guard<std::mutex> lock(g_pool_mutex);
         g_pool_size[p] = size;
+        g_stat_allocs++;
+        g_stat_driver_allocs++;
+        g_stat_bytes_alloc += (int64_t)size;
     }
     return p;
 }
@@ -256,16 +267,35 @@ void axhip_free(void *p) {
     {
         std::lock_guard<std::mutex> lock(g_pool_mutex);
         auto it = g_pool_size.find(p);
-        if (it == g_pool_size.end()) return;             // not ours (or freed twice): leave it alone
+        if (it == g_pool_size.end() || g_pool_idle.count(p)) return;   // not ours, or freed twice: leave it alone
         size = it->second;
+        g_stat_frees++;
+        g_stat_bytes_free += (int64_t)size;
         if (size <= kPoolMaxBlock && g_pool_cached + size <= kPoolMaxCached) {
             g_pool_free[size].push_back(p);
+            g_pool_idle.insert(p);
             g_pool_cached += size;
             return;
         }
         g_pool_size.erase(it);
     }
     (void)hipFree(p);
+}
+
+void axhip_alloc_stats(int64_t *allocs, int64_t *frees, int64_t *bytes_alloc, int64_t *bytes_free,
+                       int64_t *driver_allocs, int64_t *bytes_cached) {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    if (allocs) *allocs = g_stat_allocs;
+    if (frees) *frees = g_stat_frees;
+    if (bytes_alloc) *bytes_alloc = g_stat_bytes_alloc;
+    if (bytes_free) *bytes_free = g_stat_bytes_free;
+    if (driver_allocs) *driver_allocs = g_stat_driver_allocs;
+    if (bytes_cached) *bytes_cached = (int64_t)g_pool_cached;
+}
+
+void axhip_reset_alloc_stats(void) {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    g_stat_allocs = g_stat_frees = g_stat_bytes_alloc = g_stat_bytes_free = g_stat_driver_allocs = 0;
 }
 
 int axhip_memset(void *p, int v, size_t bytes) {

@@ -257,6 +257,13 @@ ax_status_t ax_model_save(ax_model_t *model, const char *path) {
     return AX_OK;
 }
 
+/* rows x cols floats stay under the per-tensor cap; each factor is bounded first so the product
+ * cannot wrap (extents come straight from the file) */
+static bool floats_fit(int64_t rows, int64_t cols) {
+    const uint64_t cap = MAX_TENSOR_BYTES / 4;
+    return rows > 0 && cols > 0 && (uint64_t)rows <= cap && (uint64_t)cols <= cap && (uint64_t)rows * (uint64_t)cols <= cap;
+}
+
 /* one layer from its descriptor (serialize.c:540-660); NULL with the error set */
 static ax_layer_t *read_layer(stream_t *s, uint32_t type, uint32_t index) {
     switch (type) {
@@ -264,7 +271,7 @@ static ax_layer_t *read_layer(stream_t *s, uint32_t type, uint32_t index) {
             int64_t in_f, out_f;
             uint8_t bias;
             if (!get_i64(s, &in_f) || !get_i64(s, &out_f) || !get_u8(s, &bias)) return NULL;
-            if (in_f <= 0 || out_f <= 0 || (uint64_t)in_f * (uint64_t)out_f * 4 > MAX_TENSOR_BYTES) {
+            if (!floats_fit(in_f, out_f)) {
                 ax_err_set(AX_ERR_INVALID_SHAPE, "layer %u: dense %" PRId64 " x %" PRId64 " is not acceptable", index, in_f, out_f);
                 return NULL;
             }
@@ -274,7 +281,7 @@ static ax_layer_t *read_layer(stream_t *s, uint32_t type, uint32_t index) {
             int64_t nf;
             float eps;
             if (!get_i64(s, &nf) || !get_f32(s, &eps)) return NULL;
-            if (nf <= 0 || (uint64_t)nf * 4 > MAX_TENSOR_BYTES) {
+            if (!floats_fit(nf, 1)) {
                 ax_err_set(AX_ERR_INVALID_SHAPE, "layer %u: layernorm over %" PRId64 " features", index, nf);
                 return NULL;
             }
@@ -295,8 +302,8 @@ static ax_layer_t *read_layer(stream_t *s, uint32_t type, uint32_t index) {
             uint32_t n_heads;
             uint8_t use_bias, causal;
             if (!get_i64(s, &d_model) || !get_u32(s, &n_heads) || !get_u8(s, &use_bias) || !get_u8(s, &causal)) return NULL;
-            if (d_model <= 0 || n_heads == 0 || n_heads > (uint32_t)INT_MAX || d_model % (int64_t)n_heads != 0 ||
-                (uint64_t)d_model * (uint64_t)d_model * 4 > MAX_TENSOR_BYTES) {
+            if (!floats_fit(d_model, d_model) || n_heads == 0 || n_heads > (uint32_t)INT_MAX ||
+                d_model % (int64_t)n_heads != 0) {
                 ax_err_set(AX_ERR_INVALID_SHAPE, "layer %u: attention with d_model %" PRId64 " and %u heads", index, d_model, n_heads);
                 return NULL;
             }

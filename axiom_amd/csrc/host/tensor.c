@@ -1,6 +1,7 @@
 /* Refcounted storage and tensor views (the subset of Axiom's src/core/tensor.c the GEMM path
  * uses).  Device memory is never touched here: allocation, release and copies go through the
  * hooks of the backend that owns the device (src/core/tensor.c:201-286, 1016-1085). */
+#include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -94,7 +95,7 @@ static ax_tensor_t *tensor_create(const int64_t *shape, int ndim, ax_dtype_t dty
     }
     size_t esz = ax_dtype_size(dtype);
     int64_t n = numel_of(shape, ndim);
-    if (!esz || n < 0) {
+    if (!esz || n < 0 || (uint64_t)n > (SIZE_MAX >> 1) / esz) {          /* n * esz must not wrap */
         ax_err_set(esz ? AX_ERR_INVALID_SHAPE : AX_ERR_INVALID_DTYPE, "tensor_create: bad dtype or extent");
         return NULL;
     }

@@ -23,6 +23,8 @@ SIGNATURES = {
     "axhip_malloc": (vp, [C.c_size_t]),
     "axhip_malloc_uninit": (vp, [C.c_size_t]),
     "axhip_free": (None, [vp]),
+    "axhip_alloc_stats": (None, [C.POINTER(C.c_int64)] * 6),
+    "axhip_reset_alloc_stats": (None, []),
     "axhip_memset": (C.c_int, [vp, C.c_int, C.c_size_t]),
     "axhip_memcpy_h2d": (C.c_int, [vp, vp, C.c_size_t]),
     "axhip_memcpy_d2h": (C.c_int, [vp, vp, C.c_size_t]),

@@ -54,7 +54,15 @@ const char *axhip_device_name(void);          /* gcnArchName of device 0, "" wit
  *      neither call waits for the device; axhip_shutdown returns everything to the driver. ------ */
 void *axhip_malloc(size_t bytes);
 void *axhip_malloc_uninit(size_t bytes);   /* contents undefined: for results that are fully overwritten */
-void  axhip_free(void *device_ptr);
+void  axhip_free(void *device_ptr);             /* NULL, foreign and already-freed pointers are ignored */
+/* Allocation counters for leak diagnosis (ax_cuda_alloc_stats / ax_cuda_reset_alloc_stats,
+ * cuda/memory.cu:13-29): requests served and blocks given back, in calls and in bytes of their size
+ * classes, so allocs == frees and bytes_alloc == bytes_free once every tensor is destroyed; plus
+ * how many of the requests needed the driver (the rest were pool hits) and the bytes the pool holds
+ * back now.  Any pointer may be NULL. */
+void  axhip_alloc_stats(int64_t *allocs, int64_t *frees, int64_t *bytes_alloc, int64_t *bytes_free,
+                        int64_t *driver_allocs, int64_t *bytes_cached);
+void  axhip_reset_alloc_stats(void);
 int   axhip_memset(void *device_ptr, int byte_value, size_t bytes);
 int   axhip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes);
 int   axhip_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes);   /* blocking */

@@ -966,3 +966,17 @@ def test_allocation_pool(hip):
     out = hip.empty((16,))
     hip.check(hip.L.axhip_fill_f32(out.ptr, 2.0, 16))
     assert np.array_equal(out.numpy(), np.full(16, 2.0, np.float32))
+    # a block freed twice is handed out once; the counters balance and tell pool hits from driver calls
+    hip.L.axhip_reset_alloc_stats()
+    x = hip.empty((3000,))
+    xp = x.ptr
+    hip.L.axhip_free(xp)
+    hip.L.axhip_free(xp)                                       # second free: ignored
+    x.ptr = None
+    y, z = hip.empty((3000,)), hip.empty((3000,))
+    assert y.ptr == xp and z.ptr != xp
+    del y, z
+    st = [C.c_int64() for _ in range(6)]
+    hip.L.axhip_alloc_stats(*[C.byref(v) for v in st])
+    allocs, frees, b_alloc, b_free, driver, cached = (v.value for v in st)
+    assert allocs == 3 and frees == 3 and b_alloc == b_free == 3 * 16384 and driver <= 2 and cached >= 2 * 16384
