@@ -1,6 +1,7 @@
-"""The host library's file code (model, tensor files) compiled with AddressSanitizer and
-UndefinedBehaviorSanitizer and driven over the reference-written fixtures, their truncations, bit
-flips and crafted headers (tests/host_sanitize_driver.c).  No GPU; the sanitizers abort on a finding."""
+"""The host library's C (tensors, layers, model container, quantized weights, model / tensor /
+quantized-weight files) compiled with AddressSanitizer, LeakSanitizer and UndefinedBehaviorSanitizer and
+driven on the CPU device: object lifetimes and refused arguments, then the reference-written fixtures with
+their truncations, bit flips and crafted headers (tests/host_sanitize_driver.c).  No GPU; a finding aborts."""
 import glob
 import os
 import subprocess
@@ -27,4 +28,4 @@ def test_file_code_is_clean_under_asan_and_ubsan(tmp_path):
     r = subprocess.run([str(exe), str(tmp_path / "scratch.bin")] + files, env=env, capture_output=True, text=True,
                        timeout=600)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
-    assert r.stdout.count("round trip ok") == len(files)
+    assert r.stdout.count("round trip ok") == len(files) and "api section: 0 findings" in r.stdout
