@@ -768,6 +768,51 @@ int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     return fail(AXHIP_ERR_NOT_IMPLEMENTED, "sgemm: A^T * B^T is not provided");
 }
 
+// A large fp32 shape off the tile grid would run whole on the register-staged guarded kernel
+// (4000^3: 101 TFLOP/s against 141 on the grid).  Its grid-aligned interior goes to the
+// direct-to-LDS kernels instead and only the right and bottom fringes to the guarded one; every
+// block is a sub-matrix reached by pointer offsets.  Returns -1 when the shape is left alone.
+int try_interior_and_fringes(const SgemmArgs &g, int transa, int transb) {
+    if ((transa && transb) || g.K % 32 != 0 || g.K <= 0) return -1;
+    if ((((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.C | (uintptr_t)g.bias) & 15) != 0 || g.lda % 4 != 0 ||
+        g.ldb % 4 != 0 || g.ldc % 4 != 0)
+        return -1;                                           // the interior would not qualify for the fast kernels either
+    int64_t gm, gn;
+    if ((g.M / 128) * (g.N / 256) >= 256) gm = 128, gn = 256;
+    else if ((g.M / 64) * (g.N / 64) >= 256) gm = gn = 64;
+    else return -1;
+    const int64_t Mi = g.M / gm * gm, Ni = g.N / gn * gn;
+    if (Mi == g.M && Ni == g.N) return -1;
+    const float *A = static_cast<const float *>(g.A), *B = static_cast<const float *>(g.B);
+    // a fringe is a strip of few tiles with the whole K: the split-K route when it qualifies
+    auto fringe = [&](const SgemmArgs &f) {
+        const int rc = try_split_k<float>(f, transa, transb, "sgemm_splitk", nullptr);
+        return rc >= 0 ? rc : dispatch_f32(f, transa, transb, 1);
+    };
+    SgemmArgs p = g;
+    p.M = Mi;
+    p.N = Ni;
+    int rc = dispatch_f32(p, transa, transb, 1);
+    if (rc == AXHIP_OK && Ni < g.N) {                       // columns Ni.. of the interior's rows
+        p = g;
+        p.M = Mi;
+        p.N = g.N - Ni;
+        p.B = transb ? B + Ni * g.ldb : B + Ni;
+        p.C = g.C + Ni;
+        if (g.bias) p.bias = g.bias + Ni;
+        rc = fringe(p);
+    }
+    if (rc == AXHIP_OK && Mi < g.M) {                       // rows Mi.., every column
+        p = g;
+        p.M = g.M - Mi;
+        p.A = transa ? A + Mi : A + Mi * g.lda;
+        p.C = g.C + Mi * g.ldc;
+        rc = fringe(p);
+    }
+    note_kernel("sgemm_interior+fringes");
+    return rc;
+}
+
 }  // namespace
 
 namespace axhip {
@@ -793,7 +838,9 @@ extern "C" int axhip_sgemm(int transa, int transb, int64_t M, int64_t N, int64_t
         return axhip_sgemm_skinny(M, N, K, A, lda, B, ldb, C, ldc, bias, act);
     SgemmArgs g{A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, alpha, beta, nullptr, bias, act};
     if (!(transa && transb)) {
-        const int rc = try_split_k<float>(g, transa, transb, "sgemm_splitk", nullptr);
+        int rc = try_split_k<float>(g, transa, transb, "sgemm_splitk", nullptr);
+        if (rc >= 0) return rc;
+        rc = try_interior_and_fringes(g, transa, transb);
         if (rc >= 0) return rc;
     }
     return dispatch_f32(g, transa, transb, 1);

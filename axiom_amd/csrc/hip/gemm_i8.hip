@@ -29,12 +29,17 @@ __device__ __forceinline__ int swz(int row, int chunk) {
 
 template <bool GUARD>
 __device__ __forceinline__ v4i load_chunk(const int8_t *base, int64_t row, int64_t rows,
-                                          int64_t k, int64_t K, bool vec_ok) {
+                                          int64_t k, int64_t K) {
     if (!GUARD) return *reinterpret_cast<const v4i *>(base + row * K + k);
     v4i r = {0, 0, 0, 0};
     if (row >= rows || k >= K) return r;
     const int8_t *p = base + row * K + k;
-    if (vec_ok && k + 16 <= K) return *reinterpret_cast<const v4i *>(p);
+    if (k + 16 <= K) {
+        // a whole chunk inside the row: one 16-byte load at whatever alignment K leaves the row
+        // (global memory takes unaligned vector loads; byte loads made K % 16 != 0 24x slower)
+        __builtin_memcpy(&r, p, 16);
+        return r;
+    }
     int64_t left = K - k;
     unsigned w[4] = {0, 0, 0, 0};
     for (int b = 0; b < 16; b++)
@@ -48,7 +53,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64)
 k_qgemm_w8a8(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
              int64_t K, float x_scale, const float *__restrict__ w_scales,
              const float *__restrict__ bias, int act, float *__restrict__ out,
-             int32_t *__restrict__ acc_out) {
+             int32_t *__restrict__ acc_out, int64_t ldc) {
     constexpr int T = WAVES_M * WAVES_N * 64;
     constexpr int CA = BM * 8 / T, CB = BN * 8 / T;       // 16-byte chunks per thread per slab
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N; // wave tile
@@ -69,7 +74,6 @@ k_qgemm_w8a8(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t
     tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
 
-    const bool vec_ok = !GUARD || ((((uintptr_t)X | (uintptr_t)W | (uintptr_t)K) & 15) == 0);
     const int64_t slabs = (K + BK - 1) / BK;
 
     v4i ra[CA], rb[CB];
@@ -78,12 +82,12 @@ k_qgemm_w8a8(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t
 #pragma unroll
         for (int i = 0; i < CA; i++) {
             int c = tid + i * T;
-            ra[i] = load_chunk<GUARD>(X, m0 + (c >> 3), M, k0 + ((c & 7) << 4), K, vec_ok);
+            ra[i] = load_chunk<GUARD>(X, m0 + (c >> 3), M, k0 + ((c & 7) << 4), K);
         }
 #pragma unroll
         for (int i = 0; i < CB; i++) {
             int c = tid + i * T;
-            rb[i] = load_chunk<GUARD>(W, n0 + (c >> 3), N, k0 + ((c & 7) << 4), K, vec_ok);
+            rb[i] = load_chunk<GUARD>(W, n0 + (c >> 3), N, k0 + ((c & 7) << 4), K);
         }
     };
     auto stash = [&](int stage) {
@@ -155,11 +159,11 @@ k_qgemm_w8a8(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t
                 const int64_t row = m0 + wm * WTM + i * 32 + (v & 3) + 8 * (v >> 2) + 4 * fhalf;
                 if (GUARD && (row >= M || !col_ok)) continue;
                 const int a = acc[i][j][v];
-                if (acc_out) acc_out[row * N + col] = a;
+                if (acc_out) acc_out[row * ldc + col] = a;
                 if (out) {
                     float f = (float)a;
                     float r = bias ? __builtin_fmaf(f, scale, bv) : f * scale;
-                    out[row * N + col] = apply_act(r, act);
+                    out[row * ldc + col] = apply_act(r, act);
                 }
             }
         }
@@ -169,7 +173,7 @@ k_qgemm_w8a8(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool GUARD>
 int launch(const char *name, const int8_t *x, float x_scale, const int8_t *w,
            const float *w_scales, const float *bias, int act, float *out, int32_t *acc_out,
-           int64_t M, int64_t N, int64_t K) {
+           int64_t M, int64_t N, int64_t K, int64_t ldc) {
     auto kern = k_qgemm_w8a8<BM, BN, WAVES_M, WAVES_N, GUARD>;
     constexpr int smem = 2 * (BM + BN) * BK;
     static bool attr_set = false;
@@ -183,7 +187,7 @@ int launch(const char *name, const int8_t *x, float x_scale, const int8_t *w,
     if (tiles > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: too many tiles");
     note_kernel(name);
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(WAVES_M * WAVES_N * 64), smem, kStream, x,
-                       w, M, N, K, x_scale, w_scales, bias, act, out, acc_out);
+                       w, M, N, K, x_scale, w_scales, bias, act, out, acc_out, ldc);
     return check_launch(name);
 }
 
@@ -226,7 +230,7 @@ __global__ void __launch_bounds__(512)
 k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
                  int64_t K, float x_scale, const float *__restrict__ w_scales,
                  const float *__restrict__ bias, float *__restrict__ out,
-                 int32_t *__restrict__ acc_out) {
+                 int32_t *__restrict__ acc_out, int64_t ldc) {
     constexpr int BM = 256, BN = 256, BKB = 128, WAVES_N = 4, WTM = 128, WTN = 64, TM = 4, TN = 2;
     constexpr int OPER = BM * BKB;   // bytes of one operand in one stage
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -408,7 +412,7 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 #pragma unroll
             for (int q = 0; q < 2; q++) {
                 const int src = 2 * (wave - 4) + q;                     // wave whose sub-tile this is
-                auto *dst = base + (m0 + (src / WAVES_N) * WTM + i * 32) * N + n0 + (src % WAVES_N) * WTN + j * 32;
+                auto *dst = base + (m0 + (src / WAVES_N) * WTM + i * 32) * ldc + n0 + (src % WAVES_N) * WTN + j * 32;
 #pragma unroll
                 for (int p = 0; p < 4; p++) {
                     const int row = p * 8 + (lane >> 3);
@@ -416,7 +420,7 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
                                                                (((lane & 7) ^ ((row >> 1) & 7)) << 4));
                     // streaming store: the 256 KB a tile writes must not evict the operand panels the
                     // XCD's other workgroups are re-reading from its 4 MB L2 (plain stores: +30 us)
-                    __builtin_nontemporal_store(v, reinterpret_cast<V4 *>(dst + (int64_t)row * N + (lane & 7) * 4));
+                    __builtin_nontemporal_store(v, reinterpret_cast<V4 *>(dst + (int64_t)row * ldc + (lane & 7) * 4));
                 }
             }
         }
@@ -534,7 +538,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64)
 k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
                  int64_t K, float x_scale, const float *__restrict__ w_scales,
                  const float *__restrict__ bias, float *__restrict__ out,
-                 int32_t *__restrict__ acc_out) {
+                 int32_t *__restrict__ acc_out, int64_t ldc) {
     constexpr int NW = WAVES_M * WAVES_N, BKB = 128;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
     constexpr int XS = BM * BKB, WS = BN * BKB;          // bytes of one stage of each operand
@@ -681,7 +685,7 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 #pragma unroll
                 for (int g = 0; g < 4; g++)
                     r[g] = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                turn_tile_and_store(turn, lane, r, acc_out + (trow + i * 32) * N + tcol + j * 32, N);
+                turn_tile_and_store(turn, lane, r, acc_out + (trow + i * 32) * ldc + tcol + j * 32, ldc);
             }
     }
     if (out) {
@@ -705,7 +709,7 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
                         const float f = (float)acc[i][j][4 * g + e];
                         r[g][e] = apply_act(has_bias ? __builtin_fmaf(f, sc[g][e], bv[g][e]) : f * sc[g][e], ACT);
                     }
-                turn_tile_and_store(turn, lane, r, out + (trow + i * 32) * N + tcol + j * 32, N);
+                turn_tile_and_store(turn, lane, r, out + (trow + i * 32) * ldc + tcol + j * 32, ldc);
             }
         }
     }
@@ -713,10 +717,11 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
 int launch_dma(const char *name, const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
-               const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K) {
+               const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K,
+               int64_t ldc) {
     constexpr int smem = NST * (BM + BN) * 128 + 2 * BN * 4;
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
-                           const float *, float *, int32_t *);
+                           const float *, float *, int32_t *, int64_t);
     static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE>,
                                     k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU>,
                                     k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU>};
@@ -732,16 +737,16 @@ int launch_dma(const char *name, const int8_t *x, float x_scale, const int8_t *w
     if (tiles > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: too many tiles");
     note_kernel(name);
     hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles), dim3(WAVES_M * WAVES_N * 64), smem, kStream, x, w,
-                       M, N, K, x_scale, w_scales, bias, out, acc_out);
+                       M, N, K, x_scale, w_scales, bias, out, acc_out, ldc);
     return check_launch(name);
 }
 
 int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
                const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N,
-               int64_t K) {
+               int64_t K, int64_t ldc) {
     constexpr int smem = 4 * 256 * 128 + 2 * 2 * 256 * 4;   // two stages of both operands + two slots of scale and bias
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
-                           const float *, float *, int32_t *);
+                           const float *, float *, int32_t *, int64_t);
     static const kern_t kerns[3] = {k_qgemm_w8a8_256<AXHIP_ACT_NONE>, k_qgemm_w8a8_256<AXHIP_ACT_RELU>,
                                     k_qgemm_w8a8_256<AXHIP_ACT_GELU>};
     static bool attr_set = false;
@@ -757,7 +762,7 @@ int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_s
     note_kernel("qgemm_w8a8_256x256_dma");
     const int64_t grid = tiles < cu_count() ? tiles : cu_count();     // one persistent workgroup per CU
     hipLaunchKernelGGL(kerns[act], dim3((unsigned)grid), dim3(512), smem, kStream, x, w, M, N, K,
-                       x_scale, w_scales, bias, out, acc_out);
+                       x_scale, w_scales, bias, out, acc_out, ldc);
     return check_launch("qgemm_w8a8_256x256_dma");
 }
 
@@ -822,6 +827,34 @@ int launch_gemv(const int8_t *x, float x_scale, const int8_t *w, const float *w_
     return check_launch("qgemm_w8a8_gemv");
 }
 
+
+// One block of the output, rows of pitch ldc: picks the kernel for its shape and alignment.
+int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_scales, const float *bias, int act,
+                float *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldc) {
+    const bool aligned = ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) && (K % BK == 0) && K > 0;
+    const bool vec_out = (!out || (((uintptr_t)out | (uintptr_t)w_scales | (uintptr_t)bias) & 15) == 0) &&
+                         (((uintptr_t)acc_out & 15) == 0) && ldc % 4 == 0;
+    if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128 &&
+        K < (int64_t(1) << 24))   // per-lane 32-bit byte offsets span 256 rows
+        return launch_256(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K, ldc);
+    // aligned but too few 256x256 tiles: direct-to-LDS kernel over smaller tiles
+    if (aligned && vec_out && K % 128 == 0 && M % 64 == 0 && N % 64 == 0 && K < (int64_t(1) << 24)) {
+        if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 512)
+            return launch_dma<128, 128, 2, 2, 3>("qgemm_w8a8_128x128_dma", x, x_scale, w, w_scales, bias,
+                                                 act, out, acc_out, M, N, K, ldc);
+        return launch_dma<64, 64, 2, 2, 4>("qgemm_w8a8_64x64_dma", x, x_scale, w, w_scales, bias, act,
+                                           out, acc_out, M, N, K, ldc);
+    }
+    // fewer than ~3/4 of the 256 CUs busy with 128x128 tiles: quarter the tile instead
+    if (aligned && M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 192)
+        return launch<128, 128, 2, 2, false>("qgemm_w8a8_128x128", x, x_scale, w, w_scales, bias,
+                                             act, out, acc_out, M, N, K, ldc);
+    if (aligned && M % 64 == 0 && N % 64 == 0)
+        return launch<64, 64, 2, 2, false>("qgemm_w8a8_64x64", x, x_scale, w, w_scales, bias, act,
+                                           out, acc_out, M, N, K, ldc);
+    return launch<64, 64, 2, 2, true>("qgemm_w8a8_64x64_guarded", x, x_scale, w, w_scales, bias,
+                                      act, out, acc_out, M, N, K, ldc);
+}
 }  // namespace
 
 extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
@@ -848,27 +881,24 @@ extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
             default: return launch_gemv<8>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
         }
     }
-    const bool aligned = ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) && (K % BK == 0) && K > 0;
-    const bool vec_out = (!out || (((uintptr_t)out | (uintptr_t)w_scales | (uintptr_t)bias) & 15) == 0) &&
-                         (((uintptr_t)acc_out & 15) == 0);
-    if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128 &&
-        K < (int64_t(1) << 24))   // per-lane 32-bit byte offsets span 256 rows
-        return launch_256(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K);
-    // aligned but too few 256x256 tiles: direct-to-LDS kernel over smaller tiles
-    if (aligned && vec_out && K % 128 == 0 && M % 64 == 0 && N % 64 == 0 && K < (int64_t(1) << 24)) {
-        if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 512)
-            return launch_dma<128, 128, 2, 2, 3>("qgemm_w8a8_128x128_dma", x, x_scale, w, w_scales, bias,
-                                                 act, out, acc_out, M, N, K);
-        return launch_dma<64, 64, 2, 2, 4>("qgemm_w8a8_64x64_dma", x, x_scale, w, w_scales, bias, act,
-                                           out, acc_out, M, N, K);
+    const bool fast = ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) && K % BK == 0 && K > 0 && K < (int64_t(1) << 24) &&
+                      N % 4 == 0 && (!out || (((uintptr_t)out | (uintptr_t)w_scales | (uintptr_t)bias) & 15) == 0) &&
+                      (((uintptr_t)acc_out & 15) == 0);
+    // A large shape off the 256 grid: the 256-aligned interior goes to the persistent kernel and
+    // the right and bottom fringes to the smaller tiles, each block addressed inside the full
+    // output through its row pitch (whole shape on 64x64 tiles: 8000^2 x 8192 at 0.93 POP/s).
+    const int64_t Mi = M / 256 * 256, Ni = N / 256 * 256;
+    if (fast && (Mi != M || Ni != N) && (Mi / 256) * (Ni / 256) >= 128) {
+        int rc = qgemm_block(x, x_scale, w, w_scales, bias, act, out, acc_out, Mi, Ni, K, N);
+        if (rc == AXHIP_OK && Ni < N)
+            rc = qgemm_block(x, x_scale, w + Ni * K, w_scales ? w_scales + Ni : nullptr, bias ? bias + Ni : nullptr, act,
+                             out ? out + Ni : nullptr, acc_out ? acc_out + Ni : nullptr, Mi, N - Ni, K, N);
+        if (rc == AXHIP_OK && Mi < M)
+            rc = qgemm_block(x + Mi * K, x_scale, w, w_scales, bias, act, out ? out + Mi * N : nullptr,
+                             acc_out ? acc_out + Mi * N : nullptr, M - Mi, N, K, N);
+        note_kernel("qgemm_w8a8_256x256_dma+fringes");
+        return rc;
     }
-    // fewer than ~3/4 of the 256 CUs busy with 128x128 tiles: quarter the tile instead
-    if (aligned && M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 192)
-        return launch<128, 128, 2, 2, false>("qgemm_w8a8_128x128", x, x_scale, w, w_scales, bias,
-                                             act, out, acc_out, M, N, K);
-    if (aligned && M % 64 == 0 && N % 64 == 0)
-        return launch<64, 64, 2, 2, false>("qgemm_w8a8_64x64", x, x_scale, w, w_scales, bias, act,
-                                           out, acc_out, M, N, K);
-    return launch<64, 64, 2, 2, true>("qgemm_w8a8_64x64_guarded", x, x_scale, w, w_scales, bias,
-                                      act, out, acc_out, M, N, K);
+    return qgemm_block(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K, N);
 }
+

@@ -31,7 +31,11 @@ INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300
                (2048, 4096, 512), (256, 4096, 4096),
                # M <= 8 with whole 16-byte steps of K: the wave-per-rows dot-product route
                (1, 768, 3072), (1, 4096, 4096), (8, 768, 768), (3, 5, 16), (7, 1001, 1040), (2, 3, 4112),
-               (4, 33, 64), (5, 9, 48), (6, 130, 256)]
+               (4, 33, 64), (5, 9, 48), (6, 130, 256),
+               # off the 256 grid with a large interior: persistent kernel inside, smaller tiles on the fringes
+               (2112, 4128, 256), (4100, 2304, 128), (2048, 4100, 128),
+               # rows that start at odd byte offsets (K % 16 != 0)
+               (70, 90, 1037), (130, 257, 4099)]
 
 
 @pytest.mark.parametrize("M,N,K", INT8_SHAPES)
@@ -119,7 +123,9 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               # shapes that take the 128x256 tile, and ones just short of it in N or in tile count
               (2048, 4096, 64), (4096, 2176, 64), (4096, 1088, 32), (128, 64, 4096),
               # few output tiles and a long K: the split-K route (bench_qgemm.c shapes among them)
-              (32, 768, 768), (64, 1024, 4096), (128, 4096, 1024), (9, 100, 512), (16, 16, 8192), (70, 130, 1536)]
+              (32, 768, 768), (64, 1024, 4096), (128, 4096, 1024), (9, 100, 512), (16, 16, 8192), (70, 130, 1536),
+              # off the tile grid with a large interior: fast kernels inside, guarded kernel on the fringes
+              (1032, 1100, 96), (2100, 4200, 64), (1024, 1092, 160)]
 
 
 @pytest.mark.parametrize("M,N,K", F32_SHAPES)
@@ -221,7 +227,7 @@ def test_sgemm_config0_1024_cube(hip, oracle, golden):
         assert np.array_equal(hip.sgemm(da, db).numpy(), c)
 
 
-@pytest.mark.parametrize("M,N,K", [(130, 200, 96), (256, 320, 96), (2048, 4096, 32), (64, 128, 2048), (33, 70, 512)])
+@pytest.mark.parametrize("M,N,K", [(130, 200, 96), (256, 320, 96), (2048, 4096, 32), (64, 128, 2048), (33, 70, 512), (1032, 1100, 96)])
 def test_sgemm_alpha_beta_bias_act(hip, oracle, M, N, K):
     say("sgemm epilogue", M, N, K)
     oracle.seed(21)
