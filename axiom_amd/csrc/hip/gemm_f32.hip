@@ -43,7 +43,7 @@ struct Operand {
     // element (r, k) of the logical [R, K] operand lives at src[r*ld + k] (KCONTIG) or
     // src[k*ld + r]
     __device__ __forceinline__ void fetch(const SRC *src, int64_t ld, int64_t r0, int64_t rows,
-                                          int64_t k0, int64_t K, int tid, bool vec_ok) {
+                                          int64_t k0, int64_t K, int tid) {
 #pragma unroll
         for (int i = 0; i < CHUNKS; i++) {
             const int c = tid + i * T;
@@ -53,9 +53,12 @@ struct Operand {
             const SRC *p = KCONTIG ? src + r * ld + k : src + k * ld + r;
             v4f v = {0.f, 0.f, 0.f, 0.f};
             if (sizeof(SRC) == 1) {                        // int8 source, K-contiguous only
-                const bool whole = !GUARD || (r < rows && k + 4 <= K && vec_ok);
+                // four elements wholly inside the row: one load at whatever alignment the row has
+                // (global memory takes unaligned vector loads)
+                const bool whole = !GUARD || (r < rows && k + 4 <= K);
                 if (whole) {
-                    int w = *reinterpret_cast<const int *>(p);
+                    int w;
+                    __builtin_memcpy(&w, p, 4);
                     v.x = (float)(signed char)(w & 0xff);
                     v.y = (float)(signed char)((w >> 8) & 0xff);
                     v.z = (float)(signed char)((w >> 16) & 0xff);
@@ -69,7 +72,7 @@ struct Operand {
                 v = *reinterpret_cast<const v4f *>(p);
             } else if (KCONTIG) {
                 if (r < rows) {
-                    if (vec_ok && k + 4 <= K) v = *reinterpret_cast<const v4f *>(p);
+                    if (k + 4 <= K) __builtin_memcpy(&v, p, 16);
                     else {
 #pragma unroll
                         for (int e = 0; e < 4; e++)
@@ -78,7 +81,7 @@ struct Operand {
                 }
             } else {
                 if (k < K) {
-                    if (vec_ok && r + 4 <= rows) v = *reinterpret_cast<const v4f *>(p);
+                    if (r + 4 <= rows) __builtin_memcpy(&v, p, 16);
                     else {
 #pragma unroll
                         for (int e = 0; e < 4; e++)
@@ -133,15 +136,6 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm(SgemmArgs g) {
     const BSRC *B = static_cast<const BSRC *>(g.B) + batch * g.stride_b;
     float *C = g.C + batch * g.stride_c;
 
-    bool vec_a = true, vec_b = true;
-    if (GUARD) {
-        vec_a = ((((uintptr_t)A >> 2) | (uintptr_t)g.lda | (uintptr_t)g.stride_a) & 3) == 0 &&
-                ((uintptr_t)A & 3) == 0;
-        vec_b = sizeof(BSRC) == 1
-                    ? ((((uintptr_t)B) | (uintptr_t)g.ldb) & 3) == 0
-                    : ((((uintptr_t)B >> 2) | (uintptr_t)g.ldb | (uintptr_t)g.stride_b) & 3) == 0;
-    }
-
     OpA opa;
     OpB opb;
     const int64_t slabs = (g.K + BK - 1) / BK;
@@ -153,8 +147,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm(SgemmArgs g) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    opa.fetch(A, g.lda, m0, g.M, 0, g.K, tid, vec_a);
-    opb.fetch(B, g.ldb, n0, g.N, 0, g.K, tid, vec_b);
+    opa.fetch(A, g.lda, m0, g.M, 0, g.K, tid);
+    opb.fetch(B, g.ldb, n0, g.N, 0, g.K, tid);
     opa.stash(lds_f, tid);
     opb.stash(lds_f + OpA::FLOATS, tid);
     __syncthreads();
@@ -163,8 +157,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) k_sgemm(SgemmArgs g) {
     for (int64_t s = 0; s < slabs; s++) {
         const int cur = (int)(s & 1);
         if (s + 1 < slabs) {
-            opa.fetch(A, g.lda, m0, g.M, (s + 1) * BK, g.K, tid, vec_a);
-            opb.fetch(B, g.ldb, n0, g.N, (s + 1) * BK, g.K, tid, vec_b);
+            opa.fetch(A, g.lda, m0, g.M, (s + 1) * BK, g.K, tid);
+            opb.fetch(B, g.ldb, n0, g.N, (s + 1) * BK, g.K, tid);
         }
         const float *sa = lds_f + cur * STAGE;
         const float *sb = sa + OpA::FLOATS;

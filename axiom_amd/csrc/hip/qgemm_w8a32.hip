@@ -1,7 +1,7 @@
 // W8A32: out[m,n] = w_scales[n] * sum_k a[m,k] * (float)w[n,k], fp32 accumulation.
 //
 // M <= 8 (the bandwidth-bound inference case): one wave owns 4 weight rows.  Lanes walk K in
-// 16-byte steps (a wave-wide load covers 1 KiB of one row), each lane keeps the activations of
+// 16-element steps (a wave-wide load covers 1 KiB of one row), each lane keeps the activations of
 // its k positions in registers across the 4 rows, and the 4*M partial sums are reduced over
 // the wave together, in a fixed tree order, ending one per lane for the write-back.  Larger M goes through the fp32
 // matrix-core GEMM with the int8 operand converted while it is staged in LDS.
@@ -17,7 +17,7 @@ using namespace axhip;
 
 constexpr int ROWS = 4;   // weight rows per wave
 
-template <int MR, bool VEC>
+template <int MR>
 __global__ void __launch_bounds__(64)
 k_w8a32_gemv(const float *__restrict__ a, const int8_t *__restrict__ w,
              const float *__restrict__ w_scales, float *__restrict__ out, int64_t N, int64_t K) {
@@ -30,13 +30,18 @@ k_w8a32_gemv(const float *__restrict__ a, const int8_t *__restrict__ w,
         for (int m = 0; m < MR; m++) acc[r][m] = 0.0f;
 
     for (int64_t k = (int64_t)lane * 16; k < K; k += 64 * 16) {
+        // A step wholly inside the row is fetched with 16-byte loads at whatever alignment K and
+        // the base pointers leave (global memory takes unaligned vector loads); only the last,
+        // partial step of a row goes element by element.
+        const bool whole = k + 16 <= K;
         float xa[MR][16];
-        if (VEC) {
+        if (whole) {
 #pragma unroll
             for (int m = 0; m < MR; m++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    v4f t = *reinterpret_cast<const v4f *>(a + m * K + k + 4 * q);
+                    v4f t;
+                    __builtin_memcpy(&t, a + m * K + k + 4 * q, 16);
                     xa[m][4 * q] = t.x; xa[m][4 * q + 1] = t.y; xa[m][4 * q + 2] = t.z; xa[m][4 * q + 3] = t.w;
                 }
         } else {
@@ -50,8 +55,9 @@ k_w8a32_gemv(const float *__restrict__ a, const int8_t *__restrict__ w,
             const int64_t n = n0 + r;
             if (n >= N) break;
             float wf[16];
-            if (VEC) {
-                v4i p = *reinterpret_cast<const v4i *>(w + n * K + k);
+            if (whole) {
+                v4i p;
+                __builtin_memcpy(&p, w + n * K + k, 16);
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const int word = p[q];
@@ -81,11 +87,9 @@ k_w8a32_gemv(const float *__restrict__ a, const int8_t *__restrict__ w,
 }
 
 template <int MR>
-int launch_gemv(bool vec, const float *a, const int8_t *w, const float *s, float *out, int64_t N,
-                int64_t K) {
+int launch_gemv(const float *a, const int8_t *w, const float *s, float *out, int64_t N, int64_t K) {
     dim3 grid((unsigned)((N + ROWS - 1) / ROWS));
-    if (vec) hipLaunchKernelGGL((k_w8a32_gemv<MR, true>), grid, dim3(64), 0, kStream, a, w, s, out, N, K);
-    else hipLaunchKernelGGL((k_w8a32_gemv<MR, false>), grid, dim3(64), 0, kStream, a, w, s, out, N, K);
+    hipLaunchKernelGGL(k_w8a32_gemv<MR>, grid, dim3(64), 0, kStream, a, w, s, out, N, K);
     return check_launch("qgemm_w8a32_gemv");
 }
 }  // namespace
@@ -98,16 +102,15 @@ extern "C" int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w
     if (M == 0 || N == 0) return AXHIP_OK;
     if (M > 8) return axhip::sgemm_i8w(M, N, K, a, w, w_scales, out);
     if ((N + ROWS - 1) / ROWS > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a32: N too large");
-    const bool vec = (K % 16 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
-    note_kernel(vec ? "qgemm_w8a32_gemv_vec16" : "qgemm_w8a32_gemv_scalar");
+    note_kernel("qgemm_w8a32_gemv");
     switch (M) {
-        case 1: return launch_gemv<1>(vec, a, w, w_scales, out, N, K);
-        case 2: return launch_gemv<2>(vec, a, w, w_scales, out, N, K);
-        case 3: return launch_gemv<3>(vec, a, w, w_scales, out, N, K);
-        case 4: return launch_gemv<4>(vec, a, w, w_scales, out, N, K);
-        case 5: return launch_gemv<5>(vec, a, w, w_scales, out, N, K);
-        case 6: return launch_gemv<6>(vec, a, w, w_scales, out, N, K);
-        case 7: return launch_gemv<7>(vec, a, w, w_scales, out, N, K);
-        default: return launch_gemv<8>(vec, a, w, w_scales, out, N, K);
+        case 1: return launch_gemv<1>(a, w, w_scales, out, N, K);
+        case 2: return launch_gemv<2>(a, w, w_scales, out, N, K);
+        case 3: return launch_gemv<3>(a, w, w_scales, out, N, K);
+        case 4: return launch_gemv<4>(a, w, w_scales, out, N, K);
+        case 5: return launch_gemv<5>(a, w, w_scales, out, N, K);
+        case 6: return launch_gemv<6>(a, w, w_scales, out, N, K);
+        case 7: return launch_gemv<7>(a, w, w_scales, out, N, K);
+        default: return launch_gemv<8>(a, w, w_scales, out, N, K);
     }
 }

@@ -125,7 +125,8 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               # few output tiles and a long K: the split-K route (bench_qgemm.c shapes among them)
               (32, 768, 768), (64, 1024, 4096), (128, 4096, 1024), (9, 100, 512), (16, 16, 8192), (70, 130, 1536),
               # off the tile grid with a large interior: fast kernels inside, guarded kernel on the fringes
-              (1032, 1100, 96), (2100, 4200, 64), (1024, 1092, 160)]
+              (1032, 1100, 96), (2100, 4200, 64), (1024, 1092, 160),
+              (130, 257, 1027), (67, 1001, 129)]                  # rows off the 16-byte grid in every form
 
 
 @pytest.mark.parametrize("M,N,K", F32_SHAPES)
@@ -377,7 +378,8 @@ def test_config4b_attention_shapes_full_size(hip, oracle):
 W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 1024), (3, 17, 45),
                 (1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024),
                 (64, 1024, 4096), (1, 4096, 4096), (5, 33, 100),
-                (2, 130, 256), (6, 67, 1040), (7, 5, 2064)]       # every row count of the wave-per-rows form
+                (2, 130, 256), (6, 67, 1040), (7, 5, 2064),
+                (32, 128, 517), (70, 260, 1031), (3, 64, 1037)]   # rows at odd byte offsets       # every row count of the wave-per-rows form
 
 
 @pytest.mark.parametrize("M,N,K", W8A32_SHAPES)
