@@ -121,14 +121,19 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
             }
         }
     } else {
-        // all loads of a batch of rows are issued before the first use, as in the vector form
+        // rows off the 16-byte grid (N or ldb not a multiple of 4): whole column groups still take one
+        // 16-byte load each, at the alignment the row has; the last, partial group goes by element.
+        // All loads of a batch of rows are issued before the first use, as in the vector form.
         for (; k + (UNROLL - 1) * KGROUPS < klen; k += UNROLL * KGROUPS) {
             float w[UNROLL][4];
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++)
+            for (int u = 0; u < UNROLL; u++) {
+                const float *rp = bp + (k_begin + k + u * KGROUPS) * ldb;
+                if (col + 4 <= N) __builtin_memcpy(w[u], rp, 16);      // one load, whatever the row's alignment
+                else
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    w[u][e] = (col + e < N) ? bp[(k_begin + k + u * KGROUPS) * ldb + e] : 0.0f;
+                    for (int e = 0; e < 4; e++) w[u][e] = (col + e < N) ? rp[e] : 0.0f;
+            }
 #pragma unroll
             for (int u = 0; u < UNROLL; u++)
 #pragma unroll
@@ -140,8 +145,11 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
         }
         for (; k < klen; k += KGROUPS) {
             float w[4];
+            const float *rp = bp + (k_begin + k) * ldb;
+            if (col + 4 <= N) __builtin_memcpy(w, rp, 16);
+            else
 #pragma unroll
-            for (int e = 0; e < 4; e++) w[e] = (col + e < N) ? bp[(k_begin + k) * ldb + e] : 0.0f;
+                for (int e = 0; e < 4; e++) w[e] = (col + e < N) ? rp[e] : 0.0f;
 #pragma unroll
             for (int m = 0; m < MR; m++) {
                 const float xv = xs[m * k_per_split + k];
