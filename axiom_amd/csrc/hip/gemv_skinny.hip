@@ -20,7 +20,7 @@ constexpr int COLS = 64;        // columns per workgroup
 constexpr int KGROUPS = 16;     // lane groups per workgroup, each 16 lanes x float4
 constexpr int UNROLL = 8;
 // workgroups to aim for: enough to cover 256 CUs a few times over; partial-sum traffic grows with M
-int64_t g_want_blocks_m12 = 1024, g_want_blocks_m38 = 512;
+constexpr int64_t kWantBlocksM12 = 1024, kWantBlocksM38 = 512;
 
 template <int MR, bool VEC>
 __global__ void __launch_bounds__(256)
@@ -275,7 +275,7 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
 
     const int64_t col_blocks = (N + COLS - 1) / COLS;
     // enough workgroups to cover 256 CUs a few times over, each with at least 128 k rows
-    const int64_t want_blocks = M <= 2 ? g_want_blocks_m12 : g_want_blocks_m38;
+    const int64_t want_blocks = M <= 2 ? kWantBlocksM12 : kWantBlocksM38;
     int64_t splits = (want_blocks + col_blocks - 1) / col_blocks;
     const int64_t max_splits = K >= 128 ? K / 128 : 1;
     if (splits > max_splits) splits = max_splits;
