@@ -269,6 +269,14 @@ def secondary(hip):
     res["streaming_slots_16384x4096"] = stream
     del xa, xb, xo, vec, rowv, colv, m2
 
+    # what this box charges per launch, whatever the kernel does: back-to-back fills of 64 floats on the
+    # stream.  The latency-bound figures above and below (bs=1 layers, few-tile GEMMs, the encoder) are
+    # read against it, as the streaming ones are against the read / copy rates measured just above.
+    tiny = hip.empty((64,))
+    _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_fill_f32(tiny.ptr, 1.0, 64)))
+    res["launch_floor_us"] = ms * 1e3
+    del tiny
+
     # the seven shapes of the reference's benchmarks/bench_qgemm.c:76-82 (fp32 GEMM against W8A32 on the
     # same weights), on device-resident operands, plus W8A8 with the activations quantized per tensor
     qshapes = {}
