@@ -694,13 +694,23 @@ int64_t split_count(int64_t M, int64_t N, int64_t K) {
     const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
     const int64_t cus = cu_count();
     if (tiles * 2 > cus || K < 256 || K % 32 != 0) return 1;
-    // One workgroup per CU measured best (32x768x768: 10.5 us against 27 unsplit; 64x1024x4096:
-    // 12 against 70; 128x4096x1024: 16.5 against 20); more ranges only add partial sums to move.
-    int64_t want = (cus + tiles - 1) / tiles;
-    if (want > K / 64) want = K / 64;                      // ranges of at least 64
+    // Tiles on the 64 grid run the direct-to-LDS kernel, for which one workgroup per CU measured
+    // best (32x768x768: 10.5 us against 27 unsplit; 64x1024x4096: 12 against 70; 128x4096x1024: 16.5
+    // against 20; more ranges only add partial sums to move).  Ragged tiles run the register-staged
+    // kernel, whose slabs each wait out a load: four workgroups per CU cover one another's waits
+    // (4x4100x4096: 65 -> 36 us; 9x8000x8192: 123 -> 85).
+    const bool ragged = M % 64 != 0 || N % 64 != 0;
+    int64_t want = ((ragged ? 4 : 1) * cus + tiles - 1) / tiles;
+    const int64_t most = K / 64;                             // ranges of at least 64
+    if (want > most) want = most;
+    // K / 32 must divide into the ranges: the nearest count at or below the wish, or, when that is
+    // under half of it (K = 4000 has only 5, 25 and 125), the nearest above up to twice the wish
+    int64_t below = 1, above = 0;
     for (int64_t s = want; s >= 2; s--)
-        if (K % (s * 32) == 0) return s;
-    return 1;
+        if (K % (s * 32) == 0) { below = s; break; }
+    for (int64_t s = want + 1; s <= 2 * want && s <= most; s++)
+        if (K % (s * 32) == 0) { above = s; break; }
+    return (below * 2 < want && above) ? above : below;
 }
 
 // returns -1 when the shape is left to the ordinary path
@@ -766,21 +776,24 @@ int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
 // (4000^3: 101 TFLOP/s against 141 on the grid).  Its grid-aligned interior goes to the
 // direct-to-LDS kernels instead and only the right and bottom fringes to the guarded one; every
 // block is a sub-matrix reached by pointer offsets.  Returns -1 when the shape is left alone.
-int try_interior_and_fringes(const SgemmArgs &g, int transa, int transb) {
+int try_interior_and_fringes(const SgemmArgs &g, int transa, int transb, int64_t min_tiles = 256) {
     if ((transa && transb) || g.K % 32 != 0 || g.K <= 0) return -1;
     if ((((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.C | (uintptr_t)g.bias) & 15) != 0 || g.lda % 4 != 0 ||
         g.ldb % 4 != 0 || g.ldc % 4 != 0)
         return -1;                                           // the interior would not qualify for the fast kernels either
     int64_t gm, gn;
     if ((g.M / 128) * (g.N / 256) >= 256) gm = 128, gn = 256;
-    else if ((g.M / 64) * (g.N / 64) >= 256) gm = gn = 64;
+    else if ((g.M / 64) * (g.N / 64) >= min_tiles) gm = gn = 64;
     else return -1;
     const int64_t Mi = g.M / gm * gm, Ni = g.N / gn * gn;
     if (Mi == g.M && Ni == g.N) return -1;
     const float *A = static_cast<const float *>(g.A), *B = static_cast<const float *>(g.B);
-    // a fringe is a strip of few tiles with the whole K: the split-K route when it qualifies
+    // a fringe is a strip of few tiles with the whole K: the split-K route when it qualifies; a
+    // wide one (up to 255 columns beside 128x256 tiles) is itself cut into its part on the 64 grid
+    // and a narrower fringe
     auto fringe = [&](const SgemmArgs &f) {
-        const int rc = try_split_k<float>(f, transa, transb, "sgemm_splitk", nullptr);
+        int rc = try_split_k<float>(f, transa, transb, "sgemm_splitk", nullptr);
+        if (rc < 0 && min_tiles == 256) rc = try_interior_and_fringes(f, transa, transb, 64);
         return rc >= 0 ? rc : dispatch_f32(f, transa, transb, 1);
     };
     SgemmArgs p = g;
@@ -807,6 +820,45 @@ int try_interior_and_fringes(const SgemmArgs &g, int transa, int transb) {
     return rc;
 }
 
+int run_f32(const SgemmArgs &g, int transa, int transb);
+
+// K off the 32 grid keeps a large product off every fast kernel.  It is run as the product over the
+// first K / 32 * 32 columns (alpha and beta as given, no bias or activation yet) followed by the
+// few remaining columns accumulated on top (beta = 1) with the bias and activation of the whole.
+// Returns -1 when the shape is left alone.
+int try_k_tail(const SgemmArgs &g, int transa, int transb) {
+    const int64_t Km = g.K / 32 * 32;
+    if ((transa && transb) || Km == g.K || Km < 512 || (g.M / 64) * (g.N / 64) < 256) return -1;
+    const float *A = static_cast<const float *>(g.A), *B = static_cast<const float *>(g.B);
+    SgemmArgs p = g;
+    p.K = Km;
+    p.bias = nullptr;
+    p.act = AXHIP_ACT_NONE;
+    int rc = run_f32(p, transa, transb);
+    if (rc != AXHIP_OK) return rc;
+    p = g;
+    p.K = g.K - Km;
+    p.A = transa ? A + Km * g.lda : A + Km;
+    p.B = transb ? B + Km : B + Km * g.ldb;
+    p.beta = 1.0f;
+    rc = dispatch_f32(p, transa, transb, 1);
+    note_kernel("sgemm_main+k_tail");
+    return rc;
+}
+
+// a single product: the route for its shape
+int run_f32(const SgemmArgs &g, int transa, int transb) {
+    if (!(transa && transb)) {
+        int rc = try_split_k<float>(g, transa, transb, "sgemm_splitk", nullptr);
+        if (rc >= 0) return rc;
+        rc = try_interior_and_fringes(g, transa, transb);
+        if (rc >= 0) return rc;
+        rc = try_k_tail(g, transa, transb);
+        if (rc >= 0) return rc;
+    }
+    return dispatch_f32(g, transa, transb, 1);
+}
+
 }  // namespace
 
 namespace axhip {
@@ -831,13 +883,7 @@ extern "C" int axhip_sgemm(int transa, int transb, int64_t M, int64_t N, int64_t
     if (M <= 8 && !transa && !transb && alpha == 1.0f && beta == 0.0f)
         return axhip_sgemm_skinny(M, N, K, A, lda, B, ldb, C, ldc, bias, act);
     SgemmArgs g{A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, alpha, beta, nullptr, bias, act};
-    if (!(transa && transb)) {
-        int rc = try_split_k<float>(g, transa, transb, "sgemm_splitk", nullptr);
-        if (rc >= 0) return rc;
-        rc = try_interior_and_fringes(g, transa, transb);
-        if (rc >= 0) return rc;
-    }
-    return dispatch_f32(g, transa, transb, 1);
+    return run_f32(g, transa, transb);
 }
 
 extern "C" int axhip_sgemm_strided_batched(int transa, int transb, int64_t M, int64_t N, int64_t K,

@@ -126,7 +126,8 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               (32, 768, 768), (64, 1024, 4096), (128, 4096, 1024), (9, 100, 512), (16, 16, 8192), (70, 130, 1536),
               # off the tile grid with a large interior: fast kernels inside, guarded kernel on the fringes
               (1032, 1100, 96), (2100, 4200, 64), (1024, 1092, 160),
-              (130, 257, 1027), (67, 1001, 129)]                  # rows off the 16-byte grid in every form
+              (130, 257, 1027), (67, 1001, 129),                  # rows off the 16-byte grid in every form
+              (1024, 1088, 1045), (1030, 1100, 600)]              # K off the 32 grid: main product, then the K tail on top
 
 
 @pytest.mark.parametrize("M,N,K", F32_SHAPES)
@@ -228,7 +229,7 @@ def test_sgemm_config0_1024_cube(hip, oracle, golden):
         assert np.array_equal(hip.sgemm(da, db).numpy(), c)
 
 
-@pytest.mark.parametrize("M,N,K", [(130, 200, 96), (256, 320, 96), (2048, 4096, 32), (64, 128, 2048), (33, 70, 512), (1032, 1100, 96)])
+@pytest.mark.parametrize("M,N,K", [(130, 200, 96), (256, 320, 96), (2048, 4096, 32), (64, 128, 2048), (33, 70, 512), (1032, 1100, 96), (1024, 1088, 1045)])
 def test_sgemm_alpha_beta_bias_act(hip, oracle, M, N, K):
     say("sgemm epilogue", M, N, K)
     oracle.seed(21)
