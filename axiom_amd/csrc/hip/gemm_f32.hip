@@ -868,9 +868,28 @@ int sgemm_i8w(int64_t M, int64_t N, int64_t K, const float *a, const int8_t *w,
     static const char *const names[3] = {"qgemm_w8a32_mfma_128x128", "qgemm_w8a32_mfma_64x64",
                                          "qgemm_w8a32_mfma_64x64_guarded"};
     SgemmArgs g{a, w, out, M, N, K, K, K, N, 0, 0, 0, 1.0f, 0.0f, w_scales, nullptr, AXHIP_ACT_NONE};
-    const int rc = try_split_k<int8_t>(g, 0, 1, "qgemm_w8a32_mfma_splitk", names);
-    if (rc >= 0) return rc;
-    return pick_tile<true, true, int8_t>(names, g, 1);
+    auto run = [&](const SgemmArgs &p) {
+        const int rc = try_split_k<int8_t>(p, 0, 1, "qgemm_w8a32_mfma_splitk", names);
+        return rc >= 0 ? rc : pick_tile<true, true, int8_t>(names, p, 1);
+    };
+    // K off the 32 grid cannot be cut into ranges: the first K / 32 * 32 columns as above, then the
+    // remaining few accumulated on top (the column scale applies to each part's sum alike)
+    const int64_t Km = K / 32 * 32;
+    if (Km != K && Km >= 512) {
+        SgemmArgs p = g;
+        p.K = Km;
+        int rc = run(p);
+        if (rc != AXHIP_OK) return rc;
+        p = g;
+        p.K = K - Km;
+        p.A = a + Km;
+        p.B = w + Km;
+        p.beta = 1.0f;
+        rc = pick_tile<true, true, int8_t>(names, p, 1);
+        note_kernel("qgemm_w8a32_mfma_main+k_tail");
+        return rc;
+    }
+    return run(g);
 }
 }  // namespace axhip
 
