@@ -16,6 +16,8 @@
 // LDS rows are 128 bytes = 32 banks, so the 16-byte chunk index is XOR-swizzled with
 // (row >> 1) & 7: the 16 lanes served together by a ds_read_b128 (16 consecutive rows, one
 // chunk) and the 16 lanes of a ds_write_b128 (2 rows x 8 chunks) then touch 64 distinct banks.
+#include <cstring>
+
 #include "common.h"
 
 namespace {
@@ -828,6 +830,16 @@ int launch_gemv(const int8_t *x, float x_scale, const int8_t *w, const float *w_
 }
 
 
+// rows of K bytes -> rows of Kp >= K bytes (Kp a multiple of 16), the tail of each row zero
+__global__ void __launch_bounds__(256)
+k_pad_rows_i8(const int8_t *__restrict__ src, int8_t *__restrict__ dst, int64_t rows, int64_t K, int64_t Kp) {
+    const int64_t per_row = Kp / 16, items = rows * per_row, stride = (int64_t)gridDim.x * 256;
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < items; t += stride) {
+        const int64_t r = t / per_row, k = (t - r * per_row) * 16;
+        *reinterpret_cast<v4i *>(dst + r * Kp + k) = load_chunk<true>(src, r, rows, k, K);
+    }
+}
+
 // One block of the output, rows of pitch ldc: picks the kernel for its shape and alignment.
 int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_scales, const float *bias, int act,
                 float *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K, int64_t ldc) {
@@ -880,6 +892,23 @@ extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
             case 7: return launch_gemv<7>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
             default: return launch_gemv<8>(x, x_scale, w, w_scales, bias, act, out, acc_out, N, K);
         }
+    }
+    // K off the 128 grid would keep a large product off the direct-to-LDS kernels (8192^2 x 8200:
+    // 0.85 POP/s).  Both operands are copied once into rows padded with zeros to the next multiple
+    // of 128 — zeros add nothing to an integer sum — and the product runs on the copies.
+    const int64_t Kp = (K + BK - 1) / BK * BK;
+    if (K % BK != 0 && K >= 512 && (M / 256) * (N / 256) >= 128 && (uint64_t)(M + N) * (uint64_t)Kp <= (uint64_t(1) << 30)) {
+        int8_t *xp = static_cast<int8_t *>(workspace((size_t)(M + N) * (size_t)Kp));
+        if (!xp) return AXHIP_ERR_ALLOC;
+        int8_t *wp = xp + M * Kp;
+        const int64_t bx = (M * (Kp / 16) + 255) / 256, bw = (N * (Kp / 16) + 255) / 256;
+        hipLaunchKernelGGL(k_pad_rows_i8, dim3((unsigned)(bx < 65536 ? bx : 65536)), dim3(256), 0, kStream, x, xp, M, K, Kp);
+        hipLaunchKernelGGL(k_pad_rows_i8, dim3((unsigned)(bw < 65536 ? bw : 65536)), dim3(256), 0, kStream, w, wp, N, K, Kp);
+        if (int rc = check_launch("qgemm_w8a8 row padding")) return rc;
+        const int rc = axhip_qgemm_w8a8(xp, x_scale, wp, w_scales, bias, act, out, acc_out, M, N, Kp);
+        note_kernel(strstr(axhip_last_kernel(), "fringes") ? "qgemm_w8a8_256x256_dma+fringes+k_padded"
+                                                           : "qgemm_w8a8_256x256_dma+k_padded");
+        return rc;
     }
     const bool fast = ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) && K % BK == 0 && K > 0 && K < (int64_t(1) << 24) &&
                       N % 4 == 0 && (!out || (((uintptr_t)out | (uintptr_t)w_scales | (uintptr_t)bias) & 15) == 0) &&

@@ -35,7 +35,9 @@ INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300
                # off the 256 grid with a large interior: persistent kernel inside, smaller tiles on the fringes
                (2112, 4128, 256), (4100, 2304, 128), (2048, 4100, 128),
                # rows that start at odd byte offsets (K % 16 != 0)
-               (70, 90, 1037), (130, 257, 4099)]
+               (70, 90, 1037), (130, 257, 4099),
+               # large with K off the 128 grid: zero-padded copies of both operands, then the fast kernels
+               (2048, 4096, 520), (2112, 4128, 600)]
 
 
 @pytest.mark.parametrize("M,N,K", INT8_SHAPES)
