@@ -1,7 +1,8 @@
 // Scaled dot-product attention forward: O = softmax(scale * Q K^T [+ causal mask]) V per head,
 // Q, K, V, O [BH, S, dk] row-major fp32, L [BH, S] = log-sum-exp of each score row (or NULL).
 //
-// Fused kernel (dk = 32, 64 or 128, any S): the score matrix never leaves the chip.  A
+// Fused kernel (dk a multiple of 4 up to 128, on the geometry of the next size among 32, 64 and
+// 128; any S): the score matrix never leaves the chip.  A
 // workgroup of 4 waves owns 128 query rows of one head, a wave 32 of them; keys and values
 // stream through LDS in blocks of 64 (direct-to-LDS loads, two stages).  Both products run on
 // v_mfma_f32_32x32x2_f32 with the query index on the MFMA's column side, so lane l of a wave
@@ -72,11 +73,16 @@ struct SdGeom {
 // RAG: S is not a multiple of 128.  Rows past the end of a head are never loaded (the load of such
 // a row is redirected to the head's last row, which keeps V finite), keys past the end are masked
 // like causal ones, and queries past the end are computed but not stored.
-template <int DK, bool CAUSAL, bool RAG>
+// PAD: the head size dkr is below DK (a multiple of 4).  Lanes whose 16-byte chunk lies past column
+// dkr issue no load, so nothing outside a row is read; their places in the K stages are zeroed once
+// and never written again, Q's are zeroed in registers, V's feed output columns that are not stored.
+// The padded k-blocks and output tiles are multiplied like the others: branching around them
+// measured slower than the MFMAs they save (dk 96: 303 us with the branches, 268 without).
+template <int DK, bool CAUSAL, bool RAG, bool PAD>
 __global__ void __launch_bounds__(256)
 k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__restrict__ V,
        float *__restrict__ O, float *__restrict__ L, int64_t BH, int64_t S, float scale_log2e,
-       int64_t H, int64_t ld, int64_t ldo) {
+       int64_t H, int64_t ld, int64_t ldo, int dkr) {
     using G = SdGeom<DK>;
     constexpr int KB = DK / 8;                   // 8-wide k-blocks of the score product
     constexpr int DT = DK / 32;                  // 32-wide column tiles of the output
@@ -100,18 +106,26 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
     // and ldo (O): H = 1, ld = DK is one matrix per head; H heads side by side in rows of
     // ld >= H * DK floats is the layout a fused projection writes and the output projection reads
     const int64_t hb = head / H, hh = head - hb * H;
-    const int64_t in0 = hb * S * ld + hh * DK;
+    const int64_t in0 = hb * S * ld + hh * (PAD ? dkr : DK);
     const float *Qh = Q + in0, *Kh = K + in0, *Vh = V + in0;
     const unsigned rowb = (unsigned)ld * 4;      // bytes between rows in global memory
     const unsigned lds0 = (unsigned)(uintptr_t)lds;
+    if (PAD) {                                   // the K stages' never-loaded chunks must read as zero
+        for (int o = tid * 16; o < 2 * G::KSTAGE; o += 256 * 16)
+            *reinterpret_cast<v4f *>(lds + o) = v4f{0.f, 0.f, 0.f, 0.f};
+        __syncthreads();
+    }
 
     // per-lane byte offsets of the direct-to-LDS loads: instruction i of this wave is number
     // 4*i + wave of a 64-row block and covers rows RPI*(4*i + wave) .. + RPI-1
     unsigned koff[G::IPW], voff[G::IPW];
+    bool kact[G::IPW];                           // PAD: does this lane's chunk of a K / Q row exist
+    const bool vact = !PAD || (lane % G::CH) * 4 < dkr;
 #pragma unroll
     for (int i = 0; i < G::IPW; i++) {
         const int slot = lane / G::CH, c = lane % G::CH;
         const int krow = G::RPI * (4 * i + wave) + slot;
+        kact[i] = !PAD || (c ^ G::swz(krow)) * 4 < dkr;
         koff[i] = (unsigned)(krow * rowb + ((c ^ G::swz(krow)) << 4));
         const int vrow = G::RPI * (4 * i + wave) + G::v_row_of_slot(slot);
         voff[i] = (unsigned)(vrow * rowb + (c << 4));
@@ -145,10 +159,11 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
             if (RAG && valid < SD_BKV) {
 #pragma unroll
                 for (int i = 0; i < G::IPW; i++)
-                    AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff_clamped(i, (int)valid), kg);
+                    if (kact[i]) AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff_clamped(i, (int)valid), kg);
             } else {
 #pragma unroll
-                for (int i = 0; i < G::IPW; i++) AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
+                for (int i = 0; i < G::IPW; i++)
+                    if (kact[i]) AXS_LOAD_LDS(lds0 + stage * G::KSTAGE + (4 * i + wave) * 1024, koff[i], kg);
             }
         };
         auto issue_v = [&](int64_t blk, int stage) {
@@ -157,11 +172,11 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
             if (RAG && valid < SD_BKV) {
 #pragma unroll
                 for (int i = 0; i < G::IPW; i++)
-                    AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff_clamped(i, (int)valid), vg);
+                    if (vact) AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff_clamped(i, (int)valid), vg);
             } else {
 #pragma unroll
                 for (int i = 0; i < G::IPW; i++)
-                    AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff[i], vg);
+                    if (vact) AXS_LOAD_LDS(lds0 + 2 * G::KSTAGE + stage * G::VSTAGE + (4 * i + wave) * G::VGROUP, voff[i], vg);
             }
         };
         if (RAG && q0 + SD_BQ > S) {
@@ -170,6 +185,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
             const int64_t base1 = left1 > 0 ? q0 + 64 : q0, valid1 = left1 > 0 ? (left1 < 64 ? left1 : 64) : valid0;
 #pragma unroll
             for (int i = 0; i < G::IPW; i++) {
+                if (!kact[i]) continue;
                 AXS_LOAD_LDS(lds0 + Q_BASE + (4 * i + wave) * 1024, koff_clamped(i, (int)valid0),
                              reinterpret_cast<const char *>(Qh + q0 * ld));
                 AXS_LOAD_LDS(lds0 + Q_BASE + G::KSTAGE + (4 * i + wave) * 1024, koff_clamped(i, (int)valid1),
@@ -178,6 +194,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
         } else {
 #pragma unroll
             for (int i = 0; i < G::IPW; i++) {
+                if (!kact[i]) continue;
                 AXS_LOAD_LDS(lds0 + Q_BASE + (4 * i + wave) * 1024, koff[i], reinterpret_cast<const char *>(Qh + q0 * ld));
                 AXS_LOAD_LDS(lds0 + Q_BASE + G::KSTAGE + (4 * i + wave) * 1024, koff[i],
                              reinterpret_cast<const char *>(Qh + (q0 + 64) * ld));
@@ -192,7 +209,10 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
             const unsigned char *qrow = lds + Q_BASE + (r >> 6) * G::KSTAGE + (r & 63) * G::ROWB;
 #pragma unroll
             for (int kb = 0; kb < KB; kb++)      // scale * log2(e) goes into Q once: scores come out in log2 units
+            {
                 qf[kb] = *reinterpret_cast<const v4f *>(qrow + (((kb * 2 + fhalf) ^ G::swz(r & 63)) << 4)) * scale_log2e;
+                if (PAD && kb * 8 + 4 * fhalf >= dkr) qf[kb] = v4f{0.f, 0.f, 0.f, 0.f};   // whatever the unloaded chunk held
+            }
         }
         __syncthreads();
         issue_v(0, 0);
@@ -313,7 +333,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
         // ---- normalise and write: lane owns query qg, dk columns 32*d + 8*g + 4*fhalf .. +3 ----
         const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
         const float inv = 1.0f / l_tot;
-        float *orow = O + (hb * S + qg) * ldo + hh * DK;
+        float *orow = O + (hb * S + qg) * ldo + hh * (PAD ? dkr : DK);
         if (!RAG || qg < S) {
 #pragma unroll
             for (int d = 0; d < DT; d++)
@@ -322,22 +342,22 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
                     v4f r;
 #pragma unroll
                     for (int e = 0; e < 4; e++) r[e] = acc_o[d][4 * g + e] * inv;
-                    *reinterpret_cast<v4f *>(orow + d * 32 + 8 * g + 4 * fhalf) = r;
+                    if (!PAD || d * 32 + 8 * g + 4 * fhalf < dkr) *reinterpret_cast<v4f *>(orow + d * 32 + 8 * g + 4 * fhalf) = r;
                 }
             if (L && fhalf == 0) L[head * S + qg] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
         }
     }
 }
 
-template <int DK>
-int launch_sdpa(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH, int64_t S,
-                float scale, int causal, int64_t H, int64_t ld, int64_t ldo) {
+template <int DK, bool PAD>
+int launch_sdpa_p(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH, int64_t S,
+                  float scale, int causal, int64_t H, int64_t ld, int64_t ldo, int dkr) {
     using G = SdGeom<DK>;
     static bool attr_set = false;
-    const void *kernels[4] = {reinterpret_cast<const void *>(k_sdpa<DK, false, false>),
-                              reinterpret_cast<const void *>(k_sdpa<DK, true, false>),
-                              reinterpret_cast<const void *>(k_sdpa<DK, false, true>),
-                              reinterpret_cast<const void *>(k_sdpa<DK, true, true>)};
+    const void *kernels[4] = {reinterpret_cast<const void *>(k_sdpa<DK, false, false, PAD>),
+                              reinterpret_cast<const void *>(k_sdpa<DK, true, false, PAD>),
+                              reinterpret_cast<const void *>(k_sdpa<DK, false, true, PAD>),
+                              reinterpret_cast<const void *>(k_sdpa<DK, true, true, PAD>)};
     if (!attr_set) {
         for (const void *k : kernels)
             AXHIP_HIP_TRY(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, G::SMEM), "hipFuncSetAttribute");
@@ -347,11 +367,22 @@ int launch_sdpa(const float *Q, const float *K, const float *V, float *O, float 
     const int64_t nq = (S + SD_BQ - 1) / SD_BQ;
     dim3 grid((unsigned)((causal ? (nq + 1) / 2 : nq) * BH));
     const bool rag = S % SD_BQ != 0;
-    if (causal && rag) hipLaunchKernelGGL((k_sdpa<DK, true, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, ldo);
-    else if (causal) hipLaunchKernelGGL((k_sdpa<DK, true, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, ldo);
-    else if (rag) hipLaunchKernelGGL((k_sdpa<DK, false, true>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, ldo);
-    else hipLaunchKernelGGL((k_sdpa<DK, false, false>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, ldo);
+#define AXS_GO(C, R)                                                                                              \
+    hipLaunchKernelGGL((k_sdpa<DK, C, R, PAD>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, \
+                       ldo, dkr)
+    if (causal && rag) AXS_GO(true, true);
+    else if (causal) AXS_GO(true, false);
+    else if (rag) AXS_GO(false, true);
+    else AXS_GO(false, false);
+#undef AXS_GO
     return check_launch("sdpa_fwd");
+}
+
+template <int DK>
+int launch_sdpa(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH, int64_t S,
+                float scale, int causal, int64_t H, int64_t ld, int64_t ldo, int dkr) {
+    return dkr == DK ? launch_sdpa_p<DK, false>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo, dkr)
+                     : launch_sdpa_p<DK, true>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo, dkr);
 }
 
 // One workgroup per score row: mask, maximum, exponentials, sum, normalise in place; L = max + log(sum).
@@ -419,18 +450,21 @@ int sdpa_unfused(const float *Q, const float *K, const float *V, float *O, float
 
 }  // namespace
 
-// shared by both entry points: H heads side by side in rows of ld (Q, K, V) / ldo (O) floats
+// shared by both entry points: H heads side by side in rows of ld (Q, K, V) / ldo (O) floats.  A head
+// size that is a multiple of 4 up to 128 runs on the kernel of the next size among 32, 64, 128.
+static bool sdpa_fusable(int64_t dk) { return dk >= 4 && dk <= 128 && dk % 4 == 0; }
+
 static int sdpa_fused(const float *Q, const float *K, const float *V, float *O, float *L, int64_t BH, int64_t S,
                       int64_t dk, float scale, int causal, int64_t H, int64_t ld, int64_t ldo) {
     int rc;
-    if (dk == 32) {
-        rc = launch_sdpa<32>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo);
+    if (dk <= 32) {
+        rc = launch_sdpa<32>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo, (int)dk);
         axhip::note_kernel(causal ? "sdpa_fused_dk32_causal" : "sdpa_fused_dk32");
-    } else if (dk == 64) {
-        rc = launch_sdpa<64>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo);
+    } else if (dk <= 64) {
+        rc = launch_sdpa<64>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo, (int)dk);
         axhip::note_kernel(causal ? "sdpa_fused_dk64_causal" : "sdpa_fused_dk64");
     } else {
-        rc = launch_sdpa<128>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo);
+        rc = launch_sdpa<128>(Q, K, V, O, L, BH, S, scale, causal, H, ld, ldo, (int)dk);
         axhip::note_kernel(causal ? "sdpa_fused_dk128_causal" : "sdpa_fused_dk128");
     }
     return rc;
@@ -443,7 +477,7 @@ extern "C" int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, fl
     if (BH < 0 || S < 0 || dk <= 0) return fail(AXHIP_ERR_SHAPE, "sdpa_fwd: bad extent");
     if (BH == 0 || S == 0) return AXHIP_OK;
     const bool aligned = ((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O) & 15) == 0);
-    if ((dk == 32 || dk == 64 || dk == 128) && aligned && (S + SD_BQ - 1) / SD_BQ * BH <= 0x7fffffff)
+    if (sdpa_fusable(dk) && aligned && (S + SD_BQ - 1) / SD_BQ * BH <= 0x7fffffff)
         return sdpa_fused(Q, K, V, O, L, BH, S, dk, scale, causal, 1, dk, dk);
     return sdpa_unfused(Q, K, V, O, L, BH, S, dk, scale, causal);
 }
@@ -453,8 +487,8 @@ extern "C" int axhip_sdpa_fwd_rows(const float *Q, const float *K, const float *
     if (int rc = axhip::ensure_ready()) return rc;
     if (!Q || !K || !V || !O) return fail(AXHIP_ERR_NULL_ARG, "sdpa_fwd_rows: NULL tensor");
     if (B < 0 || H <= 0 || S < 0) return fail(AXHIP_ERR_SHAPE, "sdpa_fwd_rows: bad extent");
-    if (dk != 32 && dk != 64 && dk != 128)
-        return fail(AXHIP_ERR_NOT_IMPLEMENTED, "sdpa_fwd_rows: head size %lld (32, 64 or 128 only)", (long long)dk);
+    if (!sdpa_fusable(dk))
+        return fail(AXHIP_ERR_NOT_IMPLEMENTED, "sdpa_fwd_rows: head size %lld (multiples of 4 up to 128 only)", (long long)dk);
     if (ld < H * dk || ldo < H * dk || ld % 4 != 0 || ldo % 4 != 0 || ld > (1 << 22))
         return fail(AXHIP_ERR_SHAPE, "sdpa_fwd_rows: row pitch must hold H * dk floats and be a multiple of 4");
     if ((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O) & 15) != 0)

@@ -78,11 +78,11 @@ static ax_tensor_t *mha_forward(ax_layer_t *self, ax_tensor_t *x) {
                 *out = NULL;
     int64_t flat_sh[2] = {rows, D}, qkv_sh[2] = {rows, 3 * D}, head_sh[3] = {B * H, S, dk};
     ax_status_t st = refresh_fused_qkv(m, ext);
-    /* Head sizes the fused kernel covers: attention reads the heads where the projection wrote
+    /* Head sizes the fused kernel covers (multiples of 4 up to 128): attention reads the heads where the projection wrote
      * them (columns h*dk.. of the q, k and v thirds of qkv) and writes them where the output
      * projection reads them, so the three layout passes of attention.c:211-262, 391-400 and their
      * four [B*H, S, dk] temporaries fall away; the projection bias moves into the GEMM write-back. */
-    const bool direct = ext->sdpa_fwd_rows && (dk == 32 || dk == 64 || dk == 128) &&
+    const bool direct = ext->sdpa_fwd_rows && dk % 4 == 0 && dk <= 128 &&
                         (!m->use_bias || ax_compute_has_gemm_bias_act());
     if (direct) {
         if (st == AX_OK && (!(x_flat = ax_tensor_reshape(x, flat_sh, 2)) || !(qkv = on_device_of(x, qkv_sh, 2)) ||

@@ -203,8 +203,9 @@ int axhip_sgd_update(float *w, const float *g, float *momentum_buf, int64_t n, f
  * causal != 0: query i sees keys j <= i.  Replaces ax_cuda_sdpa_fwd
  * (cuda/ops_attention.cu:299-392) and the device form of ax_fused_attention_fwd /
  * ax_fused_attention_fwd_causal (include/axiom/attention.h:273-283,
- * src/core/fused_attention.c:559-573).  dk of 32, 64 or 128 (16-byte aligned tensors, any S) runs
- * fused, with no score matrix in memory; other head sizes go through batched GEMMs and a row softmax. */
+ * src/core/fused_attention.c:559-573).  dk a multiple of 4 up to 128 (16-byte aligned tensors, any S)
+ * runs fused, with no score matrix in memory, on the kernel of the next size among 32, 64 and 128;
+ * other head sizes go through batched GEMMs and a row softmax. */
 int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, float *L,
                    int64_t BH, int64_t S, int64_t dk, float scale, int causal);
 /* The same attention on heads that lie side by side in the rows of wider matrices: head (b, h)
@@ -213,8 +214,8 @@ int axhip_sdpa_fwd(const float *Q, const float *K, const float *V, float *O, flo
  * V = qkv + 2D, ld = 3D, ldo = D this consumes the fused projection [B*S, 3D] and produces the
  * [B*S, D] input of the output projection directly, i.e. it stands for the sequence
  * head_interleave_qkv_split -> sdpa_fwd -> head_deinterleave of the reference's MHA forward
- * (src/core/attention.c:211-262, 391-400) without the three layout passes.  dk must be 32, 64 or
- * 128, pitches multiples of 4 floats, tensors 16-byte aligned (AXHIP_ERR_NOT_IMPLEMENTED /
+ * (src/core/attention.c:211-262, 391-400) without the three layout passes.  dk must be a multiple
+ * of 4 up to 128, pitches multiples of 4 floats, tensors 16-byte aligned (AXHIP_ERR_NOT_IMPLEMENTED /
  * AXHIP_ERR_SHAPE otherwise). */
 int axhip_sdpa_fwd_rows(const float *Q, const float *K, const float *V, int64_t ld, float *O, int64_t ldo,
                         float *L, int64_t B, int64_t H, int64_t S, int64_t dk, float scale, int causal);

@@ -438,7 +438,8 @@ def test_reference_model_file_runs_on_device(ax, oracle, golden, tag, in_shape, 
 
 
 @pytest.mark.parametrize("B,S,D,H,bias,causal", [(2, 128, 128, 2, True, True), (1, 256, 256, 4, False, False),
-                                                 (3, 40, 96, 6, True, False), (2, 77, 64, 2, True, True)])
+                                                 (3, 40, 96, 6, True, False), (2, 77, 64, 2, True, True),
+                                                 (2, 50, 90, 6, True, False), (2, 130, 288, 3, False, True)])
 def test_attention_layer_forward(ax, oracle, B, S, D, H, bias, causal):
     """ax_mha_create + forward on the device against the layer restated from the oracle's pieces
     (pinned to the reference's own layer output in test_oracle.py)."""

@@ -548,7 +548,12 @@ def run_sdpa(hip, q, k, v, scale, causal, want_l=True):
                                             (2, 384, 128, 0), (11, 640, 64, 1), (19, 256, 32, 0), (9, 512, 128, 1),
                                             (17, 128, 64, 1), (3, 200, 64, 0), (2, 1000, 64, 1), (5, 63, 32, 0),
                                             (2, 191, 128, 1), (9, 65, 64, 0), (2, 64, 64, 1), (3, 127, 32, 1),
-                                            (1, 897, 128, 0)])
+                                            (1, 897, 128, 0),
+                                            # head sizes between the kernels' own (lanes past the row end load nothing)
+                                            (3, 256, 96, 0), (2, 200, 80, 1), (5, 128, 40, 0), (2, 333, 100, 1),
+                                            (3, 64, 4, 0), (2, 129, 124, 1), (4, 512, 48, 0), (2, 77, 20, 1),
+                                            # and ones no fused kernel takes: batched GEMMs and a row softmax
+                                            (2, 64, 6, 0), (2, 100, 256, 1), (3, 50, 130, 0)])
 def test_sdpa_forward(hip, oracle, golden, BH, S, dk, causal):
     say("sdpa", BH, S, dk, causal)
     oracle.seed(5000 + BH * 100 + S + dk + causal)
@@ -572,7 +577,9 @@ def test_sdpa_forward(hip, oracle, golden, BH, S, dk, causal):
 @pytest.mark.parametrize("B,H,S,dk,causal,pad_in,pad_out", [(2, 4, 128, 64, 0, 0, 0), (2, 4, 128, 64, 1, 0, 0),
                                                             (3, 2, 77, 32, 1, 8, 4), (1, 3, 200, 128, 0, 4, 12),
                                                             (2, 5, 256, 32, 0, 0, 8), (1, 2, 1, 64, 0, 0, 0),
-                                                            (9, 4, 128, 64, 0, 0, 0), (2, 3, 321, 64, 1, 16, 0)])
+                                                            (9, 4, 128, 64, 0, 0, 0), (2, 3, 321, 64, 1, 16, 0),
+                                                            (2, 3, 200, 96, 0, 0, 0), (1, 5, 130, 40, 1, 4, 8),
+                                                            (3, 2, 64, 12, 0, 0, 4)])
 def test_sdpa_on_the_fused_projection_layout(hip, oracle, B, H, S, dk, causal, pad_in, pad_out):
     """Heads side by side in the rows of qkv [B*S, 3D (+ padding)]: the same numbers as the same
     heads handed over one matrix each, bit for bit, written into [B*S, D (+ padding)] with the
@@ -601,7 +608,7 @@ def test_sdpa_on_the_fused_projection_layout(hip, oracle, B, H, S, dk, causal, p
     assert np.array_equal(got_heads, want_o)
     assert np.array_equal(l.numpy(), want_l)
     # refusals: a head size without a fused kernel, a pitch shorter than the heads, a pitch off the 16-byte grid
-    assert hip.L.axhip_sdpa_fwd_rows(base, base, base, ld, out.ptr, ldo, None, B, H, S, 48, scale, 0) == 10
+    assert hip.L.axhip_sdpa_fwd_rows(base, base, base, ld, out.ptr, ldo, None, B, H, S, 50, scale, 0) == 10
     assert hip.L.axhip_sdpa_fwd_rows(base, base, base, D - 4, out.ptr, ldo, None, B, H, S, dk, scale, 0) == 3
     assert hip.L.axhip_sdpa_fwd_rows(base, base, base, ld + 2, out.ptr, ldo, None, B, H, S, dk, scale, 0) == 3
 
