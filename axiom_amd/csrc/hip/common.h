@@ -154,6 +154,32 @@ __device__ __forceinline__ void turn_tile_and_store(unsigned char *turn, int lan
         *reinterpret_cast<V4 *>(dst + (int64_t)(p * 8 + (lane >> 3)) * ld + (lane & 7) * 4) = o[p];
 }
 
+// The same write-back for a tile that may hang over the matrix edge: only rows below `rows` and
+// 4-column groups that begin below `cols` (a multiple of 4) are stored.
+template <typename V4, typename T>
+__device__ __forceinline__ void turn_tile_and_store_edge(unsigned char *turn, int lane, const V4 (&r)[4],
+                                                         T *dst, int64_t ld, int64_t rows, int64_t cols) {
+    static_assert(sizeof(V4) == 16 && sizeof(T) == 4, "32-bit elements in 16-byte vectors");
+    const int frow = lane & 31, fhalf = lane >> 5;
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+        *reinterpret_cast<V4 *>(turn + frow * 128 + (((2 * g + fhalf) ^ ((frow >> 1) & 7)) << 4)) = r[g];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    V4 o[4];
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const int row = p * 8 + (lane >> 3);
+        o[p] = *reinterpret_cast<const V4 *>(turn + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int p = 0; p < 4; p++)
+        if (p * 8 + (lane >> 3) < rows && (lane & 7) * 4 < cols)
+            *reinterpret_cast<V4 *>(dst + (int64_t)(p * 8 + (lane >> 3)) * ld + (lane & 7) * 4) = o[p];
+}
+
 }  // namespace axhip
 
 #define AXHIP_HIP_TRY(expr, what)                                                         \

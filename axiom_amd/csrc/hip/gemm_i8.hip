@@ -535,7 +535,10 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 // 128 MFMA cycles of work per slab and wave: the loop is bound by load latency and by the
 // CU's L1 bandwidth, not by the matrix core).  LDS: NST stages of X (BM rows x 128 B), NST
 // stages of W, then BN scales and BN biases.  Not persistent.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int ACT>
+// EDGE: M and N need not be multiples of the tile.  A row past the end of X or W is fetched from
+// the last row instead (its products land in outputs that are not stored), and the write-back
+// keeps to rows below M and 4-column groups below N (N a multiple of 4).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int ACT, bool EDGE = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64)
 k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
                  int64_t K, float x_scale, const float *__restrict__ w_scales,
@@ -558,21 +561,24 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     int tm, tn;
-    tile_of_block(blockIdx.x, (int)(M / BM), (int)(N / BN), tm, tn);
+    tile_of_block(blockIdx.x, (int)((M + BM - 1) / BM), (int)((N + BN - 1) / BN), tm, tn);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int slabs = (int)(K / BKB);
+    // rows of this tile that exist (EDGE; the last tile row / column may hang over)
+    const int mrows = EDGE && M - m0 < BM ? (int)(M - m0) : BM, nrows = EDGE && N - n0 < BN ? (int)(N - n0) : BN;
 
-    // load instruction q fills rows q*8 .. q*8+7 of an operand stage; wave w issues q = j*NW + w
+    // load instruction q fills rows q*8 .. q*8+7 of an operand stage; wave w issues q = j*NW + w.
+    // The LDS place (and so the swizzle) is that of the nominal row; the source row is clamped.
     unsigned vx[IPW_X], vw[IPW_W];
 #pragma unroll
     for (int j = 0; j < IPW_X; j++) {
         const int row = (j * NW + wave) * 8 + (lane >> 3);
-        vx[j] = (unsigned)(row * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+        vx[j] = (unsigned)((row < mrows ? row : mrows - 1) * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
     }
 #pragma unroll
     for (int j = 0; j < IPW_W; j++) {
         const int row = (j * NW + wave) * 8 + (lane >> 3);
-        vw[j] = (unsigned)(row * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+        vw[j] = (unsigned)((row < nrows ? row : nrows - 1) * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
     }
     const int8_t *gx = X + m0 * K, *gw = W + n0 * K;
     const unsigned lds0 = (unsigned)(uintptr_t)lds, lds_w = lds0 + wave * 1024;
@@ -590,8 +596,9 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     float *lds_scale = reinterpret_cast<float *>(lds + NST * (XS + WS)), *lds_bias = lds_scale + BN;
     if (out) {
         for (int c = tid; c < BN; c += NW * 64) {
-            lds_scale[c] = x_scale * w_scales[n0 + c];
-            lds_bias[c] = bias ? bias[n0 + c] : 0.0f;
+            const bool live = c < nrows;
+            lds_scale[c] = live ? x_scale * w_scales[n0 + c] : 0.0f;
+            lds_bias[c] = live && bias ? bias[n0 + c] : 0.0f;
         }
     }
 
@@ -687,7 +694,11 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 #pragma unroll
                 for (int g = 0; g < 4; g++)
                     r[g] = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                turn_tile_and_store(turn, lane, r, acc_out + (trow + i * 32) * ldc + tcol + j * 32, ldc);
+                if (EDGE)
+                    turn_tile_and_store_edge(turn, lane, r, acc_out + (trow + i * 32) * ldc + tcol + j * 32, ldc,
+                                             M - trow - i * 32, N - tcol - j * 32);
+                else
+                    turn_tile_and_store(turn, lane, r, acc_out + (trow + i * 32) * ldc + tcol + j * 32, ldc);
             }
     }
     if (out) {
@@ -711,22 +722,26 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
                         const float f = (float)acc[i][j][4 * g + e];
                         r[g][e] = apply_act(has_bias ? __builtin_fmaf(f, sc[g][e], bv[g][e]) : f * sc[g][e], ACT);
                     }
-                turn_tile_and_store(turn, lane, r, out + (trow + i * 32) * ldc + tcol + j * 32, ldc);
+                if (EDGE)
+                    turn_tile_and_store_edge(turn, lane, r, out + (trow + i * 32) * ldc + tcol + j * 32, ldc,
+                                             M - trow - i * 32, N - tcol - j * 32);
+                else
+                    turn_tile_and_store(turn, lane, r, out + (trow + i * 32) * ldc + tcol + j * 32, ldc);
             }
         }
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool EDGE = false>
 int launch_dma(const char *name, const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
                const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K,
                int64_t ldc) {
     constexpr int smem = NST * (BM + BN) * 128 + 2 * BN * 4;
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
                            const float *, float *, int32_t *, int64_t);
-    static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE>,
-                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU>,
-                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU>};
+    static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU, EDGE>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE>};
     static bool attr_set = false;
     if (!attr_set) {
         for (kern_t kf : kerns)
@@ -735,7 +750,7 @@ int launch_dma(const char *name, const int8_t *x, float x_scale, const int8_t *w
                           "hipFuncSetAttribute");
         attr_set = true;
     }
-    const int64_t tiles = (M / BM) * (N / BN);
+    const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     if (tiles > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: too many tiles");
     note_kernel(name);
     hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles), dim3(WAVES_M * WAVES_N * 64), smem, kStream, x, w,
@@ -856,6 +871,14 @@ int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_
                                                  act, out, acc_out, M, N, K, ldc);
         return launch_dma<64, 64, 2, 2, 4>("qgemm_w8a8_64x64_dma", x, x_scale, w, w_scales, bias, act,
                                            out, acc_out, M, N, K, ldc);
+    }
+    // the same kernel for M or N off the 64 grid: edge tiles clamp their loads and guard their stores
+    if (aligned && vec_out && K % 128 == 0 && N % 4 == 0 && K < (int64_t(1) << 24)) {
+        if (((M + 127) / 128) * ((N + 127) / 128) >= 512)
+            return launch_dma<128, 128, 2, 2, 3, true>("qgemm_w8a8_128x128_dma_edge", x, x_scale, w, w_scales, bias,
+                                                       act, out, acc_out, M, N, K, ldc);
+        return launch_dma<64, 64, 2, 2, 4, true>("qgemm_w8a8_64x64_dma_edge", x, x_scale, w, w_scales, bias, act,
+                                                 out, acc_out, M, N, K, ldc);
     }
     // fewer than ~3/4 of the 256 CUs busy with 128x128 tiles: quarter the tile instead
     if (aligned && M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 192)

@@ -37,7 +37,10 @@ INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300
                # rows that start at odd byte offsets (K % 16 != 0)
                (70, 90, 1037), (130, 257, 4099),
                # large with K off the 128 grid: zero-padded copies of both operands, then the fast kernels
-               (2048, 4096, 520), (2112, 4128, 600)]
+               (2048, 4096, 520), (2112, 4128, 600),
+               # M or N off the 64 grid with K on the 128 grid: the direct-to-LDS kernel with clamped edge tiles
+               (100, 4096, 512), (130, 260, 256), (2000, 2000, 128), (63, 60, 128), (9, 4, 128), (500, 1000, 1024),
+               (65, 64, 256), (64, 68, 384), (2900, 3000, 128)]
 
 
 @pytest.mark.parametrize("M,N,K", INT8_SHAPES)
