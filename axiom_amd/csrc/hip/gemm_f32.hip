@@ -297,14 +297,18 @@ struct DmaOperand {
     static constexpr int READS = KC ? 1 : 4;                           // ds_reads per 32-wide tile per k-block
     static_assert(IPW * NW == NINSTR && IPW >= 1, "slab must divide over the waves");
 
-    // byte offset, from the operand's slab origin, of what lane `lane` of instruction q fetches
-    __device__ static unsigned lane_offset(int q, int lane, int64_t ld) {
+    // byte offset, from the operand's slab origin, of what lane `lane` of instruction q fetches.
+    // `valid` (<= R; a multiple of 4 for an M/N-contiguous operand) is how many of the tile's R
+    // rows / columns exist: a lane whose row or 4-column group lies past them fetches the last
+    // existing one instead, into its own LDS place (swizzle of the nominal row).
+    __device__ static unsigned lane_offset(int q, int lane, int64_t ld, int valid = R) {
         if (KC) {
             const int row = q * 8 + (lane >> 3);
-            return (unsigned)(row * ld * 4 + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+            return (unsigned)((row < valid ? row : valid - 1) * ld * 4 + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
         }
         constexpr int LPR = 64 / (256 / R);                            // lanes per k-row
-        return (unsigned)((q * (256 / R) + lane / LPR) * ld * 4 + (lane % LPR) * 16);
+        const int chunk = lane % LPR;
+        return (unsigned)((q * (256 / R) + lane / LPR) * ld * 4 + (chunk * 4 < valid ? chunk : valid / 4 - 1) * 16);
     }
     // LDS byte address (within a stage) a lane reads its fragments from, for k-block index kbi
     // (KC) or for all k-blocks (MC, kbi ignored); `first` = first row/column of the wave's tile
@@ -329,7 +333,11 @@ template <> struct Frag<false> {
 #define AXF_DS128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 #define AXF_DS32(dst, addr, off) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI, int WAVES_K>
+// EDGE: M and N need not be multiples of the tile (N a multiple of 4, and M too when A is stored
+// M-contiguous).  Edge tiles fetch the last existing row / column group in place of the missing
+// ones — their products land in outputs that are not stored — and guard the write-back.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI, int WAVES_K,
+          bool EDGE = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(SgemmArgs g) {
     // WAVES_K == 2: a second set of waves shares each tile; set 0 multiplies k-blocks 0 and 1 of
     // every slab, set 1 k-blocks 2 and 3, and the two accumulators are added through LDS at the
@@ -355,9 +363,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     const int wm = wmn / WAVES_N, wn = wmn % WAVES_N;
     int tm, tn;
     int64_t batch = 0;
-    if (gridDim.y == 1) tile_of_block(blockIdx.x, (int)(g.M / BM), (int)(g.N / BN), tm, tn);
-    else tile_of_batched_block((int)(g.M / BM), (int)(g.N / BN), tm, tn, batch);
+    if (gridDim.y == 1) tile_of_block(blockIdx.x, (int)((g.M + BM - 1) / BM), (int)((g.N + BN - 1) / BN), tm, tn);
+    else tile_of_batched_block((int)((g.M + BM - 1) / BM), (int)((g.N + BN - 1) / BN), tm, tn, batch);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int mvalid = EDGE && g.M - m0 < BM ? (int)(g.M - m0) : BM, nvalid = EDGE && g.N - n0 < BN ? (int)(g.N - n0) : BN;
     const float *A = static_cast<const float *>(g.A) + batch * g.stride_a;
     const float *B = static_cast<const float *>(g.B) + batch * g.stride_b;
     float *C = g.C + batch * g.stride_c;
@@ -366,9 +375,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     // ---- global -> LDS ----
     unsigned va[OA::IPW], vb[OB::IPW];
 #pragma unroll
-    for (int j = 0; j < OA::IPW; j++) va[j] = OA::lane_offset(j * NW + wave, lane, g.lda);
+    for (int j = 0; j < OA::IPW; j++) va[j] = OA::lane_offset(j * NW + wave, lane, g.lda, mvalid);
 #pragma unroll
-    for (int j = 0; j < OB::IPW; j++) vb[j] = OB::lane_offset(j * NW + wave, lane, g.ldb);
+    for (int j = 0; j < OB::IPW; j++) vb[j] = OB::lane_offset(j * NW + wave, lane, g.ldb, nvalid);
     const char *ga = reinterpret_cast<const char *>(A_KC ? A + m0 * g.lda : A + m0);
     const char *gb = reinterpret_cast<const char *>(B_KC ? B + n0 * g.ldb : B + n0);
     const int64_t step_a = A_KC ? 128 : 128 * g.lda, step_b = B_KC ? 128 : 128 * g.ldb;   // bytes per slab
@@ -556,8 +565,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         const float *bp = g.bias ? g.bias + col0 : nullptr;
 #pragma unroll
         for (int j = 0; j < TN; j++) {
+            const bool col_in = !EDGE || col0 + j * 32 < g.N;          // N % 4 == 0: the whole group or none of it
             v4f bv = {0.f, 0.f, 0.f, 0.f};
-            if (bp) bv = *reinterpret_cast<const v4f *>(bp + j * 32);
+            if (bp && col_in) bv = *reinterpret_cast<const v4f *>(bp + j * 32);
 #pragma unroll
             for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -579,6 +589,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
                 __builtin_amdgcn_wave_barrier();
 #pragma unroll
                 for (int p = 0; p < 4; p++) {
+                    if (EDGE && (!col_in || m0 + wm * WTM + rrow + i * 32 + p * 8 >= g.M)) continue;
                     float *cp = dst + (int64_t)(i * 32 + p * 8) * g.ldc + j * 32;
                     v4f o = r[p];
                     if (g.alpha != 1.0f) o *= g.alpha;
@@ -595,9 +606,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI = 1, int WAVES_K = 1>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI = 1, int WAVES_K = 1,
+          bool EDGE = false>
 int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
-    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K>;
+    static_assert(!EDGE || EPI == 1, "the edge form guards the turned write-back only");
+    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K, EDGE>;
     constexpr int NW = WAVES_M * WAVES_N * WAVES_K;
     constexpr int smem = NST * (DmaOperand<BM, A_KC, NW>::BYTES + DmaOperand<BN, B_KC, NW>::BYTES);
     static bool attr_set = false;
@@ -607,7 +620,7 @@ int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
                       "hipFuncSetAttribute");
         attr_set = true;
     }
-    const int64_t tiles = (g.M / BM) * (g.N / BN);
+    const int64_t tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     note_kernel(name);
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)batch), dim3(NW * 64), smem, kStream, g);
     return check_launch(name);
@@ -622,8 +635,13 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
                     ((uintptr_t)g.C % 16 == 0) && ((uintptr_t)g.bias % 16 == 0) && g.lda % 4 == 0 &&
                     g.ldb % 4 == 0 && g.ldc % 4 == 0 && g.stride_a % 4 == 0 && g.stride_b % 4 == 0 &&
                     g.stride_c % 4 == 0 && g.lda < (1 << 20) && g.ldb < (1 << 20) && batch <= 65535 &&
-                    g.M % 64 == 0 && g.N % 64 == 0 && (g.M / 64) * (g.N / 64) <= 0x7fffffff;
+                    g.N % 4 == 0 && (A_KC || g.M % 4 == 0) && ((g.M + 63) / 64) * ((g.N + 63) / 64) <= 0x7fffffff;
     if (!ok) return -1;
+    if (g.M % 64 != 0 || g.N % 64 != 0) {                   // off the tile grid: 64x64 tiles with guarded edges
+        static const char *const edge_names[2] = {"sgemm_64x64_dma_edge", "sgemm_64x64k2_dma_edge"};
+        if (g.K > 128) return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2, true>(edge_names[1], g, batch);
+        return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 1, true>(edge_names[0], g, batch);
+    }
     auto count = [&](int64_t bm, int64_t bn) { return (g.M / bm) * (g.N / bn) * batch; };
     // Sustained timings over the benchmark shapes: 128x256 (8 waves, one workgroup per CU) wins
     // once it fills the chip; below that 64x64 tiles with the k split beat 128x128 and 128x64
@@ -694,13 +712,12 @@ int64_t split_count(int64_t M, int64_t N, int64_t K) {
     const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
     const int64_t cus = cu_count();
     if (tiles * 2 > cus || K < 256 || K % 32 != 0) return 1;
-    // Tiles on the 64 grid run the direct-to-LDS kernel, for which one workgroup per CU measured
-    // best (32x768x768: 10.5 us against 27 unsplit; 64x1024x4096: 12 against 70; 128x4096x1024: 16.5
-    // against 20; more ranges only add partial sums to move).  Ragged tiles run the register-staged
-    // kernel, whose slabs each wait out a load: four workgroups per CU cover one another's waits
-    // (4x4100x4096: 65 -> 36 us; 9x8000x8192: 123 -> 85).
+    // One workgroup per CU measured best for tiles on the 64 grid (32x768x768: 10.5 us against 27
+    // unsplit; 64x1024x4096: 12 against 70; 128x4096x1024: 16.5 against 20; more ranges only add
+    // partial sums to move); strips off the grid, part of whose tiles is padding, gain from two
+    // (4x4100x4096: 38 -> 30 us; 9x8000x8192: 78 -> 69).
     const bool ragged = M % 64 != 0 || N % 64 != 0;
-    int64_t want = ((ragged ? 4 : 1) * cus + tiles - 1) / tiles;
+    int64_t want = ((ragged ? 2 : 1) * cus + tiles - 1) / tiles;
     const int64_t most = K / 64;                             // ranges of at least 64
     if (want > most) want = most;
     // K / 32 must divide into the ranges: the nearest count at or below the wish, or, when that is
@@ -772,28 +789,23 @@ int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     return fail(AXHIP_ERR_NOT_IMPLEMENTED, "sgemm: A^T * B^T is not provided");
 }
 
-// A large fp32 shape off the tile grid would run whole on the register-staged guarded kernel
-// (4000^3: 101 TFLOP/s against 141 on the grid).  Its grid-aligned interior goes to the
-// direct-to-LDS kernels instead and only the right and bottom fringes to the guarded one; every
-// block is a sub-matrix reached by pointer offsets.  Returns -1 when the shape is left alone.
-int try_interior_and_fringes(const SgemmArgs &g, int transa, int transb, int64_t min_tiles = 256) {
+// A large fp32 shape off the tile grid runs on 64x64 tiles with guarded edges (4000^3: 125
+// TFLOP/s against 141 for 128x256 tiles on the grid).  When it is large enough for 128x256
+// tiles, its interior on that grid goes to them and only the right and bottom fringes to the
+// edge form; every block is a sub-matrix reached by pointer offsets.  Returns -1 when the shape
+// is left alone.
+int try_interior_and_fringes(const SgemmArgs &g, int transa, int transb) {
     if ((transa && transb) || g.K % 32 != 0 || g.K <= 0) return -1;
     if ((((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.C | (uintptr_t)g.bias) & 15) != 0 || g.lda % 4 != 0 ||
         g.ldb % 4 != 0 || g.ldc % 4 != 0)
         return -1;                                           // the interior would not qualify for the fast kernels either
-    int64_t gm, gn;
-    if ((g.M / 128) * (g.N / 256) >= 256) gm = 128, gn = 256;
-    else if ((g.M / 64) * (g.N / 64) >= min_tiles) gm = gn = 64;
-    else return -1;
-    const int64_t Mi = g.M / gm * gm, Ni = g.N / gn * gn;
+    if ((g.M / 128) * (g.N / 256) < 256) return -1;
+    const int64_t Mi = g.M / 128 * 128, Ni = g.N / 256 * 256;
     if (Mi == g.M && Ni == g.N) return -1;
     const float *A = static_cast<const float *>(g.A), *B = static_cast<const float *>(g.B);
-    // a fringe is a strip of few tiles with the whole K: the split-K route when it qualifies; a
-    // wide one (up to 255 columns beside 128x256 tiles) is itself cut into its part on the 64 grid
-    // and a narrower fringe
+    // a fringe is a strip of few tiles with the whole K: the split-K route when it qualifies
     auto fringe = [&](const SgemmArgs &f) {
-        int rc = try_split_k<float>(f, transa, transb, "sgemm_splitk", nullptr);
-        if (rc < 0 && min_tiles == 256) rc = try_interior_and_fringes(f, transa, transb, 64);
+        const int rc = try_split_k<float>(f, transa, transb, "sgemm_splitk", nullptr);
         return rc >= 0 ? rc : dispatch_f32(f, transa, transb, 1);
     };
     SgemmArgs p = g;

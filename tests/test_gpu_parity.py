@@ -132,7 +132,9 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               # off the tile grid with a large interior: fast kernels inside, guarded kernel on the fringes
               (1032, 1100, 96), (2100, 4200, 64), (1024, 1092, 160),
               (130, 257, 1027), (67, 1001, 129),                  # rows off the 16-byte grid in every form
-              (1024, 1088, 1045), (1030, 1100, 600)]              # K off the 32 grid: main product, then the K tail on top
+              (1024, 1088, 1045), (1030, 1100, 600),              # K off the 32 grid: main product, then the K tail on top
+              # M or N off the 64 grid with K on the 32 grid and N % 4 == 0: direct-to-LDS tiles with guarded edges
+              (65, 68, 64), (9, 4, 32), (63, 60, 96), (200, 36, 128), (500, 1000, 256), (12, 2052, 160)]
 
 
 @pytest.mark.parametrize("M,N,K", F32_SHAPES)
