@@ -929,7 +929,13 @@ extern "C" int axhip_sgemm_strided_batched(int transa, int transb, int64_t M, in
     if (batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0)
         return fail(AXHIP_ERR_SHAPE, "sgemm_strided_batched: negative batch or stride");
     if (M == 0 || N == 0 || batch == 0) return AXHIP_OK;
-    SgemmArgs g{A, B, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c,
-                alpha, beta, nullptr, nullptr, AXHIP_ACT_NONE};
-    return dispatch_f32(g, transa, transb, batch);
+    // the batch index is the grid's second dimension (at most 65535): longer batches go in pieces
+    constexpr int64_t kMostPerLaunch = 65535;
+    for (int64_t b0 = 0; b0 < batch; b0 += kMostPerLaunch) {
+        const int64_t nb = batch - b0 < kMostPerLaunch ? batch - b0 : kMostPerLaunch;
+        SgemmArgs g{A + b0 * stride_a, B + b0 * stride_b, C + b0 * stride_c, M, N, K, lda, ldb, ldc, stride_a, stride_b,
+                    stride_c, alpha, beta, nullptr, nullptr, AXHIP_ACT_NONE};
+        if (int rc = dispatch_f32(g, transa, transb, nb)) return rc;
+    }
+    return AXHIP_OK;
 }

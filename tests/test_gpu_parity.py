@@ -360,6 +360,17 @@ def test_strided_batched_qkt_and_pv(hip, oracle):
         check_fp32(oracle, c[h], a[h], b[h])
 
 
+def test_strided_batched_beyond_one_launch(hip, oracle):
+    """More batch members than a launch's second grid dimension holds (65535): done in pieces."""
+    oracle.seed(56)
+    Bn = 70000
+    a, b = oracle.normal((Bn, 4, 8)), oracle.normal((Bn, 8, 4))
+    c = hip.sgemm_batched(hip.array(a), hip.array(b)).numpy()
+    want = np.einsum("bik,bkj->bij", a.astype(np.float64), b.astype(np.float64))
+    assert np.abs(c - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.abs(c[-1] - want[-1]).max() <= 1e-5 and np.abs(c[65535] - want[65535]).max() <= 1e-5
+
+
 def test_config4b_attention_shapes_full_size(hip, oracle):
     """512 heads of [512,64]: sampled heads against the oracle, all heads by a linearity check."""
     oracle.seed(44)
