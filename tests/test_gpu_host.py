@@ -485,3 +485,42 @@ def test_attention_layer_forward(ax, oracle, B, S, D, H, bias, causal):
     assert not L.ax_layer_forward(layer, bad)
     ax.free(tx, y, y2, y3, tw, bad)
     L.ax_layer_destroy(layer)
+
+
+@pytest.mark.gpu
+def test_no_device_memory_is_left_behind(ax):
+    """Build, run and destroy an encoder-shaped model (layer norm, attention with bias on both of its
+    forward routes, dense + GELU) and a quantized weight: every device block the host core asked for comes
+    back, counted by the allocator itself."""
+    import ctypes as C
+    from axiom_amd import AxHip
+    hip = AxHip()
+    L = ax.L
+    L.ax_set_default_device(2)
+    st = [C.c_int64() for _ in range(6)]
+
+    def stats():
+        hip.L.axhip_alloc_stats(*[C.byref(v) for v in st])
+        return [v.value for v in st]
+
+    hip.L.axhip_reset_alloc_stats()
+    for (D, H) in ((128, 2), (90, 6)):                           # dk 64: direct route; dk 15: split route
+        seq = L.ax_sequential_create()
+        for layer in (L.ax_layernorm_create(D, 1e-5), L.ax_mha_create(D, H, True, True), L.ax_layernorm_create(D, 1e-5),
+                      L.ax_dense_create(D, 4 * D, True), L.ax_gelu_layer_create(), L.ax_dense_create(4 * D, D, True),
+                      L.ax_softmax_layer_create(-1)):
+            assert L.ax_sequential_add(seq, layer)
+        model = L.ax_model_create(seq)
+        x = ax.from_numpy(np.random.default_rng(D).uniform(-1, 1, (3, 70, D)).astype(np.float32))
+        for _ in range(3):
+            y = L.ax_model_predict(model, x)
+            assert y, ax.err()
+            assert np.isfinite(ax.to_numpy(y)).all()
+            ax.free(y)
+        bad = ax.from_numpy(np.zeros((3, 70, D + 4), np.float32))   # a refused input must not strand temporaries
+        assert not L.ax_model_predict(model, bad)
+        ax.free(x, bad)
+        L.ax_model_destroy(model)
+    allocs, frees, b_alloc, b_free, _, _ = stats()
+    assert allocs > 50 and allocs == frees and b_alloc == b_free, (allocs, frees, b_alloc, b_free)
+
