@@ -1,76 +1,106 @@
-/* xoshiro256** with splitmix64 seeding, per thread (Axiom's src/core/rng.c): identical
- * output sequence for a given seed, including the cached second value of the polar normal. */
+/* Per-thread pseudo-random numbers with the output sequence of Axiom's generator (src/core/rng.c):
+ * the xoshiro256** recurrence, its state filled from the seed by four splitmix64 steps; floats
+ * from the top 24 bits; normals by the polar method, which yields two values per accepted point
+ * (the second is kept for the next call).  Seeded weights therefore match the reference bit for
+ * bit (known answers in the tests). */
 #include <math.h>
 #include <time.h>
 #include <unistd.h>
 
 #include "axiom/rng.h"
 
-static _Thread_local uint64_t tl_s[4];
-static _Thread_local bool tl_seeded = false;
-static _Thread_local bool tl_have_spare = false;
-static _Thread_local float tl_spare = 0.0f;
+typedef struct {
+    uint64_t word[4];      /* xoshiro256** state */
+    float kept;            /* second value of the last accepted polar point */
+    bool ready, has_kept;
+} generator_t;
 
-static uint64_t splitmix(uint64_t *ctr) {
-    uint64_t z = (*ctr += 0x9e3779b97f4a7c15ULL);
-    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
-    z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
-    return z ^ (z >> 31);
+static _Thread_local generator_t tl_gen;
+
+/* one step of the splitmix64 sequence that starts at *counter */
+static uint64_t splitmix64_next(uint64_t *counter) {
+    *counter += UINT64_C(0x9e3779b97f4a7c15);
+    uint64_t mixed = *counter;
+    mixed ^= mixed >> 30;
+    mixed *= UINT64_C(0xbf58476d1ce4e5b9);
+    mixed ^= mixed >> 27;
+    mixed *= UINT64_C(0x94d049bb133111eb);
+    mixed ^= mixed >> 31;
+    return mixed;
 }
 
-static inline uint64_t rol(uint64_t v, int r) { return (v << r) | (v >> (64 - r)); }
+#define ROTATE_LEFT(value, bits) (((value) << (bits)) | ((value) >> (64 - (bits))))
 
 void ax_rng_seed(uint64_t seed) {
-    uint64_t ctr = seed;
-    for (int i = 0; i < 4; i++) tl_s[i] = splitmix(&ctr);
-    tl_seeded = true;
+    generator_t *g = &tl_gen;
+    uint64_t counter = seed;
+    g->word[0] = splitmix64_next(&counter);
+    g->word[1] = splitmix64_next(&counter);
+    g->word[2] = splitmix64_next(&counter);
+    g->word[3] = splitmix64_next(&counter);
+    g->ready = true;
 }
 
-bool ax_rng_is_seeded(void) { return tl_seeded; }
+bool ax_rng_is_seeded(void) { return tl_gen.ready; }
+
+/* a first draw without a seed takes one from the clock and the process id, as the reference does */
+static void seed_from_environment(void) {
+    const uint64_t now = (uint64_t)time(NULL), pid = (uint64_t)getpid();
+    ax_rng_seed(now ^ (pid << 32) ^ (pid * UINT64_C(0x517cc1b727220a95)));
+}
 
 uint64_t ax_rng_uint64(void) {
-    if (!tl_seeded) {   /* first use without a seed: time and pid, as the reference does */
-        uint64_t t = (uint64_t)time(NULL), p = (uint64_t)getpid();
-        ax_rng_seed(t ^ (p << 32) ^ (p * 0x517cc1b727220a95ULL));
-    }
-    const uint64_t out = rol(tl_s[1] * 5, 7) * 9;
-    const uint64_t sh = tl_s[1] << 17;
-    tl_s[2] ^= tl_s[0];
-    tl_s[3] ^= tl_s[1];
-    tl_s[1] ^= tl_s[2];
-    tl_s[0] ^= tl_s[3];
-    tl_s[2] ^= sh;
-    tl_s[3] = rol(tl_s[3], 45);
-    return out;
+    generator_t *g = &tl_gen;
+    if (!g->ready) seed_from_environment();
+    uint64_t a = g->word[0], b = g->word[1], c = g->word[2], d = g->word[3];
+    const uint64_t result = ROTATE_LEFT(b * 5, 7) * 9;
+    const uint64_t shifted = b << 17;
+    c ^= a;
+    d ^= b;
+    b ^= c;
+    a ^= d;
+    c ^= shifted;
+    d = ROTATE_LEFT(d, 45);
+    g->word[0] = a;
+    g->word[1] = b;
+    g->word[2] = c;
+    g->word[3] = d;
+    return result;
 }
 
-float ax_rng_float(void) { return (float)(ax_rng_uint64() >> 40) * 0x1.0p-24f; }
-float ax_rng_uniform(float low, float high) { return low + ax_rng_float() * (high - low); }
+/* [0, 1): the top 24 bits of a draw, scaled by 2^-24 */
+float ax_rng_float(void) { return ldexpf((float)(ax_rng_uint64() >> 40), -24); }
+
+float ax_rng_uniform(float low, float high) {
+    const float unit = ax_rng_float();
+    return low + unit * (high - low);
+}
 
 float ax_rng_normal(void) {
-    if (tl_have_spare) {
-        tl_have_spare = false;
-        return tl_spare;
+    generator_t *g = &tl_gen;
+    if (g->has_kept) {
+        g->has_kept = false;
+        return g->kept;
     }
-    float u, v, r2;
-    do {
-        u = ax_rng_float() * 2.0f - 1.0f;
-        v = ax_rng_float() * 2.0f - 1.0f;
-        r2 = u * u + v * v;
-    } while (r2 >= 1.0f || r2 == 0.0f);
-    const float f = sqrtf(-2.0f * logf(r2) / r2);
-    tl_spare = v * f;
-    tl_have_spare = true;
-    return u * f;
+    for (;;) {
+        const float x = ax_rng_float() * 2.0f - 1.0f;
+        const float y = ax_rng_float() * 2.0f - 1.0f;
+        const float radius2 = x * x + y * y;
+        if (radius2 >= 1.0f || radius2 == 0.0f) continue;     /* outside the unit disc, or its centre */
+        const float factor = sqrtf(-2.0f * logf(radius2) / radius2);
+        g->kept = y * factor;
+        g->has_kept = true;
+        return x * factor;
+    }
 }
 
 float ax_rng_normal_params(float mean, float std) { return mean + std * ax_rng_normal(); }
 
+/* uniform on [0, n) by rejection: draws below 2^64 mod n would make some residues more likely */
 uint64_t ax_rng_bounded(uint64_t n) {
-    if (n <= 1) return 0;
-    const uint64_t reject_below = (0 - n) % n;
-    for (;;) {
-        uint64_t r = ax_rng_uint64();
-        if (r >= reject_below) return r % n;
-    }
+    if (n < 2) return 0;
+    const uint64_t threshold = (UINT64_C(0) - n) % n;
+    uint64_t draw = ax_rng_uint64();
+    while (draw < threshold) draw = ax_rng_uint64();
+    return draw % n;
 }
