@@ -261,6 +261,68 @@ def test_sgemm_alpha_beta_bias_act(hip, oracle, M, N, K):
     assert np.isfinite(hip.sgemm(da, db, c=poison).numpy()).all()
 
 
+# dimensions around every boundary the dispatch looks at (tile edges, vector widths, K slabs, split thresholds)
+EDGY = [1, 2, 3, 4, 5, 7, 8, 9, 12, 15, 16, 17, 31, 32, 33, 36, 60, 63, 64, 65, 68, 96, 100, 127, 128, 129, 132, 160, 192,
+        255, 256, 257, 260, 320, 384, 500, 512, 516, 640, 700, 768, 1000, 1024, 1028, 1100]
+
+
+def test_sgemm_dispatch_sweep(hip, oracle):
+    """120 seeded shapes drawn from the boundary dimensions, in a random form (NN / NT / TN), with a random
+    alpha, beta, bias and activation: whichever route the dispatch takes, the result obeys the fp64 bound."""
+    rng = np.random.default_rng(20240)
+    seen = set()
+    for case in range(120):
+        M, N, K = (int(rng.choice(EDGY)) for _ in range(3))
+        if case % 3 == 0:
+            K = int(rng.choice([1024, 1536, 2048, 2052, 4096]))          # long K: split and K-tail routes
+        form = int(rng.integers(0, 3))
+        alpha = float(rng.choice([1.0, 1.0, 0.5, -2.0]))
+        beta = float(rng.choice([0.0, 0.0, 1.0, 0.25]))
+        use_bias, act = bool(rng.integers(0, 2)), int(rng.integers(0, 3))
+        a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+        b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+        c0 = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+        bias = rng.normal(0, 0.5, N).astype(np.float32)
+        say("sweep", case, M, N, K, "form", form, "alpha", alpha, "beta", beta, "bias", use_bias, "act", act)
+        da = hip.array(np.ascontiguousarray(a.T) if form == 2 else a)
+        db = hip.array(np.ascontiguousarray(b.T) if form == 1 else b)
+        got = hip.sgemm(da, db, transa=form == 2, transb=form == 1, alpha=alpha, beta=beta, c=hip.array(c0),
+                        bias=hip.array(bias) if use_bias else None, act=act).numpy()
+        seen.add(hip.last_kernel())
+        pre = alpha * (a.astype(np.float64) @ b.astype(np.float64)) + beta * c0 + (bias if use_bias else 0.0)
+        want = np.maximum(pre, 0) if act == 1 else oracle.gelu(pre.astype(np.float32)).astype(np.float64) if act == 2 else pre
+        bound = BOUND_FP32 * (abs(alpha) * (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)) + abs(beta) + 1.0)
+        assert (np.abs(got - want) <= bound + (2e-5 * (1 + np.abs(pre)) if act == 2 else 0)).all(), \
+            (case, M, N, K, form, hip.last_kernel(), float(np.abs(got - want).max()))
+    say("  routes:", sorted(seen))
+    assert len(seen) >= 6
+
+
+def test_w8a8_dispatch_sweep(hip, oracle):
+    """100 seeded int8 shapes from the boundary dimensions (K also on and off the 16- and 128-byte grids):
+    accumulators bit-exact and outputs equal to the oracle's epilogue whatever kernel ran."""
+    rng = np.random.default_rng(20241)
+    seen = set()
+    for case in range(100):
+        M, N = int(rng.choice(EDGY)), int(rng.choice(EDGY))
+        K = int(rng.choice(EDGY + [1040, 2048, 2064, 4096, 4100]))
+        act, use_bias = int(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        x = rng.integers(-127, 128, (M, K), dtype=np.int8)
+        w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+        ws = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        bias = rng.normal(0, 0.02, N).astype(np.float32)
+        xs = float(np.float32(0.0131))
+        say("sweep i8", case, M, N, K, "act", act, "bias", use_bias)
+        out, acc = hip.qgemm_w8a8(hip.array(x), xs, hip.array(w), hip.array(ws), hip.array(bias) if use_bias else None, act)
+        seen.add(hip.last_kernel())
+        want_acc = x.astype(np.int32) @ w.astype(np.int32).T
+        assert np.array_equal(acc.numpy(), want_acc), (case, M, N, K, hip.last_kernel())
+        assert np.array_equal(out.numpy(), oracle.w8a8_epilogue(want_acc, xs, ws, bias if use_bias else None, act)), \
+            (case, M, N, K, hip.last_kernel())
+    say("  routes:", sorted(seen))
+    assert len(seen) >= 3
+
+
 def test_config3_ffn_block(hip, oracle):
     """tokens 2048, d_model 1024, d_ff 4096: GEMM1 + bias + GELU -> GEMM2 + bias."""
     oracle.seed(3)
