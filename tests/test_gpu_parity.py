@@ -691,6 +691,23 @@ def test_sdpa_on_the_fused_projection_layout(hip, oracle, B, H, S, dk, causal, p
     assert hip.L.axhip_sdpa_fwd_rows(base, base, base, ld + 2, out.ptr, ldo, None, B, H, S, dk, scale, 0) == 3
 
 
+def test_sdpa_shape_sweep(hip, oracle):
+    """60 seeded (heads, S, dk, causal) draws over sequence lengths around the 64- and 128-row blocks and
+    every kind of head size (native, padded to the next kernel, unfused)."""
+    rng = np.random.default_rng(20242)
+    lengths = [1, 2, 31, 63, 64, 65, 100, 127, 128, 129, 191, 192, 193, 255, 256, 257, 300, 384, 500, 513]
+    sizes = [4, 8, 12, 16, 28, 32, 36, 40, 48, 60, 64, 68, 72, 80, 96, 100, 124, 128, 6, 130]
+    for case in range(60):
+        BH, S, dk, causal = int(rng.integers(1, 12)), int(rng.choice(lengths)), int(rng.choice(sizes)), int(rng.integers(0, 2))
+        say("sdpa sweep", case, BH, S, dk, causal)
+        q, k, v = (rng.uniform(-0.5, 0.5, (BH, S, dk)).astype(np.float32) for _ in range(3))
+        scale = float(np.float32(1.0) / np.sqrt(np.float32(dk)))
+        o, l = run_sdpa(hip, q, k, v, scale, causal)
+        o64, l64 = oracle.sdpa(q, k, v, scale, causal, f64=True)
+        assert np.abs(o - o64).max() <= SDPA_TOL, (case, BH, S, dk, causal, hip.last_kernel(), float(np.abs(o - o64).max()))
+        assert np.abs(l - l64).max() <= 1e-5 * max(1.0, np.abs(l64).max()), (case, BH, S, dk, causal)
+
+
 def test_sdpa_large_scores_and_full_size(hip, oracle):
     """Scores far from zero (the running maximum must absorb them), and the attention shape of
     the benchmark (512 heads of [512, 64]) checked on sampled heads."""
