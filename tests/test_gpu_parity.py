@@ -323,6 +323,27 @@ def test_w8a8_dispatch_sweep(hip, oracle):
     assert len(seen) >= 3
 
 
+def test_w8a32_dispatch_sweep(hip, oracle):
+    """80 seeded W8A32 shapes from the boundary dimensions: the row-per-wave form (M <= 8), the matrix-core form,
+    its split over K and its K tail all obey the fp64 bound of a correct fp32 accumulation."""
+    rng = np.random.default_rng(20243)
+    seen = set()
+    for case in range(80):
+        M, N = int(rng.choice(EDGY[:34])), int(rng.choice(EDGY))
+        K = int(rng.choice(EDGY + [1040, 2048, 2064, 4096, 4099]))
+        a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+        w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+        ws = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        say("sweep w8a32", case, M, N, K)
+        got = hip.qgemm_w8a32(hip.array(a), hip.array(w), hip.array(ws)).numpy()
+        seen.add(hip.last_kernel())
+        want = (a.astype(np.float64) @ w.astype(np.float64).T) * ws
+        bound = BOUND_FP32 * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64).T) * ws + 1e-30
+        assert (np.abs(got - want) <= bound).all(), (case, M, N, K, hip.last_kernel(), float((np.abs(got - want) / bound).max()))
+    say("  routes:", sorted(seen))
+    assert len(seen) >= 3
+
+
 def test_config3_ffn_block(hip, oracle):
     """tokens 2048, d_model 1024, d_ff 4096: GEMM1 + bias + GELU -> GEMM2 + bias."""
     oracle.seed(3)
