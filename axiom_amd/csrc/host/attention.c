@@ -57,6 +57,51 @@ static ax_status_t refresh_fused_qkv(ax_mha_t *m, const ax_cuda_extension_t *ext
     return AX_OK;
 }
 
+/* Head sizes the fused kernel covers (multiples of 4 up to 128): attention reads the heads where the
+ * projection wrote them (columns h*dk.. of the q, k and v thirds of qkv) and writes them where the
+ * output projection reads them, so the three layout passes of attention.c:211-262, 391-400 and their
+ * four [B*H, S, dk] temporaries fall away; the projection bias moves into the GEMM write-back. */
+static ax_status_t attend_on_projection(ax_mha_t *m, const ax_cuda_extension_t *ext, ax_tensor_t *x_flat, ax_tensor_t *qkv,
+                                        ax_tensor_t *attn, int64_t B, int64_t S) {
+    const int64_t D = m->d_model;
+    ax_status_t st = m->use_bias ? ax_compute_gemm_bias_act(x_flat, m->Wqkv_cache, m->bqkv_cache, AX_ACT_NONE, qkv)
+                                 : ax_compute_gemm(x_flat, m->Wqkv_cache, qkv);
+    if (st != AX_OK) return st;
+    return ext->sdpa_fwd_rows(dev_ptr(qkv), dev_ptr(qkv) + D, dev_ptr(qkv) + 2 * D, 3 * D, dev_ptr(attn), D, NULL, B, m->n_heads,
+                              S, m->d_k, 1.0f / sqrtf((float)m->d_k), m->causal);
+}
+
+/* The reference's own sequence (attention.c:211-262, 391-400): projection, split into one matrix per head
+ * (adding the fused bias), attention per head, merge back to [B*S, D]. */
+static ax_status_t attend_per_head(ax_mha_t *m, const ax_cuda_extension_t *ext, ax_tensor_t *x_flat, ax_tensor_t *qkv,
+                                   ax_tensor_t *attn, int64_t B, int64_t S) {
+    const int64_t D = m->d_model, H = m->n_heads, dk = m->d_k;
+    int64_t head_sh[3] = {B * H, S, dk};
+    ax_tensor_t *heads[4] = {NULL, NULL, NULL, NULL};         /* Q, K, V, O as [B*H, S, dk] */
+    ax_status_t st = AX_OK;
+    for (int i = 0; i < 4 && st == AX_OK; i++)
+        if (!(heads[i] = on_device_of(x_flat, head_sh, 3))) st = AX_ERR_ALLOC;
+    if (st == AX_OK) st = ax_compute_gemm(x_flat, m->Wqkv_cache, qkv);
+    if (st == AX_OK) {
+        ax_err_clear();                                      /* the layout members return nothing: read the error state */
+        if (m->use_bias)
+            ext->head_interleave_qkv_split_bias(dev_ptr(qkv), dev_ptr(m->bqkv_cache), dev_ptr(heads[0]), dev_ptr(heads[1]),
+                                                dev_ptr(heads[2]), B, S, H, dk, D);
+        else
+            ext->head_interleave_qkv_split(dev_ptr(qkv), dev_ptr(heads[0]), dev_ptr(heads[1]), dev_ptr(heads[2]), B, S, H, dk, D);
+        st = ax_err_last_status();
+    }
+    if (st == AX_OK)
+        st = ext->sdpa_fwd(dev_ptr(heads[0]), dev_ptr(heads[1]), dev_ptr(heads[2]), dev_ptr(heads[3]), NULL, B * H, S, dk,
+                           1.0f / sqrtf((float)dk), m->causal, NULL);
+    if (st == AX_OK) {
+        ext->head_deinterleave(dev_ptr(heads[3]), dev_ptr(attn), B, S, H, dk);
+        st = ax_err_last_status();
+    }
+    for (int i = 0; i < 4; i++) ax_tensor_destroy(heads[i]);
+    return st;
+}
+
 static ax_tensor_t *mha_forward(ax_layer_t *self, ax_tensor_t *x) {
     ax_mha_t *m = (ax_mha_t *)self;
     if (!x || x->ndim != 3 || x->dtype != AX_FLOAT32 || x->shape[2] != m->d_model) {
@@ -73,52 +118,19 @@ static ax_tensor_t *mha_forward(ax_layer_t *self, ax_tensor_t *x) {
         ax_err_set(AX_ERR_BACKEND, "mha: input must be contiguous and on the device that holds the weights");
         return NULL;
     }
-    const int64_t B = x->shape[0], S = x->shape[1], D = m->d_model, H = m->n_heads, dk = m->d_k, rows = B * S;
-    ax_tensor_t *x_flat = NULL, *qkv = NULL, *Qh = NULL, *Kh = NULL, *Vh = NULL, *Oh = NULL, *attn = NULL, *out_flat = NULL,
-                *out = NULL;
-    int64_t flat_sh[2] = {rows, D}, qkv_sh[2] = {rows, 3 * D}, head_sh[3] = {B * H, S, dk};
+    const int64_t B = x->shape[0], S = x->shape[1], D = m->d_model, dk = m->d_k, rows = B * S;
+    ax_tensor_t *x_flat = NULL, *qkv = NULL, *attn = NULL, *out_flat = NULL, *out = NULL;
+    int64_t flat_sh[2] = {rows, D}, qkv_sh[2] = {rows, 3 * D};
     ax_status_t st = refresh_fused_qkv(m, ext);
-    /* Head sizes the fused kernel covers (multiples of 4 up to 128): attention reads the heads where the projection wrote
-     * them (columns h*dk.. of the q, k and v thirds of qkv) and writes them where the output
-     * projection reads them, so the three layout passes of attention.c:211-262, 391-400 and their
-     * four [B*H, S, dk] temporaries fall away; the projection bias moves into the GEMM write-back. */
-    const bool direct = ext->sdpa_fwd_rows && dk % 4 == 0 && dk <= 128 &&
-                        (!m->use_bias || ax_compute_has_gemm_bias_act());
-    if (direct) {
-        if (st == AX_OK && (!(x_flat = ax_tensor_reshape(x, flat_sh, 2)) || !(qkv = on_device_of(x, qkv_sh, 2)) ||
-                            !(attn = on_device_of(x, flat_sh, 2)) || !(out_flat = on_device_of(x, flat_sh, 2))))
-            st = AX_ERR_ALLOC;
-        if (st == AX_OK)
-            st = m->use_bias ? ax_compute_gemm_bias_act(x_flat, m->Wqkv_cache, m->bqkv_cache, AX_ACT_NONE, qkv)
-                             : ax_compute_gemm(x_flat, m->Wqkv_cache, qkv);
-        if (st == AX_OK)
-            st = ext->sdpa_fwd_rows(dev_ptr(qkv), dev_ptr(qkv) + D, dev_ptr(qkv) + 2 * D, 3 * D, dev_ptr(attn), D, NULL, B, H, S,
-                                    dk, 1.0f / sqrtf((float)dk), m->causal);
-        goto project;
-    }
     if (st == AX_OK && (!(x_flat = ax_tensor_reshape(x, flat_sh, 2)) || !(qkv = on_device_of(x, qkv_sh, 2)) ||
-                        !(Qh = on_device_of(x, head_sh, 3)) || !(Kh = on_device_of(x, head_sh, 3)) ||
-                        !(Vh = on_device_of(x, head_sh, 3)) || !(Oh = on_device_of(x, head_sh, 3)) ||
                         !(attn = on_device_of(x, flat_sh, 2)) || !(out_flat = on_device_of(x, flat_sh, 2))))
         st = AX_ERR_ALLOC;
-    if (st == AX_OK) st = ax_compute_gemm(x_flat, m->Wqkv_cache, qkv);
     if (st == AX_OK) {
-        ax_err_clear();
-        if (m->use_bias)
-            ext->head_interleave_qkv_split_bias(dev_ptr(qkv), dev_ptr(m->bqkv_cache), dev_ptr(Qh), dev_ptr(Kh), dev_ptr(Vh),
-                                                B, S, H, dk, D);
-        else
-            ext->head_interleave_qkv_split(dev_ptr(qkv), dev_ptr(Qh), dev_ptr(Kh), dev_ptr(Vh), B, S, H, dk, D);
-        st = ax_err_last_status();
+        const bool on_projection = ext->sdpa_fwd_rows && dk % 4 == 0 && dk <= 128 &&
+                                   (!m->use_bias || ax_compute_has_gemm_bias_act());
+        st = on_projection ? attend_on_projection(m, ext, x_flat, qkv, attn, B, S)
+                           : attend_per_head(m, ext, x_flat, qkv, attn, B, S);
     }
-    if (st == AX_OK)
-        st = ext->sdpa_fwd(dev_ptr(Qh), dev_ptr(Kh), dev_ptr(Vh), dev_ptr(Oh), NULL, B * H, S, dk, 1.0f / sqrtf((float)dk),
-                           m->causal, NULL);
-    if (st == AX_OK) {
-        ext->head_deinterleave(dev_ptr(Oh), dev_ptr(attn), B, S, H, dk);
-        st = ax_err_last_status();
-    }
-project:
     if (st == AX_OK) {                                       /* attention.c:402-417: gemm, then bias along axis 1 */
         if (m->use_bias && ax_compute_has_gemm_bias_act()) st = ax_compute_gemm_bias_act(attn, m->Wo, m->bo, AX_ACT_NONE, out_flat);
         else {
@@ -129,10 +141,6 @@ project:
     if (st == AX_OK) out = ax_tensor_reshape(out_flat, x->shape, 3);
     ax_tensor_destroy(x_flat);
     ax_tensor_destroy(qkv);
-    ax_tensor_destroy(Qh);
-    ax_tensor_destroy(Kh);
-    ax_tensor_destroy(Vh);
-    ax_tensor_destroy(Oh);
     ax_tensor_destroy(attn);
     ax_tensor_destroy(out_flat);
     return out;
