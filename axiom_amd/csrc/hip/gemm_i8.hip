@@ -866,7 +866,8 @@ int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_
         return launch_256(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K, ldc);
     // aligned but too few 256x256 tiles: direct-to-LDS kernel over smaller tiles
     if (aligned && vec_out && K % 128 == 0 && M % 64 == 0 && N % 64 == 0 && K < (int64_t(1) << 24)) {
-        if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 512)
+        // 128x128 tiles once there is one for every CU (2048^2 x 4096: 26.2 us against 30.7 on 64x64)
+        if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 256)
             return launch_dma<128, 128, 2, 2, 3>("qgemm_w8a8_128x128_dma", x, x_scale, w, w_scales, bias,
                                                  act, out, acc_out, M, N, K, ldc);
         return launch_dma<64, 64, 2, 2, 4>("qgemm_w8a8_64x64_dma", x, x_scale, w, w_scales, bias, act,
@@ -874,7 +875,7 @@ int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_
     }
     // the same kernel for M or N off the 64 grid: edge tiles clamp their loads and guard their stores
     if (aligned && vec_out && K % 128 == 0 && N % 4 == 0 && K < (int64_t(1) << 24)) {
-        if (((M + 127) / 128) * ((N + 127) / 128) >= 512)
+        if (((M + 127) / 128) * ((N + 127) / 128) >= 256)
             return launch_dma<128, 128, 2, 2, 3, true>("qgemm_w8a8_128x128_dma_edge", x, x_scale, w, w_scales, bias,
                                                        act, out, acc_out, M, N, K, ldc);
         return launch_dma<64, 64, 2, 2, 4, true>("qgemm_w8a8_64x64_dma_edge", x, x_scale, w, w_scales, bias, act,
