@@ -861,7 +861,9 @@ int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_
     const bool aligned = ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) && (K % BK == 0) && K > 0;
     const bool vec_out = (!out || (((uintptr_t)out | (uintptr_t)w_scales | (uintptr_t)bias) & 15) == 0) &&
                          (((uintptr_t)acc_out & 15) == 0) && ldc % 4 == 0;
-    if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128 &&
+    // the persistent 256x256 kernel from about 80 tiles on (81 tiles, 2304^2 x 8192: 72 us against 82 on
+    // 128x128 tiles; 64 tiles, 2048^2 x 4096: 40 against 26)
+    if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 80 &&
         K < (int64_t(1) << 24))   // per-lane 32-bit byte offsets span 256 rows
         return launch_256(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K, ldc);
     // aligned but too few 256x256 tiles: direct-to-LDS kernel over smaller tiles
@@ -921,7 +923,7 @@ extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
     // 0.85 POP/s).  Both operands are copied once into rows padded with zeros to the next multiple
     // of 128 — zeros add nothing to an integer sum — and the product runs on the copies.
     const int64_t Kp = (K + BK - 1) / BK * BK;
-    if (K % BK != 0 && K >= 512 && (M / 256) * (N / 256) >= 128 && (uint64_t)(M + N) * (uint64_t)Kp <= (uint64_t(1) << 30)) {
+    if (K % BK != 0 && K >= 512 && (M / 256) * (N / 256) >= 80 && (uint64_t)(M + N) * (uint64_t)Kp <= (uint64_t(1) << 30)) {
         int8_t *xp = static_cast<int8_t *>(workspace((size_t)(M + N) * (size_t)Kp));
         if (!xp) return AXHIP_ERR_ALLOC;
         int8_t *wp = xp + M * Kp;
@@ -941,7 +943,7 @@ extern "C" int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w,
     // the right and bottom fringes to the smaller tiles, each block addressed inside the full
     // output through its row pitch (whole shape on 64x64 tiles: 8000^2 x 8192 at 0.93 POP/s).
     const int64_t Mi = M / 256 * 256, Ni = N / 256 * 256;
-    if (fast && (Mi != M || Ni != N) && (Mi / 256) * (Ni / 256) >= 128) {
+    if (fast && (Mi != M || Ni != N) && (Mi / 256) * (Ni / 256) >= 80) {
         int rc = qgemm_block(x, x_scale, w, w_scales, bias, act, out, acc_out, Mi, Ni, K, N);
         if (rc == AXHIP_OK && Ni < N)
             rc = qgemm_block(x, x_scale, w + Ni * K, w_scales ? w_scales + Ni : nullptr, bias ? bias + Ni : nullptr, act,
