@@ -649,7 +649,10 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
     // (K <= 128) a workgroup's life is mostly its loads and its write-back: plain 64x64 tiles,
     // several workgroups per CU.
     if (g.K > 128) {
-        if (g.M % 128 == 0 && g.N % 256 == 0 && count(128, 256) >= 256)
+        // ... provided its rounds of one tile per CU come out nearly full: 384 tiles are a full round
+        // and a half-empty one (3072x4096x2048: 106 TFLOP/s, against 130 on 64x64 tiles)
+        const int64_t big = count(128, 256), cus = cu_count(), rounds = (big + cus - 1) / cus;
+        if (g.M % 128 == 0 && g.N % 256 == 0 && big >= 256 && big * 10 >= rounds * cus * 9)
             return launch_dma<128, 256, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
         return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[2], g, batch);
     }
