@@ -334,8 +334,10 @@ template <> struct Frag<false> {
 #define AXF_DS32(dst, addr, off) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 
 // EDGE: M and N need not be multiples of the tile (N a multiple of 4, and M too when A is stored
-// M-contiguous).  Edge tiles fetch the last existing row / column group in place of the missing
-// ones — their products land in outputs that are not stored — and guard the write-back.
+// M-contiguous) nor K of the slab (K a multiple of 4).  Edge tiles fetch the last existing row /
+// column group in place of the missing ones — their products land in outputs that are not stored —
+// and guard the write-back; in the last slab, lanes whose k values lie past K write zeros to
+// their LDS place instead of loading, in both operands, so the tail adds exact zeros.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI, int WAVES_K,
           bool EDGE = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(SgemmArgs g) {
@@ -370,7 +372,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     const float *A = static_cast<const float *>(g.A) + batch * g.stride_a;
     const float *B = static_cast<const float *>(g.B) + batch * g.stride_b;
     float *C = g.C + batch * g.stride_c;
-    const int slabs = (int)(g.K / 32);
+    // EDGE also takes a K that ends inside a slab (K a multiple of 4): the last slab's lanes whose four
+    // k values lie past K load nothing and write zeros to their LDS place instead
+    const int slabs = EDGE ? (int)((g.K + 31) / 32) : (int)(g.K / 32);
+    const int ktail = EDGE ? (int)(g.K - (int64_t)(slabs - 1) * 32) : 32;     // k values in the last slab
+    int left = slabs;                                                          // slabs not yet requested
 
     // ---- global -> LDS ----
     unsigned va[OA::IPW], vb[OB::IPW];
@@ -383,6 +389,18 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     const int64_t step_a = A_KC ? 128 : 128 * g.lda, step_b = B_KC ? 128 : 128 * g.ldb;   // bytes per slab
     const unsigned lds0 = (unsigned)(uintptr_t)lds_raw;
     const unsigned dma_a = lds0 + wave * OA::PITCH, dma_b = lds0 + wave * OB::PITCH;
+    // does this lane's 16 bytes of load instruction j lie inside K in the last slab
+    bool ta[OA::IPW], tb[OB::IPW];
+#pragma unroll
+    for (int j = 0; j < OA::IPW; j++) {
+        const int q = j * NW + wave, row = q * 8 + (lane >> 3);
+        ta[j] = A_KC ? (((lane & 7) ^ ((row >> 1) & 7)) * 4 < ktail) : (q * (256 / BM) + lane / (64 / (256 / BM)) < ktail);
+    }
+#pragma unroll
+    for (int j = 0; j < OB::IPW; j++) {
+        const int q = j * NW + wave, row = q * 8 + (lane >> 3);
+        tb[j] = B_KC ? (((lane & 7) ^ ((row >> 1) & 7)) * 4 < ktail) : (q * (256 / BN) + lane / (64 / (256 / BN)) < ktail);
+    }
 
     // ---- LDS -> fragments ----
     const int frow = lane & 31, fhalf = lane >> 5;
@@ -413,10 +431,24 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
 // loads of the next unread slab into stage ST
 #define AXF_ISSUE(ST)                                                                            \
     do {                                                                                         \
-        _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                                      \
-            AXF_LOAD_LDS(dma_a + (ST) * OA::BYTES + j * NW * OA::PITCH, va[j], ga);              \
-        _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                                      \
-            AXF_LOAD_LDS(dma_b + B_BASE + (ST) * OB::BYTES + j * NW * OB::PITCH, vb[j], gb);     \
+        --left;                                                                                  \
+        if (EDGE && left == 0 && ktail < 32) {                                                   \
+            _Pragma("unroll") for (int j = 0; j < OA::IPW; j++) {                                \
+                const unsigned at = wave * OA::PITCH + (ST) * OA::BYTES + j * NW * OA::PITCH;    \
+                if (ta[j]) AXF_LOAD_LDS(lds0 + at, va[j], ga);                                   \
+                else *reinterpret_cast<v4f *>(lds_raw + at + lane * 16) = v4f{0.f, 0.f, 0.f, 0.f}; \
+            }                                                                                    \
+            _Pragma("unroll") for (int j = 0; j < OB::IPW; j++) {                                \
+                const unsigned at = B_BASE + wave * OB::PITCH + (ST) * OB::BYTES + j * NW * OB::PITCH; \
+                if (tb[j]) AXF_LOAD_LDS(lds0 + at, vb[j], gb);                                   \
+                else *reinterpret_cast<v4f *>(lds_raw + at + lane * 16) = v4f{0.f, 0.f, 0.f, 0.f}; \
+            }                                                                                    \
+        } else {                                                                                 \
+            _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                                  \
+                AXF_LOAD_LDS(dma_a + (ST) * OA::BYTES + j * NW * OA::PITCH, va[j], ga);          \
+            _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                                  \
+                AXF_LOAD_LDS(dma_b + B_BASE + (ST) * OB::BYTES + j * NW * OB::PITCH, vb[j], gb); \
+        }                                                                                        \
         ga += step_a;                                                                            \
         gb += step_b;                                                                            \
     } while (0)
@@ -488,6 +520,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     if constexpr (NST > 3) { if (slabs > 2) AXF_ISSUE(2); }
     if (!ring) AXF_ISSUE(NST - 1);
     AXF_VM(0);
+    if constexpr (EDGE) AXF_LGKM(0);             // zeros written for a K tail that is already in the first slabs
     __builtin_amdgcn_s_barrier();
     for (int s = 0; s < slabs; s += NST) {
         AXF_SLAB(0, ring && s + NST - 1 < slabs);
@@ -631,13 +664,13 @@ int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
 // names: 128x256, 64x64, 64x64 with the k split.
 template <bool A_KC, bool B_KC>
 int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
-    const bool ok = g.K % 32 == 0 && g.K > 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
+    const bool ok = g.K % 4 == 0 && g.K > 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                     ((uintptr_t)g.C % 16 == 0) && ((uintptr_t)g.bias % 16 == 0) && g.lda % 4 == 0 &&
                     g.ldb % 4 == 0 && g.ldc % 4 == 0 && g.stride_a % 4 == 0 && g.stride_b % 4 == 0 &&
                     g.stride_c % 4 == 0 && g.lda < (1 << 20) && g.ldb < (1 << 20) && batch <= 65535 &&
                     g.N % 4 == 0 && (A_KC || g.M % 4 == 0) && ((g.M + 63) / 64) * ((g.N + 63) / 64) <= 0x7fffffff;
     if (!ok) return -1;
-    if (g.M % 64 != 0 || g.N % 64 != 0) {                   // off the tile grid: 64x64 tiles with guarded edges
+    if (g.M % 64 != 0 || g.N % 64 != 0 || g.K % 32 != 0) {  // off the tile grid: 64x64 tiles with guarded edges
         static const char *const edge_names[2] = {"sgemm_64x64_dma_edge", "sgemm_64x64k2_dma_edge"};
         if (g.K > 128) return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2, true>(edge_names[1], g, batch);
         return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 1, true>(edge_names[0], g, batch);
@@ -843,7 +876,10 @@ int run_f32(const SgemmArgs &g, int transa, int transb);
 // Returns -1 when the shape is left alone.
 int try_k_tail(const SgemmArgs &g, int transa, int transb) {
     const int64_t Km = g.K / 32 * 32;
-    if ((transa && transb) || Km == g.K || Km < 512 || (g.M / 64) * (g.N / 64) < 256) return -1;
+    if ((transa && transb) || Km == g.K || Km < 256) return -1;
+    // K a multiple of 4 runs in one pass on the 64x64 tiles with guarded edges, which take a K tail
+    // themselves; two passes are for the other K and for shapes whose main part earns 128x256 tiles
+    if (g.K % 4 == 0 && (g.M / 128) * (g.N / 256) < 256) return -1;
     const float *A = static_cast<const float *>(g.A), *B = static_cast<const float *>(g.B);
     SgemmArgs p = g;
     p.K = Km;

@@ -563,22 +563,29 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     int tm, tn;
     tile_of_block(blockIdx.x, (int)((M + BM - 1) / BM), (int)((N + BN - 1) / BN), tm, tn);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
-    const int slabs = (int)(K / BKB);
+    // EDGE also takes a K that ends inside a slab (K a multiple of 16): in the last slab the lanes
+    // whose 16 bytes lie past K load nothing and write zeros to their LDS place instead
+    const int slabs = EDGE ? (int)((K + BKB - 1) / BKB) : (int)(K / BKB);
+    const int ktail = EDGE ? (int)(K - (int64_t)(slabs - 1) * BKB) : BKB;      // bytes of K in the last slab
+    int left = slabs;                                                          // slabs not yet requested
     // rows of this tile that exist (EDGE; the last tile row / column may hang over)
     const int mrows = EDGE && M - m0 < BM ? (int)(M - m0) : BM, nrows = EDGE && N - n0 < BN ? (int)(N - n0) : BN;
 
     // load instruction q fills rows q*8 .. q*8+7 of an operand stage; wave w issues q = j*NW + w.
     // The LDS place (and so the swizzle) is that of the nominal row; the source row is clamped.
     unsigned vx[IPW_X], vw[IPW_W];
+    bool tx[IPW_X], tw[IPW_W];                   // is this lane's chunk inside K in the last slab
 #pragma unroll
     for (int j = 0; j < IPW_X; j++) {
         const int row = (j * NW + wave) * 8 + (lane >> 3);
         vx[j] = (unsigned)((row < mrows ? row : mrows - 1) * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+        tx[j] = (((lane & 7) ^ ((row >> 1) & 7)) << 4) < ktail;
     }
 #pragma unroll
     for (int j = 0; j < IPW_W; j++) {
         const int row = (j * NW + wave) * 8 + (lane >> 3);
         vw[j] = (unsigned)((row < nrows ? row : nrows - 1) * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+        tw[j] = (((lane & 7) ^ ((row >> 1) & 7)) << 4) < ktail;
     }
     const int8_t *gx = X + m0 * K, *gw = W + n0 * K;
     const unsigned lds0 = (unsigned)(uintptr_t)lds, lds_w = lds0 + wave * 1024;
@@ -613,10 +620,24 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 
 #define AXI8G_ISSUE(ST)                                                                          \
     do {                                                                                         \
-        _Pragma("unroll") for (int j = 0; j < IPW_X; j++)                                        \
-            AXI8_LOAD_LDS(lds_w + (ST) * XS + j * NW * 1024, vx[j], gx);                         \
-        _Pragma("unroll") for (int j = 0; j < IPW_W; j++)                                        \
-            AXI8_LOAD_LDS(lds_w + W_BASE + (ST) * WS + j * NW * 1024, vw[j], gw);                \
+        --left;                                                                                  \
+        if (EDGE && left == 0 && ktail < BKB) {                                                  \
+            _Pragma("unroll") for (int j = 0; j < IPW_X; j++) {                                  \
+                const unsigned at = wave * 1024 + (ST) * XS + j * NW * 1024;                     \
+                if (tx[j]) AXI8_LOAD_LDS(lds0 + at, vx[j], gx);                                  \
+                else *reinterpret_cast<v4i *>(lds + at + lane * 16) = v4i{0, 0, 0, 0};           \
+            }                                                                                    \
+            _Pragma("unroll") for (int j = 0; j < IPW_W; j++) {                                  \
+                const unsigned at = wave * 1024 + W_BASE + (ST) * WS + j * NW * 1024;            \
+                if (tw[j]) AXI8_LOAD_LDS(lds0 + at, vw[j], gw);                                  \
+                else *reinterpret_cast<v4i *>(lds + at + lane * 16) = v4i{0, 0, 0, 0};           \
+            }                                                                                    \
+        } else {                                                                                 \
+            _Pragma("unroll") for (int j = 0; j < IPW_X; j++)                                    \
+                AXI8_LOAD_LDS(lds_w + (ST) * XS + j * NW * 1024, vx[j], gx);                     \
+            _Pragma("unroll") for (int j = 0; j < IPW_W; j++)                                    \
+                AXI8_LOAD_LDS(lds_w + W_BASE + (ST) * WS + j * NW * 1024, vw[j], gw);            \
+        }                                                                                        \
         gx += BKB;                                                                               \
         gw += BKB;                                                                               \
     } while (0)
@@ -661,6 +682,7 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     if constexpr (NST > 2) { if (slabs > 1) AXI8G_ISSUE(1); }
     if constexpr (NST > 3) { if (slabs > 2) AXI8G_ISSUE(2); }
     AXI8_VM(0);
+    if constexpr (EDGE) AXI8_LGKM(0);            // zeros written for a K tail that is already in the first slabs
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     for (int s = 0; s < slabs; s += NST) {
@@ -876,7 +898,8 @@ int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_
                                            out, acc_out, M, N, K, ldc);
     }
     // the same kernel for M or N off the 64 grid: edge tiles clamp their loads and guard their stores
-    if (aligned && vec_out && K % 128 == 0 && N % 4 == 0 && K < (int64_t(1) << 24)) {
+    const bool aligned16 = ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) && K % 16 == 0 && K > 0;
+    if (aligned16 && vec_out && N % 4 == 0 && K < (int64_t(1) << 24)) {
         if (((M + 127) / 128) * ((N + 127) / 128) >= 256)
             return launch_dma<128, 128, 2, 2, 3, true>("qgemm_w8a8_128x128_dma_edge", x, x_scale, w, w_scales, bias,
                                                        act, out, acc_out, M, N, K, ldc);

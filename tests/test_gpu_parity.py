@@ -40,7 +40,10 @@ INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300
                (2048, 4096, 520), (2112, 4128, 600),
                # M or N off the 64 grid with K on the 128 grid: the direct-to-LDS kernel with clamped edge tiles
                (100, 4096, 512), (130, 260, 256), (2000, 2000, 128), (63, 60, 128), (9, 4, 128), (500, 1000, 1024),
-               (65, 64, 256), (64, 68, 384), (2900, 3000, 128)]
+               (65, 64, 256), (64, 68, 384), (2900, 3000, 128),
+               # K a multiple of 16 off the 128 grid: the last slab's tail is zero-filled in LDS
+               (100, 4096, 784), (64, 64, 16), (130, 260, 144), (256, 4096, 784), (2900, 3000, 400), (9, 4, 48),
+               (64, 128, 1040), (128, 128, 112)]
 
 
 @pytest.mark.parametrize("M,N,K", INT8_SHAPES)
@@ -134,7 +137,9 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               (130, 257, 1027), (67, 1001, 129),                  # rows off the 16-byte grid in every form
               (1024, 1088, 1045), (1030, 1100, 600),              # K off the 32 grid: main product, then the K tail on top
               # M or N off the 64 grid with K on the 32 grid and N % 4 == 0: direct-to-LDS tiles with guarded edges
-              (65, 68, 64), (9, 4, 32), (63, 60, 96), (200, 36, 128), (500, 1000, 256), (12, 2052, 160)]
+              (65, 68, 64), (9, 4, 32), (63, 60, 96), (200, 36, 128), (500, 1000, 256), (12, 2052, 160),
+              # K a multiple of 4 off the 32 grid: the last slab's tail is zero-filled in LDS
+              (64, 4096, 784), (128, 64, 36), (64, 64, 4), (100, 132, 100), (256, 256, 44), (70, 64, 1000), (16, 256, 2076)]
 
 
 @pytest.mark.parametrize("M,N,K", F32_SHAPES)
@@ -236,7 +241,7 @@ def test_sgemm_config0_1024_cube(hip, oracle, golden):
         assert np.array_equal(hip.sgemm(da, db).numpy(), c)
 
 
-@pytest.mark.parametrize("M,N,K", [(130, 200, 96), (256, 320, 96), (2048, 4096, 32), (64, 128, 2048), (33, 70, 512), (1032, 1100, 96), (1024, 1088, 1045)])
+@pytest.mark.parametrize("M,N,K", [(130, 200, 96), (256, 320, 96), (2048, 4096, 32), (64, 128, 2048), (33, 70, 512), (1032, 1100, 96), (1024, 1088, 1045), (200, 260, 784)])
 def test_sgemm_alpha_beta_bias_act(hip, oracle, M, N, K):
     say("sgemm epilogue", M, N, K)
     oracle.seed(21)
