@@ -943,8 +943,11 @@ def test_softmax_rows(hip, oracle, golden):
     say("softmax")
     for (rows, cols), arr in zip(sc.SOFTMAX_SHAPES, sc.softmax_inputs(oracle)):
         assert np.abs(run_softmax(hip, arr) - golden[f"softmax_{rows}x{cols}_naive"]).max() < 1e-6
+    # 4097 .. 36864 columns: the row held in LDS (rows start off the 16-byte grid when cols is odd);
+    # beyond: two reads with the running-maximum form
     for (rows, cols) in [(1, 1), (7, 129), (1000, 512), (33, 513), (64, 1024), (5, 4096), (3, 4097), (2, 100000),
-                         (8192, 512), (4097, 64)]:
+                         (8192, 512), (4097, 64), (5, 10001), (3, 36864), (3, 36865), (7, 50257), (2, 131075),
+                         (300, 4100), (1, 36863)]:
         oracle.seed(rows + cols)
         x = oracle.uniform((rows, cols), -8, 8)
         got = run_softmax(hip, x)
@@ -953,6 +956,10 @@ def test_softmax_rows(hip, oracle, golden):
         assert (np.abs(got - want) <= 2e-6 * want + 1e-12).all(), (rows, cols)
         if rows * cols <= 1 << 20:
             assert np.abs(got - oracle.softmax_rows(x)).max() < 1e-6
+        if cols > 4096:                                   # in place (the slot allows in == out)
+            dx = hip.array(x)
+            hip.check(hip.L.axhip_softmax_rows(dx.ptr, dx.ptr, rows, cols))
+            assert np.array_equal(dx.numpy(), got)
 
 
 def run_layernorm(hip, x, gamma, beta, eps, save=True):
@@ -973,7 +980,8 @@ def test_layernorm_forward(hip, oracle, golden):
         o_out, o_xh, o_inv = oracle.layernorm(x, gamma, beta, 1e-5)
         assert np.abs(out - o_out).max() < 5e-6 and np.abs(xh - o_xh).max() < 5e-6
         assert np.allclose(inv, o_inv, rtol=2e-6)
-    for shp in [(4096, 1024), (2048, 768), (100, 4096), (3, 5000), (9, 1), (4097, 96)]:
+    for shp in [(4096, 1024), (2048, 768), (100, 4096), (3, 5000), (9, 1), (4097, 96), (5, 10001), (2, 36864),
+                (3, 36867), (3, 50257), (130, 4099)]:
         oracle.seed(sum(shp))
         x, gamma, beta = oracle.uniform(shp, -3, 5), oracle.uniform((shp[-1],), 0.5, 1.5), oracle.uniform((shp[-1],), -1, 1)
         out, xh, inv = run_layernorm(hip, x, gamma, beta, 1e-5)
