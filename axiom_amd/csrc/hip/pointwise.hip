@@ -60,28 +60,36 @@ __device__ __forceinline__ void row_offsets(const Bcast &g, IDX row, int64_t &oa
     }
 }
 
-// VEC: every thread owns 4 consecutive elements of the inner dimension (inner % 4 == 0, every
-// address a multiple of 16 bytes, inner strides 0 or 1).  Otherwise one element per thread.
+// VEC: every thread owns 4 consecutive elements of the inner dimension (inner strides 0 or 1),
+// moved as 16 bytes at whatever alignment the row has (global memory takes unaligned vector
+// accesses); the last group of a row whose length is not a multiple of 4 goes by element.
+// Otherwise one element per thread.
 template <int OP, bool VEC, typename IDX>
 __global__ void __launch_bounds__(256)
 k_binary(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out, Bcast g,
          int64_t items) {
     const int64_t stride = (int64_t)gridDim.x * 256;
-    const IDX per_row = (IDX)(VEC ? g.inner / 4 : g.inner);
+    const IDX per_row = (IDX)(VEC ? (g.inner + 3) / 4 : g.inner);
     for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < items; t += stride) {
         const IDX row = (IDX)t / per_row, col = (IDX)t - row * per_row;
         int64_t oa, ob;
         row_offsets<IDX>(g, row, oa, ob);
         if (VEC) {
             const int64_t c = (int64_t)col * 4;
-            v4f va, vb, r;
-            if (g.ia) va = *reinterpret_cast<const v4f *>(a + oa + c);
-            else va = v4f{a[oa], a[oa], a[oa], a[oa]};
-            if (g.ib) vb = *reinterpret_cast<const v4f *>(b + ob + c);
-            else vb = v4f{b[ob], b[ob], b[ob], b[ob]};
+            float *dst = out + (int64_t)row * g.inner + c;
+            if (c + 4 <= g.inner) {
+                v4f va, vb, r;
+                if (g.ia) __builtin_memcpy(&va, a + oa + c, 16);
+                else va = v4f{a[oa], a[oa], a[oa], a[oa]};
+                if (g.ib) __builtin_memcpy(&vb, b + ob + c, 16);
+                else vb = v4f{b[ob], b[ob], b[ob], b[ob]};
 #pragma unroll
-            for (int e = 0; e < 4; e++) r[e] = binop<OP>(va[e], vb[e]);
-            *reinterpret_cast<v4f *>(out + (int64_t)row * g.inner + c) = r;
+                for (int e = 0; e < 4; e++) r[e] = binop<OP>(va[e], vb[e]);
+                __builtin_memcpy(dst, &r, 16);
+            } else {
+                for (int64_t e = 0; c + e < g.inner; e++)
+                    dst[e] = binop<OP>(a[oa + (c + e) * g.ia], b[ob + (c + e) * g.ib]);
+            }
         } else {
             out[t] = binop<OP>(a[oa + (int64_t)col * g.ia], b[ob + (int64_t)col * g.ib]);
         }
@@ -96,10 +104,11 @@ k_unary_p(const float *__restrict__ in, float *__restrict__ out, int64_t n, floa
     if (vec) {
         const int64_t n4 = n >> 2;
         for (int64_t j = i; j < n4; j += stride) {
-            v4f v = reinterpret_cast<const v4f *>(in)[j];
+            v4f v;
+            __builtin_memcpy(&v, in + 4 * j, 16);         // any alignment
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] = unop<OP>(v[e], p);
-            reinterpret_cast<v4f *>(out)[j] = v;
+            __builtin_memcpy(out + 4 * j, &v, 16);
         }
         for (int64_t j = (n4 << 2) + i; j < n; j += stride) out[j] = unop<OP>(in[j], p);
     } else {
@@ -152,11 +161,8 @@ unsigned blocks_for(int64_t items) {
 
 template <int OP>
 int launch_binary(const float *a, const float *b, float *out, const Bcast &g, int64_t rows) {
-    const bool aligned = ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)out) & 15) == 0);
-    bool vec = aligned && g.inner % 4 == 0 && (g.ia == 0 || g.ia == 1) && (g.ib == 0 || g.ib == 1);
-    for (int d = 0; d < g.nouter && vec; d++)
-        vec = (g.ia == 0 || g.sa[d] % 4 == 0) && (g.ib == 0 || g.sb[d] % 4 == 0);
-    const int64_t items = rows * (vec ? g.inner / 4 : g.inner);
+    const bool vec = g.inner >= 4 && (g.ia == 0 || g.ia == 1) && (g.ib == 0 || g.ib == 1);
+    const int64_t items = rows * (vec ? (g.inner + 3) / 4 : g.inner);
     const bool narrow = items < 0x7fffffff && rows < 0x7fffffff && g.inner < 0x7fffffff;
     const dim3 grid(blocks_for(items)), block(256);
     if (vec && narrow) hipLaunchKernelGGL((k_binary<OP, true, unsigned>), grid, block, 0, kStream, a, b, out, g, items);
@@ -168,7 +174,7 @@ int launch_binary(const float *a, const float *b, float *out, const Bcast &g, in
 
 template <int OP>
 int launch_unary(const float *in, float *out, int64_t n, float p) {
-    const int vec = (((uintptr_t)in | (uintptr_t)out) & 15) == 0;
+    const int vec = 1;
     hipLaunchKernelGGL(k_unary_p<OP>, dim3(blocks_for(vec ? n / 4 + 1 : n)), dim3(256), 0, kStream, in, out, n, p, vec);
     return check_launch("unary");
 }
