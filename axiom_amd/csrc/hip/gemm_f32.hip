@@ -950,7 +950,7 @@ extern "C" int axhip_sgemm(int transa, int transb, int64_t M, int64_t N, int64_t
     if (int rc = axhip::ensure_ready()) return rc;
     if (int rc = validate("sgemm", transa, transb, M, N, K, A, lda, B, ldb, C, ldc, act)) return rc;
     if (M == 0 || N == 0) return AXHIP_OK;
-    if (M <= 8 && !transa && !transb && alpha == 1.0f && beta == 0.0f)
+    if (M <= 16 && !transa && !transb && alpha == 1.0f && beta == 0.0f)
         return axhip_sgemm_skinny(M, N, K, A, lda, B, ldb, C, ldc, bias, act);
     SgemmArgs g{A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, alpha, beta, nullptr, bias, act};
     return run_f32(g, transa, transb);

@@ -1,4 +1,4 @@
-// Skinny-M (1 <= M <= 8) fp32 route: C[M,N] = act(A[M,K] * B[K,N] + bias[n]).
+// Skinny-M (1 <= M <= 16) fp32 route: C[M,N] = act(A[M,K] * B[K,N] + bias[n]).
 //
 // The work is one pass over B (K*N*4 bytes): HBM-bound.  A workgroup of 256 threads owns 64
 // columns (16 lanes x float4 = 256 contiguous bytes per B row) and a K range; its 16 lane
@@ -6,7 +6,7 @@
 // 256-byte row segments and eight of them are kept in flight per lane.  The M activations of
 // a k row are wave-uniform only per lane group, so they come from LDS (staged once per
 // workgroup); the first batch of weight loads is issued before that staging so HBM latency
-// overlaps it.  Lane groups are summed through LDS in a fixed order.  When K is split over
+// overlaps it.  Lane groups are summed inside their wave, waves through LDS, in a fixed order.  When K is split over
 // several workgroups each writes its partial tile to a workspace and bumps a per-strip
 // counter; the workgroup that arrives last adds the partials in split order (not arrival
 // order) and applies bias and activation.  The sum order is fixed, so results are
@@ -29,7 +29,7 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
          int64_t k_per_split, const float *__restrict__ bias, int act, int splits,
          float *__restrict__ C, int64_t ldc, int *__restrict__ counters) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
-    // sm: [MR][k_per_split] activations, then [KGROUPS][MR][COLS] partial sums
+    // sm: [MR][k_per_split] activations, then [KGROUPS or 4][MR][COLS] partial sums
     const int tid = threadIdx.x;
     const int cg = tid & 15;            // column group: columns 4*cg .. 4*cg+3 of the 64
     const int kg = tid >> 4;            // lane group
@@ -159,11 +159,31 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
         }
     }
 
+    // Lane groups are joined through LDS.  From M = 9 on the four lane groups of a wave (lanes l,
+    // l^16, l^32, l^48 hold the same columns) are first added with the row-swap instructions, so
+    // that one partial per wave goes through LDS and the buffer stays small enough for three
+    // workgroups per CU; up to M = 8 every lane group writes its own partial (measured faster there).
+    constexpr bool PRE = MR > 8;
+    constexpr int NPART = PRE ? 4 : KGROUPS;
     float *red = sm + (int64_t)MR * k_per_split;
 #pragma unroll
-    for (int m = 0; m < MR; m++)
-        *reinterpret_cast<v4f *>(red + (kg * MR + m) * COLS + 4 * cg) =
-            v4f{acc[m][0], acc[m][1], acc[m][2], acc[m][3]};
+    for (int m = 0; m < MR; m++) {
+        if (PRE) {
+            v4f r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const unsigned u = __builtin_bit_cast(unsigned, acc[m][e]);
+                const auto p32 = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+                const float h = __builtin_bit_cast(float, (unsigned)p32[0]) + __builtin_bit_cast(float, (unsigned)p32[1]);
+                const unsigned u2 = __builtin_bit_cast(unsigned, h);
+                const auto p16 = __builtin_amdgcn_permlane16_swap(u2, u2, false, false);
+                r[e] = __builtin_bit_cast(float, (unsigned)p16[0]) + __builtin_bit_cast(float, (unsigned)p16[1]);
+            }
+            if ((tid & 63) < 16) *reinterpret_cast<v4f *>(red + ((tid >> 6) * MR + m) * COLS + 4 * cg) = r;
+        } else {
+            *reinterpret_cast<v4f *>(red + (kg * MR + m) * COLS + 4 * cg) = v4f{acc[m][0], acc[m][1], acc[m][2], acc[m][3]};
+        }
+    }
     __syncthreads();
 
     float *part = dst + (int64_t)blockIdx.y * dst_split_stride;   // == C itself when splits == 1
@@ -171,7 +191,7 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
         const int m = i / COLS, c = i % COLS;
         float s = 0.0f;
 #pragma unroll
-        for (int g2 = 0; g2 < KGROUPS; g2++) s += red[(g2 * MR + m) * COLS + c];
+        for (int w = 0; w < NPART; w++) s += red[(w * MR + m) * COLS + c];
         const int64_t n = n0 + c;
         if (n < N) {
             if (splits == 1) {
@@ -266,7 +286,7 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
                                   const float *bias, int act) {
     if (int rc = axhip::ensure_ready()) return rc;
     if (!A || !B || !C) return fail(AXHIP_ERR_NULL_ARG, "sgemm_skinny: NULL matrix");
-    if (M < 1 || M > 8) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: M=%lld outside 1..8", (long long)M);
+    if (M < 1 || M > 16) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: M=%lld outside 1..16", (long long)M);
     if (N < 0 || K < 0 || lda < K || ldb < N || ldc < N)
         return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: bad dimension or leading dimension");
     if (act < AXHIP_ACT_NONE || act > AXHIP_ACT_GELU)
@@ -283,9 +303,12 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
     int64_t kps = (K + splits - 1) / splits;
     kps = (kps + KGROUPS - 1) / KGROUPS * KGROUPS;
     // the activations of one split must fit LDS next to the reduction buffer
-    const int64_t red_floats = (int64_t)KGROUPS * M * COLS;
-    const int64_t max_kps = ((int64_t)(96 * 1024 / 4) - red_floats) / M / KGROUPS * KGROUPS;
+    const int64_t red_floats = (int64_t)(M > 8 ? 4 : KGROUPS) * M * COLS;   // partials per workgroup, as in the kernel
+    // ... within 52 KiB, so that three workgroups share a CU whatever M is (4096 x 11008 at M = 16: 95 us
+    // with one 96 KiB workgroup per CU, 60 us this way)
+    const int64_t max_kps = ((int64_t)(52 * 1024 / 4) - red_floats) / M / KGROUPS * KGROUPS;
     if (kps > max_kps) kps = max_kps;
+    if (kps > 512) kps = 512;      // at most 128 KiB of weights per workgroup: wide matrices get more workgroups, not longer ones
     if (kps < KGROUPS) kps = KGROUPS;
     splits = K > 0 ? (K + kps - 1) / kps : 1;
     if (splits > 65535) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: K=%lld too large", (long long)K);
@@ -310,7 +333,13 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
             (const void *)k_skinny<7, true>, (const void *)k_skinny<8, true>,
             (const void *)k_skinny<1, false>, (const void *)k_skinny<2, false>, (const void *)k_skinny<3, false>,
             (const void *)k_skinny<4, false>, (const void *)k_skinny<5, false>, (const void *)k_skinny<6, false>,
-            (const void *)k_skinny<7, false>, (const void *)k_skinny<8, false>};
+            (const void *)k_skinny<7, false>, (const void *)k_skinny<8, false>,
+            (const void *)k_skinny<9, true>, (const void *)k_skinny<10, true>, (const void *)k_skinny<11, true>,
+            (const void *)k_skinny<12, true>, (const void *)k_skinny<13, true>, (const void *)k_skinny<14, true>,
+            (const void *)k_skinny<15, true>, (const void *)k_skinny<16, true>,
+            (const void *)k_skinny<9, false>, (const void *)k_skinny<10, false>, (const void *)k_skinny<11, false>,
+            (const void *)k_skinny<12, false>, (const void *)k_skinny<13, false>, (const void *)k_skinny<14, false>,
+            (const void *)k_skinny<15, false>, (const void *)k_skinny<16, false>};
         for (const void *k : ks)
             AXHIP_HIP_TRY(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024),
                           "hipFuncSetAttribute");
@@ -326,6 +355,7 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
                          bias, act, (int)splits, C, ldc, counters);                           \
         break;
         AX_CASE(1) AX_CASE(2) AX_CASE(3) AX_CASE(4) AX_CASE(5) AX_CASE(6) AX_CASE(7) AX_CASE(8)
+        AX_CASE(9) AX_CASE(10) AX_CASE(11) AX_CASE(12) AX_CASE(13) AX_CASE(14) AX_CASE(15) AX_CASE(16)
 #undef AX_CASE
         default: rc = AXHIP_ERR_SHAPE;
     }

@@ -79,8 +79,8 @@ int   axhip_memcpy_d2d(void *device_dst, const void *device_src, size_t bytes);
  *      transa = 0: A is [M,K] (lda >= K);  1: A is [K,M] (lda >= M)
  *      transb = 0: B is [K,N] (ldb >= N);  1: B is [N,K] (ldb >= K)
  *      bias may be NULL; beta == 0 never reads C (C may be uninitialised).
- *      True fp32 MFMA arithmetic; M <= 8 with transa = transb = 0 takes the
- *      weight-streaming route below. ------------------------------------------------- */
+ *      True fp32 MFMA arithmetic; M <= 16 with transa = transb = 0, alpha = 1, beta = 0 takes
+ *      the weight-streaming route below. ------------------------------------------------- */
 int axhip_sgemm(int transa, int transb, int64_t M, int64_t N, int64_t K, float alpha,
                 const float *A, int64_t lda, const float *B, int64_t ldb, float beta,
                 float *C, int64_t ldc, const float *bias, int act);
@@ -93,7 +93,7 @@ int axhip_sgemm_strided_batched(int transa, int transb, int64_t M, int64_t N, in
                                 const float *B, int64_t ldb, int64_t stride_b, float beta,
                                 float *C, int64_t ldc, int64_t stride_c, int64_t batch);
 
-/* Skinny-M route (1 <= M <= 8): C[M,N] = act(A[M,K] * B[K,N] + bias[n]), B streamed once
+/* Skinny-M route (1 <= M <= 16): C[M,N] = act(A[M,K] * B[K,N] + bias[n]), B streamed once
  * for all M rows.  The GPU counterpart of the small/skinny-M AXPY route of opt_gemm
  * (src/compute/backends/cpu_opt.c:3499-3567).  Results are deterministic run to run. */
 int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,

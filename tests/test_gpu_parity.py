@@ -367,7 +367,7 @@ def test_config3_ffn_block(hip, oracle):
 
 
 # ------------------------------------------------------------------ skinny-M route
-@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("M", list(range(1, 17)))
 def test_skinny_against_oracle(hip, oracle, M):
     oracle.seed(100 + M)
     # (100, 3076) and (5000, 3072): a ragged last strip with K below one batch of rows, and splits longer
@@ -388,7 +388,7 @@ def test_skinny_against_oracle(hip, oracle, M):
         assert np.array_equal(hip.sgemm_skinny(da, db).numpy(), got)  # deterministic
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 1030, 4096), (3, 2048, 3104), (8, 777, 4100)])
+@pytest.mark.parametrize("M,K,N", [(1, 1030, 4096), (3, 2048, 3104), (8, 777, 4100), (13, 1500, 2052), (16, 4096, 1028)])
 def test_skinny_padded_leading_dimensions(hip, oracle, M, K, N):
     """Sub-matrices of wider buffers (lda > K, ldb > N, ldc > N): the padding is neither read into
     the result nor written."""
@@ -766,7 +766,7 @@ def test_error_paths(hip):
     assert L.axhip_sgemm(0, 0, 8, 8, 8, 1.0, None, 8, a.ptr, 8, 0.0, a.ptr, 8, None, 0) == 1
     assert L.axhip_sgemm(0, 0, 8, 8, 8, 1.0, a.ptr, 4, a.ptr, 8, 0.0, a.ptr, 8, None, 0) == 3
     assert L.axhip_sgemm(1, 1, 8, 8, 8, 1.0, a.ptr, 8, a.ptr, 8, 0.0, a.ptr, 8, None, 0) == 10
-    assert L.axhip_sgemm_skinny(9, 8, 8, a.ptr, 8, a.ptr, 8, a.ptr, 8, None, 0) == 3
+    assert L.axhip_sgemm_skinny(17, 8, 8, a.ptr, 8, a.ptr, 8, a.ptr, 8, None, 0) == 3
     assert L.axhip_qgemm_w8a8(a.ptr, 1.0, a.ptr, None, None, 0, None, None, 8, 8, 8) == 1
     assert L.axhip_qgemm_w8a8(a.ptr, 1.0, a.ptr, None, None, 7, None, a.ptr, 8, 8, 8) == 3
     assert "activation" in hip.last_error()
