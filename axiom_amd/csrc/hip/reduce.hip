@@ -3,7 +3,9 @@
 // [outer, axis_len, inner] (the reference's reduction_dims, cuda/ops_reduce.cu:246-251).
 // HBM-bound: one pass over the input.  Sums:
 //
-//   inner > 1  (column sums; axis 0 of [rows, cols] is the dense layer's bias gradient):
+//   inner > 1  (column sums; axis 0 of [rows, cols] is the dense layer's bias gradient), wide
+//              (2048 columns and up; narrower ones take the column kernel below, which is the
+//              faster of the two there):
 //              the skinny-M GEMM with a row of ones as the activations, out = 1^T * in.  A
 //              fused multiply-add by 1.0 is an exact addition, so this is a plain sum in the
 //              kernel's fixed order, streamed at the skinny route's rate.
@@ -162,8 +164,13 @@ int launch_cols(const float *in, int64_t outer, int64_t axis_len, int64_t inner,
     const int64_t groups = vec ? inner / 4 : inner;
     int tx_log2 = 0;
     while (tx_log2 < 8 && (int64_t(1) << tx_log2) < groups) tx_log2++;
-    const int64_t col_blocks = (groups + (int64_t(1) << tx_log2) - 1) >> tx_log2;
     const int64_t slice = (axis_len + splits - 1) / splits;
+    // Few workgroups over a long axis (the join of a split reduction is the usual case): narrower
+    // column blocks, so that more threads share the axis and the serial walk of each is short.
+    while (tx_log2 > 2 && ((groups + (int64_t(1) << tx_log2) - 1) >> tx_log2) * splits * outer < 256 &&
+           slice >= 4 * (256 >> (tx_log2 - 1)))
+        tx_log2--;
+    const int64_t col_blocks = (groups + (int64_t(1) << tx_log2) - 1) >> tx_log2;
     const int64_t blocks = col_blocks * splits * outer;
     if (blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "reduce: too many column blocks");
     if (vec)
@@ -180,9 +187,9 @@ int reduce_cols(const float *in, int64_t outer, int64_t axis_len, int64_t inner,
     // enough workgroups to stream from every CU: cut the axis when outer x column blocks is small
     const int64_t groups = (inner + 3) / 4, col_blocks = (groups + 255) / 256;
     int64_t splits = 1;
-    if (outer * col_blocks < 1024) {
-        splits = 1024 / (outer * col_blocks);
-        const int64_t most = axis_len / 64;
+    if (outer * col_blocks < 2048) {
+        splits = 2048 / (outer * col_blocks);
+        const int64_t most = axis_len / (axis_len >= 8192 ? 32 : 64);       // rows per slice, at least
         if (splits > most) splits = most;
         if (splits < 1) splits = 1;
     }
@@ -315,7 +322,7 @@ extern "C" int axhip_sum_axis(const float *in, int64_t outer, int64_t axis_len, 
     if (outer == 0 || inner == 0) return AXHIP_OK;
     if (axis_len == 0) return axhip_fill_f32(out, 0.0f, outer * inner);
     if (inner == 1) return reduce_rows<AXHIP_RED_SUM>(in, outer, axis_len, out);
-    if (outer > 4 || inner < 64) return reduce_cols<AXHIP_RED_SUM>(in, outer, axis_len, inner, out);
+    if (outer > 4 || inner < 2048) return reduce_cols<AXHIP_RED_SUM>(in, outer, axis_len, inner, out);
     float *ones = axhip::ones_vector((size_t)axis_len);
     if (!ones) return AXHIP_ERR_ALLOC;
     for (int64_t o = 0; o < outer; o++) {
