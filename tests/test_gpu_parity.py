@@ -1087,6 +1087,41 @@ def test_binary_and_reductions_beyond_2_31_elements(hip, oracle, N, M):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kind,M,N,K", [("f32", 66000, 33000, 8), ("f32", 65664, 32768, 64), ("i8", 65600, 32768, 128),
+                                        ("i8", 66001, 33000, 64)])
+def test_gemm_outputs_beyond_2_31_elements(hip, kind, M, N, K):
+    """A product with more than 2^31 output elements (8.6 GB of fp32): element offsets into C must be
+    64-bit in every kernel of the route (edge tiles, interior + fringes, the persistent int8 tiles).
+    Operands are small integers, so every product and every row or column sum of C is an exact fp32
+    integer whatever the order: row sums of C are A . rowsum(B), column sums are colsum(A) . B, and
+    rows at the start, around flat index 2^31 and at the end are read back."""
+    say("gemm beyond 2^31 outputs", kind, M, N, K)
+    assert M * N > 2 ** 31
+    rng = np.random.default_rng(M + N + K)
+    a = rng.integers(-2, 3, (M, K))
+    out = hip.empty((M, N))
+    if kind == "f32":
+        b = rng.integers(-2, 3, (K, N))
+        da, db = hip.array(a.astype(np.float32)), hip.array(b.astype(np.float32))
+        hip.check(hip.L.axhip_sgemm(0, 0, M, N, K, 1.0, da.ptr, K, db.ptr, N, 0.0, out.ptr, N, None, 0))
+    else:
+        w = rng.integers(-2, 3, (N, K))
+        b = w.T
+        da, dw = hip.array(a.astype(np.int8)), hip.array(w.astype(np.int8))
+        ones = hip.array(np.ones(N, np.float32))
+        hip.check(hip.L.axhip_qgemm_w8a8(da.ptr, 1.0, dw.ptr, ones.ptr, None, 0, out.ptr, None, M, N, K))
+    rows, cols = hip.empty((M,)), hip.empty((N,))
+    hip.check(hip.L.axhip_sum_axis(out.ptr, M, N, 1, rows.ptr))
+    assert np.array_equal(rows.numpy(), (a @ b.sum(axis=1)).astype(np.float32))
+    hip.check(hip.L.axhip_sum_axis(out.ptr, 1, M, N, cols.ptr))
+    assert np.array_equal(cols.numpy(), (a.sum(axis=0) @ b).astype(np.float32))
+    for r0 in (0, 2 ** 31 // N - 1, M - 3):
+        window = np.empty((3, N), np.float32)
+        hip.check(hip.L.axhip_memcpy_d2h(window.ctypes.data, out.ptr + r0 * N * 4, window.nbytes))
+        assert np.array_equal(window, (a[r0:r0 + 3] @ b).astype(np.float32)), r0
+
+
+@pytest.mark.gpu
 def test_allocation_pool(hip):
     """Freed blocks come back for the next request of their size class, zero-filled, with earlier
     work on them finished first (one stream); foreign pointers and double frees are ignored."""
