@@ -397,25 +397,27 @@ def cpu_baseline():
     import oracle_bind as ob
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     rng = np.random.default_rng(2)
-    M, N, K = 4096, 8192, 8192          # half of the headline's rows: ~10 s of CPU work
+    M, N, K = 8192, 8192, 8192          # the headline shape itself: ~4 s a run on 16 cores
     a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
     q = rand_i8(rng, (N, K))
     s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
     if ob.ref_available():
         lib, kind = ob.RefLib(), "reference"
-        run = lambda: lib.qgemm_w8a32(a, q, s)
     else:
         lib, kind = ob.Oracle(), "port"
-        run = lambda: lib.qgemm_w8a32(a, q, s)
-    t0 = time.perf_counter()
-    run()
-    dt = time.perf_counter() - t0
+    runs, spent = [], 0.0
+    while len(runs) < 3 and spent < 20.0:                # a bounded sample: three runs, 20 s at most
+        t0 = time.perf_counter()
+        lib.qgemm_w8a32(a, q, s)
+        runs.append(time.perf_counter() - t0)
+        spent += runs[-1]
+    dt = min(runs)
     tops = 2.0 * M * N * K / dt / 1e12
     result_line("cpu", f"q8a32_{M}x{N}x{K}", "gflops", tops * 1e3)
     return {"value": tops, "unit": "TOP/s", "cores": cores, "kind": kind,
             "sample": f"ax_qgemm_w8a32 (the reference's only quantized GEMM: int8 weights x fp32 "
-                      f"activations, fp32 accumulate; it has no W8A8) on M={M} of the headline's 8192 "
-                      f"rows, N=K=8192, one run of {dt:.1f} s"}
+                      f"activations, fp32 accumulate; it has no W8A8) on the headline shape M=N=K=8192, "
+                      f"best of {len(runs)} runs ({', '.join('%.1f' % r for r in runs)} s)"}
 
 
 def main():
