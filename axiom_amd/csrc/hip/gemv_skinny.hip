@@ -6,7 +6,9 @@
 // 256-byte row segments and eight of them are kept in flight per lane.  The M activations of
 // a k row are wave-uniform only per lane group, so they come from LDS (staged once per
 // workgroup); the first batch of weight loads is issued before that staging so HBM latency
-// overlaps it.  Lane groups are summed inside their wave, waves through LDS, in a fixed order.  When K is split over
+// overlaps it.  The 16 lane groups' sums are joined through LDS in a fixed order; from M = 9 on the
+// four lane groups of a wave are first added inside the wave (row swaps), which keeps the LDS
+// buffer at four partial tiles whatever M is.  When K is split over
 // several workgroups each writes its partial tile to a workspace and bumps a per-strip
 // counter; the workgroup that arrives last adds the partials in split order (not arrival
 // order) and applies bias and activation.  The sum order is fixed, so results are
@@ -20,7 +22,7 @@ constexpr int COLS = 64;        // columns per workgroup
 constexpr int KGROUPS = 16;     // lane groups per workgroup, each 16 lanes x float4
 constexpr int UNROLL = 8;
 // workgroups to aim for: enough to cover 256 CUs a few times over; partial-sum traffic grows with M
-constexpr int64_t kWantBlocksM12 = 1024, kWantBlocksM38 = 512;
+constexpr int64_t kWantBlocksM12 = 1024, kWantBlocksM3up = 512;      // M = 1, 2 / M >= 3
 
 template <int MR, bool VEC>
 __global__ void __launch_bounds__(256)
@@ -295,7 +297,7 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
 
     const int64_t col_blocks = (N + COLS - 1) / COLS;
     // enough workgroups to cover 256 CUs a few times over, each with at least 128 k rows
-    const int64_t want_blocks = M <= 2 ? kWantBlocksM12 : kWantBlocksM38;
+    const int64_t want_blocks = M <= 2 ? kWantBlocksM12 : kWantBlocksM3up;
     int64_t splits = (want_blocks + col_blocks - 1) / col_blocks;
     const int64_t max_splits = K >= 128 ? K / 128 : 1;
     if (splits > max_splits) splits = max_splits;
