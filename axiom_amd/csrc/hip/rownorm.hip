@@ -81,6 +81,15 @@ k_rows_cached(const float *__restrict__ in, float *__restrict__ out, int64_t row
         for (int i = 0; i < VPT; i++)
             if (t + i * TPR < cols) out[row * cols + t + i * TPR] = v[i] * inv;
     } else {
+        // scale and shift are requested now (L2 hits), so that they have arrived when the row's
+        // sums are joined rather than being waited for after the barrier
+        float gam[VPT], bet[VPT];
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int c = t + i * TPR;
+            gam[i] = c < cols ? ln.gamma[c] : 0.0f;
+            bet[i] = c < cols ? ln.beta[c] : 0.0f;
+        }
         float s = 0.0f, s2 = 0.0f;
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
@@ -98,7 +107,7 @@ k_rows_cached(const float *__restrict__ in, float *__restrict__ out, int64_t row
             const int c = t + i * TPR;
             if (c < cols) {
                 const float xh = (v[i] - mean) * inv_std;
-                out[row * cols + c] = __builtin_fmaf(ln.gamma[c], xh, ln.beta[c]);
+                out[row * cols + c] = __builtin_fmaf(gam[i], xh, bet[i]);
                 if (ln.x_hat) ln.x_hat[row * cols + c] = xh;
             }
         }
