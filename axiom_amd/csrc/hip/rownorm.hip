@@ -1,7 +1,7 @@
 // Row softmax (the .softmax_rowwise vtable slot; cpu_naive.c:235-270, cuda/ops_fused.cu:44-91)
 // and layer normalisation forward (src/core/norm.c:1278-1399) over contiguous [rows, cols] fp32.
 // HBM-bound.  A row of up to TPR*VPT columns is read once into registers (one wave per row up to
-// 1024 columns, one workgroup per row up to 4096), reduced, and written once; a row of up to 36864
+// 1024 columns, one workgroup per row up to 6144), reduced, and written once; a row of up to 36864
 // columns is held in LDS by a workgroup of 1024 threads; longer rows are read twice.
 #include <float.h>
 
@@ -323,6 +323,9 @@ int launch_rows(const float *in, float *out, int64_t rows, int64_t cols, const L
         if (rows > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "%s: too many rows", what);
         if (cols <= 4096) {
             hipLaunchKernelGGL((k_rows_cached<256, 16, KIND>), dim3((unsigned)rows), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
+        } else if (cols <= 6144) {
+            // still in registers (24 values a thread): faster than the LDS form up to here, slower from about 8192
+            hipLaunchKernelGGL((k_rows_cached<256, 24, KIND>), dim3((unsigned)rows), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
         } else if (cols <= 36864) {
             static bool attr_set = false;
             if (!attr_set) {
