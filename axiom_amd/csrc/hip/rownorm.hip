@@ -1,6 +1,7 @@
 // Row softmax (the .softmax_rowwise vtable slot; cpu_naive.c:235-270, cuda/ops_fused.cu:44-91)
 // and layer normalisation forward (src/core/norm.c:1278-1399) over contiguous [rows, cols] fp32.
-// HBM-bound.  A row of up to TPR*VPT columns is read once into registers (one wave per row up to
+// HBM-bound.  A row of up to TPR*VPT columns is read once into registers (several rows per wave up
+// to 128 columns, one wave per row up to
 // 1024 columns, one workgroup per row up to 6144), reduced, and written once; a row of up to 36864
 // columns is held in LDS by a workgroup of 1024 threads; longer rows are read twice.
 #include <float.h>
@@ -308,13 +309,87 @@ k_rows_streamed(const float *__restrict__ in, float *__restrict__ out, int64_t c
     }
 }
 
+// Short rows (up to 64 * VPT <= 128 columns): a wave per row has too few bytes in flight to cover
+// HBM latency, so a wave takes RPW consecutive rows and requests all of them before it reduces any.
+template <int VPT, int RPW, int KIND>
+__global__ void __launch_bounds__(256)
+k_rows_short(const float *__restrict__ in, float *__restrict__ out, int64_t rows, int cols, LnArgs ln) {
+    const int t = threadIdx.x & 63;
+    const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW;
+    if (row0 >= rows) return;
+    float v[RPW][VPT];
+#pragma unroll
+    for (int r = 0; r < RPW; r++)
+#pragma unroll
+        for (int i = 0; i < VPT; i++)
+            v[r][i] = (row0 + r < rows && t + i * 64 < cols) ? in[(row0 + r) * cols + t + i * 64]
+                                                             : (KIND == 0 ? -FLT_MAX : 0.0f);
+    float gam[VPT], bet[VPT];
+    if (KIND == 1) {
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int c = t + i * 64;
+            gam[i] = c < cols ? ln.gamma[c] : 0.0f;
+            bet[i] = c < cols ? ln.beta[c] : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; r++) {
+        const int64_t row = row0 + r;
+        if (row >= rows) break;
+        if (KIND == 0) {
+            float mx = -FLT_MAX;
+#pragma unroll
+            for (int i = 0; i < VPT; i++) mx = fmaxf(mx, v[r][i]);
+            mx = row_join<64, true>(mx, nullptr, 0);
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < VPT; i++) {
+                v[r][i] = (t + i * 64 < cols) ? expf(v[r][i] - mx) : 0.0f;
+                sum += v[r][i];
+            }
+            sum = row_join<64, false>(sum, nullptr, 0);
+            const float inv = 1.0f / sum;
+#pragma unroll
+            for (int i = 0; i < VPT; i++)
+                if (t + i * 64 < cols) out[row * cols + t + i * 64] = v[r][i] * inv;
+        } else {
+            float s = 0.0f, s2 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < VPT; i++) {
+                s += v[r][i];
+                s2 = __builtin_fmaf(v[r][i], v[r][i], s2);
+            }
+            row_join2<64>(s, s2, nullptr, 0);
+            const float mean = s / (float)cols;
+            float var = s2 / (float)cols - mean * mean;
+            if (var < 0.0f) var = 0.0f;
+            const float inv_std = 1.0f / sqrtf(var + ln.eps);
+            if (ln.inv_std && t == 0) ln.inv_std[row] = inv_std;
+#pragma unroll
+            for (int i = 0; i < VPT; i++) {
+                const int c = t + i * 64;
+                if (c < cols) {
+                    const float xh = (v[r][i] - mean) * inv_std;
+                    out[row * cols + c] = __builtin_fmaf(gam[i], xh, bet[i]);
+                    if (ln.x_hat) ln.x_hat[row * cols + c] = xh;
+                }
+            }
+        }
+    }
+}
+
 template <int KIND>
 int launch_rows(const float *in, float *out, int64_t rows, int64_t cols, const LnArgs &ln, const char *what) {
     if (cols <= 1024) {
         const int64_t blocks = (rows + 3) / 4;
         if (blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "%s: too many rows", what);
-        if (cols <= 128)
-            hipLaunchKernelGGL((k_rows_cached<64, 2, KIND>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
+        if (cols <= 64)
+            hipLaunchKernelGGL((k_rows_short<1, 8, KIND>), dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
+        else if (cols <= 128)
+            hipLaunchKernelGGL((k_rows_short<2, 4, KIND>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
+        else if (cols <= 256)
+            hipLaunchKernelGGL((k_rows_cached<64, 4, KIND>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
         else if (cols <= 512)
             hipLaunchKernelGGL((k_rows_cached<64, 8, KIND>), dim3((unsigned)blocks), dim3(256), 0, kStream, in, out, rows, (int)cols, ln);
         else

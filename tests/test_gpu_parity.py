@@ -949,7 +949,8 @@ def test_softmax_rows(hip, oracle, golden):
     # beyond: two reads with the running-maximum form
     for (rows, cols) in [(1, 1), (7, 129), (1000, 512), (33, 513), (64, 1024), (5, 4096), (3, 4097), (2, 100000),
                          (8192, 512), (4097, 64), (5, 10001), (3, 36864), (3, 36865), (7, 50257), (2, 131075),
-                         (300, 4100), (1, 36863), (9, 6144), (9, 6145), (17, 6143)]:
+                         (300, 4100), (1, 36863), (9, 6144), (9, 6145), (17, 6143), (1003, 128), (33, 65), (35, 64),
+                         (29, 33), (2, 256), (70, 200)]:
         oracle.seed(rows + cols)
         x = oracle.uniform((rows, cols), -8, 8)
         got = run_softmax(hip, x)
@@ -983,7 +984,8 @@ def test_layernorm_forward(hip, oracle, golden):
         assert np.abs(out - o_out).max() < 5e-6 and np.abs(xh - o_xh).max() < 5e-6
         assert np.allclose(inv, o_inv, rtol=2e-6)
     for shp in [(4096, 1024), (2048, 768), (100, 4096), (3, 5000), (9, 1), (4097, 96), (5, 10001), (2, 36864),
-                (3, 36867), (3, 50257), (130, 4099), (9, 6144), (9, 6145), (17, 6141)]:
+                (3, 36867), (3, 50257), (130, 4099), (9, 6144), (9, 6145), (17, 6141), (1003, 128), (33, 65),
+                (35, 64), (29, 33), (70, 200)]:
         oracle.seed(sum(shp))
         x, gamma, beta = oracle.uniform(shp, -3, 5), oracle.uniform((shp[-1],), 0.5, 1.5), oracle.uniform((shp[-1],), -1, 1)
         out, xh, inv = run_layernorm(hip, x, gamma, beta, 1e-5)
