@@ -1,9 +1,9 @@
 // Row softmax (the .softmax_rowwise vtable slot; cpu_naive.c:235-270, cuda/ops_fused.cu:44-91)
 // and layer normalisation forward (src/core/norm.c:1278-1399) over contiguous [rows, cols] fp32.
 // HBM-bound.  A row of up to TPR*VPT columns is read once into registers (several rows per wave up
-// to 128 columns, one wave per row up to
-// 1024 columns, one workgroup per row up to 6144), reduced, and written once; a row of up to 36864
-// columns is held in LDS by a workgroup of 1024 threads; longer rows are read twice.
+// to 128 columns, one wave per row up to 1024, one workgroup per row up to 6144), reduced, and
+// written once; a row of up to 36864 columns is held in LDS by a workgroup of 1024 threads; longer
+// rows are read twice.
 #include <float.h>
 
 #include "common.h"

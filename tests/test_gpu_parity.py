@@ -559,7 +559,8 @@ SUM_BOUND = 1e-5     # |gpu - sum64| <= SUM_BOUND * sum |x|   (fp32 sums in a fi
 @pytest.mark.parametrize("shape,axis", [((37, 19), 0), ((37, 19), 1), ((4, 9, 10), 0), ((4, 9, 10), 1),
                                         ((4, 9, 10), 2), ((2048, 4096), 0), ((2048, 4096), 1),
                                         ((1000, 7), 0), ((3, 100003), 1), ((1, 64), 0), ((5000, 64), 0),
-                                        ((16384, 772), 0), ((20000, 1000), 0), ((3000, 2044), 0), ((3000, 2052), 0)])
+                                        ((16384, 772), 0), ((20000, 1000), 0), ((3000, 2044), 0), ((3000, 2052), 0),
+                                        ((100003, 10), 1), ((70001, 33), 1), ((50001, 127), 1), ((1001, 3), 1)])
 def test_sum_axis(hip, oracle, golden, shape, axis):
     say("sum", shape, axis)
     oracle.seed(4343 if shape in ((37, 19), (4, 9, 10)) else sum(shape) + axis)
@@ -904,7 +905,9 @@ def test_reductions_golden(hip, oracle, golden):
 @pytest.mark.parametrize("shape,axis", [((4096, 4096), 0), ((4096, 4096), 1), ((3, 100000, 5), 1), ((64, 7, 64), 1),
                                         ((2, 3000001), 1), ((1 << 22,), 0), ((5, 4, 3, 130), 2), ((33, 1000), 0),
                                         ((1000, 33), 1), ((100000, 8), 0), ((17, 1), 0), ((20000, 1000), 0), ((16384, 772), 0),
-                                        ((2048, 1024), 0), ((3, 9000, 36), 1), ((9001, 2050), 0)])
+                                        ((2048, 1024), 0), ((3, 9000, 36), 1), ((9001, 2050), 0),
+                                        ((100003, 10), 1), ((70001, 32), 1), ((70001, 33), 1), ((50001, 128), 1),
+                                        ((50001, 129), 1), ((1001, 3), 1), ((65, 17), 1)])
 def test_reductions_shapes(hip, oracle, shape, axis):
     say("reduce", shape, axis)
     oracle.seed(sum(shape) + axis)
