@@ -243,18 +243,20 @@ k_argmax(const float *__restrict__ in, int64_t outer, int64_t axis_len, int64_t 
     }
 }
 
-// one wave per row, for rows along the contiguous axis
+// LPR lanes per row (a wave; 16 or 4 lanes for short rows, as in the row reductions), for rows
+// along the contiguous axis
+template <int LPR>
 __global__ void __launch_bounds__(256)
 k_argmax_rows(const float *__restrict__ in, int64_t rows, int64_t len, int64_t *__restrict__ out) {
-    const int lane = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & (LPR - 1);
+    const int64_t r = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
     if (r >= rows) return;
     const float *p = in + r * len;
     // lanes scan interleaved positions in ascending order, so each keeps its first maximum;
     // a lane without elements, or with NaNs only ahead of row element 0's rule, defers below
     float bestv = p[0];
     int64_t best = 0;
-    for (int64_t c = lane; c < len; c += 64) {
+    for (int64_t c = lane; c < len; c += LPR) {
         const float v = p[c];
         if (v > bestv || (v == bestv && c < best)) {
             bestv = v;
@@ -262,7 +264,7 @@ k_argmax_rows(const float *__restrict__ in, int64_t rows, int64_t len, int64_t *
         }
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
+    for (int off = LPR / 2; off > 0; off >>= 1) {          // lane 0 of a row only ever takes in its own lanes
         const float ov = __shfl_down(bestv, off, 64);
         const int64_t oi = __shfl_down(best, off, 64);
         if (ov > bestv || (ov == bestv && oi < best)) {
@@ -313,10 +315,16 @@ extern "C" int axhip_argmax_axis(const float *in, int64_t outer, int64_t axis_le
     if (!in || !out) return fail(AXHIP_ERR_NULL_ARG, "argmax: NULL");
     if (outer < 0 || axis_len <= 0 || inner < 0) return fail(AXHIP_ERR_SHAPE, "argmax: bad extent");
     if (outer == 0 || inner == 0) return AXHIP_OK;
-    if (inner == 1 && axis_len >= 64) {
-        const int64_t blocks = (outer + 3) / 4;
+    if (inner == 1 && axis_len >= 8) {      // shorter rows: a thread per row, below
+        const int lpr = axis_len > 128 ? 64 : axis_len > 32 ? 16 : 4;      // 2 Mi rows of 32: 1062 us a thread per row, 90 us so
+        const int64_t per_block = 256 / lpr, blocks = (outer + per_block - 1) / per_block;
         if (blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "argmax: too many rows");
-        hipLaunchKernelGGL(k_argmax_rows, dim3((unsigned)blocks), dim3(256), 0, kStream, in, outer, axis_len, out);
+        if (lpr == 64)
+            hipLaunchKernelGGL(k_argmax_rows<64>, dim3((unsigned)blocks), dim3(256), 0, kStream, in, outer, axis_len, out);
+        else if (lpr == 16)
+            hipLaunchKernelGGL(k_argmax_rows<16>, dim3((unsigned)blocks), dim3(256), 0, kStream, in, outer, axis_len, out);
+        else
+            hipLaunchKernelGGL(k_argmax_rows<4>, dim3((unsigned)blocks), dim3(256), 0, kStream, in, outer, axis_len, out);
         return check_launch("argmax_rows");
     }
     int64_t blocks = (outer * inner + 255) / 256;

@@ -907,7 +907,7 @@ def test_reductions_golden(hip, oracle, golden):
                                         ((1000, 33), 1), ((100000, 8), 0), ((17, 1), 0), ((20000, 1000), 0), ((16384, 772), 0),
                                         ((2048, 1024), 0), ((3, 9000, 36), 1), ((9001, 2050), 0),
                                         ((100003, 10), 1), ((70001, 32), 1), ((70001, 33), 1), ((50001, 128), 1),
-                                        ((50001, 129), 1), ((1001, 3), 1), ((65, 17), 1)])
+                                        ((50001, 129), 1), ((1001, 3), 1), ((65, 17), 1), ((3001, 8), 1), ((3001, 7), 1)])
 def test_reductions_shapes(hip, oracle, shape, axis):
     say("reduce", shape, axis)
     oracle.seed(sum(shape) + axis)
