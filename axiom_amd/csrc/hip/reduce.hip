@@ -243,6 +243,77 @@ k_argmax(const float *__restrict__ in, int64_t outer, int64_t axis_len, int64_t 
     }
 }
 
+// Argmax down columns (inner > 1) of a long axis, in two steps like the column reductions: a
+// workgroup of TX columns by TY axis positions walks one slice of the axis and leaves, per column,
+// the first index of the slice's maximum among its non-NaN values (-1: none); the finishing pass
+// takes the slices in ascending order.  The rule reproduced is the scan that starts from element 0
+// and replaces on strictly greater: NaNs are passed over, except that a NaN in element 0 is never
+// replaced and the answer is then 0.
+__global__ void __launch_bounds__(256)
+k_argmax_cols_part(const float *__restrict__ in, int64_t axis_len, int64_t inner, int tx_log2, int64_t col_blocks,
+                   int64_t splits, int64_t slice, float *__restrict__ part_v, int64_t *__restrict__ part_i) {
+    __shared__ float jv[256];
+    __shared__ int64_t ji[256];
+    const int tx = threadIdx.x & ((1 << tx_log2) - 1), ty = threadIdx.x >> tx_log2, TY = 256 >> tx_log2;
+    int64_t b = blockIdx.x;
+    const int64_t cb = b % col_blocks;
+    b /= col_blocks;
+    const int64_t s = b % splits, o = b / splits;
+    const int64_t col = (cb << tx_log2) + tx;
+    int64_t a1 = (s + 1) * slice;
+    if (a1 > axis_len) a1 = axis_len;
+    float bestv = 0.0f;
+    int64_t best = -1;
+    if (col < inner) {
+        const float *base = in + o * axis_len * inner + col;
+#pragma unroll 8
+        for (int64_t a = s * slice + ty; a < a1; a += TY) {
+            const float v = base[a * inner];
+            if (best < 0 ? v == v : v > bestv) {
+                bestv = v;
+                best = a;
+            }
+        }
+    }
+    jv[threadIdx.x] = bestv;
+    ji[threadIdx.x] = best;
+    __syncthreads();
+    if (ty == 0 && col < inner) {
+        for (int y = 1; y < TY; y++) {
+            const float ov = jv[(y << tx_log2) + tx];
+            const int64_t oi = ji[(y << tx_log2) + tx];
+            if (oi >= 0 && (best < 0 || ov > bestv || (ov == bestv && oi < best))) {
+                bestv = ov;
+                best = oi;
+            }
+        }
+        const int64_t at = (o * splits + s) * inner + col;
+        part_v[at] = bestv;
+        part_i[at] = best;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+k_argmax_cols_finish(const float *__restrict__ in, const float *__restrict__ part_v, const int64_t *__restrict__ part_i,
+                     int64_t outer, int64_t axis_len, int64_t inner, int64_t splits, int64_t *__restrict__ out) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= outer * inner) return;
+    const int64_t o = t / inner, i = t - o * inner;
+    const float first = in[o * axis_len * inner + i];
+    float bestv = 0.0f;
+    int64_t best = -1;
+#pragma unroll 4
+    for (int64_t s = 0; s < splits; s++) {
+        const int64_t at = (o * splits + s) * inner + i, oi = part_i[at];
+        const float ov = part_v[at];
+        if (oi >= 0 && (best < 0 || ov > bestv)) {
+            bestv = ov;
+            best = oi;
+        }
+    }
+    out[t] = (first != first || best < 0) ? 0 : best;
+}
+
 // LPR lanes per row (a wave; 16 or 4 lanes for short rows, as in the row reductions), for rows
 // along the contiguous axis
 template <int LPR>
@@ -326,6 +397,26 @@ extern "C" int axhip_argmax_axis(const float *in, int64_t outer, int64_t axis_le
         else
             hipLaunchKernelGGL(k_argmax_rows<4>, dim3((unsigned)blocks), dim3(256), 0, kStream, in, outer, axis_len, out);
         return check_launch("argmax_rows");
+    }
+    if (inner > 1 && axis_len >= 64) {      // a long axis: slices of it in parallel, then a join
+        int tx_log2 = 2;
+        while (tx_log2 < 6 && (int64_t(1) << tx_log2) < inner) tx_log2++;      // at least 4 axis positions a workgroup: fewer slices to join
+        const int64_t col_blocks = (inner + (int64_t(1) << tx_log2) - 1) >> tx_log2;
+        int64_t splits = 2048 / (outer * col_blocks);
+        if (splits > axis_len / 64) splits = axis_len / 64;
+        if (splits < 1) splits = 1;
+        const int64_t slice = (axis_len + splits - 1) / splits, cells = outer * splits * inner;
+        const int64_t part_blocks = col_blocks * splits * outer, out_blocks = (outer * inner + 255) / 256;
+        if (part_blocks > 0x7fffffff || out_blocks > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "argmax: too many columns");
+        char *ws = static_cast<char *>(axhip::workspace((size_t)cells * 12));
+        if (!ws) return AXHIP_ERR_ALLOC;
+        int64_t *part_i = reinterpret_cast<int64_t *>(ws);
+        float *part_v = reinterpret_cast<float *>(ws + (size_t)cells * 8);
+        hipLaunchKernelGGL(k_argmax_cols_part, dim3((unsigned)part_blocks), dim3(256), 0, kStream, in, axis_len, inner,
+                           tx_log2, col_blocks, splits, slice, part_v, part_i);
+        hipLaunchKernelGGL(k_argmax_cols_finish, dim3((unsigned)out_blocks), dim3(256), 0, kStream, in, part_v, part_i,
+                           outer, axis_len, inner, splits, out);
+        return check_launch("argmax_cols");
     }
     int64_t blocks = (outer * inner + 255) / 256;
     if (blocks > 16384) blocks = 16384;

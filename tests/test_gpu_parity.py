@@ -937,6 +937,31 @@ def test_reduce_starting_values(hip):
     assert np.array_equal(run_reduce(hip, "min", -x, 1), np.array([np.finfo(np.float32).max, -2.0], np.float32))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,cols", [(1000, 37), (70, 300), (4099, 5), (63, 9)])
+def test_argmax_down_columns_scan_rule(hip, oracle, rows, cols):
+    """The reference's argmax scans from element 0 and replaces on strictly greater (opt_argmax,
+    cpu_opt.c:7202-7249): NaNs are passed over, a NaN in element 0 is never replaced (answer 0),
+    ties keep the first index.  Long axes are cut into slices on the GPU; the rule must survive."""
+    say("argmax scan rule", rows, cols)
+    oracle.seed(rows + cols)
+    x = oracle.uniform((rows, cols), -1, 1)
+    x[::7] = 0.5                                               # ties across slices
+    x[0, 1] = np.nan                                           # NaN first: stays
+    x[5:rows // 2, 2] = np.nan                                 # NaNs inside: skipped
+    x[:, 3] = np.nan
+    x[:, 4] = -np.inf
+    x[rows - 1, 0] = 2.0                                       # maximum in the last slice
+    want = np.zeros(cols, np.int64)
+    for c in range(cols):
+        bestv, best = x[0, c], 0
+        for a in range(1, rows):
+            if x[a, c] > bestv:
+                bestv, best = x[a, c], a
+        want[c] = best
+    assert np.array_equal(run_argmax(hip, x, 0), want)
+
+
 def run_softmax(hip, x):
     dx, out = hip.array(x), hip.empty(x.shape)
     hip.check(hip.L.axhip_softmax_rows(dx.ptr, out.ptr, x.shape[0], x.shape[1]))
