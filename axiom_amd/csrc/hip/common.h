@@ -29,6 +29,9 @@ size_t pool_class(size_t bytes);
 void pool_release_all();
 // At least `n` device floats, all 1.0f, owned by the runtime (grown on demand).
 float *ones_vector(size_t n);
+// Per-device set-up of the skinny-M kernels (LDS limits, address of the static scratch); the device
+// must be current.  Called by axhip_init.
+int skinny_setup();
 
 constexpr hipStream_t kStream = nullptr;
 

@@ -281,80 +281,73 @@ int launch_m(bool vec, dim3 grid, size_t smem, const float *A, int64_t lda, cons
     return check_launch("sgemm_skinny");
 }
 
-}  // namespace
 
-extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
-                                  const float *B, int64_t ldb, float *C, int64_t ldc,
-                                  const float *bias, int act) {
-    if (int rc = axhip::ensure_ready()) return rc;
-    if (!A || !B || !C) return fail(AXHIP_ERR_NULL_ARG, "sgemm_skinny: NULL matrix");
-    if (M < 1 || M > 16) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: M=%lld outside 1..16", (long long)M);
-    if (N < 0 || K < 0 || lda < K || ldb < N || ldc < N)
-        return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: bad dimension or leading dimension");
-    if (act < AXHIP_ACT_NONE || act > AXHIP_ACT_GELU)
-        return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: unknown activation %d", act);
-    if (N == 0) return AXHIP_OK;
+// What one call launches: grid, split length, LDS bytes and the size of the partial-sum area.
+struct SkinnyPlan {
+    int64_t col_blocks, splits, kps, red_floats;
+    bool vec;
+    size_t smem, partial_bytes;
+};
 
-    const int64_t col_blocks = (N + COLS - 1) / COLS;
+int plan_skinny(int64_t M, int64_t N, int64_t K, const float *B, int64_t ldb, SkinnyPlan &p) {
+    p.col_blocks = (N + COLS - 1) / COLS;
     // enough workgroups to cover 256 CUs a few times over, each with at least 128 k rows
     const int64_t want_blocks = M <= 2 ? kWantBlocksM12 : kWantBlocksM3up;
-    int64_t splits = (want_blocks + col_blocks - 1) / col_blocks;
+    int64_t splits = (want_blocks + p.col_blocks - 1) / p.col_blocks;
     const int64_t max_splits = K >= 128 ? K / 128 : 1;
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
     int64_t kps = (K + splits - 1) / splits;
     kps = (kps + KGROUPS - 1) / KGROUPS * KGROUPS;
     // the activations of one split must fit LDS next to the reduction buffer
-    const int64_t red_floats = (int64_t)(M > 8 ? 4 : KGROUPS) * M * COLS;   // partials per workgroup, as in the kernel
+    p.red_floats = (int64_t)(M > 8 ? 4 : KGROUPS) * M * COLS;   // partials per workgroup, as in the kernel
     // ... within 52 KiB, so that three workgroups share a CU whatever M is (4096 x 11008 at M = 16: 95 us
     // with one 96 KiB workgroup per CU, 60 us this way)
-    const int64_t max_kps = ((int64_t)(52 * 1024 / 4) - red_floats) / M / KGROUPS * KGROUPS;
+    const int64_t max_kps = ((int64_t)(52 * 1024 / 4) - p.red_floats) / M / KGROUPS * KGROUPS;
     if (kps > max_kps) kps = max_kps;
     if (kps > 512) kps = 512;      // at most 128 KiB of weights per workgroup: wide matrices get more workgroups, not longer ones
     if (kps < KGROUPS) kps = KGROUPS;
     splits = K > 0 ? (K + kps - 1) / kps : 1;
     if (splits > 65535) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: K=%lld too large", (long long)K);
+    p.splits = splits;
+    p.kps = kps;
+    p.vec = (N % 4 == 0) && (ldb % 4 == 0) && ((uintptr_t)B % 16 == 0);
+    p.smem = (size_t)(M * kps + p.red_floats) * sizeof(float);
+    p.partial_bytes = splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+    return AXHIP_OK;
+}
 
-    const bool vec = (N % 4 == 0) && (ldb % 4 == 0) && ((uintptr_t)B % 16 == 0);
-    const size_t smem = (size_t)(M * kps + red_floats) * sizeof(float);
+int check_skinny_args(const char *who, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                      const float *B, int64_t ldb, const float *C, int64_t ldc, int act) {
+    if (!A || !B || !C) return fail(AXHIP_ERR_NULL_ARG, "%s: NULL matrix", who);
+    if (M < 1 || M > 16) return fail(AXHIP_ERR_SHAPE, "%s: M=%lld outside 1..16", who, (long long)M);
+    if (N < 0 || K < 0 || lda < K || ldb < N || ldc < N)
+        return fail(AXHIP_ERR_SHAPE, "%s: bad dimension or leading dimension", who);
+    if (act < AXHIP_ACT_NONE || act > AXHIP_ACT_GELU)
+        return fail(AXHIP_ERR_SHAPE, "%s: unknown activation %d", who, act);
+    return AXHIP_OK;
+}
+
+// `partials` holds plan.partial_bytes, `counters` plan.col_blocks ints that are zero (both unused when
+// the plan has one split); the kernel leaves the counters at zero.
+int run_skinny(const SkinnyPlan &p, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+               const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int act,
+               float *partials, int *counters) {
     float *dst = C;
     int64_t dst_ld = ldc, dst_split = 0;
-    int *counters = nullptr;
-    if (splits > 1) {
-        dst = static_cast<float *>(axhip::workspace((size_t)splits * M * N * sizeof(float)));
-        counters = axhip::strip_counters((size_t)col_blocks);
-        if (!dst || !counters) return AXHIP_ERR_ALLOC;
+    if (p.splits > 1) {
+        dst = partials;
         dst_ld = N;
         dst_split = M * N;
     }
-    static bool attr_set = false;
-    if (!attr_set) {
-        const void *ks[] = {
-            (const void *)k_skinny<1, true>, (const void *)k_skinny<2, true>, (const void *)k_skinny<3, true>,
-            (const void *)k_skinny<4, true>, (const void *)k_skinny<5, true>, (const void *)k_skinny<6, true>,
-            (const void *)k_skinny<7, true>, (const void *)k_skinny<8, true>,
-            (const void *)k_skinny<1, false>, (const void *)k_skinny<2, false>, (const void *)k_skinny<3, false>,
-            (const void *)k_skinny<4, false>, (const void *)k_skinny<5, false>, (const void *)k_skinny<6, false>,
-            (const void *)k_skinny<7, false>, (const void *)k_skinny<8, false>,
-            (const void *)k_skinny<9, true>, (const void *)k_skinny<10, true>, (const void *)k_skinny<11, true>,
-            (const void *)k_skinny<12, true>, (const void *)k_skinny<13, true>, (const void *)k_skinny<14, true>,
-            (const void *)k_skinny<15, true>, (const void *)k_skinny<16, true>,
-            (const void *)k_skinny<9, false>, (const void *)k_skinny<10, false>, (const void *)k_skinny<11, false>,
-            (const void *)k_skinny<12, false>, (const void *)k_skinny<13, false>, (const void *)k_skinny<14, false>,
-            (const void *)k_skinny<15, false>, (const void *)k_skinny<16, false>};
-        for (const void *k : ks)
-            AXHIP_HIP_TRY(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024),
-                          "hipFuncSetAttribute");
-        attr_set = true;
-    }
-    dim3 grid((unsigned)col_blocks, (unsigned)splits);
-    note_kernel(vec ? "sgemm_skinny_vec4" : "sgemm_skinny_scalar");
+    dim3 grid((unsigned)p.col_blocks, (unsigned)p.splits);
+    note_kernel(p.vec ? "sgemm_skinny_vec4" : "sgemm_skinny_scalar");
     int rc;
     switch (M) {
-#define AX_CASE(m)                                                                            \
-    case m:                                                                                   \
-        rc = launch_m<m>(vec, grid, smem, A, lda, B, ldb, dst, dst_ld, dst_split, N, K, kps,  \
-                         bias, act, (int)splits, C, ldc, counters);                           \
+#define AX_CASE(m)                                                                                  \
+    case m:                                                                                         \
+        rc = launch_m<m>(p.vec, grid, p.smem, A, lda, B, ldb, dst, dst_ld, dst_split, N, K, p.kps,  \
+                         bias, act, (int)p.splits, C, ldc, counters);                               \
         break;
         AX_CASE(1) AX_CASE(2) AX_CASE(3) AX_CASE(4) AX_CASE(5) AX_CASE(6) AX_CASE(7) AX_CASE(8)
         AX_CASE(9) AX_CASE(10) AX_CASE(11) AX_CASE(12) AX_CASE(13) AX_CASE(14) AX_CASE(15) AX_CASE(16)
@@ -362,4 +355,90 @@ extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *
         default: rc = AXHIP_ERR_SHAPE;
     }
     return rc;
+}
+
+// Scratch of axhip_sgemm_skinny_static: split-K partial tiles, then the per-strip arrival counters.
+// Every GPU that loads this library holds its own copy until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; the device address is looked up once per
+// device in skinny_setup() and kept in g_scratch_dev.
+constexpr size_t kScratchPartialBytes = size_t(8) << 20;
+constexpr size_t kScratchCounters = 4096;
+static __device__ __align__(256) unsigned char scratch[kScratchPartialBytes + kScratchCounters * sizeof(int)];
+constexpr int kMaxDevices = 16;
+unsigned char *g_scratch_dev[kMaxDevices] = {};
+
+}  // namespace
+
+namespace axhip {
+// Once per device, with that device current (called from axhip_init): raises the kernels' dynamic LDS
+// limit and looks up where this device keeps the static scratch array.
+int skinny_setup() {
+    int dev = 0;
+    AXHIP_HIP_TRY(hipGetDevice(&dev), "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(AXHIP_ERR_BACKEND, "device index %d not supported", dev);
+    const void *ks[] = {
+        (const void *)k_skinny<1, true>, (const void *)k_skinny<2, true>, (const void *)k_skinny<3, true>,
+        (const void *)k_skinny<4, true>, (const void *)k_skinny<5, true>, (const void *)k_skinny<6, true>,
+        (const void *)k_skinny<7, true>, (const void *)k_skinny<8, true>,
+        (const void *)k_skinny<1, false>, (const void *)k_skinny<2, false>, (const void *)k_skinny<3, false>,
+        (const void *)k_skinny<4, false>, (const void *)k_skinny<5, false>, (const void *)k_skinny<6, false>,
+        (const void *)k_skinny<7, false>, (const void *)k_skinny<8, false>,
+        (const void *)k_skinny<9, true>, (const void *)k_skinny<10, true>, (const void *)k_skinny<11, true>,
+        (const void *)k_skinny<12, true>, (const void *)k_skinny<13, true>, (const void *)k_skinny<14, true>,
+        (const void *)k_skinny<15, true>, (const void *)k_skinny<16, true>,
+        (const void *)k_skinny<9, false>, (const void *)k_skinny<10, false>, (const void *)k_skinny<11, false>,
+        (const void *)k_skinny<12, false>, (const void *)k_skinny<13, false>, (const void *)k_skinny<14, false>,
+        (const void *)k_skinny<15, false>, (const void *)k_skinny<16, false>};
+    for (const void *k : ks)
+        AXHIP_HIP_TRY(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024),
+                      "hipFuncSetAttribute");
+    void *ptr = nullptr;
+    AXHIP_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+    if (!ptr) return fail(AXHIP_ERR_BACKEND, "static scratch has no device address");
+    g_scratch_dev[dev] = static_cast<unsigned char *>(ptr);
+    return AXHIP_OK;
+}
+}  // namespace axhip
+
+extern "C" int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                                  const float *B, int64_t ldb, float *C, int64_t ldc,
+                                  const float *bias, int act) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (int rc = check_skinny_args("sgemm_skinny", M, N, K, A, lda, B, ldb, C, ldc, act)) return rc;
+    if (N == 0) return AXHIP_OK;
+    SkinnyPlan p;
+    if (int rc = plan_skinny(M, N, K, B, ldb, p)) return rc;
+    float *partials = nullptr;
+    int *counters = nullptr;
+    if (p.splits > 1) {
+        partials = static_cast<float *>(axhip::workspace(p.partial_bytes));
+        counters = axhip::strip_counters((size_t)p.col_blocks);
+        if (!partials || !counters) return AXHIP_ERR_ALLOC;
+    }
+    return run_skinny(p, M, N, K, A, lda, B, ldb, C, ldc, bias, act, partials, counters);
+}
+
+extern "C" int axhip_sgemm_skinny_static(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                                         const float *B, int64_t ldb, float *C, int64_t ldc,
+                                         const float *bias, int act) {
+    if (int rc = axhip::ensure_ready()) return rc;      // no-op after axhip_init
+    if (int rc = check_skinny_args("sgemm_skinny_static", M, N, K, A, lda, B, ldb, C, ldc, act)) return rc;
+    if (N == 0) return AXHIP_OK;
+    SkinnyPlan p;
+    if (int rc = plan_skinny(M, N, K, B, ldb, p)) return rc;
+    int dev = 0;
+    AXHIP_HIP_TRY(hipGetDevice(&dev), "hipGetDevice");
+    unsigned char *base = (dev >= 0 && dev < kMaxDevices) ? g_scratch_dev[dev] : nullptr;
+    if (!base) return fail(AXHIP_ERR_BACKEND, "sgemm_skinny_static: axhip_init has not run on device %d", dev);
+    if (p.partial_bytes > kScratchPartialBytes || (size_t)p.col_blocks > kScratchCounters)
+        return fail(AXHIP_ERR_SHAPE,
+                    "sgemm_skinny_static: M=%lld N=%lld K=%lld needs %zu bytes of partial sums and %lld counters; "
+                    "the static scratch holds %zu bytes and %zu counters (use axhip_sgemm_skinny)",
+                    (long long)M, (long long)N, (long long)K, p.partial_bytes, (long long)p.col_blocks,
+                    kScratchPartialBytes, kScratchCounters);
+    // Partials are fully written before they are read.  The counters start at zero when the code object
+    // is loaded and every launch's last-arriving workgroups put theirs back to zero, so nothing needs
+    // clearing between calls that run one after another.
+    return run_skinny(p, M, N, K, A, lda, B, ldb, C, ldc, bias, act, reinterpret_cast<float *>(base),
+                      reinterpret_cast<int *>(base + kScratchPartialBytes));
 }

@@ -176,6 +176,7 @@ int axhip_init(void) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(AXHIP_ERR_BACKEND, "device 0 is %s; this library holds gfx950 code only",
                     prop.gcnArchName);
+    if (int rc = axhip::skinny_setup()) return rc;
     g_ready = 1;
     return AXHIP_OK;
 }

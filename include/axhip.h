@@ -100,6 +100,19 @@ int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *A, int64_t 
                        const float *B, int64_t ldb, float *C, int64_t ldc,
                        const float *bias, int act);
 
+/* The same route for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Arguments, results and kernels are those of axhip_sgemm_skinny — outputs are bit-identical —
+ * but the split-K partial sums and arrival counters live in an 8 MiB + 16 KiB array that is part of
+ * the library's device code (one copy per GPU, held until the process ends), and the call makes no
+ * hipMalloc / hipFree.  axhip_init must have run on the current device.  A shape whose partial sums
+ * exceed 8 MiB or that spans more than 4096 strips of 64 columns (N > 262144) is refused with
+ * AXHIP_ERR_SHAPE.  All calls on one GPU share the array: calls that overlap in time on one GPU
+ * (two streams, two host threads) race; calls issued one after another do not. */
+int axhip_sgemm_skinny_static(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                              const float *B, int64_t ldb, float *C, int64_t ldc,
+                              const float *bias, int act);
+
 /* ---- int8 -------------------------------------------------------------------------- */
 /* W8A8: acc[m,n] = sum_k (int32)x[m,k] * (int32)w[n,k]   (exact, int32 MFMA)
  *       out[m,n] = act( (float)acc * (x_scale * w_scales[n]) + bias[n] )
