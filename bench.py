@@ -27,11 +27,29 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, TOP/s
 PEAK_FP32_TFLOPS = 157.3     # MI355X fp32 matrix, TFLOP/s
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
-# Bytes that cross the L2 boundary per headline launch, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of `bench.py --counter-probe`, each scaled by what the same counter reads for
-# the probe's copy-shaped kernel of known size (profiles/qgemm_w8a8_256_8192cube_hbm_counters.txt):
-# 806.5 MB fetched (the counter under-reads by 2.000) + 268.9 MB written (scale 1.000).
-HEADLINE_TRAFFIC_BYTES = 806.5e6 + 268.9e6
+# Bytes that cross the L2 boundary per headline launch come from the committed counter summary of
+# `bench.py --counter-probe` (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each scaled by what the same
+# counter reads for the probe's copy-shaped kernel of known size).  The summary names the kernel
+# variant it was taken on; for any other variant the figure is unknown and reported as null.
+HEADLINE_COUNTERS = os.path.join(ROOT, "profiles", "qgemm_w8a8_256_8192cube_hbm_counters.txt")
+PREHEAT_SECONDS = 0.6        # untimed launches before warm-up: the GPU leaves its idle clock only under load
+
+
+def headline_traffic_bytes(kernel):
+    """(bytes per launch, note) from the lines `bench_kernel: <name>` and `traffic_bytes_per_launch:
+    <number>` of the counter summary; (None, why) when the file is missing or was taken on another
+    kernel variant."""
+    try:
+        fields = {}
+        for ln in open(HEADLINE_COUNTERS):
+            key, sep, val = ln.partition(":")
+            if sep and key.strip() in ("bench_kernel", "traffic_bytes_per_launch"):
+                fields[key.strip()] = val.strip()
+        if fields.get("bench_kernel") != kernel:
+            return None, f"counter summary is for {fields.get('bench_kernel')!r}, this run used {kernel!r}"
+        return float(fields["traffic_bytes_per_launch"]), os.path.relpath(HEADLINE_COUNTERS, ROOT)
+    except (OSError, KeyError, ValueError) as e:
+        return None, f"no usable counter summary: {e}"
 
 
 def result_line(suite, case, metric, value):
@@ -77,6 +95,39 @@ def time_calls(hip, fn, steps=None, warmup=None, seconds=0.3):
     return host_ms, ms.value / steps
 
 
+def time_each(hip, fn, steps, warmup, preheat_s):
+    """Times `steps` calls one by one: an event on the kernels' stream before the first call and
+    after every call, so each launch has its own duration (the reference's per-iteration samples,
+    benchmarks/bench_comprehensive.c:90-95).  Before that, `preheat_s` seconds of untimed calls
+    bring the GPU to its sustained clock, then `warmup` more untimed calls.  Returns (host ms per
+    step between device syncs, per-launch event ms as an array, seconds actually pre-heated)."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < preheat_s:
+        for _ in range(8):
+            fn()
+        hip.sync()
+    preheated = time.perf_counter() - t0
+    for _ in range(warmup):
+        fn()
+    hip.sync()
+    ev = [hip.L.axhip_event_create() for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    hip.check(hip.L.axhip_event_record(ev[0]))
+    for i in range(steps):
+        fn()
+        hip.check(hip.L.axhip_event_record(ev[i + 1]))
+    hip.sync()
+    host_ms = (time.perf_counter() - t0) * 1e3 / steps
+    each = np.empty(steps)
+    ms = C.c_float()
+    for i in range(steps):
+        hip.check(hip.L.axhip_event_elapsed_ms(ev[i], ev[i + 1], C.byref(ms)))
+        each[i] = ms.value
+    for e in ev:
+        hip.L.axhip_event_destroy(e)
+    return host_ms, each, preheated
+
+
 def headline(hip, steps, warmup):
     M = N = K = 8192
     rng = np.random.default_rng(0)
@@ -88,10 +139,11 @@ def headline(hip, steps, warmup):
     def step():
         hip.check(hip.L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, bias.ptr, 0, out.ptr, None, M, N, K))
 
-    host_ms, ev_ms = time_calls(hip, step, steps, warmup)
+    host_ms, each, preheated = time_each(hip, step, steps, warmup, PREHEAT_SECONDS)
     ops = 2.0 * M * N * K
-    return {"M": M, "N": N, "K": K, "host_ms": host_ms, "event_ms": ev_ms, "ops": ops,
-            "kernel": hip.last_kernel(),
+    return {"M": M, "N": N, "K": K, "host_ms": host_ms, "event_ms": float(each.mean()),
+            "median_ms": float(np.median(each)), "min_ms": float(each.min()), "max_ms": float(each.max()),
+            "preheat_s": preheated, "ops": ops, "kernel": hip.last_kernel(),
             "algorithmic_bytes": M * K + N * K + 4 * M * N + 8 * N}
 
 
@@ -420,6 +472,46 @@ def cpu_baseline():
                       f"best of {len(runs)} runs ({', '.join('%.1f' % r for r in runs)} s)"}
 
 
+def cpu_baseline_fp32():
+    """The fp32 half of the metric on the host cores: the reference's cpu_opt GEMM
+    (src/compute/backends/cpu_opt.c:3446) at M=N=K=1024, configs[0], with the harness shape of
+    benchmarks/bench_comprehensive.c:26-36 (5 warm + 40 timed runs, per-run samples)."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_bind as ob
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    rng = np.random.default_rng(3)
+    n = 1024
+    a = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    b = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    if ob.ref_available():
+        lib, kind = ob.RefLib(), "reference"
+        lib.backend(lib.CPU_SIMD)
+        ta, tb, to = lib.tensor(a), lib.tensor(b), lib.empty(n, n)       # operands placed once, outside the timing
+
+        def run():
+            assert lib.L.ax_compute_gemm(ta, tb, to) == 0
+    else:
+        lib, kind = ob.Oracle(), "port"
+        c = np.empty((n, n), np.float32)
+
+        def run():
+            lib.L.axo_gemm_opt(a, b, c, n, n, n)
+    for _ in range(5):
+        run()
+    runs = []
+    for _ in range(40):
+        t0 = time.perf_counter()
+        run()
+        runs.append(time.perf_counter() - t0)
+    runs = np.array(runs)
+    tf = 2.0 * n ** 3 / np.median(runs) / 1e12
+    result_line("cpu", f"f32_nn_{n}x{n}x{n}", "gflops", tf * 1e3)
+    return {"value": tf, "unit": "TFLOP/s", "cores": cores, "kind": kind,
+            "median_ms": float(np.median(runs) * 1e3), "min_ms": float(runs.min() * 1e3),
+            "sample": f"cpu_opt fp32 GEMM (opt_gemm through ax_compute_gemm) at M=N=K={n}, operands in place, "
+                      f"median of 40 runs after 5 warm-up runs"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -442,6 +534,7 @@ def main():
     h = headline(hip, args.steps, args.warmup)
     tops = h["ops"] / h["host_ms"] / 1e9
     achieved = h["ops"] / h["event_ms"] / 1e9
+    traffic, traffic_source = headline_traffic_bytes(h["kernel"])
     result_line("axhip", "q8a8_8192x8192x8192", "gflops", tops * 1e3)
     line = {
         "metric": "int8 qgemm TOP/s on 1 MI355X (W8A8, M=N=K=8192, fused dequant+bias)",
@@ -453,16 +546,19 @@ def main():
                    "M": h["M"], "N": h["N"], "K": h["K"], "device": hip.L.axhip_device_name().decode()},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": achieved / PEAK_INT8_TOPS,
-                     "traffic": HEADLINE_TRAFFIC_BYTES if h["kernel"] == "qgemm_w8a8_256x256_dma" else None,
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": h["kernel"],
-                     "kernel_us": h["event_ms"] * 1e3, "algorithmic_ops": h["ops"],
-                     "algorithmic_bytes": h["algorithmic_bytes"]},
+                     "kernel_us": h["event_ms"] * 1e3, "median_us": h["median_ms"] * 1e3,
+                     "min_us": h["min_ms"] * 1e3, "max_us": h["max_ms"] * 1e3,
+                     "algorithmic_ops": h["ops"], "algorithmic_bytes": h["algorithmic_bytes"]},
+        "preheat_s": round(h["preheat_s"], 3),
     }
     if not args.no_secondary:
         line["secondary"] = secondary(hip)
     hip.sync()
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
+        line["cpu_baseline_fp32"] = cpu_baseline_fp32()
     print(json.dumps(line), flush=True)
 
 
