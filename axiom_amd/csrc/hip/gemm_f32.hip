@@ -681,6 +681,11 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
     // everywhere, and two stages are as good as three or four.  With only a few slabs per tile
     // (K <= 128) a workgroup's life is mostly its loads and its write-back: plain 64x64 tiles,
     // several workgroups per CU.
+    const int force = tuning().f32_tile;         // 0 = by shape; 128, 64 or 642 (64x64 with the k split) where the shape permits
+    if (force == 128 && g.M % 128 == 0 && g.N % 256 == 0 && g.K >= 64)
+        return launch_dma<128, 256, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
+    if (force == 642 && g.K >= 64) return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[2], g, batch);
+    if (force == 64) return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
     if (g.K > 128) {
         // ... provided its rounds of one tile per CU come out nearly full: 384 tiles are a full round
         // and a half-empty one (3072x4096x2048: 106 TFLOP/s, against 130 on 64x64 tiles)
@@ -754,6 +759,8 @@ int64_t split_count(int64_t M, int64_t N, int64_t K) {
     // (4x4100x4096: 38 -> 30 us; 9x8000x8192: 78 -> 69).
     const bool ragged = M % 64 != 0 || N % 64 != 0;
     int64_t want = ((ragged ? 2 : 1) * cus + tiles - 1) / tiles;
+    if (tuning().f32_splitk == 1) return 1;
+    if (tuning().f32_splitk > 1) want = tuning().f32_splitk;
     const int64_t most = K / 64;                             // ranges of at least 64
     if (want > most) want = most;
     // K / 32 must divide into the ranges: the nearest count at or below the wish, or, when that is

@@ -538,13 +538,20 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 // EDGE: M and N need not be multiples of the tile.  A row past the end of X or W is fetched from
 // the last row instead (its products land in outputs that are not stored), and the write-back
 // keeps to rows below M and 4-column groups below N (N a multiple of 4).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int ACT, bool EDGE = false>
-__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64)
+// WAVES_K = 2: a second set of WAVES_M x WAVES_N waves takes k-steps 2 and 3 of every slab (the first
+// set keeps 0 and 1) and hands its accumulators over through LDS at the end.  A tile then has two
+// waves on every SIMD with no more global traffic, so one wave's waits for LDS and for the slab
+// barrier are covered by the other's MFMAs: for a launch of at most one small tile per CU, whose
+// time is the chain of those waits rather than memory or matrix-core throughput.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int ACT, bool EDGE = false, int WAVES_K = 1>
+__global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64)
 k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
                  int64_t K, float x_scale, const float *__restrict__ w_scales,
                  const float *__restrict__ bias, float *__restrict__ out,
-                 int32_t *__restrict__ acc_out, int64_t ldc) {
-    constexpr int NW = WAVES_M * WAVES_N, BKB = 128;
+                 int32_t *__restrict__ acc_out, int64_t ldc, int splits, int32_t *partials,
+                 int *__restrict__ counters) {
+    constexpr int NWO = WAVES_M * WAVES_N, NW = NWO * WAVES_K, BKB = 128;      // waves that own outputs / all waves
+    constexpr int KSTEPS = 4 / WAVES_K;                                        // k-steps of a slab per wave
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
     constexpr int XS = BM * BKB, WS = BN * BKB;          // bytes of one stage of each operand
     constexpr int W_BASE = NST * XS;
@@ -552,21 +559,28 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     constexpr int NREADS = TM + TN;
     constexpr int VM_KEEP = (NST - 2) * (IPW_X + IPW_W);
     static_assert(IPW_X * 8 * NW == BM && IPW_W * 8 * NW == BN, "slab must divide over the waves");
-    static_assert(NST >= 2 && NST <= 4 && VM_KEEP < 64, "stage count");
+    static_assert(NST >= 2 && NST <= 8 && VM_KEEP < 64, "stage count");
     static_assert((NST - 1) * XS + (TM - 1) * 4096 < 65536 && (NST - 1) * WS + (TN - 1) * 4096 < 65536,
                   "ds_read immediates are 16 bits");
-    static_assert(NW * 4096 <= NST * XS, "write-back turn area");
+    static_assert(WAVES_K == 1 || WAVES_K == 2, "one or two wave sets over k");
+    static_assert(NWO * 4096 + (WAVES_K - 1) * NWO * TM * TN * 4096 <= NST * XS, "write-back turn area and k hand-over");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int wk = wave / NWO, wo = wave % NWO;          // wave set over k, output wave inside the set
+    const int wm = wo / WAVES_N, wn = wo % WAVES_N;
     int tm, tn;
     tile_of_block(blockIdx.x, (int)((M + BM - 1) / BM), (int)((N + BN - 1) / BN), tm, tn);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     // EDGE also takes a K that ends inside a slab (K a multiple of 16): in the last slab the lanes
     // whose 16 bytes lie past K load nothing and write zeros to their LDS place instead
-    const int slabs = EDGE ? (int)((K + BKB - 1) / BKB) : (int)(K / BKB);
-    const int ktail = EDGE ? (int)(K - (int64_t)(slabs - 1) * BKB) : BKB;      // bytes of K in the last slab
+    const int slabs_all = EDGE ? (int)((K + BKB - 1) / BKB) : (int)(K / BKB);
+    // Split over K (gridDim.y = splits > 1): workgroup y of a tile multiplies slabs [slab0, slab0 + slabs);
+    // the host picks splits so that none is empty.  The int32 partial tiles are added by whichever
+    // workgroup of the tile finishes last: integer sums are exact in any order.
+    const int per_split = (slabs_all + splits - 1) / splits, slab0 = (int)blockIdx.y * per_split;
+    const int slabs = slabs_all - slab0 < per_split ? slabs_all - slab0 : per_split;
+    const int ktail = EDGE && slab0 + slabs == slabs_all ? (int)(K - (int64_t)(slabs_all - 1) * BKB) : BKB;   // bytes of K in this range's last slab
     int left = slabs;                                                          // slabs not yet requested
     // rows of this tile that exist (EDGE; the last tile row / column may hang over)
     const int mrows = EDGE && M - m0 < BM ? (int)(M - m0) : BM, nrows = EDGE && N - n0 < BN ? (int)(N - n0) : BN;
@@ -587,16 +601,17 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         vw[j] = (unsigned)((row < nrows ? row : nrows - 1) * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
         tw[j] = (((lane & 7) ^ ((row >> 1) & 7)) << 4) < ktail;
     }
-    const int8_t *gx = X + m0 * K, *gw = W + n0 * K;
+    const int8_t *gx = X + m0 * K + (int64_t)slab0 * BKB, *gw = W + n0 * K + (int64_t)slab0 * BKB;
     const unsigned lds0 = (unsigned)(uintptr_t)lds, lds_w = lds0 + wave * 1024;
 
     const int frow = lane & 31, fhalf = lane >> 5;
-    unsigned rx[4], rw[4];
+    unsigned rx[KSTEPS], rw[KSTEPS];                     // this wave's k-steps: wk * KSTEPS + 0 ..
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
+    for (int i = 0; i < KSTEPS; i++) {
+        const int ks = wk * KSTEPS + i;
         const unsigned inrow = (unsigned)(frow * BKB + (((ks * 2 + fhalf) ^ ((frow >> 1) & 7)) << 4));
-        rx[ks] = lds0 + wm * WTM * BKB + inrow;
-        rw[ks] = lds0 + W_BASE + wn * WTN * BKB + inrow;
+        rx[i] = lds0 + wm * WTM * BKB + inrow;
+        rw[i] = lds0 + W_BASE + wn * WTN * BKB + inrow;
     }
 
     typedef float v4f_t __attribute__((ext_vector_type(4)));
@@ -665,12 +680,14 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         AXI8G_FRAGS(1, ST, 1);                                                                   \
         AXI8_LGKM(NREADS);                                                                       \
         AXI8G_MFMAS(0);                                                                          \
-        AXI8G_FRAGS(0, ST, 2);                                                                   \
-        AXI8_LGKM(NREADS);                                                                       \
-        AXI8G_MFMAS(1);                                                                          \
-        AXI8G_FRAGS(1, ST, 3);                                                                   \
-        AXI8_LGKM(NREADS);                                                                       \
-        AXI8G_MFMAS(0);                                                                          \
+        if constexpr (KSTEPS == 4) {                                                             \
+            AXI8G_FRAGS(0, ST, 2);                                                               \
+            AXI8_LGKM(NREADS);                                                                   \
+            AXI8G_MFMAS(1);                                                                      \
+            AXI8G_FRAGS(1, ST, 3);                                                               \
+            AXI8_LGKM(NREADS);                                                                   \
+            AXI8G_MFMAS(0);                                                                      \
+        }                                                                                        \
         AXI8_LGKM(0);                                                                            \
         AXI8G_MFMAS(1);                                                                          \
         if (VM_KEEP > 0 && (more)) AXI8_VM(VM_KEEP); else AXI8_VM(0);                            \
@@ -678,31 +695,103 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         __builtin_amdgcn_sched_barrier(0);                                                       \
     } while (0)
 
+    // prologue: the first NST-1 slabs are requested; compute starts as soon as the first has landed
     AXI8G_ISSUE(0);
     if constexpr (NST > 2) { if (slabs > 1) AXI8G_ISSUE(1); }
     if constexpr (NST > 3) { if (slabs > 2) AXI8G_ISSUE(2); }
-    AXI8_VM(0);
+    if constexpr (NST > 4) { if (slabs > 3) AXI8G_ISSUE(3); }
+    if constexpr (NST > 5) { if (slabs > 4) AXI8G_ISSUE(4); }
+    if constexpr (NST > 6) { if (slabs > 5) AXI8G_ISSUE(5); }
+    if constexpr (NST > 7) { if (slabs > 6) AXI8G_ISSUE(6); }
+    if (VM_KEEP > 0 && slabs >= NST - 1) AXI8_VM(VM_KEEP); else AXI8_VM(0);
     if constexpr (EDGE) AXI8_LGKM(0);            // zeros written for a K tail that is already in the first slabs
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     for (int s = 0; s < slabs; s += NST) {
         AXI8G_SLAB(0, s + NST - 1 < slabs);
-        if (s + 1 < slabs) {
-            AXI8G_SLAB(1, s + NST < slabs);
-            if constexpr (NST > 2) {
-                if (s + 2 < slabs) {
-                    AXI8G_SLAB(2, s + NST + 1 < slabs);
-                    if constexpr (NST > 3) {
-                        if (s + 3 < slabs) AXI8G_SLAB(3, s + NST + 2 < slabs);
-                    }
-                }
-            }
-        }
+        if (s + 1 >= slabs) break;
+        AXI8G_SLAB(1, s + NST < slabs);
+        if constexpr (NST > 2) { if (s + 2 >= slabs) break; AXI8G_SLAB(2, s + NST + 1 < slabs); }
+        if constexpr (NST > 3) { if (s + 3 >= slabs) break; AXI8G_SLAB(3, s + NST + 2 < slabs); }
+        if constexpr (NST > 4) { if (s + 4 >= slabs) break; AXI8G_SLAB(4, s + NST + 3 < slabs); }
+        if constexpr (NST > 5) { if (s + 5 >= slabs) break; AXI8G_SLAB(5, s + NST + 4 < slabs); }
+        if constexpr (NST > 6) { if (s + 6 >= slabs) break; AXI8G_SLAB(6, s + NST + 5 < slabs); }
+        if constexpr (NST > 7) { if (s + 7 >= slabs) break; AXI8G_SLAB(7, s + NST + 6 < slabs); }
     }
 #undef AXI8G_ISSUE
 #undef AXI8G_FRAGS
 #undef AXI8G_MFMAS
 #undef AXI8G_SLAB
+
+    if constexpr (WAVES_K == 2) {
+        // the second wave set hands its sums to the first through the dead stages, register by register
+        // ([wave][16-byte group][lane], past the turn area), and is done
+        v4i *hand = reinterpret_cast<v4i *>(lds + NWO * 4096) + wo * (TM * TN * 4 * 64) + lane;
+        if (wk == 1) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++)
+                        hand[((i * TN + j) * 4 + g) * 64] =
+                            v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+        }
+        __syncthreads();
+        if (wk == 1) return;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const v4i t = hand[((i * TN + j) * 4 + g) * 64];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[i][j][4 * g + e] += t[e];
+                }
+    }
+    // from here on only the NWO output waves are alive (a finished wave no longer counts at barriers)
+    if (splits > 1) {
+        // Partial tiles are kept register by register, [tile][split][wave][register][lane]: whoever reads
+        // them back has the same wave / lane / register roles, so the layout never has to mean rows and
+        // columns.  Partials, the arrival counter and the reads below are device-scope accesses (the
+        // workgroups of one tile run on different XCDs, each with its own L2); the wait makes this thread's
+        // stores complete before the barrier, the barrier orders them before thread 0's increment.
+        constexpr int REGS = TM * TN * 16;
+        int32_t *tile_part = partials + (int64_t)blockIdx.x * splits * (NWO * REGS * 64);
+        int32_t *mine = tile_part + ((int64_t)blockIdx.y * NWO + wave) * (REGS * 64);
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    __hip_atomic_store(mine + ((i * TN + j) * 16 + v) * 64 + lane, acc[i][j][v], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        int *last_flag = reinterpret_cast<int *>(lds_bias + BN);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (tid == 0) {
+            const int arrived = __hip_atomic_fetch_add(counters + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *last_flag = (arrived == splits - 1);
+        }
+        __syncthreads();
+        if (!*last_flag) return;
+        for (int p = 0; p < splits; p++) {
+            if (p == (int)blockIdx.y) continue;
+            const int32_t *theirs = tile_part + ((int64_t)p * NWO + wave) * (REGS * 64);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++)
+                        acc[i][j][v] += __hip_atomic_load(theirs + ((i * TN + j) * 16 + v) * 64 + lane, __ATOMIC_RELAXED,
+                                                          __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (tid == 0)                                   // ready for the next launch
+            __hip_atomic_store(counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 
     // write-back as in the 256x256 kernel: through 4 KiB of dead stage per wave
     unsigned char *turn = lds + wave * 4096;
@@ -754,16 +843,36 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool EDGE = false>
-int launch_dma(const char *name, const int8_t *x, float x_scale, const int8_t *w, const float *w_scales,
-               const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N, int64_t K,
-               int64_t ldc) {
-    constexpr int smem = NST * (BM + BN) * 128 + 2 * BN * 4;
+// Workgroups over K for a launch of `tiles` output tiles and `slabs` slabs of 128 bytes.  The join
+// costs a store, an atomic and a load in a row at the end of every workgroup, about 4 us, so a split
+// pays only when the tiles leave at least half the CUs idle and K is long: up to one workgroup per CU,
+// at most 8, each with at least 8 slabs (64 x 1024 x 4096: 8.6 -> 6.4 us with 4; 256 x 2048 x 8192:
+// 14.8 -> 12.3 with 2; M = 256, N = K = 4096, one tile per CU already: 9.8 -> 12.8 with 2).
+int pick_splits(int64_t tiles, int64_t slabs) {
+    const Tuning &tune = tuning();
+    int64_t splits = 1;
+    if (tune.i8_splitk > 0) splits = tune.i8_splitk;
+    else if (tiles * 2 <= cu_count() && slabs >= 16) {
+        splits = cu_count() / tiles;
+        if (splits > slabs / 8) splits = slabs / 8;
+        if (splits > 8) splits = 8;
+    }
+    if (splits > slabs) splits = slabs;
+    if (splits < 1) splits = 1;
+    const int64_t per = (slabs + splits - 1) / splits;
+    return (int)((slabs + per - 1) / per);          // drop ranges that would be empty
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool EDGE = false, int WAVES_K = 1>
+int launch_dma(const char *name, const char *split_name, const int8_t *x, float x_scale, const int8_t *w,
+               const float *w_scales, const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N,
+               int64_t K, int64_t ldc) {
+    constexpr int smem = NST * (BM + BN) * 128 + 2 * BN * 4 + 16;      // stages, scale and bias rows, the split join's flag
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
-                           const float *, float *, int32_t *, int64_t);
-    static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE>,
-                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU, EDGE>,
-                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE>};
+                           const float *, float *, int32_t *, int64_t, int, int32_t *, int *);
+    static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE, WAVES_K>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU, EDGE, WAVES_K>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE, WAVES_K>};
     static bool attr_set = false;
     if (!attr_set) {
         for (kern_t kf : kerns)
@@ -774,9 +883,17 @@ int launch_dma(const char *name, const int8_t *x, float x_scale, const int8_t *w
     }
     const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     if (tiles > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: too many tiles");
-    note_kernel(name);
-    hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles), dim3(WAVES_M * WAVES_N * 64), smem, kStream, x, w,
-                       M, N, K, x_scale, w_scales, bias, out, acc_out, ldc);
+    const int splits = pick_splits(tiles, (K + 127) / 128);
+    int32_t *partials = nullptr;
+    int *counters = nullptr;
+    if (splits > 1) {
+        partials = static_cast<int32_t *>(workspace((size_t)tiles * splits * BM * BN * sizeof(int32_t)));
+        counters = strip_counters((size_t)tiles);
+        if (!partials || !counters) return AXHIP_ERR_ALLOC;
+    }
+    note_kernel(splits > 1 ? split_name : name);
+    hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles, (unsigned)splits), dim3(WAVES_M * WAVES_N * WAVES_K * 64), smem, kStream,
+                       x, w, M, N, K, x_scale, w_scales, bias, out, acc_out, ldc, splits, partials, counters);
     return check_launch(name);
 }
 
@@ -885,26 +1002,38 @@ int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_
                          (((uintptr_t)acc_out & 15) == 0) && ldc % 4 == 0;
     // the persistent 256x256 kernel from about 80 tiles on (81 tiles, 2304^2 x 8192: 72 us against 82 on
     // 128x128 tiles; 64 tiles, 2048^2 x 4096: 40 against 26)
-    if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 80 &&
-        K < (int64_t(1) << 24))   // per-lane 32-bit byte offsets span 256 rows
+    if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && K < (int64_t(1) << 24) &&   // per-lane 32-bit byte offsets span 256 rows
+        (tuning().i8_tile == 256 || (tuning().i8_tile == 0 && (M / 256) * (N / 256) >= 80)))
         return launch_256(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K, ldc);
     // aligned but too few 256x256 tiles: direct-to-LDS kernel over smaller tiles
+    const int force = tuning().i8_tile;             // 0 = by shape, else 64 / 128 where the shape permits
     if (aligned && vec_out && K % 128 == 0 && M % 64 == 0 && N % 64 == 0 && K < (int64_t(1) << 24)) {
         // 128x128 tiles once there is one for every CU (2048^2 x 4096: 26.2 us against 30.7 on 64x64)
-        if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 256)
-            return launch_dma<128, 128, 2, 2, 3>("qgemm_w8a8_128x128_dma", x, x_scale, w, w_scales, bias,
-                                                 act, out, acc_out, M, N, K, ldc);
-        return launch_dma<64, 64, 2, 2, 4>("qgemm_w8a8_64x64_dma", x, x_scale, w, w_scales, bias, act,
-                                           out, acc_out, M, N, K, ldc);
+        const bool fits128 = M % 128 == 0 && N % 128 == 0;
+        if (fits128 && (force == 128 || (force == 0 && (M / 128) * (N / 128) >= 256)))
+            return launch_dma<128, 128, 2, 2, 3>("qgemm_w8a8_128x128_dma", "qgemm_w8a8_128x128_dma_splitk", x, x_scale, w,
+                                                 w_scales, bias, act, out, acc_out, M, N, K, ldc);
+        // at most one 64x64 tile per CU: the whole LDS goes to slabs in flight (M = 256, N = K = 4096: 8 stages
+        // xx us against 9.6 with four), since a lone workgroup's loads are bound by latency, not by the CU's fill rate
+        // at most one 64x64 tile per CU: two wave sets share each slab's k-steps (M = 256, N = K = 4096: 9.8 us
+        // against 10.5; 256 x 2048 x 8192: 14.8 against 17.7)
+        if (force == 642 || (force == 0 && (M / 64) * (N / 64) <= cu_count()))
+            return launch_dma<64, 64, 2, 2, 4, false, 2>("qgemm_w8a8_64x64k2_dma", "qgemm_w8a8_64x64k2_dma_splitk", x, x_scale, w,
+                                                         w_scales, bias, act, out, acc_out, M, N, K, ldc);
+        return launch_dma<64, 64, 2, 2, 4>("qgemm_w8a8_64x64_dma", "qgemm_w8a8_64x64_dma_splitk", x, x_scale, w, w_scales,
+                                           bias, act, out, acc_out, M, N, K, ldc);
     }
     // the same kernel for M or N off the 64 grid: edge tiles clamp their loads and guard their stores
     const bool aligned16 = ((((uintptr_t)x | (uintptr_t)w) & 15) == 0) && K % 16 == 0 && K > 0;
     if (aligned16 && vec_out && N % 4 == 0 && K < (int64_t(1) << 24)) {
-        if (((M + 127) / 128) * ((N + 127) / 128) >= 256)
-            return launch_dma<128, 128, 2, 2, 3, true>("qgemm_w8a8_128x128_dma_edge", x, x_scale, w, w_scales, bias,
-                                                       act, out, acc_out, M, N, K, ldc);
-        return launch_dma<64, 64, 2, 2, 4, true>("qgemm_w8a8_64x64_dma_edge", x, x_scale, w, w_scales, bias, act,
-                                                 out, acc_out, M, N, K, ldc);
+        if (force == 128 || (force == 0 && ((M + 127) / 128) * ((N + 127) / 128) >= 256))
+            return launch_dma<128, 128, 2, 2, 3, true>("qgemm_w8a8_128x128_dma_edge", "qgemm_w8a8_128x128_dma_edge_splitk", x,
+                                                       x_scale, w, w_scales, bias, act, out, acc_out, M, N, K, ldc);
+        if (force == 642 || (force == 0 && ((M + 63) / 64) * ((N + 63) / 64) <= cu_count()))
+            return launch_dma<64, 64, 2, 2, 4, true, 2>("qgemm_w8a8_64x64k2_dma_edge", "qgemm_w8a8_64x64k2_dma_edge_splitk", x,
+                                                        x_scale, w, w_scales, bias, act, out, acc_out, M, N, K, ldc);
+        return launch_dma<64, 64, 2, 2, 4, true>("qgemm_w8a8_64x64_dma_edge", "qgemm_w8a8_64x64_dma_edge_splitk", x, x_scale, w,
+                                                 w_scales, bias, act, out, acc_out, M, N, K, ldc);
     }
     // fewer than ~3/4 of the 256 CUs busy with 128x128 tiles: quarter the tile instead
     if (aligned && M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) >= 192)

@@ -292,7 +292,7 @@ struct SkinnyPlan {
 int plan_skinny(int64_t M, int64_t N, int64_t K, const float *B, int64_t ldb, SkinnyPlan &p) {
     p.col_blocks = (N + COLS - 1) / COLS;
     // enough workgroups to cover 256 CUs a few times over, each with at least 128 k rows
-    const int64_t want_blocks = M <= 2 ? kWantBlocksM12 : kWantBlocksM3up;
+    const int64_t want_blocks = tuning().skinny_blocks > 0 ? tuning().skinny_blocks : M <= 2 ? kWantBlocksM12 : kWantBlocksM3up;
     int64_t splits = (want_blocks + p.col_blocks - 1) / p.col_blocks;
     const int64_t max_splits = K >= 128 ? K / 128 : 1;
     if (splits > max_splits) splits = max_splits;

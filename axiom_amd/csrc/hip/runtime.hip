@@ -1,6 +1,7 @@
 // Lifecycle, memory and timing entry points of libaxhip.so.
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include <mutex>
@@ -34,6 +35,29 @@ int64_t g_stat_allocs = 0, g_stat_frees = 0, g_stat_bytes_alloc = 0, g_stat_byte
 size_t g_pool_cached = 0;
 constexpr size_t kPoolMaxBlock = size_t(1) << 30;        // larger blocks go straight back to the driver
 constexpr size_t kPoolMaxCached = size_t(16) << 30;      // bytes the pool may hold back
+
+axhip::Tuning g_tuning = {0, 0, 0, 0, 0};
+
+// "64x64" / "128x128" / "256x256" / "128x256" / "64x64k2" or the bare first number; 0 when absent or not one of `allowed`
+int parse_tile(const char *name, const int *allowed, int n_allowed) {
+    const char *v = getenv(name);
+    if (!v || !*v) return 0;
+    char *end = nullptr;
+    long t = strtol(v, &end, 10);
+    if (end == v) return 0;
+    if (strstr(v, "k2")) t = t * 10 + 2;
+    for (int i = 0; i < n_allowed; i++)
+        if (allowed[i] == t) return (int)t;
+    return 0;
+}
+
+int parse_count(const char *name, long lo, long hi) {
+    const char *v = getenv(name);
+    if (!v || !*v) return 0;
+    char *end = nullptr;
+    const long t = strtol(v, &end, 10);
+    return (end != v && *end == 0 && t >= lo && t <= hi) ? (int)t : 0;
+}
 }  // namespace
 
 namespace axhip {
@@ -47,6 +71,8 @@ int fail(int code, const char *fmt, ...) {
 }
 
 int cu_count() { return g_cu_count; }
+
+const Tuning &tuning() { return g_tuning; }
 
 // sizes are rounded so that blocks get reused: powers of two up to 1 MiB, then multiples of 1 MiB
 size_t pool_class(size_t bytes) {
@@ -164,8 +190,30 @@ int axhip_device_count(void) {
     return n;
 }
 
+int axhip_tuning_reload(void) {
+    static const int i8_tiles[] = {64, 642, 128, 256}, f32_tiles[] = {64, 642, 128};
+    g_tuning.i8_tile = parse_tile("AX_HIP_I8_TILE", i8_tiles, 4);
+    g_tuning.i8_splitk = parse_count("AX_HIP_I8_SPLITK", 1, 16);
+    g_tuning.f32_tile = parse_tile("AX_HIP_F32_TILE", f32_tiles, 3);
+    g_tuning.f32_splitk = parse_count("AX_HIP_F32_SPLITK", 1, 4096);
+    g_tuning.skinny_blocks = parse_count("AX_HIP_SKINNY_BLOCKS", 1, 65535);
+    return (g_tuning.i8_tile != 0) + (g_tuning.i8_splitk != 0) + (g_tuning.f32_tile != 0) + (g_tuning.f32_splitk != 0) +
+           (g_tuning.skinny_blocks != 0);
+}
+
+int axhip_tuning_get(const char *name) {
+    if (!name) return -1;
+    if (!strcmp(name, "AX_HIP_I8_TILE")) return g_tuning.i8_tile;
+    if (!strcmp(name, "AX_HIP_I8_SPLITK")) return g_tuning.i8_splitk;
+    if (!strcmp(name, "AX_HIP_F32_TILE")) return g_tuning.f32_tile;
+    if (!strcmp(name, "AX_HIP_F32_SPLITK")) return g_tuning.f32_splitk;
+    if (!strcmp(name, "AX_HIP_SKINNY_BLOCKS")) return g_tuning.skinny_blocks;
+    return -1;
+}
+
 int axhip_init(void) {
     if (g_ready) return AXHIP_OK;
+    (void)axhip_tuning_reload();
     if (axhip_device_count() <= 0)
         return fail(AXHIP_ERR_BACKEND, "no HIP device visible: libaxhip has no CPU fallback");
     AXHIP_HIP_TRY(hipSetDevice(0), "hipSetDevice");

@@ -20,6 +20,8 @@ SIGNATURES = {
     "axhip_device_count": (C.c_int, []),
     "axhip_last_error": (C.c_char_p, []),
     "axhip_device_name": (C.c_char_p, []),
+    "axhip_tuning_reload": (C.c_int, []),
+    "axhip_tuning_get": (C.c_int, [C.c_char_p]),
     "axhip_malloc": (vp, [C.c_size_t]),
     "axhip_malloc_uninit": (vp, [C.c_size_t]),
     "axhip_free": (None, [vp]),

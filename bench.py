@@ -9,8 +9,10 @@ and the skinny-M route's GB/s, each with its own roofline fraction.  RESULT line
 reference's benchmark format (benchmarks/bench_common.h:25-42) go to stderr.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu]
-    python bench.py --counter-probe     # for hardware-counter runs: 3 headline launches and 3
+    python bench.py --counter-probe [headline|skinny|fp32|config2|attention]
+                                        # for hardware-counter runs: a few launches of one case's kernels and 3
                                         # launches of a copy-shaped kernel of known size, no output line
+    python bench.py --sustain 8 [--operands zeros]   # back-to-back headline launches, for clock sampling
 """
 import argparse
 import ctypes as C
@@ -421,26 +423,109 @@ def secondary(hip):
     return res
 
 
-def counter_probe(hip):
-    """Workload for per-dispatch hardware counters (HBM bytes fetched / written): the headline
-    kernel, and for scale the elementwise ReLU kernel over 64 Mi floats, which reads 256 MiB
-    and writes 256 MiB exactly once (a plain copy as far as memory traffic goes)."""
-    M = N = K = 8192
+def counter_probe(hip, case, repeat=1):
+    """Workloads for per-dispatch hardware counters and kernel traces: a few launches of the kernels of
+    one case, then for scale the elementwise ReLU kernel over 64 Mi floats, which reads 256 MiB and
+    writes 256 MiB exactly once (a plain copy as far as memory traffic goes).
+      headline  W8A8 8192^3
+      skinny    the 4096 x 4096 layer of the bs=1 MLP at M = 1 and M = 8 over 8 rotating weight sets
+                (537 MB, so every launch streams its 67.1 MB from HBM and not from the Infinity Cache)
+      fp32      1024^3, then the FFN pair 2048 x 1024 x 4096 (bias + GELU fused) and back
+      config2   W8A8 M = 256, N = K = 4096
+      attention batched Q K^T and P V over 512 heads of [512, 64], then the fused forward"""
     rng = np.random.default_rng(0)
-    x, w = hip.array(rand_i8(rng, (M, K))), hip.array(rand_i8(rng, (N, K)))
-    ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
-    bias = hip.array(rng.normal(0.0, 0.02, N).astype(np.float32))
-    out = hip.empty((M, N))
-    for _ in range(3):
-        hip.check(hip.L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, bias.ptr, 0, out.ptr, None, M, N, K))
+    L = hip.L
+    reps = 3 * repeat                # `repeat` > 1 (--probe-repeat): long enough for sustained clocks, for kernel traces
+    if case == "headline":
+        M = N = K = 8192
+        x, w = hip.array(rand_i8(rng, (M, K))), hip.array(rand_i8(rng, (N, K)))
+        ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+        bias = hip.array(rng.normal(0.0, 0.02, N).astype(np.float32))
+        out = hip.empty((M, N))
+        for _ in range(reps):
+            hip.check(L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, bias.ptr, 0, out.ptr, None, M, N, K))
+        what = f"{reps} x qgemm_w8a8 8192^3 ({hip.last_kernel()})"
+    elif case == "skinny":
+        sets = [hip.array(rng.uniform(-0.04, 0.04, (4096, 4096)).astype(np.float32)) for _ in range(8)]
+        zeros = hip.empty((4096,))
+        what = ""
+        for M in (1, 8):
+            xin, h2 = hip.array(rng.uniform(0, 1, (M, 4096)).astype(np.float32)), hip.empty((M, 4096))
+            for i in range(16 * repeat):
+                hip.check(L.axhip_sgemm(0, 0, M, 4096, 4096, 1.0, xin.ptr, 4096, sets[i % 8].ptr, 4096, 0.0,
+                                        h2.ptr, 4096, zeros.ptr, 1))
+            what += f"{16 * repeat} x sgemm M={M} 4096x4096 ({hip.last_kernel()}) "
+    elif case == "fp32":
+        a = hip.array(rng.uniform(-1, 1, (1024, 1024)).astype(np.float32))
+        b = hip.array(rng.uniform(-1, 1, (1024, 1024)).astype(np.float32))
+        c = hip.empty((1024, 1024))
+        for _ in range(8 * repeat):
+            hip.check(L.axhip_sgemm(0, 0, 1024, 1024, 1024, 1.0, a.ptr, 1024, b.ptr, 1024, 0.0, c.ptr, 1024, None, 0))
+        what = f"{8 * repeat} x sgemm 1024^3 ({hip.last_kernel()}) "
+        x = hip.array(rng.normal(0, 1, (2048, 1024)).astype(np.float32))
+        w1 = hip.array(rng.normal(0, 0.02, (1024, 4096)).astype(np.float32))
+        w2 = hip.array(rng.normal(0, 0.02, (4096, 1024)).astype(np.float32))
+        b1 = hip.array(rng.normal(0, 0.02, 4096).astype(np.float32))
+        b2 = hip.array(rng.normal(0, 0.02, 1024).astype(np.float32))
+        hbuf, y = hip.empty((2048, 4096)), hip.empty((2048, 1024))
+        for _ in range(8 * repeat):
+            hip.check(L.axhip_sgemm(0, 0, 2048, 4096, 1024, 1.0, x.ptr, 1024, w1.ptr, 4096, 0.0, hbuf.ptr, 4096, b1.ptr, 2))
+            k1 = hip.last_kernel()
+            hip.check(L.axhip_sgemm(0, 0, 2048, 1024, 4096, 1.0, hbuf.ptr, 4096, w2.ptr, 1024, 0.0, y.ptr, 1024, b2.ptr, 0))
+        what += f"{8 * repeat} x FFN pair ({k1}, {hip.last_kernel()})"
+    elif case == "config2":
+        xi, wi = hip.array(rand_i8(rng, (256, 4096))), hip.array(rand_i8(rng, (4096, 4096)))
+        ws = hip.array(rng.uniform(1e-3, 1e-2, 4096).astype(np.float32))
+        bi = hip.array(rng.normal(0, 0.02, 4096).astype(np.float32))
+        oi = hip.empty((256, 4096))
+        for _ in range(16 * repeat):
+            hip.check(L.axhip_qgemm_w8a8(xi.ptr, 0.01, wi.ptr, ws.ptr, bi.ptr, 0, oi.ptr, None, 256, 4096, 4096))
+        what = f"{16 * repeat} x qgemm_w8a8 256x4096x4096 ({hip.last_kernel()})"
+    elif case == "attention":
+        Bn, S, D = 512, 512, 64
+        q, k, v = (hip.array(rng.normal(0, 1, (Bn, S, D)).astype(np.float32)) for _ in range(3))
+        sc, o, l = hip.empty((Bn, S, S)), hip.empty((Bn, S, D)), hip.empty((Bn, S))
+        for _ in range(reps):
+            hip.check(L.axhip_sgemm_strided_batched(0, 1, S, S, D, 1.0, q.ptr, D, S * D, k.ptr, D, S * D, 0.0,
+                                                    sc.ptr, S, S * S, Bn))
+            k1 = hip.last_kernel()
+            hip.check(L.axhip_sgemm_strided_batched(0, 0, S, D, S, 1.0, sc.ptr, S, S * S, v.ptr, D, S * D, 0.0,
+                                                    o.ptr, D, S * D, Bn))
+            k2 = hip.last_kernel()
+            hip.check(L.axhip_sdpa_fwd(q.ptr, k.ptr, v.ptr, o.ptr, l.ptr, Bn, S, D, 0.125, 0))
+        what = f"{reps} x (QK^T {k1}, PV {k2}, fused {hip.last_kernel()}) over 512 heads of [512, 64]"
+    else:
+        sys.exit(f"unknown counter-probe case {case!r}")
     hip.sync()
     n = 64 << 20
     src, dst = hip.empty((n,)), hip.empty((n,))
     for _ in range(3):
-        hip.check(hip.L.axhip_relu(src.ptr, dst.ptr, n))
+        hip.check(L.axhip_relu(src.ptr, dst.ptr, n))
     hip.sync()
-    print(f"counter probe: 3 x {hip.last_kernel()} over {n} floats after 3 x qgemm_w8a8 8192^3",
-          file=sys.stderr, flush=True)
+    print(f"counter probe: {what}, then 3 x ReLU (k_unary<0>) over {n} floats", file=sys.stderr, flush=True)
+
+
+def sustain(hip, seconds, operands):
+    """The headline GEMM launched back to back for `seconds`, over random int8 operands or all-zero ones
+    (same instruction stream, no switching activity in the matrix core), so that clock and power can be
+    sampled from outside (rocm-smi) while it runs.  Prints the average time per launch once a second."""
+    M = N = K = 8192
+    rng = np.random.default_rng(0)
+    if operands == "zeros":
+        x, w = hip.empty((M, K), np.int8), hip.empty((N, K), np.int8)
+    else:
+        x, w = hip.array(rand_i8(rng, (M, K))), hip.array(rand_i8(rng, (N, K)))
+    ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+    bias = hip.array(rng.normal(0.0, 0.02, N).astype(np.float32))
+    out = hip.empty((M, N))
+    t_end = time.perf_counter() + seconds
+    while time.perf_counter() < t_end:
+        t0 = time.perf_counter()
+        for _ in range(2000):
+            hip.check(hip.L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, bias.ptr, 0, out.ptr, None, M, N, K))
+        hip.sync()
+        print(f"sustain {operands}: {(time.perf_counter() - t0) / 2000 * 1e6:.1f} us per launch "
+              f"({hip.last_kernel()})", flush=True)
 
 
 def cpu_baseline():
@@ -519,7 +604,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--counter-probe", action="store_true")
+    ap.add_argument("--counter-probe", nargs="?", const="headline", default=None,
+                    choices=["headline", "skinny", "fp32", "config2", "attention"])
+    ap.add_argument("--probe-repeat", type=int, default=1, help="multiplies the launch counts of --counter-probe")
+    ap.add_argument("--sustain", type=float, default=0.0, help="seconds of back-to-back headline launches")
+    ap.add_argument("--operands", choices=["random", "zeros"], default="random")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -528,7 +617,10 @@ def main():
     hip = AxHip()
     hip.init()
     if args.counter_probe:
-        counter_probe(hip)
+        counter_probe(hip, args.counter_probe, args.probe_repeat)
+        return
+    if args.sustain > 0:
+        sustain(hip, args.sustain, args.operands)
         return
 
     h = headline(hip, args.steps, args.warmup)

@@ -47,6 +47,29 @@ int         axhip_device_count(void);         /* .device_count  */
 const char *axhip_last_error(void);           /* thread-local message of the last failure */
 const char *axhip_device_name(void);          /* gcnArchName of device 0, "" without a GPU */
 
+/* Tile-selection overrides, for re-measuring the dispatch thresholds without recompiling — the
+ * counterpart of AX_GEMM_MC / AX_GEMM_NC / AX_GEMM_KC (src/compute/backends/cpu_opt.c:512-539).
+ * Read from the environment by axhip_init and again by axhip_tuning_reload (which needs no GPU and
+ * returns how many variables were recognised); unset, empty or invalid values mean "choose by shape".
+ * A forced choice applies only where the shape permits that kernel; results do not depend on it.
+ *   AX_HIP_I8_TILE       64x64 | 64x64k2 | 128x128 | 256x256   W8A8 tile (256x256: M, N multiples of 256; k2: two
+ *                        wave sets split each K slab)
+ *   AX_HIP_I8_SPLITK     1..16      workgroups over K per W8A8 tile of 64x64 / 128x128 (1: never split)
+ *   AX_HIP_F32_TILE      64x64 | 64x64k2 | 128x256   fp32 tile on the aligned fast path (k2: two wave sets split each K slab)
+ *   AX_HIP_F32_SPLITK    1..4096    K ranges of the fp32 few-tile route (1: never split)
+ *   AX_HIP_SKINNY_BLOCKS 1..65535   workgroups the skinny-M route aims for
+ * axhip_tuning_get returns the value in effect (0: automatic; tiles as their first number, 64x64k2 as
+ * 642), or -1 for an unknown name. */
+int axhip_tuning_reload(void);
+int axhip_tuning_get(const char *name);
+
+/* Threading: compute entry points must be called from one host thread at a time.  They share a
+ * device workspace, arrival counters and a vector of ones that several of them keep data in across
+ * two or more launches (split-K partial sums, reduction partials, padded operand copies), all on the
+ * HIP null stream; a second thread issuing such a call in between would overwrite them.  This is the
+ * contract of the reference's backends (include/axiom/ops.h:17-19, cuda/internal.h:70-74).  Only
+ * axhip_malloc / axhip_free / axhip_alloc_stats may be called concurrently with anything. */
+
 /* ---- memory: .storage_alloc/.storage_free/.memcpy_* hooks
  *      (src/compute/backends/cuda/memory.cu:78-140).  axhip_malloc returns zero-filled
  *      memory like the reference's allocator (memory.cu:90), or NULL.  Blocks are pooled: axhip_free

@@ -43,7 +43,10 @@ INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300
                (65, 64, 256), (64, 68, 384), (2900, 3000, 128),
                # K a multiple of 16 off the 128 grid: the last slab's tail is zero-filled in LDS
                (100, 4096, 784), (64, 64, 16), (130, 260, 144), (256, 4096, 784), (2900, 3000, 400), (9, 4, 48),
-               (64, 128, 1040), (128, 128, 112)]
+               (64, 128, 1040), (128, 128, 112),
+               # few tiles against a long K: workgroups split K and the last one of a tile adds the int32 partials
+               (64, 1024, 4096), (64, 64, 8192), (256, 2048, 8192), (512, 1024, 4096), (100, 4096, 4096), (70, 200, 2064),
+               (128, 128, 2048)]
 
 
 @pytest.mark.parametrize("M,N,K", INT8_SHAPES)
@@ -326,6 +329,59 @@ def test_w8a8_dispatch_sweep(hip, oracle):
             (case, M, N, K, hip.last_kernel())
     say("  routes:", sorted(seen))
     assert len(seen) >= 3
+
+
+def test_forced_tiles_and_splits_keep_parity(hip, oracle):
+    """The environment overrides change which kernel runs, never the result: W8A8 accumulators and outputs stay
+    bit-exact and fp32 / skinny products stay inside their gates under every forced tile, split and block count."""
+    import os
+    names = ("AX_HIP_I8_TILE", "AX_HIP_I8_SPLITK", "AX_HIP_F32_TILE", "AX_HIP_F32_SPLITK", "AX_HIP_SKINNY_BLOCKS")
+    saved = {n: os.environ.get(n) for n in names}
+    rng = np.random.default_rng(77)
+    M, N, K = 256, 512, 2048
+    x, w = rng.integers(-127, 128, (M, K), dtype=np.int8), rng.integers(-127, 128, (N, K), dtype=np.int8)
+    ws, bias = rng.uniform(1e-3, 1e-2, N).astype(np.float32), rng.normal(0, 0.02, N).astype(np.float32)
+    want_acc = x.astype(np.int32) @ w.astype(np.int32).T
+    want_out = oracle.w8a8_epilogue(want_acc, np.float32(0.02), ws, bias, 1)
+    a, b = rng.uniform(-1, 1, (256, 1024)).astype(np.float32), rng.uniform(-1, 1, (1024, 512)).astype(np.float32)
+    ref = oracle.gemm_opt(a, b)
+    sa = rng.uniform(-1, 1, (3, 1024)).astype(np.float32)
+    sref = oracle.gemm_opt(sa, b)
+    dx, dw, dws, db, da, dbm, dsa = (hip.array(v) for v in (x, w, ws, bias, a, b, sa))
+    seen = set()
+    try:
+        for tile, split in (("64x64", "1"), ("64x64", "4"), ("64x64k2", "1"), ("64x64k2", "3"), ("128x128", "2"),
+                            ("256x256", "1"), ("", "16"), ("bogus", "99")):
+            os.environ["AX_HIP_I8_TILE"], os.environ["AX_HIP_I8_SPLITK"] = tile, split
+            hip.L.axhip_tuning_reload()
+            say("forced i8", tile, split)
+            out, acc = hip.qgemm_w8a8(dx, 0.02, dw, dws, db, 1)
+            seen.add(hip.last_kernel())
+            assert np.array_equal(acc.numpy(), want_acc), (tile, split, hip.last_kernel())
+            assert np.array_equal(out.numpy(), want_out), (tile, split, hip.last_kernel())
+        assert {"qgemm_w8a8_64x64_dma", "qgemm_w8a8_64x64_dma_splitk", "qgemm_w8a8_64x64k2_dma", "qgemm_w8a8_64x64k2_dma_splitk",
+                "qgemm_w8a8_128x128_dma_splitk", "qgemm_w8a8_256x256_dma"} <= seen, seen
+        seen = set()
+        for tile, split in (("64x64", "1"), ("64x64k2", "1"), ("128x256", "1"), ("", "4"), ("64x64", "8")):
+            os.environ["AX_HIP_F32_TILE"], os.environ["AX_HIP_F32_SPLITK"] = tile, split
+            hip.L.axhip_tuning_reload()
+            say("forced f32", tile, split)
+            got = hip.sgemm(da, dbm).numpy()
+            seen.add(hip.last_kernel())
+            check_fp32(oracle, got, a, b, ref=ref)
+        assert {"sgemm_nn_64x64_dma", "sgemm_nn_64x64k2_dma", "sgemm_nn_128x256_dma", "sgemm_splitk"} <= seen, seen
+        for blocks in ("8", "64", "4000"):
+            os.environ["AX_HIP_SKINNY_BLOCKS"] = blocks
+            hip.L.axhip_tuning_reload()
+            say("forced skinny blocks", blocks)
+            check_fp32(oracle, hip.sgemm_skinny(dsa, dbm).numpy(), sa, b, ref=sref)
+    finally:
+        for n, v in saved.items():
+            if v is None:
+                os.environ.pop(n, None)
+            else:
+                os.environ[n] = v
+        hip.L.axhip_tuning_reload()
 
 
 def test_w8a32_dispatch_sweep(hip, oracle):
