@@ -72,18 +72,27 @@ __device__ __forceinline__ float apply_act(float v, int act) {
 // Workgroup id -> output tile.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs,
 // each with its own L2; renumbering so that every XCD walks one contiguous run of tiles, in
 // bands of 4 tile-rows, keeps the operand panels an XCD re-reads inside that XCD's L2.
+// (An integer division by a run-time value costs some thirty vector instructions even when every
+// operand is the same for the whole workgroup, and in an fp32 MFMA kernel vector instructions take
+// the matrix core's issue slots: the common cases — a power-of-two tile count, full bands and full
+// groups — are therefore done with shifts, and the general division is kept for the rest.)
+__device__ __forceinline__ unsigned div_by(unsigned n, unsigned d) {
+    return (d & (d - 1)) == 0 ? n >> (31 - __builtin_clz(d)) : n / d;
+}
+
 __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int &tm, int &tn) {
-    const int total = tiles_m * tiles_n;
-    int id = bid;
-    if ((total & 7) == 0) id = (bid & 7) * (total >> 3) + (bid >> 3);
-    constexpr int BAND = 4;
-    const int per_band = BAND * tiles_n;
-    const int band = id / per_band;
-    const int first = band * BAND;
-    const int rows = (tiles_m - first) < BAND ? (tiles_m - first) : BAND;
-    const int in_band = id - band * per_band;
-    tm = first + in_band % rows;
-    tn = in_band / rows;
+    const unsigned total = (unsigned)tiles_m * (unsigned)tiles_n;
+    unsigned id = (unsigned)bid;
+    if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+    constexpr unsigned BAND = 4;
+    const unsigned per_band = BAND * (unsigned)tiles_n;
+    const unsigned band = div_by(id, per_band);
+    const unsigned first = band * BAND;
+    const unsigned rows = ((unsigned)tiles_m - first) < BAND ? ((unsigned)tiles_m - first) : BAND;
+    const unsigned in_band = id - band * per_band;
+    const unsigned q = rows == BAND ? in_band >> 2 : in_band / rows;
+    tm = (int)(first + (in_band - q * rows));
+    tn = (int)q;
 }
 
 // The same for a batched launch with grid (tiles, batch): the hardware numbers workgroups x
@@ -92,15 +101,22 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // batch entry runs on the same XCD, back to back, and that entry's operands are fetched into one
 // L2 only (a partial last group of `left` entries uses r % left, r / left).
 __device__ __forceinline__ void tile_of_batched_block(int tiles_m, int tiles_n, int &tm, int &tn, int64_t &batch) {
-    const int64_t tiles = (int64_t)tiles_m * tiles_n, entries = gridDim.y;
-    const int64_t lin = blockIdx.x + tiles * blockIdx.y;
-    const int64_t group = lin / (8 * tiles), r = lin - group * 8 * tiles;
-    const int64_t left = entries - group * 8, per = left < 8 ? left : 8;
-    batch = group * 8 + r % per;
-    const int tile = (int)(r / per);
+    const unsigned tiles = (unsigned)tiles_m * (unsigned)tiles_n, entries = gridDim.y;
+    // lin = x + tiles * y with x < tiles, so lin / (8 * tiles) = y / 8 and the remainder is x + tiles * (y % 8)
+    const unsigned group = blockIdx.y >> 3, r = blockIdx.x + tiles * (blockIdx.y & 7);
+    const unsigned left = entries - group * 8;
+    unsigned tile;
+    if (left >= 8) {
+        batch = (int64_t)(group * 8 + (r & 7));
+        tile = r >> 3;
+    } else {
+        tile = r / left;
+        batch = (int64_t)(group * 8 + (r - tile * left));
+    }
     // consecutive workgroups walk along a tile row: their write-backs fill whole output rows
-    tm = tile / tiles_n;
-    tn = tile - tm * tiles_n;
+    const unsigned row = div_by(tile, (unsigned)tiles_n);
+    tm = (int)row;
+    tn = (int)(tile - row * (unsigned)tiles_n);
 }
 
 // Sums NV per-lane values over the 64 lanes of a wave, all NV at once.  A butterfly per value

@@ -6,7 +6,7 @@ namespace {
 using namespace axhip;
 
 template <int OP>   // 0 relu, 1 gelu
-__global__ void __launch_bounds__(256) k_unary(const float *__restrict__ in, float *__restrict__ out,
+__global__ void __launch_bounds__(256) k_unary(const float *in, float *out,
                                                int64_t n, int vec) {
     const int64_t stride = (int64_t)gridDim.x * 256;
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -31,8 +31,8 @@ __global__ void __launch_bounds__(256) k_fill(float *__restrict__ dst, float val
 }
 
 __global__ void __launch_bounds__(256)
-k_bias_add(const float *__restrict__ in, const float *__restrict__ bias, int64_t axis_len,
-           int64_t inner, int64_t total, float *__restrict__ out) {
+k_bias_add(const float *in, const float *__restrict__ bias, int64_t axis_len,
+           int64_t inner, int64_t total, float *out) {
     const int64_t stride = (int64_t)gridDim.x * 256;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
         out[i] = in[i] + bias[(i / inner) % axis_len];

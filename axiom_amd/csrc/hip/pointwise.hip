@@ -66,7 +66,7 @@ __device__ __forceinline__ void row_offsets(const Bcast &g, IDX row, int64_t &oa
 // Otherwise one element per thread.
 template <int OP, bool VEC, typename IDX>
 __global__ void __launch_bounds__(256)
-k_binary(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out, Bcast g,
+k_binary(const float *a, const float *b, float *out, Bcast g,
          int64_t items) {
     const int64_t stride = (int64_t)gridDim.x * 256;
     const IDX per_row = (IDX)(VEC ? (g.inner + 3) / 4 : g.inner);
@@ -98,7 +98,7 @@ k_binary(const float *__restrict__ a, const float *__restrict__ b, float *__rest
 
 template <int OP>
 __global__ void __launch_bounds__(256)
-k_unary_p(const float *__restrict__ in, float *__restrict__ out, int64_t n, float p, int vec) {
+k_unary_p(const float *in, float *out, int64_t n, float p, int vec) {
     const int64_t stride = (int64_t)gridDim.x * 256;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (vec) {

@@ -55,7 +55,7 @@ struct LnArgs {
 // KIND 0: softmax, 1: layer norm.  Thread t of a row holds columns t, t + TPR, ...
 template <int TPR, int VPT, int KIND>
 __global__ void __launch_bounds__(256)
-k_rows_cached(const float *__restrict__ in, float *__restrict__ out, int64_t rows, int cols, LnArgs ln) {
+k_rows_cached(const float *in, float *out, int64_t rows, int cols, LnArgs ln) {
     __shared__ float lds[8];
     constexpr int RPB = 256 / TPR;
     const int t = threadIdx.x % TPR, wave = threadIdx.x >> 6;
@@ -149,7 +149,7 @@ constexpr int kBig = 1024, kBigWaves = kBig / 64;   // threads of the long-row k
 // columns of the ragged tail it picks up, in every pass, so it only ever re-reads its own LDS entries.
 template <int KIND>
 __global__ void __launch_bounds__(kBig)
-k_rows_lds(const float *__restrict__ in, float *__restrict__ out, int64_t cols, LnArgs ln) {
+k_rows_lds(const float *in, float *out, int64_t cols, LnArgs ln) {
     extern __shared__ __attribute__((aligned(16))) float rowbuf[];
     __shared__ float lds[2 * kBigWaves];
     const int t = threadIdx.x, wave = t >> 6;
@@ -233,7 +233,7 @@ k_rows_lds(const float *__restrict__ in, float *__restrict__ out, int64_t cols, 
 // spent on the maximum alone; the threads' pairs are joined as sum_i s_i * exp(m_i - M).
 template <int KIND>
 __global__ void __launch_bounds__(kBig)
-k_rows_streamed(const float *__restrict__ in, float *__restrict__ out, int64_t cols, LnArgs ln) {
+k_rows_streamed(const float *in, float *out, int64_t cols, LnArgs ln) {
     __shared__ float lds[2 * kBigWaves];
     const int t = threadIdx.x, wave = t >> 6;
     const int64_t row = blockIdx.x;
@@ -313,7 +313,7 @@ k_rows_streamed(const float *__restrict__ in, float *__restrict__ out, int64_t c
 // HBM latency, so a wave takes RPW consecutive rows and requests all of them before it reduces any.
 template <int VPT, int RPW, int KIND>
 __global__ void __launch_bounds__(256)
-k_rows_short(const float *__restrict__ in, float *__restrict__ out, int64_t rows, int cols, LnArgs ln) {
+k_rows_short(const float *in, float *out, int64_t rows, int cols, LnArgs ln) {
     const int t = threadIdx.x & 63;
     const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW;
     if (row0 >= rows) return;

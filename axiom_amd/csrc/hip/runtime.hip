@@ -225,6 +225,9 @@ int axhip_init(void) {
         return fail(AXHIP_ERR_BACKEND, "device 0 is %s; this library holds gfx950 code only",
                     prop.gcnArchName);
     if (int rc = axhip::skinny_setup()) return rc;
+    // the shared workspace and the arrival counters exist from the start (64 MiB, 4096 counters): a first
+    // call at a new shape then pays no allocation or device-wide wait unless it needs more than that
+    if (!axhip::workspace(size_t(64) << 20) || !axhip::strip_counters(4096)) return AXHIP_ERR_ALLOC;
     g_ready = 1;
     return AXHIP_OK;
 }

@@ -54,8 +54,13 @@ static ax_status_t as_matrix(const ax_tensor_t *t, const char *who, const char *
     m->p = (float *)t->storage->data + t->offset;
     m->rows = t->shape[0];
     m->cols = t->shape[1];
+    /* a view whose rows overlap or repeat (a stride-0 expanded row, say) is not a dense matrix with a pitch */
+    if (t->shape[0] > 1 && t->strides[0] < t->shape[1]) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "%s: rows of %s overlap (row stride %lld < %lld columns)", who, which,
+                   (long long)t->strides[0], (long long)t->shape[1]);
+        return AX_ERR_SHAPE_MISMATCH;
+    }
     m->ld = t->shape[0] > 1 ? t->strides[0] : t->shape[1];
-    if (m->ld < m->cols) m->ld = m->cols;
     return AX_OK;
 }
 

@@ -316,7 +316,16 @@ def test_elementwise_reduction_optimizer_slots(ax, oracle, golden):
     bad = ax.empty((7, 6))
     assert L.ax_compute_add(tm, tn, bad) == 3                      # [6,10] does not broadcast to [7,6]
     v.shape[0], v.shape[1], v.strides[0], v.strides[1] = 6, 10, 10, 1
-    ax.free(tm, tn, view, out, bad)
+    # a GEMM operand whose rows overlap (row stride below the row length, e.g. an expanded row) is refused,
+    # not read as a dense matrix
+    ga, gb, gout = ax.from_numpy(m), ax.from_numpy(oracle.uniform((10, 4), -1, 1)), ax.empty((6, 4))
+    assert L.ax_compute_gemm(ga, gb, gout) == 0
+    ga.contents.strides[0] = 0
+    assert L.ax_compute_gemm(ga, gb, gout) == 3 and "overlap" in ax.err()[1]
+    ga.contents.strides[0] = 5
+    assert L.ax_compute_gemm(ga, gb, gout) == 3
+    ga.contents.strides[0] = 10
+    ax.free(tm, tn, view, out, bad, ga, gb, gout)
     # unary / scalar / activation slots
     x = sc.unary_input(oracle)
     tx, out = ax.from_numpy(x), ax.empty(x.shape)

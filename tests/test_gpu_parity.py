@@ -608,6 +608,34 @@ def test_elementwise_slots(hip, oracle, golden):
     assert not z.numpy().any()
 
 
+def test_elementwise_in_place(hip, oracle):
+    """Calls whose output is their input (the host core does this for fused activations, residual bias adds and
+    the mean's final scale): same values as the out-of-place call."""
+    oracle.seed(81)
+    x = oracle.normal((513, 1027), 0, 2)            # odd row length: vector and element paths
+    n = x.size
+    bias = oracle.normal((1027,), 0, 1)
+    dbias = hip.array(bias)
+
+    def both(call):
+        src, dst = hip.array(x), hip.empty(x.shape)
+        call(src.ptr, dst.ptr)
+        want = dst.numpy()
+        call(src.ptr, src.ptr)
+        assert np.array_equal(src.numpy(), want, equal_nan=True)
+
+    both(lambda i, o: hip.check(hip.L.axhip_relu(i, o, n)))
+    both(lambda i, o: hip.check(hip.L.axhip_gelu(i, o, n)))
+    both(lambda i, o: hip.check(hip.L.axhip_unary(7, i, o, n, 0.0)))                  # tanh
+    both(lambda i, o: hip.check(hip.L.axhip_unary(12, i, o, n, 0.25)))                # mul_scalar
+    both(lambda i, o: hip.check(hip.L.axhip_bias_add(i, dbias.ptr, 513, 1027, 1, o)))
+    both(lambda i, o: hip.check(hip.L.axhip_softmax_rows(i, o, 513, 1027)))
+    import ctypes as C
+    shape, dense = (C.c_int64 * 2)(513, 1027), (C.c_int64 * 2)(1027, 1)
+    other = hip.array(oracle.normal((513, 1027), 0, 1))
+    both(lambda i, o: hip.check(hip.L.axhip_binary(0, i, other.ptr, o, 2, shape, dense, dense)))
+
+
 # ------------------------------------------------------------------ dense backward blocks
 SUM_BOUND = 1e-5     # |gpu - sum64| <= SUM_BOUND * sum |x|   (fp32 sums in a fixed parallel order)
 
