@@ -320,6 +320,35 @@ struct DmaOperand {
     static constexpr int k_imm(int k) { return KC ? 0 : (k / (256 / R)) * PITCH + (k % (256 / R)) * R * 4; }
 };
 
+// An int8 operand stored [rows, K] (K contiguous; the weights of the W8A32 product): a slab is 32 bytes
+// per row, one load instruction carries 32 rows (lane l -> row l >> 1, 16-byte half l & 1), and only the
+// first NINSTR waves have one to issue.  A fragment is one ds_read_b32 — the four k values a lane feeds
+// to the four MFMAs of a k-block — converted to fp32 in registers right before use, so LDS and the
+// loads carry a quarter of the bytes of an fp32 operand.  (Rows 32 bytes apart put the 32 lanes of a
+// read on 8 banks: a 4-way conflict on a read that is a quarter of the other operand's.)
+template <int R, int NW>
+struct DmaOperandI8 {
+    static constexpr int PITCH = 1024;
+    static constexpr int NINSTR = R / 32;
+    static constexpr int IPW = (NINSTR + NW - 1) / NW;
+    static constexpr int BYTES = NINSTR * PITCH;
+    static constexpr int READS = 1;
+    static_assert(R % 32 == 0, "whole load instructions");
+    __device__ static unsigned lane_offset(int q, int lane, int64_t ld, int valid = R) {
+        const int row = q * 32 + (lane >> 1);
+        return (unsigned)((row < valid ? row : valid - 1) * ld + (lane & 1) * 16);
+    }
+    __device__ static unsigned frag_base(int first, int frow, int fhalf, int kbi) {
+        return (unsigned)((first + frow) * 32 + kbi * 8 + fhalf * 4);
+    }
+    static constexpr int k_imm(int) { return 0; }
+};
+
+struct FragI8 {
+    int raw;       // k = 4 * (lane >> 5) + e of the k-block in byte e
+    __device__ __forceinline__ float get(int e) const { return (float)(signed char)(raw >> (8 * e)); }
+};
+
 template <bool KC> struct Frag;
 template <> struct Frag<true> {
     v4f q;
@@ -339,7 +368,7 @@ template <> struct Frag<false> {
 // and guard the write-back; in the last slab, lanes whose k values lie past K write zeros to
 // their LDS place instead of loading, in both operands, so the tail adds exact zeros.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI, int WAVES_K,
-          bool EDGE = false>
+          bool EDGE = false, typename BSRC = float>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(SgemmArgs g) {
     // WAVES_K == 2: a second set of waves shares each tile; set 0 multiplies k-blocks 0 and 1 of
     // every slab, set 1 k-blocks 2 and 3, and the two accumulators are added through LDS at the
@@ -348,8 +377,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     constexpr int NW = WAVES_M * WAVES_N * WAVES_K;
     static_assert(WAVES_K == 1 || WAVES_K == 2, "k split");
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
+    constexpr bool B_I8 = sizeof(BSRC) == 1;     // int8 B, [N, K]: W8A32 (K a multiple of 32, so no K tail)
+    static_assert(!B_I8 || (B_KC && NST == 2 && EPI == 1), "int8 B is K-contiguous, two stages, turned write-back");
     using OA = DmaOperand<BM, A_KC, NW>;
-    using OB = DmaOperand<BN, B_KC, NW>;
+    using OB = typename std::conditional<B_I8, DmaOperandI8<BN, NW>, DmaOperand<BN, B_KC, NW>>::type;
     // LDS: NST stages of A, then NST stages of B
     constexpr int B_BASE = NST * OA::BYTES;
     constexpr int NREADS = TM * OA::READS + TN * OB::READS;
@@ -370,7 +401,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int mvalid = EDGE && g.M - m0 < BM ? (int)(g.M - m0) : BM, nvalid = EDGE && g.N - n0 < BN ? (int)(g.N - n0) : BN;
     const float *A = static_cast<const float *>(g.A) + batch * g.stride_a;
-    const float *B = static_cast<const float *>(g.B) + batch * g.stride_b;
+    const BSRC *B = static_cast<const BSRC *>(g.B) + batch * g.stride_b;
     float *C = g.C + batch * g.stride_c;
     // EDGE also takes a K that ends inside a slab (K a multiple of 4): the last slab's lanes whose four
     // k values lie past K load nothing and write zeros to their LDS place instead
@@ -386,7 +417,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     for (int j = 0; j < OB::IPW; j++) vb[j] = OB::lane_offset(j * NW + wave, lane, g.ldb, nvalid);
     const char *ga = reinterpret_cast<const char *>(A_KC ? A + m0 * g.lda : A + m0);
     const char *gb = reinterpret_cast<const char *>(B_KC ? B + n0 * g.ldb : B + n0);
-    const int64_t step_a = A_KC ? 128 : 128 * g.lda, step_b = B_KC ? 128 : 128 * g.ldb;   // bytes per slab
+    const int64_t step_a = A_KC ? 128 : 128 * g.lda, step_b = B_KC ? 32 * (int64_t)sizeof(BSRC) : 128 * g.ldb;   // bytes per slab
     const unsigned lds0 = (unsigned)(uintptr_t)lds_raw;
     const unsigned dma_a = lds0 + wave * OA::PITCH, dma_b = lds0 + wave * OB::PITCH;
     // does this lane's 16 bytes of load instruction j lie inside K in the last slab
@@ -399,7 +430,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
 #pragma unroll
     for (int j = 0; j < OB::IPW; j++) {
         const int q = j * NW + wave, row = q * 8 + (lane >> 3);
-        tb[j] = B_KC ? (((lane & 7) ^ ((row >> 1) & 7)) * 4 < ktail) : (q * (256 / BN) + lane / (64 / (256 / BN)) < ktail);
+        tb[j] = B_I8 ? true
+                : B_KC ? (((lane & 7) ^ ((row >> 1) & 7)) * 4 < ktail) : (q * (256 / BN) + lane / (64 / (256 / BN)) < ktail);
     }
 
     // ---- LDS -> fragments ----
@@ -426,7 +458,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     Frag<A_KC> fa[2][TM];
-    Frag<B_KC> fb[2][TN];
+    typename std::conditional<B_I8, FragI8, Frag<B_KC>>::type fb[2][TN];
 
 // loads of the next unread slab into stage ST
 #define AXF_ISSUE(ST)                                                                            \
@@ -447,7 +479,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
             _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                                  \
                 AXF_LOAD_LDS(dma_a + (ST) * OA::BYTES + j * NW * OA::PITCH, va[j], ga);          \
             _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                                  \
-                AXF_LOAD_LDS(dma_b + B_BASE + (ST) * OB::BYTES + j * NW * OB::PITCH, vb[j], gb); \
+                if (!B_I8 || j * NW + wave < OB::NINSTR)                                         \
+                    AXF_LOAD_LDS(dma_b + B_BASE + (ST) * OB::BYTES + j * NW * OB::PITCH, vb[j], gb); \
         }                                                                                        \
         ga += step_a;                                                                            \
         gb += step_b;                                                                            \
@@ -467,7 +500,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
             }                                                                                    \
         }                                                                                        \
         _Pragma("unroll") for (int t = 0; t < TN; t++) {                                         \
-            if constexpr (B_KC) {                                                                \
+            if constexpr (B_I8) {                                                                \
+                AXF_DS32(fb[BUF][t].raw, rb[ST][KBI], t * 1024);                                 \
+            } else if constexpr (B_KC) {                                                         \
                 AXF_DS128(fb[BUF][t].q, rb[ST][KBI], t * 4096);                                  \
             } else {                                                                             \
                 AXF_DS32(fb[BUF][t].s0, rb[ST][0], OB::k_imm((KBI) * 8 + 0) + t * 128);          \
@@ -599,8 +634,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const bool col_in = !EDGE || col0 + j * 32 < g.N;          // N % 4 == 0: the whole group or none of it
-            v4f bv = {0.f, 0.f, 0.f, 0.f};
+            v4f bv = {0.f, 0.f, 0.f, 0.f}, cs = {1.f, 1.f, 1.f, 1.f};
             if (bp && col_in) bv = *reinterpret_cast<const v4f *>(bp + j * 32);
+            if (g.col_scale && col_in) cs = *reinterpret_cast<const v4f *>(g.col_scale + col0 + j * 32);
 #pragma unroll
             for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -626,6 +662,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
                     float *cp = dst + (int64_t)(i * 32 + p * 8) * g.ldc + j * 32;
                     v4f o = r[p];
                     if (g.alpha != 1.0f) o *= g.alpha;
+                    if (g.col_scale) o *= cs;
                     if (use_beta) o += g.beta * *reinterpret_cast<const v4f *>(cp);
                     if (bp) o += bv;
 #pragma unroll
@@ -640,12 +677,15 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI = 1, int WAVES_K = 1,
-          bool EDGE = false>
+          bool EDGE = false, typename BSRC = float>
 int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
     static_assert(!EDGE || EPI == 1, "the edge form guards the turned write-back only");
-    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K, EDGE>;
+    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K, EDGE, BSRC>;
     constexpr int NW = WAVES_M * WAVES_N * WAVES_K;
-    constexpr int smem = NST * (DmaOperand<BM, A_KC, NW>::BYTES + DmaOperand<BN, B_KC, NW>::BYTES);
+    using OB = typename std::conditional<sizeof(BSRC) == 1, DmaOperandI8<BN, NW>, DmaOperand<BN, B_KC, NW>>::type;
+    constexpr int stage_bytes = NST * (DmaOperand<BM, A_KC, NW>::BYTES + OB::BYTES);
+    // the write-back turns 4 KiB per output wave through the dead stages
+    constexpr int smem = stage_bytes > WAVES_M * WAVES_N * 4096 ? stage_bytes : WAVES_M * WAVES_N * 4096;
     static bool attr_set = false;
     if (!attr_set) {
         AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -695,6 +735,30 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
         return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[2], g, batch);
     }
     return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
+}
+
+// The same fast path with int8 weights as the B operand (W8A32: A fp32 [M,K], B int8 [N,K], the
+// per-column scale applied in the write-back).  K must be a multiple of 32 (whole slabs, rows of B on
+// 16-byte boundaries); M and N may be off the tile grid.  Returns -1 when the shape does not qualify.
+const char *const kI8DmaNames[3] = {"qgemm_w8a32_mfma_128x256_dma", "qgemm_w8a32_mfma_64x64_dma", "qgemm_w8a32_mfma_64x64k2_dma"};
+int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
+    const bool ok = g.K % 32 == 0 && g.K > 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
+                    ((uintptr_t)g.C % 16 == 0) && ((uintptr_t)g.bias % 16 == 0) && ((uintptr_t)g.col_scale % 16 == 0) &&
+                    g.lda % 4 == 0 && g.ldb % 16 == 0 && g.ldc % 4 == 0 && g.stride_a % 4 == 0 && g.stride_b % 16 == 0 &&
+                    g.stride_c % 4 == 0 && g.lda < (1 << 20) && g.ldb < (1 << 22) && batch <= 65535 && g.N % 4 == 0 &&
+                    ((g.M + 63) / 64) * ((g.N + 63) / 64) <= 0x7fffffff;
+    if (!ok) return -1;
+    if (g.M % 64 != 0 || g.N % 64 != 0) {
+        if (g.K > 128) return launch_dma<64, 64, 2, 2, 2, true, true, 1, 2, true, int8_t>(names[2], g, batch);
+        return launch_dma<64, 64, 2, 2, 2, true, true, 1, 1, true, int8_t>(names[1], g, batch);
+    }
+    if (g.K > 128) {
+        const int64_t big = (g.M / 128) * (g.N / 256) * batch, cus = cu_count(), rounds = (big + cus - 1) / cus;
+        if (g.M % 128 == 0 && g.N % 256 == 0 && big >= 256 && big * 10 >= rounds * cus * 9)
+            return launch_dma<128, 256, 2, 4, 2, true, true, 1, 1, false, int8_t>(names[0], g, batch);
+        return launch_dma<64, 64, 2, 2, 2, true, true, 1, 2, false, int8_t>(names[2], g, batch);
+    }
+    return launch_dma<64, 64, 2, 2, 2, true, true, 1, 1, false, int8_t>(names[1], g, batch);
 }
 
 // ---- split-K for shapes with few output tiles -----------------------------------------
@@ -794,7 +858,10 @@ int try_split_k(const SgemmArgs &g, int transa, int transb, const char *name, co
     p.act = AXHIP_ACT_NONE;
     int rc;
     if (std::is_same<BSRC, float>::value) rc = dispatch_f32(p, transa, transb, splits);
-    else rc = pick_tile<true, true, int8_t>(i8_names, p, splits);
+    else {
+        rc = try_dma_i8(kI8DmaNames, p, splits);
+        if (rc < 0) rc = pick_tile<true, true, int8_t>(i8_names, p, splits);
+    }
     if (rc) return rc;
     const bool vec = g.N % 4 == 0 && g.ldc % 4 == 0 && (((uintptr_t)g.C | (uintptr_t)g.bias) & 15) == 0;
     const int64_t items = g.M * (vec ? g.N / 4 : g.N);
@@ -928,7 +995,9 @@ int sgemm_i8w(int64_t M, int64_t N, int64_t K, const float *a, const int8_t *w,
     SgemmArgs g{a, w, out, M, N, K, K, K, N, 0, 0, 0, 1.0f, 0.0f, w_scales, nullptr, AXHIP_ACT_NONE};
     auto run = [&](const SgemmArgs &p) {
         const int rc = try_split_k<int8_t>(p, 0, 1, "qgemm_w8a32_mfma_splitk", names);
-        return rc >= 0 ? rc : pick_tile<true, true, int8_t>(names, p, 1);
+        if (rc >= 0) return rc;
+        const int rd = try_dma_i8(kI8DmaNames, p, 1);
+        return rd >= 0 ? rd : pick_tile<true, true, int8_t>(names, p, 1);
     };
     // K off the 32 grid cannot be cut into ranges: the first K / 32 * 32 columns as above, then the
     // remaining few accumulated on top (the column scale applies to each part's sum alike)
