@@ -699,6 +699,203 @@ int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
     return check_launch(name);
 }
 
+// =====================================================================================
+// C = alpha * A * B^T with a short K (32, 64, 96 or 128: the scores Q K^T of attention heads), both
+// operands K-contiguous.  A product this shape writes eight times what it reads per workgroup and has
+// only a few dozen MFMAs per output tile, so a workgroup per tile spends its life in its prologue, its
+// load latency and its write-back.  Here a workgroup keeps a 128-row block of A in LDS for its whole
+// life and walks the 64-column blocks of B^T through two buffers: the loads of block j+1 and the stores
+// of tile j-1 are in flight while tile j is multiplied, and the address arithmetic is paid once per
+// workgroup.  Within a wave, loads are issued before the stores they must not wait behind (loads and
+// stores retire in issue order), so the wait for block j+1 never includes the stores of tile j-1.
+// 4 waves as 2 (M) x 2 (N), wave tile 64 x 32.  LDS: A block KS x 16 KiB, two B blocks KS x 8 KiB each,
+// 4 KiB per wave to turn the write-back into whole 128-byte rows; two workgroups share a CU up to K = 64.
+template <int KS>
+__global__ void __launch_bounds__(256) k_sgemm_nt_rows(SgemmArgs g) {
+    constexpr int BM = 128, BN = 64, NW = 4, TM = 2;
+    using OA = DmaOperand<BM, true, NW>;
+    using OB = DmaOperand<BN, true, NW>;
+    constexpr int A_BYTES = KS * OA::BYTES, B_BYTES = KS * OB::BYTES;     // the resident block, one B buffer
+    constexpr int B_BASE = A_BYTES, TURN_BASE = A_BYTES + 2 * B_BYTES;
+    constexpr int NSTORES = TM * 4;                                       // store instructions of a wave per tile
+    static_assert(KS >= 1 && KS <= 4 && TURN_BASE + NW * 4096 <= 160 * 1024, "LDS budget");
+    static_assert(3 * OA::BYTES + 4096 < 65536 && B_BYTES + 3 * OB::BYTES < 65536, "ds_read immediates are 16 bits");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    int tm = (int)blockIdx.x, tn = 0;
+    int64_t batch = 0;
+    if (gridDim.y > 1) tile_of_batched_block((int)(g.M / BM), 1, tm, tn, batch);
+    const int64_t m0 = (int64_t)tm * BM;
+    const float *A = static_cast<const float *>(g.A) + batch * g.stride_a + m0 * g.lda;
+    const float *B = static_cast<const float *>(g.B) + batch * g.stride_b;
+    float *C = g.C + batch * g.stride_c + m0 * g.ldc;
+    const int nblk = (int)(g.N / BN);
+
+    unsigned va[OA::IPW], vb[OB::IPW];
+#pragma unroll
+    for (int j = 0; j < OA::IPW; j++) va[j] = OA::lane_offset(j * NW + wave, lane, g.lda);
+#pragma unroll
+    for (int j = 0; j < OB::IPW; j++) vb[j] = OB::lane_offset(j * NW + wave, lane, g.ldb);
+    const char *ga = reinterpret_cast<const char *>(A), *gb = reinterpret_cast<const char *>(B);
+    const int64_t step_b = (int64_t)BN * g.ldb * 4;                       // bytes from one block of B to the next
+    const unsigned lds0 = (unsigned)(uintptr_t)lds_raw;
+    const unsigned dma_a = lds0 + wave * OA::PITCH, dma_b = lds0 + B_BASE + wave * OB::PITCH;
+
+    const int frow = lane & 31, fhalf = lane >> 5;
+    unsigned ra[4], rb[4];
+#pragma unroll
+    for (int kbi = 0; kbi < 4; kbi++) {
+        ra[kbi] = lds0 + OA::frag_base(wm * 64, frow, fhalf, kbi);
+        rb[kbi] = lds0 + B_BASE + OB::frag_base(wn * 32, frow, fhalf, kbi);
+    }
+    unsigned char *turn = lds_raw + TURN_BASE + wave * 4096;
+    const int rrow = lane >> 3, rchunk = lane & 7;
+    // where this lane's 16 bytes of a write-back row go, relative to the tile's first row and column block
+    float *cdst = C + (int64_t)(wm * 64 + rrow) * g.ldc + wn * 32 + rchunk * 4;
+
+    v16f acc[TM];
+    Frag<true> fa[2][TM], fb[2];
+
+// loads of the next block of B into buffer BUFK
+#define AXN_ISSUE_B(BUFK)                                                                        \
+    do {                                                                                         \
+        _Pragma("unroll") for (int s = 0; s < KS; s++)                                           \
+            _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                                  \
+                AXF_LOAD_LDS(dma_b + (BUFK) * B_BYTES + s * OB::BYTES + j * NW * OB::PITCH, vb[j], gb + s * 128); \
+        gb += step_b;                                                                            \
+    } while (0)
+// fragments of k-block KK (slab KK >> 2, block KK & 3) out of B buffer BUFK
+#define AXN_FRAGS(BUF, BUFK, KK)                                                                 \
+    do {                                                                                         \
+        AXF_DS128(fa[BUF][0].q, ra[(KK) & 3], ((KK) >> 2) * OA::BYTES);                          \
+        AXF_DS128(fa[BUF][1].q, ra[(KK) & 3], ((KK) >> 2) * OA::BYTES + 4096);                   \
+        AXF_DS128(fb[BUF].q, rb[(KK) & 3], (BUFK) * B_BYTES + ((KK) >> 2) * OB::BYTES);          \
+    } while (0)
+// one tile out of B buffer BUFK: 4 * KS k-blocks, the fragments of the next one requested before the
+// MFMAs of the current; the first MFMA of each accumulator starts from zero
+#define AXN_TILE(BUFK)                                                                           \
+    do {                                                                                         \
+        AXN_FRAGS(0, BUFK, 0);                                                                   \
+        _Pragma("unroll") for (int kk = 0; kk < 4 * KS; kk++) {                                  \
+            if (kk + 1 < 4 * KS) {                                                               \
+                AXN_FRAGS((kk + 1) & 1, BUFK, kk + 1);                                           \
+                AXF_LGKM(3);                                                                     \
+            } else {                                                                             \
+                AXF_LGKM(0);                                                                     \
+            }                                                                                    \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+            _Pragma("unroll") for (int e = 0; e < 4; e++)                                        \
+                _Pragma("unroll") for (int i = 0; i < TM; i++)                                   \
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[kk & 1].get(e), fa[kk & 1][i].get(e), \
+                                                                  (kk == 0 && e == 0) ? zero : acc[i], 0, 0, 0); \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+        }                                                                                        \
+    } while (0)
+
+    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // Write-back of the tile in `acc` (columns n0 ..): each 32x32 sub-tile is turned through the wave's
+    // 4 KiB of LDS (16-byte chunk c of row r at chunk c ^ ((r >> 1) & 7), conflict-free both ways) so
+    // that a store instruction writes 8 rows of 128 contiguous bytes; streaming stores, the scores are
+    // not read again by this kernel.
+    auto write_back = [&](int64_t n0) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int gq = 0; gq < 4; gq++)
+                *reinterpret_cast<v4f *>(turn + frow * 128 + (((2 * gq + fhalf) ^ ((frow >> 1) & 7)) << 4)) =
+                    v4f{acc[i][4 * gq], acc[i][4 * gq + 1], acc[i][4 * gq + 2], acc[i][4 * gq + 3]};
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            v4f r[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const int row = p * 8 + rrow;
+                r[p] = *reinterpret_cast<const v4f *>(turn + row * 128 + ((rchunk ^ ((row >> 1) & 7)) << 4));
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                v4f o = r[p];
+                if (g.alpha != 1.0f) o *= g.alpha;
+                __builtin_nontemporal_store(o, reinterpret_cast<v4f *>(cdst + (int64_t)(i * 32 + p * 8) * g.ldc + n0));
+            }
+        }
+    };
+    // One tile.  Order inside a wave: the loads of the block after this one, then the stores of the tile
+    // before this one, then this tile's MFMAs; the wait that follows passes over the stores (NSTORES of
+    // them are younger than the loads) and the barrier makes every wave's part of the next block visible
+    // and frees this tile's buffer for the loads after next.
+#define AXN_STEP(BUFK, j)                                                                        \
+    do {                                                                                         \
+        const bool more = (j) + 1 < nblk;                                                        \
+        if (more) AXN_ISSUE_B(1 - (BUFK));                                                       \
+        if ((j) > 0) write_back((int64_t)((j) - 1) * BN);                                        \
+        AXN_TILE(BUFK);                                                                          \
+        if (more) {                                                                              \
+            if ((j) > 0) AXF_VM(NSTORES); else AXF_VM(0);                                        \
+            __builtin_amdgcn_s_barrier();                                                        \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+        }                                                                                        \
+    } while (0)
+
+#pragma unroll
+    for (int s = 0; s < KS; s++)
+#pragma unroll
+        for (int j = 0; j < OA::IPW; j++)
+            AXF_LOAD_LDS(dma_a + s * OA::BYTES + j * NW * OA::PITCH, va[j], ga + s * 128);
+    AXN_ISSUE_B(0);
+    AXF_VM(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    for (int j = 0; j < nblk; j += 2) {
+        AXN_STEP(0, j);
+        if (j + 1 >= nblk) break;
+        AXN_STEP(1, j + 1);
+    }
+    write_back((int64_t)(nblk - 1) * BN);
+#undef AXN_ISSUE_B
+#undef AXN_FRAGS
+#undef AXN_TILE
+#undef AXN_STEP
+}
+
+template <int KS>
+int launch_nt_rows(const SgemmArgs &g, int64_t batch) {
+    constexpr int smem = KS * (16 + 2 * 8) * 1024 + 4 * 4096;
+    static bool attr_set = false;
+    if (!attr_set) {
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sgemm_nt_rows<KS>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem),
+                      "hipFuncSetAttribute");
+        attr_set = true;
+    }
+    note_kernel("sgemm_nt_rows128_dma");
+    hipLaunchKernelGGL((k_sgemm_nt_rows<KS>), dim3((unsigned)(g.M / 128), (unsigned)batch), dim3(256), smem, kStream, g);
+    return check_launch("sgemm_nt_rows128_dma");
+}
+
+// The short-K NT route: K a multiple of 32 up to 128, M on the 128 grid, N on the 64 grid with at least
+// four column blocks, no beta / bias / activation, enough row blocks for the chip.  -1: not taken.
+int try_nt_rows(const SgemmArgs &g, int64_t batch) {
+    if (tuning().f32_tile != 0) return -1;
+    if (g.K % 32 != 0 || g.K < 32 || g.K > 128 || g.M % 128 != 0 || g.N % 64 != 0 || g.N < 256) return -1;
+    if (g.beta != 0.0f || g.bias || g.col_scale || g.act != AXHIP_ACT_NONE) return -1;
+    if ((g.M / 128) * batch < 2 * cu_count() || batch > 65535 || g.M / 128 > 0x7fffffff) return -1;
+    if ((((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.C) & 15) != 0 || g.lda % 4 != 0 || g.ldb % 4 != 0 || g.ldc % 4 != 0 ||
+        g.stride_a % 4 != 0 || g.stride_b % 4 != 0 || g.stride_c % 4 != 0 || g.lda >= (1 << 20) || g.ldb >= (1 << 20))
+        return -1;
+    switch (g.K / 32) {
+        case 1: return launch_nt_rows<1>(g, batch);
+        case 2: return launch_nt_rows<2>(g, batch);
+        case 3: return launch_nt_rows<3>(g, batch);
+        default: return launch_nt_rows<4>(g, batch);
+    }
+}
+
 // Chooses the largest tile that still leaves about eight waves per CU; returns -1 when the
 // shape does not qualify for the fast path (the caller then uses the register-staged kernel).
 // names: 128x256, 64x64, 64x64 with the k split.
@@ -889,6 +1086,8 @@ int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     static const char *const nt_d[3] = {"sgemm_nt_128x256_dma", "sgemm_nt_64x64_dma", "sgemm_nt_64x64k2_dma"};
     static const char *const tn_d[3] = {"sgemm_tn_128x256_dma", "sgemm_tn_64x64_dma", "sgemm_tn_64x64k2_dma"};
     int rc = -1;
+    if (!transa && transb) rc = try_nt_rows(g, batch);
+    if (rc >= 0) return rc;
     if (!transa && !transb) rc = try_dma<true, false>(nn_d, g, batch);
     else if (!transa && transb) rc = try_dma<true, true>(nt_d, g, batch);
     else if (transa && !transb) rc = try_dma<false, false>(tn_d, g, batch);

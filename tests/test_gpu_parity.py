@@ -537,6 +537,33 @@ def test_config4b_attention_shapes_full_size(hip, oracle):
     assert (np.abs(got - want) <= 1e-5 * scale).all()
 
 
+@pytest.mark.parametrize("Bn,M,N,K,alpha", [(600, 128, 256, 64, 1.0), (300, 256, 320, 32, 0.5), (130, 512, 512, 96, 0.125),
+                                             (520, 128, 448, 128, 1.0), (1, 65536, 256, 64, 2.0), (513, 128, 256, 64, 1.0)])
+def test_short_k_nt_row_blocks(hip, oracle, Bn, M, N, K, alpha):
+    """A B^T with K of 32..128 and many row blocks: the kernel that keeps a 128-row block of A in LDS and
+    walks the column blocks; against the fp64 bound and, on sampled batch entries, the CPU path."""
+    say("short-k nt", Bn, M, N, K, alpha)
+    oracle.seed(Bn + M + N + K)
+    a, b = oracle.normal((Bn, M, K)), oracle.normal((Bn, N, K))
+    da, db = hip.array(a), hip.array(b)
+    c = hip.empty((Bn, M, N))
+    hip.check(hip.L.axhip_memset(c.ptr, 0xFF, c.nbytes))                 # every output must be written
+    hip.check(hip.L.axhip_sgemm_strided_batched(0, 1, M, N, K, alpha, da.ptr, K, M * K, db.ptr, K, N * K, 0.0,
+                                                c.ptr, N, M * N, Bn))
+    assert hip.last_kernel() == "sgemm_nt_rows128_dma"
+    got = c.numpy()
+    assert not np.isnan(got).any()
+    for h in sorted({0, Bn // 2, Bn - 1}):
+        rows = slice(0, min(M, 1024))
+        want = oracle.gemm_opt_nt(a[h][rows], b[h]) * np.float32(alpha)
+        assert np.abs(got[h][rows] - want).max() <= REL_FP32 * np.abs(want).max()
+    # every entry: row sums of C equal alpha * A . (sum of B's rows), to fp32 accumulation accuracy
+    bsum = b.astype(np.float64).sum(axis=1)
+    want = alpha * np.einsum("hmk,hk->hm", a.astype(np.float64), bsum)
+    scale = abs(alpha) * np.einsum("hmk,hk->hm", np.abs(a).astype(np.float64), np.abs(b).astype(np.float64).sum(axis=1))
+    assert (np.abs(got.astype(np.float64).sum(axis=2) - want) <= 1e-5 * scale).all()
+
+
 # ------------------------------------------------------------------ W8A32
 W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 1024), (3, 17, 45),
                 (1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024),
