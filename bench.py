@@ -9,7 +9,7 @@ and the skinny-M route's GB/s, each with its own roofline fraction.  RESULT line
 reference's benchmark format (benchmarks/bench_common.h:25-42) go to stderr.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu]
-    python bench.py --counter-probe [headline|skinny|fp32|config2|attention]
+    python bench.py --counter-probe [headline|skinny|gemm1024|fp32|config2|attention]
                                         # for hardware-counter runs: a few launches of one case's kernels and 3
                                         # launches of a copy-shaped kernel of known size, no output line
     python bench.py --sustain 8 [--operands zeros]   # back-to-back headline launches, for clock sampling
@@ -430,7 +430,8 @@ def counter_probe(hip, case, repeat=1):
       headline  W8A8 8192^3
       skinny    the 4096 x 4096 layer of the bs=1 MLP at M = 1 and M = 8 over 8 rotating weight sets
                 (537 MB, so every launch streams its 67.1 MB from HBM and not from the Infinity Cache)
-      fp32      1024^3, then the FFN pair 2048 x 1024 x 4096 (bias + GELU fused) and back
+      gemm1024  fp32 1024^3
+      fp32      the FFN pair 2048 x 1024 x 4096 (bias + GELU fused into the first GEMM) and back
       config2   W8A8 M = 256, N = K = 4096
       attention batched Q K^T and P V over 512 heads of [512, 64], then the fused forward"""
     rng = np.random.default_rng(0)
@@ -455,13 +456,15 @@ def counter_probe(hip, case, repeat=1):
                 hip.check(L.axhip_sgemm(0, 0, M, 4096, 4096, 1.0, xin.ptr, 4096, sets[i % 8].ptr, 4096, 0.0,
                                         h2.ptr, 4096, zeros.ptr, 1))
             what += f"{16 * repeat} x sgemm M={M} 4096x4096 ({hip.last_kernel()}) "
-    elif case == "fp32":
+    elif case == "gemm1024":
         a = hip.array(rng.uniform(-1, 1, (1024, 1024)).astype(np.float32))
         b = hip.array(rng.uniform(-1, 1, (1024, 1024)).astype(np.float32))
         c = hip.empty((1024, 1024))
-        for _ in range(8 * repeat):
+        for _ in range(16 * repeat):
             hip.check(L.axhip_sgemm(0, 0, 1024, 1024, 1024, 1.0, a.ptr, 1024, b.ptr, 1024, 0.0, c.ptr, 1024, None, 0))
-        what = f"{8 * repeat} x sgemm 1024^3 ({hip.last_kernel()}) "
+        what = f"{16 * repeat} x sgemm 1024^3 ({hip.last_kernel()})"
+    elif case == "fp32":
+        what = ""
         x = hip.array(rng.normal(0, 1, (2048, 1024)).astype(np.float32))
         w1 = hip.array(rng.normal(0, 0.02, (1024, 4096)).astype(np.float32))
         w2 = hip.array(rng.normal(0, 0.02, (4096, 1024)).astype(np.float32))
@@ -605,7 +608,7 @@ def main():
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--counter-probe", nargs="?", const="headline", default=None,
-                    choices=["headline", "skinny", "fp32", "config2", "attention"])
+                    choices=["headline", "skinny", "gemm1024", "fp32", "config2", "attention"])
     ap.add_argument("--probe-repeat", type=int, default=1, help="multiplies the launch counts of --counter-probe")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of back-to-back headline launches")
     ap.add_argument("--operands", choices=["random", "zeros"], default="random")
