@@ -87,6 +87,9 @@ SIGNATURES = {
     "ax_compute_has_gemm_relu": (C.c_int, []), "ax_compute_has_gemm_nt": (C.c_int, []),
     "ax_compute_has_gemm_tn": (C.c_int, []), "ax_compute_has_gemm_ex": (C.c_int, []),
     "ax_compute_has_bias_add": (C.c_int, []), "ax_compute_has_gemm_bias_act": (C.c_int, []),
+    "ax_compute_has_gemm_act_head": (C.c_int, []),
+    "ax_compute_gemm_act_head": (C.c_int, [TP, TP, TP, C.c_int, TP, TP, C.c_int, TP]),
+    "ax_matmul_bias_act_head": (TP, [TP, TP, TP, C.c_int, TP, TP, C.c_int]),
     "ax_device_count": (C.c_int, [C.c_int]), "ax_device_synchronize": (None, [C.c_int]),
     "ax_device_is_available": (C.c_int, [C.c_int]),
     "ax_err_clear": (None, []), "ax_err_last_status": (C.c_int, []),

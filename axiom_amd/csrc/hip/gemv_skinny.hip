@@ -24,14 +24,32 @@ constexpr int UNROLL = 8;
 // workgroups to aim for: enough to cover 256 CUs a few times over; partial-sum traffic grows with M
 constexpr int64_t kWantBlocksM12 = 1024, kWantBlocksM3up = 512;      // M = 1, 2 / M >= 3
 
+// A narrow layer riding on this one: out2[m, j] = act2(sum_n C[m, n] * W[n, j] + bias2[j]), j < nh <= 16
+// (a hidden layer followed by a classifier head).  The workgroup that finishes a strip has that strip's 64
+// finished outputs per row in hand and multiplies them by the head's 64 x nh block of weights at once;
+// the strips' contributions are joined like the splits of a strip: partial vectors out, an arrival counter,
+// the last strip adds them in strip order.  That is one more join at the end of this launch instead of a
+// launch of its own, whose time would be almost all fixed cost.
+struct SkinnyHead {
+    const float *W;        // [N, nh] dense; null: no head
+    const float *bias;     // [nh] or null
+    float *out;            // [MR, nh] dense
+    float *part;           // [strips][MR][nh] partial vectors
+    int *counter;          // one arrival counter, zero between launches
+    int nh, act, strips;
+    int keep;              // also write this layer's own output C
+};
+
 template <int MR, bool VEC>
 __global__ void __launch_bounds__(256)
 k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, int64_t ldb,
          float *__restrict__ dst, int64_t dst_ld, int64_t dst_split_stride, int64_t N, int64_t K,
          int64_t k_per_split, const float *__restrict__ bias, int act, int splits,
-         float *__restrict__ C, int64_t ldc, int *__restrict__ counters) {
+         float *__restrict__ C, int64_t ldc, int *__restrict__ counters, SkinnyHead head) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
-    // sm: [MR][k_per_split] activations, then [KGROUPS or 4][MR][COLS] partial sums
+    __shared__ int head_last;
+    // sm: [MR][k_per_split] activations, then [KGROUPS or 4][MR][COLS] partial sums, then (with a head)
+    // [MR][COLS] finished outputs of the strip
     const int tid = threadIdx.x;
     const int cg = tid & 15;            // column group: columns 4*cg .. 4*cg+3 of the 64
     const int kg = tid >> 4;            // lane group
@@ -64,6 +82,18 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
 #pragma unroll
         for (int u = 0; u < UNROLL; u++)
             w0[u] = *reinterpret_cast<const v4f *>(bp + (k_begin + k + u * KGROUPS) * ldb);
+    }
+
+    // the head's block of weights for this strip (64 rows x nh <= 1024 floats), requested now so that it
+    // is in LDS long before a finishing workgroup needs it
+    float hw[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (head.W) {
+        const int cols = N - n0 < COLS ? (int)(N - n0) : COLS;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int e = tid + q * 256;
+            if (e < cols * head.nh) hw[q] = head.W[n0 * head.nh + e];
+        }
     }
 
     float *xs = sm;
@@ -188,6 +218,54 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
     }
     __syncthreads();
 
+    float *hs = red + NPART * MR * COLS;                          // the strip's finished outputs, for the head
+    float *hws = hs + MR * COLS;                                  // the head's [64][nh] block of weights
+    // The head's share of a finished strip (every thread of the finishing workgroup calls this).
+    auto head_tail = [&]() {
+        const int nh = head.nh, hm = tid / nh, hj = tid - hm * nh;
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (tid + q * 256 < COLS * nh) hws[tid + q * 256] = hw[q];
+        __syncthreads();                                          // hs and hws are complete
+        const bool mine = tid < MR * nh;
+        if (mine) {
+            float sum = 0.0f;
+            const int cols = N - n0 < COLS ? (int)(N - n0) : COLS;
+#pragma unroll 16
+            for (int c = 0; c < cols; c++) sum = __builtin_fmaf(hs[hm * COLS + c], hws[c * nh + hj], sum);
+            __hip_atomic_store(reinterpret_cast<int *>(head.part + ((int64_t)blockIdx.x * MR + hm) * nh + hj), __float_as_int(sum),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (tid == 0) {
+            const int arrived = __hip_atomic_fetch_add(head.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            head_last = (arrived == head.strips - 1);
+        }
+        __syncthreads();
+        if (!head_last) return;
+        if (mine) {
+            float sum = 0.0f;
+            const float *pp = head.part + (int64_t)hm * nh + hj;
+            const int64_t step = (int64_t)MR * nh;
+            for (int s0 = 0; s0 < head.strips; s0 += 64) {        // strip order; 64 requests in flight at a time
+                float v[64];
+#pragma unroll
+                for (int u = 0; u < 64; u++)
+                    v[u] = s0 + u < head.strips
+                               ? __int_as_float(__hip_atomic_load(reinterpret_cast<const int *>(pp + (s0 + u) * step),
+                                                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                               : 0.0f;
+#pragma unroll
+                for (int u = 0; u < 64; u++)
+                    if (s0 + u < head.strips) sum += v[u];
+            }
+            if (head.bias) sum += head.bias[hj];
+            head.out[hm * nh + hj] = apply_act(sum, head.act);
+        }
+        if (tid == 0) __hip_atomic_store(head.counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+
     float *part = dst + (int64_t)blockIdx.y * dst_split_stride;   // == C itself when splits == 1
     for (int i = tid; i < MR * COLS; i += 256) {
         const int m = i / COLS, c = i % COLS;
@@ -198,7 +276,9 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
         if (n < N) {
             if (splits == 1) {
                 if (bias) s += bias[n];
-                part[m * dst_ld + n] = apply_act(s, act);
+                s = apply_act(s, act);
+                if (!head.W || head.keep) part[m * dst_ld + n] = s;
+                if (head.W) hs[i] = s;
             } else {
                 // device-scope store: written through to the point all XCDs' L2s agree on
                 __hip_atomic_store(reinterpret_cast<int *>(part + m * dst_ld + n), __float_as_int(s),
@@ -206,7 +286,10 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
             }
         }
     }
-    if (splits == 1) return;
+    if (splits == 1) {
+        if (head.W) head_tail();
+        return;
+    }
 
     // Publish this partial, then find out whether every split of this column strip is in.
     // Partials, counter and the reads below are all device-scope accesses, so no cache-wide
@@ -261,23 +344,26 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
         const int64_t n = n0 + i % COLS;
         float r = s[o];
         if (bias) r += bias[n];
-        C[m * ldc + n] = apply_act(r, act);
+        r = apply_act(r, act);
+        if (!head.W || head.keep) C[m * ldc + n] = r;
+        if (head.W) hs[i] = r;
     }
     if (tid == 0)                                   // ready for the next launch
         __hip_atomic_store(counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (head.W) head_tail();
 }
 
 template <int MR>
 int launch_m(bool vec, dim3 grid, size_t smem, const float *A, int64_t lda, const float *B,
              int64_t ldb, float *dst, int64_t dst_ld, int64_t dst_split, int64_t N, int64_t K,
              int64_t kps, const float *bias, int act, int splits, float *C, int64_t ldc,
-             int *counters) {
+             int *counters, const SkinnyHead &head) {
     if (vec)
         hipLaunchKernelGGL((k_skinny<MR, true>), grid, dim3(256), smem, kStream, A, lda, B, ldb, dst,
-                           dst_ld, dst_split, N, K, kps, bias, act, splits, C, ldc, counters);
+                           dst_ld, dst_split, N, K, kps, bias, act, splits, C, ldc, counters, head);
     else
         hipLaunchKernelGGL((k_skinny<MR, false>), grid, dim3(256), smem, kStream, A, lda, B, ldb,
-                           dst, dst_ld, dst_split, N, K, kps, bias, act, splits, C, ldc, counters);
+                           dst, dst_ld, dst_split, N, K, kps, bias, act, splits, C, ldc, counters, head);
     return check_launch("sgemm_skinny");
 }
 
@@ -332,7 +418,7 @@ int check_skinny_args(const char *who, int64_t M, int64_t N, int64_t K, const fl
 // the plan has one split); the kernel leaves the counters at zero.
 int run_skinny(const SkinnyPlan &p, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int act,
-               float *partials, int *counters) {
+               float *partials, int *counters, const SkinnyHead &head = SkinnyHead{}) {
     float *dst = C;
     int64_t dst_ld = ldc, dst_split = 0;
     if (p.splits > 1) {
@@ -341,13 +427,14 @@ int run_skinny(const SkinnyPlan &p, int64_t M, int64_t N, int64_t K, const float
         dst_split = M * N;
     }
     dim3 grid((unsigned)p.col_blocks, (unsigned)p.splits);
-    note_kernel(p.vec ? "sgemm_skinny_vec4" : "sgemm_skinny_scalar");
+    const size_t smem = p.smem + (head.W ? (size_t)(M + head.nh) * COLS * sizeof(float) : 0);
+    note_kernel(head.W ? "sgemm_skinny_with_head" : p.vec ? "sgemm_skinny_vec4" : "sgemm_skinny_scalar");
     int rc;
     switch (M) {
 #define AX_CASE(m)                                                                                  \
     case m:                                                                                         \
-        rc = launch_m<m>(p.vec, grid, p.smem, A, lda, B, ldb, dst, dst_ld, dst_split, N, K, p.kps,  \
-                         bias, act, (int)p.splits, C, ldc, counters);                               \
+        rc = launch_m<m>(p.vec, grid, smem, A, lda, B, ldb, dst, dst_ld, dst_split, N, K, p.kps,    \
+                         bias, act, (int)p.splits, C, ldc, counters, head);                         \
         break;
         AX_CASE(1) AX_CASE(2) AX_CASE(3) AX_CASE(4) AX_CASE(5) AX_CASE(6) AX_CASE(7) AX_CASE(8)
         AX_CASE(9) AX_CASE(10) AX_CASE(11) AX_CASE(12) AX_CASE(13) AX_CASE(14) AX_CASE(15) AX_CASE(16)
@@ -441,4 +528,34 @@ extern "C" int axhip_sgemm_skinny_static(int64_t M, int64_t N, int64_t K, const 
     // clearing between calls that run one after another.
     return run_skinny(p, M, N, K, A, lda, B, ldb, C, ldc, bias, act, reinterpret_cast<float *>(base),
                       reinterpret_cast<int *>(base + kScratchPartialBytes));
+}
+
+extern "C" int axhip_sgemm_skinny_head(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B,
+                                       int64_t ldb, float *C, int64_t ldc, const float *bias, int act, int64_t NH,
+                                       const float *W2, const float *bias2, int act2, float *out2) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!W2 || !out2) return fail(AXHIP_ERR_NULL_ARG, "sgemm_skinny_head: NULL head weights or output");
+    if (NH < 1 || NH > 16) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny_head: head width %lld outside 1..16", (long long)NH);
+    if (act2 < AXHIP_ACT_NONE || act2 > AXHIP_ACT_GELU)
+        return fail(AXHIP_ERR_SHAPE, "sgemm_skinny_head: unknown activation %d", act2);
+    // C may be NULL (the wide layer's output is then never written); the argument check wants a pointer
+    if (int rc = check_skinny_args("sgemm_skinny_head", M, N, K, A, lda, B, ldb, C ? C : out2, C ? ldc : N, act)) return rc;
+    if (N < 1) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny_head: the wide layer has no outputs");
+    SkinnyPlan p;
+    if (int rc = plan_skinny(M, N, K, B, ldb, p)) return rc;
+    const size_t main_bytes = (p.partial_bytes + 255) / 256 * 256, head_bytes = (size_t)p.col_blocks * M * NH * sizeof(float);
+    unsigned char *ws = static_cast<unsigned char *>(axhip::workspace(main_bytes + head_bytes));
+    int *counters = axhip::strip_counters((size_t)p.col_blocks + 1);
+    if (!ws || !counters) return AXHIP_ERR_ALLOC;
+    SkinnyHead head = {};
+    head.W = W2;
+    head.bias = bias2;
+    head.out = out2;
+    head.part = reinterpret_cast<float *>(ws + main_bytes);
+    head.counter = counters + p.col_blocks;
+    head.nh = (int)NH;
+    head.act = act2;
+    head.strips = (int)p.col_blocks;
+    head.keep = C != nullptr;
+    return run_skinny(p, M, N, K, A, lda, B, ldb, C ? C : out2, C ? ldc : N, bias, act, reinterpret_cast<float *>(ws), counters, head);
 }

@@ -197,6 +197,11 @@ ax_status_t ax_compute_gemm_bias_act(const ax_tensor_t *a, const ax_tensor_t *b,
     AX_DISPATCH(gemm_bias_act, out, gemm_bias_act(a, b, bias, (int)act, out));
 }
 
+ax_status_t ax_compute_gemm_act_head(const ax_tensor_t *a, const ax_tensor_t *b, const ax_tensor_t *bias, ax_activation_t act,
+                                     const ax_tensor_t *w2, const ax_tensor_t *bias2, ax_activation_t act2, ax_tensor_t *out2) {
+    AX_DISPATCH(gemm_act_head, out2, gemm_act_head(a, b, bias, (int)act, w2, bias2, (int)act2, out2));
+}
+
 ax_status_t ax_compute_layernorm(const ax_tensor_t *x, const ax_tensor_t *gamma, const ax_tensor_t *beta, float eps,
                                  ax_tensor_t *out, ax_tensor_t *x_hat, ax_tensor_t *inv_std) {
     AX_DISPATCH(layernorm_fwd, out, layernorm_fwd(x, gamma, beta, eps, out, x_hat, inv_std));
@@ -209,5 +214,6 @@ int ax_compute_has_gemm_tn(void) { return AX_HAS(gemm_tn); }
 int ax_compute_has_gemm_ex(void) { return AX_HAS(gemm_ex); }
 int ax_compute_has_bias_add(void) { return AX_HAS(bias_add); }
 int ax_compute_has_gemm_bias_act(void) { return AX_HAS(gemm_bias_act); }
+int ax_compute_has_gemm_act_head(void) { return AX_HAS(gemm_act_head); }
 int ax_compute_has_adam_update(void) { return AX_HAS(adam_update); }
 int ax_compute_has_sgd_update(void) { return AX_HAS(sgd_update); }

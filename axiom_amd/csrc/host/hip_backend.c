@@ -127,6 +127,34 @@ static ax_status_t hip_gemm_bias_act(const ax_tensor_t *a, const ax_tensor_t *b,
     return run_gemm("hip gemm_bias_act", 0, 0, a, b, 1.0f, 0.0f, bias, act, out);
 }
 
+/* Dense -> narrow Dense on the skinny route (at most 16 rows, second layer at most 16 wide, dense weights);
+ * anything else is left to the caller's layer-by-layer path */
+static ax_status_t hip_gemm_act_head(const ax_tensor_t *a, const ax_tensor_t *b, const ax_tensor_t *bias, int act,
+                                     const ax_tensor_t *w2, const ax_tensor_t *bias2, int act2, ax_tensor_t *out2) {
+    const char *who = "hip gemm_act_head";
+    mat_t A, B, W, O;
+    ax_status_t st;
+    if ((st = as_matrix(a, who, "a", &A)) || (st = as_matrix(b, who, "b", &B)) || (st = as_matrix(w2, who, "w2", &W)) ||
+        (st = as_matrix(out2, who, "out2", &O)))
+        return st;
+    if (A.cols != B.rows || B.cols != W.rows || O.rows != A.rows || O.cols != W.cols) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "%s shape mismatch: [%lld,%lld] x [%lld,%lld] x [%lld,%lld] -> [%lld,%lld]", who,
+                   (long long)A.rows, (long long)A.cols, (long long)B.rows, (long long)B.cols, (long long)W.rows,
+                   (long long)W.cols, (long long)O.rows, (long long)O.cols);
+        return AX_ERR_SHAPE_MISMATCH;
+    }
+    if (A.rows < 1 || A.rows > 16 || W.cols < 1 || W.cols > 16 || W.ld != W.cols || O.ld != O.cols ||
+        act < AXHIP_ACT_NONE || act > AXHIP_ACT_GELU || act2 < AXHIP_ACT_NONE || act2 > AXHIP_ACT_GELU) {
+        ax_err_set(AX_ERR_NOT_IMPLEMENTED, "%s: %lld rows into a head of %lld is not taken in one launch", who,
+                   (long long)A.rows, (long long)W.cols);
+        return AX_ERR_NOT_IMPLEMENTED;
+    }
+    const float *bp, *bp2;
+    if ((st = as_vector(bias, who, B.cols, &bp)) || (st = as_vector(bias2, who, W.cols, &bp2))) return st;
+    return lift(axhip_sgemm_skinny_head(A.rows, B.cols, A.cols, A.p, A.ld, B.p, B.ld, NULL, B.cols, bp, act, W.cols, W.p, bp2,
+                                        act2, O.p), who);
+}
+
 /* contiguous fp32 tensor on this device -> pointer + element count */
 static ax_status_t as_flat(const ax_tensor_t *t, const char *who, float **p, int64_t *n) {
     if (!t || !t->storage) {
@@ -525,6 +553,7 @@ static ax_status_t hook_d2d(void *d, const void *s, size_t n) { return lift(axhi
         .synchronize = hook_synchronize, .device_count = hook_device_count,                     \
         .storage_alloc = hook_alloc, .storage_free = hook_free, .memcpy_h2d = hook_h2d,         \
         .memcpy_d2h = hook_d2h, .memcpy_d2d = hook_d2d, .gemm_bias_act = hip_gemm_bias_act,     \
+        .gemm_act_head = hip_gemm_act_head,                                                     \
         .layernorm_fwd = hip_layernorm_fwd, .storage_alloc_uninit = hook_alloc_uninit,          \
     }
 

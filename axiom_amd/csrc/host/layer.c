@@ -3,6 +3,7 @@
 #include <stdlib.h>
 
 #include "axiom/compute.h"
+#include "axiom/error.h"
 #include "axiom/init.h"
 #include "axiom/layer.h"
 #include "axiom/ops.h"
@@ -177,6 +178,30 @@ ax_layer_t *ax_layernorm_create(int64_t num_features, float eps) {
     return &ln->base;
 }
 
+/* the activation a layer type fuses into the Dense before it, or -1 */
+static int fused_act_of(ax_layer_type_t t) {
+    return t == AX_LAYER_RELU ? AX_ACT_RELU : t == AX_LAYER_GELU ? AX_ACT_GELU : -1;
+}
+
+/* Dense [+ ReLU / GELU] followed by a Dense of at most 16 outputs [+ ReLU / GELU], on a few rows: one backend
+ * call when the backend has it (ax_matmul_bias_act_head).  Returns the result and sets *consumed to the number
+ * of layers it stands for, or NULL with *consumed = 0 when the pattern or the backend does not apply (the
+ * caller then goes layer by layer), or NULL with *consumed < 0 on a real error. */
+static ax_tensor_t *try_dense_head(ax_sequential_t *seq, int i, ax_tensor_t *x, int *consumed) {
+    *consumed = 0;
+    if (seq->layers[i]->type != AX_LAYER_DENSE || x->ndim != 2 || x->shape[0] > 16) return NULL;
+    int j = i + 1, act = AX_ACT_NONE, act2 = AX_ACT_NONE;
+    if (j < seq->n_layers && fused_act_of(seq->layers[j]->type) >= 0) act = fused_act_of(seq->layers[j++]->type);
+    if (j >= seq->n_layers || seq->layers[j]->type != AX_LAYER_DENSE || seq->layers[j]->output_features > 16) return NULL;
+    ax_dense_t *d1 = (ax_dense_t *)seq->layers[i], *d2 = (ax_dense_t *)seq->layers[j++];
+    if (j < seq->n_layers && fused_act_of(seq->layers[j]->type) >= 0) act2 = fused_act_of(seq->layers[j++]->type);
+    ax_tensor_t *y = ax_matmul_bias_act_head(x, d1->weight, dense_bias(d1), act, d2->weight, dense_bias(d2), act2);
+    if (y) *consumed = j - i;
+    else if (ax_err_last_status() != AX_ERR_NOT_IMPLEMENTED) *consumed = -1;
+    else ax_err_clear();                       /* not an error: the layers run one by one */
+    return y;
+}
+
 static ax_tensor_t *sequential_forward(ax_layer_t *self, ax_tensor_t *input) {
     ax_sequential_t *seq = (ax_sequential_t *)self;
     ax_tensor_t *x = input, *prev = NULL;
@@ -184,7 +209,10 @@ static ax_tensor_t *sequential_forward(ax_layer_t *self, ax_tensor_t *input) {
         ax_layer_t *l = seq->layers[i];
         ax_layer_type_t next_type = (i + 1 < seq->n_layers) ? seq->layers[i + 1]->type : AX_LAYER_TYPE_COUNT;
         ax_tensor_t *y;
-        if (l->type == AX_LAYER_DENSE && next_type == AX_LAYER_RELU) {
+        int consumed = 0;
+        if ((y = try_dense_head(seq, i, x, &consumed)) != NULL || consumed < 0) {
+            if (consumed > 0) i += consumed - 1;
+        } else if (l->type == AX_LAYER_DENSE && next_type == AX_LAYER_RELU) {
             ax_dense_t *d = (ax_dense_t *)l;
             y = ax_matmul_bias_relu(x, d->weight, dense_bias(d));
             i++;

@@ -77,6 +77,30 @@ ax_tensor_t *ax_matmul_bias_gelu(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bi
     return matmul_impl(a, b, bias, AX_ACT_GELU, true, "matmul_bias_gelu");
 }
 
+ax_tensor_t *ax_matmul_bias_act_head(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bias, int act, ax_tensor_t *w2,
+                                     ax_tensor_t *bias2, int act2) {
+    if (!a || !b || !w2) {
+        ax_err_set(AX_ERR_NULL_ARG, "matmul_bias_act_head: NULL tensor");
+        return NULL;
+    }
+    if (a->ndim != 2 || b->ndim != 2 || w2->ndim != 2 || a->shape[1] != b->shape[0] || b->shape[1] != w2->shape[0]) {
+        ax_err_set(AX_ERR_SHAPE_MISMATCH, "matmul_bias_act_head needs a:[M,K], b:[K,N], w2:[N,H]");
+        return NULL;
+    }
+    if (!ax_compute_has_gemm_act_head()) {
+        ax_err_set(AX_ERR_NOT_IMPLEMENTED, "matmul_bias_act_head: the active backend has no such operation");
+        return NULL;
+    }
+    int64_t oshape[2] = {a->shape[0], w2->shape[1]};
+    ax_tensor_t *out = alloc_like_device(a, oshape, 2);
+    if (!out) return NULL;
+    if (ax_compute_gemm_act_head(a, b, bias, (ax_activation_t)act, w2, bias2, (ax_activation_t)act2, out) != AX_OK) {
+        ax_tensor_destroy(out);
+        return NULL;
+    }
+    return out;
+}
+
 static ax_tensor_t *unary(ax_tensor_t *a, ax_status_t (*op)(const ax_tensor_t *, ax_tensor_t *), const char *who) {
     if (!a) {
         ax_err_set(AX_ERR_NULL_ARG, "%s: NULL tensor", who);

@@ -123,6 +123,19 @@ int axhip_sgemm_skinny(int64_t M, int64_t N, int64_t K, const float *A, int64_t 
                        const float *B, int64_t ldb, float *C, int64_t ldc,
                        const float *bias, int act);
 
+/* The skinny-M route with a narrow layer riding on it, in one launch:
+ *   C[M,N]     = act(A[M,K] * B[K,N] + bias[n])                 (C may be NULL: then it is never written)
+ *   out2[M,NH] = act2(C[M,N] * W2[N,NH] + bias2[j]),   1 <= NH <= 16, W2 and out2 dense
+ * i.e. a Dense(+activation) layer followed by a Dense layer of at most 16 outputs — the hidden layer and
+ * classifier head that end the 784-4096-4096-10 network of the reference's benchmarks — as Sequential runs
+ * them at batch sizes of a few rows (src/core/layer.c:181-230 over opt_gemm's skinny route,
+ * src/compute/backends/cpu_opt.c:3499-3567).  Whoever finishes a strip of C multiplies it by the head's rows
+ * for that strip; the strips' partial vectors are added in strip order, so results are deterministic.  C is
+ * bit-identical to axhip_sgemm_skinny; out2 is the same sum in another order. */
+int axhip_sgemm_skinny_head(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B,
+                            int64_t ldb, float *C, int64_t ldc, const float *bias, int act, int64_t NH,
+                            const float *W2, const float *bias2, int act2, float *out2);
+
 /* The same route for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * Arguments, results and kernels are those of axhip_sgemm_skinny — outputs are bit-identical —

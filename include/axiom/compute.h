@@ -103,6 +103,11 @@ ax_status_t ax_compute_gelu(const ax_tensor_t *in, ax_tensor_t *out);
 ax_status_t ax_compute_gemm_bias_act(const ax_tensor_t *a, const ax_tensor_t *b, const ax_tensor_t *bias,
                                      ax_activation_t act, ax_tensor_t *out);
 int ax_compute_has_gemm_bias_act(void);
+/* Not in the reference: two Dense layers, the second at most 16 wide, in one backend call (the appended
+ * gemm_act_head slot).  AX_ERR_NOT_IMPLEMENTED when the backend has no such slot or does not take the shape. */
+ax_status_t ax_compute_gemm_act_head(const ax_tensor_t *a, const ax_tensor_t *b, const ax_tensor_t *bias, ax_activation_t act,
+                                     const ax_tensor_t *w2, const ax_tensor_t *bias2, ax_activation_t act2, ax_tensor_t *out2);
+int ax_compute_has_gemm_act_head(void);
 /* The reference's vtable has leaky_relu / elu_op / swish_op slots (filled by its GPU backend,
  * cuda/ops_activations.cu) but no dispatch wrapper: ax_leaky_relu, ax_elu, ax_swish
  * (src/core/activations.c:79,141,363) loop over host pointers. */

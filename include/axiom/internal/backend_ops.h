@@ -7,8 +7,8 @@
  * reference's offsets and tests/test_host_core.py compares them with this header.
  * Any slot may be NULL; dispatch answers AX_ERR_NOT_IMPLEMENTED for those.
  *
- * Three slots are appended after the reference's last member (gemm_bias_act, layernorm_fwd,
- * storage_alloc_uninit); the reference never reads that far, this repository's host core does. */
+ * Four slots are appended after the reference's last member (gemm_bias_act, layernorm_fwd,
+ * storage_alloc_uninit, gemm_act_head); the reference never reads that far, this repository's host core does. */
 #ifndef AX_INTERNAL_BACKEND_OPS_H
 #define AX_INTERNAL_BACKEND_OPS_H
 
@@ -118,6 +118,12 @@ struct ax_backend_ops {
      * contract (include/axiom/tensor.h of the reference): an operator's result is overwritten in
      * full, and a fill launch per result is a sizeable share of a bs=1 layer's time */
     void *(*storage_alloc_uninit)(size_t size_bytes);
+    /* two Dense layers in one call, the second at most 16 wide (a hidden layer and its classifier head):
+     * out2 = act2(act(a x b + bias) x w2 + bias2); the wide intermediate is not materialised.  Biases may be
+     * NULL, acts are ax_activation_t.  A backend returns AX_ERR_NOT_IMPLEMENTED for shapes it does not
+     * take this way (more than a few rows, a wider second layer); the caller then runs the layers one by one. */
+    ax_status_t (*gemm_act_head)(ax_tin_t a, ax_tin_t b, ax_tin_t bias, int act, ax_tin_t w2, ax_tin_t bias2, int act2,
+                                 ax_tout_t out2);
 };
 
 /* The MI355X backend.  `device` is AX_DEVICE_HIP. */

@@ -15,6 +15,12 @@ ax_tensor_t *ax_matmul(ax_tensor_t *a, ax_tensor_t *b);                         
 ax_tensor_t *ax_matmul_bias(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bias);     /* a may be [B,S,K] */
 ax_tensor_t *ax_matmul_bias_relu(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bias);
 ax_tensor_t *ax_matmul_bias_gelu(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bias); /* not in the reference */
+/* Not in the reference: act2(act(a x b + bias) x w2 + bias2) for a second layer of at most 16 outputs, without
+ * the wide intermediate, when the active backend takes the shape in one call (a few rows of a); returns NULL
+ * with the thread's error status at AX_ERR_NOT_IMPLEMENTED when it does not — the caller then runs the two
+ * layers separately — and NULL with another status on a real error.  act, act2: ax_activation_t. */
+ax_tensor_t *ax_matmul_bias_act_head(ax_tensor_t *a, ax_tensor_t *b, ax_tensor_t *bias, int act, ax_tensor_t *w2,
+                                     ax_tensor_t *bias2, int act2);
 ax_tensor_t *ax_relu(ax_tensor_t *a);
 ax_tensor_t *ax_gelu(ax_tensor_t *a);                                                /* tanh form */
 /* src/core/ops.c:509-537, src/core/activations.c:79,141,363,598 — on the tensor's device */

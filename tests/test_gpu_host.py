@@ -208,6 +208,52 @@ def test_config1_sequential_mlp(ax, oracle, M):
     L.ax_layer_destroy(seq)
 
 
+def test_sequential_dense_with_narrow_head(ax, oracle):
+    """Sequential fuses Dense [+ act] -> Dense(<= 16) [+ act] on a few rows into one backend call and runs the
+    same layers one by one otherwise; both give the oracle's result."""
+    L = ax.L
+    from axiom_amd.axiom import TP
+    assert L.ax_compute_has_gemm_act_head()
+    for (M, hidden, head, act1, act2) in ((3, 512, 7, "gelu", "relu"), (16, 300, 16, None, None), (17, 512, 7, "relu", None),
+                                          (4, 512, 17, "relu", None)):
+        L.ax_set_seed(99)
+        seq = L.ax_sequential_create()
+        L.ax_sequential_add(seq, L.ax_dense_create(200, hidden, True))
+        if act1:
+            L.ax_sequential_add(seq, L.ax_gelu_layer_create() if act1 == "gelu" else L.ax_relu_layer_create())
+        L.ax_sequential_add(seq, L.ax_dense_create(hidden, head, True))
+        if act2:
+            L.ax_sequential_add(seq, L.ax_relu_layer_create())
+        params = (TP * 4)()
+        assert L.ax_layer_get_params(seq, params, 4) == 4
+        oracle.seed(M + hidden + head)
+        b1, b2 = oracle.normal((hidden,), 0, 0.3), oracle.normal((head,), 0, 0.3)
+        assert L.ax_tensor_write(params[1], b1.ctypes.data, b1.nbytes) == 0
+        assert L.ax_tensor_write(params[3], b2.ctypes.data, b2.nbytes) == 0
+        w1, w2 = ax.to_numpy(params[0]), ax.to_numpy(params[2])
+        x = oracle.uniform((M, 200), -1, 1)
+        tx = ax.from_numpy(x)
+        L.ax_err_clear()
+        y = L.ax_layer_forward(seq, tx)
+        assert y, ax.err()
+        code = {None: 0, "relu": 1, "gelu": 2}
+        ref = oracle.dense(oracle.dense(x, w1, b1, code[act1]), w2, b2, code[act2])
+        assert close(ax.to_numpy(y), ref), (M, hidden, head)
+        assert ax.err()[0] == 0                                # a fall-back to the layer-by-layer path is not an error
+        ax.free(tx, y)
+        L.ax_layer_destroy(seq)
+    # the operation itself: refused shapes report AX_ERR_NOT_IMPLEMENTED, bad shapes a shape error
+    oracle.seed(5)
+    a, w1, w2 = oracle.uniform((2, 64), -1, 1), oracle.uniform((64, 128), -1, 1), oracle.uniform((128, 5), -1, 1)
+    ta, tw1, tw2 = ax.from_numpy(a), ax.from_numpy(w1), ax.from_numpy(w2)
+    y = L.ax_matmul_bias_act_head(ta, tw1, None, 1, tw2, None, 0)
+    assert y and close(ax.to_numpy(y), oracle.dense(oracle.dense(a, w1, None, 1), w2, None, 0))
+    big = ax.from_numpy(oracle.uniform((40, 64), -1, 1))
+    assert not L.ax_matmul_bias_act_head(big, tw1, None, 1, tw2, None, 0) and ax.err()[0] == 10
+    assert not L.ax_matmul_bias_act_head(ta, tw2, None, 1, tw1, None, 0) and ax.err()[0] == 3
+    ax.free(ta, tw1, tw2, y, big)
+
+
 def test_config3_ffn_through_layers(ax, oracle):
     L = ax.L
     L.ax_set_seed(3)

@@ -464,6 +464,44 @@ def test_skinny_padded_leading_dimensions(hip, oracle, M, K, N):
     check_fp32(oracle, hip.sgemm_skinny(hip.array(a), hip.array(b)).numpy(), a, b)
 
 
+@pytest.mark.parametrize("M,K,N,NH,act,act2,keep,with_bias", [
+    (1, 4096, 4096, 10, 1, 0, True, True), (8, 4096, 4096, 10, 1, 0, False, True), (16, 784, 4096, 16, 2, 1, True, True),
+    (3, 100, 70, 1, 0, 0, True, False), (5, 64, 64, 7, 1, 1, True, True), (2, 2000, 1000, 3, 0, 2, False, False),
+    (9, 300, 4100, 12, 1, 0, True, True), (4, 16, 8, 16, 0, 0, True, True)])
+def test_skinny_with_head(hip, oracle, M, K, N, NH, act, act2, keep, with_bias):
+    """A skinny layer with a narrow layer riding on it: the wide output is bit-identical to the plain route,
+    the head's output is the oracle's dense layer on it (fp32 gate and fp64 bound), and calls in a row agree."""
+    say("skinny+head", M, K, N, NH, act, act2, keep, with_bias)
+    oracle.seed(M * 31 + K + N + NH)
+    a, b = oracle.uniform((M, K), 0, 1), oracle.uniform((K, N), -0.05, 0.05)
+    w2 = oracle.uniform((N, NH), -0.05, 0.05)
+    bias, bias2 = oracle.normal((N,), 0, 0.1), oracle.normal((NH,), 0, 0.1)
+    da, db, dw2 = hip.array(a), hip.array(b), hip.array(w2)
+    dbias, dbias2 = (hip.array(bias), hip.array(bias2)) if with_bias else (None, None)
+    want_c = hip.sgemm_skinny(da, db, dbias, act).numpy()
+    c, o = hip.empty((M, N)), hip.empty((M, NH))
+    outs = []
+    for _ in range(2):
+        hip.check(hip.L.axhip_memset(c.ptr, 0xFF, c.nbytes))
+        hip.check(hip.L.axhip_memset(o.ptr, 0xFF, o.nbytes))
+        hip.check(hip.L.axhip_sgemm_skinny_head(M, N, K, da.ptr, K, db.ptr, N, c.ptr if keep else None, N, hip._p(dbias), act,
+                                                NH, dw2.ptr, hip._p(dbias2), act2, o.ptr))
+        assert hip.last_kernel() == "sgemm_skinny_with_head"
+        outs.append(o.numpy())
+        if keep:
+            assert np.array_equal(c.numpy(), want_c)
+        else:
+            assert np.isnan(c.numpy()).all()                     # never written
+    assert np.array_equal(outs[0], outs[1])                      # deterministic
+    ref = oracle.dense(want_c, w2, bias2 if with_bias else None, act2)
+    assert np.abs(outs[0] - ref).max() <= REL_FP32 * max(np.abs(ref).max(), 1e-6)
+    if act2 == 0:
+        pre = outs[0] - (bias2[None, :] if with_bias else 0)
+        check_fp32(oracle, pre.astype(np.float32), want_c, w2)
+    assert hip.L.axhip_sgemm_skinny_head(M, N, K, da.ptr, K, db.ptr, N, None, N, None, 0, 17, dw2.ptr, None, 0, o.ptr) == 3
+    assert hip.L.axhip_sgemm_skinny_head(M, N, K, da.ptr, K, db.ptr, N, None, N, None, 0, NH, None, None, 0, o.ptr) == 1
+
+
 @pytest.mark.parametrize("M", [1, 2, 4, 8])
 def test_config1_mlp_inference(hip, oracle, M):
     """x[M,784] -> dense 4096 -> ReLU -> dense 4096 -> ReLU -> dense 10; Kaiming-uniform weights
