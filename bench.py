@@ -271,6 +271,27 @@ def secondary(hip):
     res["skinny_mlp_784_4096_4096_10"] = mlp
     del sets
 
+    # the same route on one large layer (8192 x 8192 fp32, 268 MB of weights, 4 rotating sets): what the
+    # kernel streams at once a launch's fixed cost (start-up, split-K join, about 5 us) is small beside its traffic
+    big_sets = [hip.array(rng.uniform(-0.03, 0.03, (8192, 8192)).astype(np.float32)) for _ in range(4)]
+    bias8k = hip.empty((8192,))
+    big = {}
+    for M in (1, 8):
+        xin = hip.array(rng.uniform(0, 1, (M, 8192)).astype(np.float32))
+        yb = hip.empty((M, 8192))
+        it = [0]
+
+        def big_step():
+            w_ = big_sets[it[0] % 4]
+            it[0] += 1
+            hip.check(hip.L.axhip_sgemm(0, 0, M, 8192, 8192, 1.0, xin.ptr, 8192, w_.ptr, 8192, 0.0, yb.ptr, 8192, bias8k.ptr, 1))
+
+        _, ms = time_calls(hip, big_step)
+        gbs = 4 * 8192 * 8192 / ms / 1e6
+        big[f"M{M}"] = {"us": ms * 1e3, "GB/s": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS, "kernel": hip.last_kernel()}
+    res["skinny_layer_8192x8192"] = big
+    del big_sets
+
     # config 4b: strided-batched attention-shaped products, 512 heads of [512,64]
     Bn, S, D = 512, 512, 64
     q = hip.array(rng.normal(0, 1, (Bn, S, D)).astype(np.float32))
