@@ -896,6 +896,235 @@ int try_nt_rows(const SgemmArgs &g, int64_t batch) {
     }
 }
 
+// =====================================================================================
+// C = alpha * A * B for batched products with many output tiles and a K of a few hundred (P V of
+// attention heads: K = 512, N = 64).  With a workgroup per tile, a third of each workgroup's life is its
+// first load latency and its write-back, and the workgroups that share a CU go through both together.
+// Here a fixed set of workgroups (one or two per CU) each walk a list of 128 x 64 output tiles and treat
+// the K slabs of all of them as one stream through a ring of three LDS stages: the first slabs of the
+// next tile are in flight while the last ones of the current tile are multiplied, and the stores of a
+// finished tile are issued after the loads of the slab that follows them, so that no wait for loads
+// includes stores.  The ring position is a run-time offset (five additions per slab), the first slab of
+// a tile is known at compile time: its first MFMAs start from zero and the accumulators never leave
+// their registers.  4 waves as 2 x 2, wave tile 64 x 32; A K-contiguous, B N-contiguous; the MFMA takes
+// the A fragment first here, so a lane owns one column n of eight rows and a store instruction writes
+// two whole 128-byte rows.  Workgroup w serves batch entries w % 8, w % 8 + 8, ... (w % 8 is the XCD it
+// runs on), tile after tile of one entry, so the tiles that share an entry's B run next to each other on
+// one XCD's L2.
+__global__ void __launch_bounds__(256) k_sgemm_nn_stream(SgemmArgs g, int batch, int slots) {
+    constexpr int BM = 128, BN = 64, NW = 4, TM = 2, NST = 3;
+    using OA = DmaOperand<BM, true, NW>;
+    using OB = DmaOperand<BN, false, NW>;
+    constexpr int B_BASE = NST * OA::BYTES;
+    constexpr int LOADS = OA::IPW + OB::IPW;       // load instructions of a wave per slab
+    constexpr int NSTORES = TM * 16;               // store instructions of a wave per tile
+    static_assert(B_BASE + NST * OB::BYTES <= 80 * 1024, "two workgroups per CU");
+    static_assert(LOADS + NSTORES < 64, "wait counts");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int xcd = (int)(blockIdx.x & 7), slot = (int)(blockIdx.x >> 3);
+    const int cbs = (int)(g.N / BN), per_entry = (int)(g.M / BM) * cbs;
+    const int items_here = xcd < batch ? ((batch - xcd + 7) / 8) * per_entry : 0;    // tiles of this XCD's entries
+    if (slot >= items_here) return;
+    const int n_items = (items_here - slot + slots - 1) / slots;                     // ... of which this workgroup's
+    const int slabs = (int)(g.K / 32);
+    const float *A = static_cast<const float *>(g.A), *B = static_cast<const float *>(g.B);
+
+    // item q of this XCD: entry xcd + 8 * (q / per_entry), row block and column block from the remainder
+    auto locate = [&](int q, const char *&pa, const char *&pb, float *&pc) {
+        const int e = q / per_entry, r = q - e * per_entry, rb = r / cbs, cb = r - rb * cbs;
+        const int64_t entry = xcd + 8 * (int64_t)e;
+        pa = reinterpret_cast<const char *>(A + entry * g.stride_a + (int64_t)rb * BM * g.lda);
+        pb = reinterpret_cast<const char *>(B + entry * g.stride_b + (int64_t)cb * BN);
+        pc = g.C + entry * g.stride_c + (int64_t)rb * BM * g.ldc + (int64_t)cb * BN;
+    };
+
+    unsigned va[OA::IPW], vb[OB::IPW];
+#pragma unroll
+    for (int j = 0; j < OA::IPW; j++) va[j] = OA::lane_offset(j * NW + wave, lane, g.lda);
+#pragma unroll
+    for (int j = 0; j < OB::IPW; j++) vb[j] = OB::lane_offset(j * NW + wave, lane, g.ldb);
+    const int64_t step_b = 128 * g.ldb;                                              // bytes per slab of B
+    const unsigned lds0 = (unsigned)(uintptr_t)lds_raw;
+    const unsigned dma_a = lds0 + wave * OA::PITCH, dma_b = lds0 + B_BASE + wave * OB::PITCH;
+
+    const int frow = lane & 31, fhalf = lane >> 5;
+    unsigned ra0[4];                               // fragment addresses in stage 0
+#pragma unroll
+    for (int kbi = 0; kbi < 4; kbi++) ra0[kbi] = lds0 + OA::frag_base(wm * 64, frow, fhalf, kbi);
+    const unsigned rb0 = lds0 + B_BASE + OB::frag_base(wn * 32, frow, fhalf, 0);
+    // register v of lane l: n = l & 31, m = i*32 + 8*(v>>2) + 4*(l>>5) + (v&3)
+    const int64_t lane_c = (int64_t)(wm * 64 + 4 * fhalf) * g.ldc + wn * 32 + frow;
+
+    // the load side of the stream runs ahead of the multiply side: each has its own item and ring position
+    const char *ga, *gb;
+    float *c_unused, *c_cur, *c_prev = nullptr;
+    int lq = slot, lk = 0, to_load = n_items * slabs;
+    unsigned load_a = 0, load_b = 0, mul_a = 0, mul_b = 0;        // byte offsets of the stage loaded / multiplied next
+    locate(lq, ga, gb, c_unused);
+    {
+        const char *ua, *ub;
+        locate(slot, ua, ub, c_cur);
+    }
+
+    v16f acc[TM];
+    Frag<true> fa[2][TM];
+    Frag<false> fb[2];
+    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < TM; i++) acc[i] = zero;
+    unsigned ra[4], rb;
+
+// loads of the stream's next slab into the ring
+#define AXS_ISSUE()                                                                              \
+    do {                                                                                         \
+        _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                                      \
+            AXF_LOAD_LDS(dma_a + load_a + j * NW * OA::PITCH, va[j], ga);                        \
+        _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                                      \
+            AXF_LOAD_LDS(dma_b + load_b + j * NW * OB::PITCH, vb[j], gb);                        \
+        load_a = load_a == (NST - 1) * OA::BYTES ? 0 : load_a + OA::BYTES;                       \
+        load_b = load_b == (NST - 1) * OB::BYTES ? 0 : load_b + OB::BYTES;                       \
+        --to_load;                                                                               \
+        if (++lk == slabs) {                                                                     \
+            lk = 0;                                                                              \
+            lq += slots;                                                                         \
+            if (to_load > 0) locate(lq, ga, gb, c_unused);                                       \
+        } else {                                                                                 \
+            ga += 128;                                                                           \
+            gb += step_b;                                                                        \
+        }                                                                                        \
+    } while (0)
+// fragments of k-block KB of the stage being multiplied
+#define AXS_FRAGS(BUF, KB)                                                                       \
+    do {                                                                                         \
+        AXF_DS128(fa[BUF][0].q, ra[KB], 0);                                                      \
+        AXF_DS128(fa[BUF][1].q, ra[KB], 4096);                                                   \
+        AXF_DS32(fb[BUF].s0, rb, OB::k_imm((KB) * 8 + 0));                                       \
+        AXF_DS32(fb[BUF].s1, rb, OB::k_imm((KB) * 8 + 1));                                       \
+        AXF_DS32(fb[BUF].s2, rb, OB::k_imm((KB) * 8 + 2));                                       \
+        AXF_DS32(fb[BUF].s3, rb, OB::k_imm((KB) * 8 + 3));                                       \
+    } while (0)
+// the eight MFMAs of a k-block; ZERO: a tile's first, which start from a clean accumulator
+#define AXS_MFMAS(BUF, ZERO)                                                                     \
+    do {                                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+        _Pragma("unroll") for (int e = 0; e < 4; e++)                                            \
+            _Pragma("unroll") for (int i = 0; i < TM; i++)                                       \
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[BUF][i].get(e), fb[BUF].get(e), \
+                                                              ((ZERO) && e == 0) ? zero : acc[i], 0, 0, 0); \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    } while (0)
+
+    // the finished tile: a store instruction writes one float per lane, two rows of 128 bytes
+    auto write_back = [&]() {
+        float *cp = c_prev + lane_c;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                float o = acc[i][v];
+                if (g.alpha != 1.0f) o *= g.alpha;
+                __builtin_nontemporal_store(o, cp + (int64_t)(i * 32 + 8 * (v >> 2) + (v & 3)) * g.ldc);
+            }
+    };
+
+// One slab; FIRST: the first of a tile.  Order inside a wave: the loads of the slab two ahead, then
+// (FIRST) the stores of the tile finished by the previous slab, then this slab's MFMAs; the wait that
+// follows passes over whatever was issued after the next slab's loads, and the barrier makes every
+// wave's part of that slab visible and frees this slab's stage for the loads issued next.
+#define AXS_SLAB(FIRST)                                                                          \
+    do {                                                                                         \
+        const bool more = to_load > 0, wrote = (FIRST) && c_prev != nullptr;                     \
+        if (more) AXS_ISSUE();                                                                   \
+        if (wrote) write_back();                                                                 \
+        _Pragma("unroll") for (int kbi = 0; kbi < 4; kbi++) ra[kbi] = ra0[kbi] + mul_a;          \
+        rb = rb0 + mul_b;                                                                        \
+        mul_a = mul_a == (NST - 1) * OA::BYTES ? 0 : mul_a + OA::BYTES;                          \
+        mul_b = mul_b == (NST - 1) * OB::BYTES ? 0 : mul_b + OB::BYTES;                          \
+        AXS_FRAGS(0, 0);                                                                         \
+        AXS_FRAGS(1, 1);                                                                         \
+        AXF_LGKM(6);                                                                             \
+        AXS_MFMAS(0, FIRST);                                                                     \
+        AXS_FRAGS(0, 2);                                                                         \
+        AXF_LGKM(6);                                                                             \
+        AXS_MFMAS(1, false);                                                                     \
+        AXS_FRAGS(1, 3);                                                                         \
+        AXF_LGKM(6);                                                                             \
+        AXS_MFMAS(0, false);                                                                     \
+        AXF_LGKM(0);                                                                             \
+        AXS_MFMAS(1, false);                                                                     \
+        if (more) {                                                                              \
+            if (wrote) AXF_VM(LOADS + NSTORES); else AXF_VM(LOADS);                              \
+        } else {                                                                                 \
+            if (wrote) AXF_VM(NSTORES); else AXF_VM(0);                                          \
+        }                                                                                        \
+        __builtin_amdgcn_s_barrier();                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    } while (0)
+
+    AXS_ISSUE();
+    AXS_ISSUE();                                   // a tile has at least four slabs
+    AXF_VM(LOADS);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    int cq = slot;
+    for (int t = 0; t < n_items; t++) {
+        AXS_SLAB(true);
+        for (int s = 1; s < slabs; s++) AXS_SLAB(false);
+        c_prev = c_cur;
+        cq += slots;
+        if (t + 1 < n_items) {
+            const char *ua, *ub;
+            locate(cq, ua, ub, c_cur);
+        }
+    }
+    write_back();
+#undef AXS_ISSUE
+#undef AXS_FRAGS
+#undef AXS_MFMAS
+#undef AXS_SLAB
+}
+
+// The streamed NN route: a batch of at least 8 entries, K a multiple of 32 from 128 to 1024, M on the 128
+// grid, N on the 64 grid, no beta / bias / activation, at least three tiles for every workgroup.  An
+// XCD's share of the tiles is dealt to one or two workgroups per CU, whichever leaves the last round of
+// tiles fuller.  -1: not taken.
+int try_nn_stream(const SgemmArgs &g, int64_t batch) {
+    if (tuning().f32_tile != 0) return -1;
+    if (g.K < 128 || g.K > 1024 || g.K % 32 != 0 || g.M % 128 != 0 || g.N % 64 != 0 || batch < 8 || batch > 65535) return -1;
+    if (g.beta != 0.0f || g.bias || g.col_scale || g.act != AXHIP_ACT_NONE) return -1;
+    if ((((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.C) & 15) != 0 || g.lda % 4 != 0 || g.ldb % 4 != 0 || g.ldc % 4 != 0 ||
+        g.stride_a % 4 != 0 || g.stride_b % 4 != 0 || g.stride_c % 4 != 0 || g.lda >= (1 << 20) || g.ldb >= (1 << 20))
+        return -1;
+    const int64_t per_entry = (g.M / 128) * (g.N / 64), per_xcd = (batch + 7) / 8 * per_entry, cus = cu_count() / 8;
+    if (per_entry > 4096 || cus < 1) return -1;
+    int64_t slots = 0, best_num = 0, best_den = 1;
+    for (int64_t w = 1; w <= 2; w++) {
+        const int64_t rounds = (per_xcd + w * cus - 1) / (w * cus);
+        // fill = per_xcd / (rounds * w * cus); two per CU wins a tie
+        if (rounds >= 3 && per_xcd * best_den >= best_num * rounds * w * cus) {
+            best_num = per_xcd;
+            best_den = rounds * w * cus;
+            slots = w * cus;
+        }
+    }
+    if (slots == 0) return -1;
+    constexpr int smem = 3 * (DmaOperand<128, true, 4>::BYTES + DmaOperand<64, false, 4>::BYTES);
+    static bool attr_set = false;
+    if (!attr_set) {
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_sgemm_nn_stream),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem),
+                      "hipFuncSetAttribute");
+        attr_set = true;
+    }
+    note_kernel("sgemm_nn_stream128x64_dma");
+    hipLaunchKernelGGL(k_sgemm_nn_stream, dim3((unsigned)(8 * slots)), dim3(256), smem, kStream, g, (int)batch, (int)slots);
+    return check_launch("sgemm_nn_stream128x64_dma");
+}
+
 // Chooses the largest tile that still leaves about eight waves per CU; returns -1 when the
 // shape does not qualify for the fast path (the caller then uses the register-staged kernel).
 // names: 128x256, 64x64, 64x64 with the k split.
@@ -1087,6 +1316,7 @@ int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     static const char *const tn_d[3] = {"sgemm_tn_128x256_dma", "sgemm_tn_64x64_dma", "sgemm_tn_64x64k2_dma"};
     int rc = -1;
     if (!transa && transb) rc = try_nt_rows(g, batch);
+    if (!transa && !transb) rc = try_nn_stream(g, batch);
     if (rc >= 0) return rc;
     if (!transa && !transb) rc = try_dma<true, false>(nn_d, g, batch);
     else if (!transa && transb) rc = try_dma<true, true>(nt_d, g, batch);

@@ -542,25 +542,42 @@ def counter_probe(hip, case, repeat=1):
 
 
 def sustain(hip, seconds, operands):
-    """The headline GEMM launched back to back for `seconds`, over random int8 operands or all-zero ones
-    (same instruction stream, no switching activity in the matrix core), so that clock and power can be
-    sampled from outside (rocm-smi) while it runs.  Prints the average time per launch once a second."""
+    """One GEMM launched back to back for `seconds`, so that clock and power can be sampled from outside
+    (rocm-smi) while it runs: the headline over random int8 operands or all-zero ones (same instruction
+    stream, no switching activity in the matrix core), or the fp32 8192^3 product over random / zero
+    operands ("fp32", "fp32zeros").  Prints the average time per launch about once a second."""
     M = N = K = 8192
     rng = np.random.default_rng(0)
-    if operands == "zeros":
-        x, w = hip.empty((M, K), np.int8), hip.empty((N, K), np.int8)
+    if operands.startswith("fp32"):
+        if operands == "fp32zeros":
+            a, b = hip.empty((M, K)), hip.empty((K, N))
+        else:
+            a = hip.array(rng.standard_normal((M, K), dtype=np.float32))
+            b = hip.array(rng.standard_normal((K, N), dtype=np.float32))
+        out = hip.empty((M, N))
+        per_print = 120
+
+        def launch():
+            hip.check(hip.L.axhip_sgemm(0, 0, M, N, K, 1.0, a.ptr, K, b.ptr, N, 0.0, out.ptr, N, None, 0))
     else:
-        x, w = hip.array(rand_i8(rng, (M, K))), hip.array(rand_i8(rng, (N, K)))
-    ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
-    bias = hip.array(rng.normal(0.0, 0.02, N).astype(np.float32))
-    out = hip.empty((M, N))
+        if operands == "zeros":
+            x, w = hip.empty((M, K), np.int8), hip.empty((N, K), np.int8)
+        else:
+            x, w = hip.array(rand_i8(rng, (M, K))), hip.array(rand_i8(rng, (N, K)))
+        ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+        bias = hip.array(rng.normal(0.0, 0.02, N).astype(np.float32))
+        out = hip.empty((M, N))
+        per_print = 2000
+
+        def launch():
+            hip.check(hip.L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, bias.ptr, 0, out.ptr, None, M, N, K))
     t_end = time.perf_counter() + seconds
     while time.perf_counter() < t_end:
         t0 = time.perf_counter()
-        for _ in range(2000):
-            hip.check(hip.L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, bias.ptr, 0, out.ptr, None, M, N, K))
+        for _ in range(per_print):
+            launch()
         hip.sync()
-        print(f"sustain {operands}: {(time.perf_counter() - t0) / 2000 * 1e6:.1f} us per launch "
+        print(f"sustain {operands}: {(time.perf_counter() - t0) / per_print * 1e6:.1f} us per launch "
               f"({hip.last_kernel()})", flush=True)
 
 
@@ -644,7 +661,7 @@ def main():
                     choices=["headline", "skinny", "gemm1024", "fp32", "config2", "attention"])
     ap.add_argument("--probe-repeat", type=int, default=1, help="multiplies the launch counts of --counter-probe")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of back-to-back headline launches")
-    ap.add_argument("--operands", choices=["random", "zeros"], default="random")
+    ap.add_argument("--operands", choices=["random", "zeros", "fp32", "fp32zeros"], default="random")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")

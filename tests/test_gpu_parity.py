@@ -1,6 +1,8 @@
 """GPU parity: the HIP path, called through the C ABI of libaxhip.so, against the CPU oracle
 on identical seeded inputs.  int32 accumulators and int8 outputs: bit-exact.  fp32: the gates
 stated next to each assert."""
+import os
+
 import numpy as np
 import pytest
 
@@ -334,7 +336,6 @@ def test_w8a8_dispatch_sweep(hip, oracle):
 def test_forced_tiles_and_splits_keep_parity(hip, oracle):
     """The environment overrides change which kernel runs, never the result: W8A8 accumulators and outputs stay
     bit-exact and fp32 / skinny products stay inside their gates under every forced tile, split and block count."""
-    import os
     names = ("AX_HIP_I8_TILE", "AX_HIP_I8_SPLITK", "AX_HIP_F32_TILE", "AX_HIP_F32_SPLITK", "AX_HIP_SKINNY_BLOCKS")
     saved = {n: os.environ.get(n) for n in names}
     rng = np.random.default_rng(77)
@@ -600,6 +601,52 @@ def test_short_k_nt_row_blocks(hip, oracle, Bn, M, N, K, alpha):
     want = alpha * np.einsum("hmk,hk->hm", a.astype(np.float64), bsum)
     scale = abs(alpha) * np.einsum("hmk,hk->hm", np.abs(a).astype(np.float64), np.abs(b).astype(np.float64).sum(axis=1))
     assert (np.abs(got.astype(np.float64).sum(axis=2) - want) <= 1e-5 * scale).all()
+
+
+@pytest.mark.parametrize("Bn,M,N,K,alpha,pad", [(200, 512, 64, 128, 1.0, 0), (67, 256, 384, 160, 0.5, 0), (280, 384, 64, 512, 1.0, 0),
+                                                 (72, 512, 128, 1024, 0.25, 0), (264, 256, 64, 224, 2.0, 8), (9, 4096, 256, 192, 1.0, 4)])
+def test_streamed_nn_tiles(hip, oracle, Bn, M, N, K, alpha, pad):
+    """Batched A B with K of a few hundred and many 128 x 64 output tiles: the kernel whose workgroups walk
+    a list of tiles with the K slabs of all of them in one stream; against the CPU path on sampled batch
+    entries and, for every entry, a row-sum identity.  `pad`: extra floats in every leading dimension."""
+    say("streamed nn", Bn, M, N, K, alpha, pad)
+    oracle.seed(Bn + M + N + K)
+    lda, ldb, ldc = K + pad, N + pad, N + pad
+    a_full, b_full = oracle.normal((Bn, M, lda)), oracle.normal((Bn, K, ldb))
+    a, b = a_full[:, :, :K], b_full[:, :, :N]
+    da, db = hip.array(a_full), hip.array(b_full)
+    c = hip.empty((Bn, M, ldc))
+    hip.check(hip.L.axhip_memset(c.ptr, 0xFF, c.nbytes))                 # every output must be written, no pad column
+    hip.check(hip.L.axhip_sgemm_strided_batched(0, 0, M, N, K, alpha, da.ptr, lda, M * lda, db.ptr, ldb, K * ldb, 0.0,
+                                                c.ptr, ldc, M * ldc, Bn))
+    assert hip.last_kernel() == "sgemm_nn_stream128x64_dma"
+    full = c.numpy()
+    got = full[:, :, :N]
+    assert not np.isnan(got).any()
+    if pad:
+        assert np.isnan(full[:, :, N:]).all()
+    for h in sorted({0, 7, Bn // 2, Bn - 1}):
+        rows = slice(max(0, M - 1024), M)
+        want = oracle.gemm_opt(np.ascontiguousarray(a[h][rows]), np.ascontiguousarray(b[h])) * np.float32(alpha)
+        assert np.abs(got[h][rows] - want).max() <= REL_FP32 * np.abs(want).max()
+    # every entry: row sums of C equal alpha * A . (row sums of B), to fp32 accumulation accuracy
+    bsum = b.astype(np.float64).sum(axis=2)
+    want = alpha * np.einsum("hmk,hk->hm", a.astype(np.float64), bsum)
+    scale = abs(alpha) * np.einsum("hmk,hk->hm", np.abs(a).astype(np.float64), np.abs(b).astype(np.float64).sum(axis=2))
+    assert (np.abs(got.astype(np.float64).sum(axis=2) - want) <= 1e-5 * scale).all()
+    # and the same product on the one-tile-per-workgroup kernels
+    os.environ["AX_HIP_F32_TILE"] = "642"
+    try:
+        hip.L.axhip_tuning_reload()
+        c2 = hip.empty((Bn, M, ldc))
+        hip.check(hip.L.axhip_sgemm_strided_batched(0, 0, M, N, K, alpha, da.ptr, lda, M * lda, db.ptr, ldb, K * ldb, 0.0,
+                                                    c2.ptr, ldc, M * ldc, Bn))
+        assert hip.last_kernel() != "sgemm_nn_stream128x64_dma"
+        other = c2.numpy()[:, :, :N]
+    finally:
+        del os.environ["AX_HIP_F32_TILE"]
+        hip.L.axhip_tuning_reload()
+    assert np.abs(got - other).max() <= REL_FP32 * np.abs(other).max()
 
 
 # ------------------------------------------------------------------ W8A32
