@@ -557,19 +557,19 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     AXF_VM(0);
     if constexpr (EDGE) AXF_LGKM(0);             // zeros written for a K tail that is already in the first slabs
     __builtin_amdgcn_s_barrier();
-    for (int s = 0; s < slabs; s += NST) {
+    // whole rounds of the ring in a loop with one way out, then the slabs % NST that remain (nothing is
+    // left to fetch by then): an exit between two slabs of the loop body makes the compiler copy the
+    // accumulators from one register set to another every round
+    int s = 0;
+    for (; s + NST <= slabs; s += NST) {
         AXF_SLAB(0, ring && s + NST - 1 < slabs);
-        if (s + 1 >= slabs) break;
         AXF_SLAB(1, s + NST < slabs);
-        if constexpr (NST > 2) {
-            if (s + 2 >= slabs) break;
-            AXF_SLAB(2, s + NST + 1 < slabs);
-        }
-        if constexpr (NST > 3) {
-            if (s + 3 >= slabs) break;
-            AXF_SLAB(3, s + NST + 2 < slabs);
-        }
+        if constexpr (NST > 2) AXF_SLAB(2, s + NST + 1 < slabs);
+        if constexpr (NST > 3) AXF_SLAB(3, s + NST + 2 < slabs);
     }
+    if (s < slabs) AXF_SLAB(0, false);
+    if (s + 1 < slabs) AXF_SLAB(1, false);
+    if constexpr (NST > 3) { if (s + 2 < slabs) AXF_SLAB(2, false); }
 #undef AXF_ISSUE
 #undef AXF_FRAGS
 #undef AXF_MFMAS

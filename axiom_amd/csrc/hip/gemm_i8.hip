@@ -559,7 +559,7 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     constexpr int NREADS = TM + TN;
     constexpr int VM_KEEP = (NST - 2) * (IPW_X + IPW_W);
     static_assert(IPW_X * 8 * NW == BM && IPW_W * 8 * NW == BN, "slab must divide over the waves");
-    static_assert(NST >= 2 && NST <= 8 && VM_KEEP < 64, "stage count");
+    static_assert(NST >= 2 && NST <= 4 && VM_KEEP < 64, "stage count");
     static_assert((NST - 1) * XS + (TM - 1) * 4096 < 65536 && (NST - 1) * WS + (TN - 1) * 4096 < 65536,
                   "ds_read immediates are 16 bits");
     static_assert(WAVES_K == 1 || WAVES_K == 2, "one or two wave sets over k");
@@ -699,25 +699,23 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     AXI8G_ISSUE(0);
     if constexpr (NST > 2) { if (slabs > 1) AXI8G_ISSUE(1); }
     if constexpr (NST > 3) { if (slabs > 2) AXI8G_ISSUE(2); }
-    if constexpr (NST > 4) { if (slabs > 3) AXI8G_ISSUE(3); }
-    if constexpr (NST > 5) { if (slabs > 4) AXI8G_ISSUE(4); }
-    if constexpr (NST > 6) { if (slabs > 5) AXI8G_ISSUE(5); }
-    if constexpr (NST > 7) { if (slabs > 6) AXI8G_ISSUE(6); }
     if (VM_KEEP > 0 && slabs >= NST - 1) AXI8_VM(VM_KEEP); else AXI8_VM(0);
     if constexpr (EDGE) AXI8_LGKM(0);            // zeros written for a K tail that is already in the first slabs
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
-    for (int s = 0; s < slabs; s += NST) {
+    // whole rounds of the ring in a loop with one way out, then the slabs % NST that remain (nothing is
+    // left to fetch by then): an exit between two slabs of the loop body makes the compiler copy the
+    // accumulators from one register set to another every round
+    int s = 0;
+    for (; s + NST <= slabs; s += NST) {
         AXI8G_SLAB(0, s + NST - 1 < slabs);
-        if (s + 1 >= slabs) break;
         AXI8G_SLAB(1, s + NST < slabs);
-        if constexpr (NST > 2) { if (s + 2 >= slabs) break; AXI8G_SLAB(2, s + NST + 1 < slabs); }
-        if constexpr (NST > 3) { if (s + 3 >= slabs) break; AXI8G_SLAB(3, s + NST + 2 < slabs); }
-        if constexpr (NST > 4) { if (s + 4 >= slabs) break; AXI8G_SLAB(4, s + NST + 3 < slabs); }
-        if constexpr (NST > 5) { if (s + 5 >= slabs) break; AXI8G_SLAB(5, s + NST + 4 < slabs); }
-        if constexpr (NST > 6) { if (s + 6 >= slabs) break; AXI8G_SLAB(6, s + NST + 5 < slabs); }
-        if constexpr (NST > 7) { if (s + 7 >= slabs) break; AXI8G_SLAB(7, s + NST + 6 < slabs); }
+        if constexpr (NST > 2) AXI8G_SLAB(2, s + NST + 1 < slabs);
+        if constexpr (NST > 3) AXI8G_SLAB(3, s + NST + 2 < slabs);
     }
+    if (s < slabs) AXI8G_SLAB(0, false);
+    if (s + 1 < slabs) AXI8G_SLAB(1, false);
+    if constexpr (NST > 3) { if (s + 2 < slabs) AXI8G_SLAB(2, false); }
 #undef AXI8G_ISSUE
 #undef AXI8G_FRAGS
 #undef AXI8G_MFMAS
