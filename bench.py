@@ -544,11 +544,30 @@ def counter_probe(hip, case, repeat=1):
 def sustain(hip, seconds, operands):
     """One GEMM launched back to back for `seconds`, so that clock and power can be sampled from outside
     (rocm-smi) while it runs: the headline over random int8 operands or all-zero ones (same instruction
-    stream, no switching activity in the matrix core), or the fp32 8192^3 product over random / zero
-    operands ("fp32", "fp32zeros").  Prints the average time per launch about once a second."""
+    stream, no switching activity in the matrix core), the fp32 8192^3 product over random / zero
+    operands ("fp32", "fp32zeros"), or the batched attention products ("qkt", "pv", each also with "zeros").
+    Prints the average time per launch about once a second."""
     M = N = K = 8192
     rng = np.random.default_rng(0)
-    if operands.startswith("fp32"):
+    if operands.startswith("qkt") or operands.startswith("pv"):
+        # the attention-shaped products of 512 heads of [512, 64]: Q K^T (writes 537 MB) or P V (reads it)
+        Bn, S, D = 512, 512, 64
+        zeros = operands.endswith("zeros")
+        mk = (lambda shape: hip.empty(shape)) if zeros else (lambda shape: hip.array(rng.normal(0, 1, shape).astype(np.float32)))
+        if operands.startswith("qkt"):
+            q, k_, s_ = mk((Bn, S, D)), mk((Bn, S, D)), hip.empty((Bn, S, S))
+
+            def launch():
+                hip.check(hip.L.axhip_sgemm_strided_batched(0, 1, S, S, D, 1.0, q.ptr, D, S * D, k_.ptr, D, S * D, 0.0,
+                                                            s_.ptr, S, S * S, Bn))
+        else:
+            p_, v_, o_ = mk((Bn, S, S)), mk((Bn, S, D)), hip.empty((Bn, S, D))
+
+            def launch():
+                hip.check(hip.L.axhip_sgemm_strided_batched(0, 0, S, D, S, 1.0, p_.ptr, S, S * S, v_.ptr, D, S * D, 0.0,
+                                                            o_.ptr, D, S * D, Bn))
+        per_print = 4000
+    elif operands.startswith("fp32"):
         if operands == "fp32zeros":
             a, b = hip.empty((M, K)), hip.empty((K, N))
         else:
@@ -661,7 +680,7 @@ def main():
                     choices=["headline", "skinny", "gemm1024", "fp32", "config2", "attention"])
     ap.add_argument("--probe-repeat", type=int, default=1, help="multiplies the launch counts of --counter-probe")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of back-to-back headline launches")
-    ap.add_argument("--operands", choices=["random", "zeros", "fp32", "fp32zeros"], default="random")
+    ap.add_argument("--operands", choices=["random", "zeros", "fp32", "fp32zeros", "qkt", "qktzeros", "pv", "pvzeros"], default="random")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
