@@ -23,6 +23,7 @@ constexpr int KGROUPS = 16;     // lane groups per workgroup, each 16 lanes x fl
 constexpr int UNROLL = 8;
 // workgroups to aim for: enough to cover 256 CUs a few times over; partial-sum traffic grows with M
 constexpr int64_t kWantBlocksM12 = 1024, kWantBlocksM3up = 512;      // M = 1, 2 / M >= 3
+constexpr int kJoinChunk = 16;              // splits whose partials the finishing workgroup requests at once
 
 // A narrow layer riding on this one: out2[m, j] = act2(sum_n C[m, n] * W[n, j] + bias2[j]), j < nh <= 16
 // (a hidden layer followed by a classifier head).  The workgroup that finishes a strip has that strip's 64
@@ -309,7 +310,7 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
     // Each thread owns up to OUTS outputs.  All partials of a chunk of splits are requested
     // before the first is used (one trip to memory per chunk, not per split); they are added
     // in split order.
-    constexpr int OUTS = (MR * COLS + 255) / 256, CHUNK = 16;
+    constexpr int OUTS = (MR * COLS + 255) / 256, CHUNK = kJoinChunk;
     const float *pp[OUTS];
     float s[OUTS];
     bool ok[OUTS];
@@ -382,6 +383,11 @@ int plan_skinny(int64_t M, int64_t N, int64_t K, const float *B, int64_t ldb, Sk
     int64_t splits = (want_blocks + p.col_blocks - 1) / p.col_blocks;
     const int64_t max_splits = K >= 128 ? K / 128 : 1;
     if (splits > max_splits) splits = max_splits;
+    // The workgroup that finishes a strip requests the partials of up to 16 splits at once: more splits
+    // mean more dependent trips to memory at the very end of the launch (M = 1, 8192 x 1024: 20.7 us with
+    // 64 splits, 11.8 with 16).  A narrow matrix gets longer workgroups instead of more of them.
+    const bool narrow = splits > kJoinChunk;
+    if (narrow) splits = kJoinChunk;
     if (splits < 1) splits = 1;
     int64_t kps = (K + splits - 1) / splits;
     kps = (kps + KGROUPS - 1) / KGROUPS * KGROUPS;
@@ -391,7 +397,8 @@ int plan_skinny(int64_t M, int64_t N, int64_t K, const float *B, int64_t ldb, Sk
     // with one 96 KiB workgroup per CU, 60 us this way)
     const int64_t max_kps = ((int64_t)(52 * 1024 / 4) - p.red_floats) / M / KGROUPS * KGROUPS;
     if (kps > max_kps) kps = max_kps;
-    if (kps > 512) kps = 512;      // at most 128 KiB of weights per workgroup: wide matrices get more workgroups, not longer ones
+    // at most 128 KiB of weights per workgroup: wide matrices get more workgroups, not longer ones
+    if (kps > (narrow ? 2048 : 512)) kps = narrow ? 2048 : 512;
     if (kps < KGROUPS) kps = KGROUPS;
     splits = K > 0 ? (K + kps - 1) / kps : 1;
     if (splits > 65535) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: K=%lld too large", (long long)K);
