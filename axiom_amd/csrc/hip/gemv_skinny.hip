@@ -24,6 +24,7 @@ constexpr int UNROLL = 8;
 // workgroups to aim for: enough to cover 256 CUs a few times over; partial-sum traffic grows with M
 constexpr int64_t kWantBlocksM12 = 1024, kWantBlocksM3up = 512;      // M = 1, 2 / M >= 3
 constexpr int kJoinChunk = 16;              // splits whose partials the finishing workgroup requests at once
+constexpr int kMfmaFromM = 9;              // from this M on the products run on the matrix cores (16-byte aligned rows); below, the vector ALU form measured faster (M = 8, 4096 x 32000: 107 us against 117)
 
 // A narrow layer riding on this one: out2[m, j] = act2(sum_n C[m, n] * W[n, j] + bias2[j]), j < nh <= 16
 // (a hidden layer followed by a classifier head).  The workgroup that finishes a strip has that strip's 64
@@ -76,13 +77,18 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
             const int kk = tid + c * 256;
             xr[m][c] = kk < klen32 ? A[m * lda + k_begin + kk] : 0.0f;
         }
-    // first batch of weights (VEC form, full batch available)
-    const bool pre = VEC && col < N && (UNROLL - 1) * KGROUPS + kg < klen;
+    // first batch of weights (VEC form, full batch available).  From M = 9 on the products run on the
+    // matrix cores, whose instructions every lane of a wave must reach together: there the batch is taken
+    // when all lane groups have it (pre_all, the same for the whole workgroup).
+    constexpr bool MFMA = VEC && MR >= kMfmaFromM;
+    const bool pre_all = UNROLL * KGROUPS <= klen;
+    const bool pre = MFMA ? pre_all : (VEC && col < N && (UNROLL - 1) * KGROUPS + kg < klen);
     v4f w0[UNROLL];
     if (pre) {
+        const float *bf = MFMA && col >= N ? B + n0 : bp;     // MFMA form: see below
 #pragma unroll
         for (int u = 0; u < UNROLL; u++)
-            w0[u] = *reinterpret_cast<const v4f *>(bp + (k_begin + k + u * KGROUPS) * ldb);
+            w0[u] = *reinterpret_cast<const v4f *>(bf + (k_begin + k + u * KGROUPS) * ldb);
     }
 
     // the head's block of weights for this strip (64 rows x nh <= 1024 floats), requested now so that it
@@ -116,7 +122,55 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
 #pragma unroll
         for (int e = 0; e < 4; e++) acc[m][e] = 0.0f;
 
-    if (VEC) {
+    // M = 9..16 on v_mfma_f32_16x16x4_f32.  The weight layout is already the instruction's: the four lane
+    // groups of a wave hold four consecutive k rows, lane cg of a group the columns 4*cg .. 4*cg+3, so
+    // element j of the loaded float4 is the B operand (k = lane / 16, n = lane % 16) of the product for
+    // columns 4*i + j, and the A operand is the activation of row m = lane % 16 at the lane group's k:
+    // one LDS read and four MFMAs per 16 bytes of weights, against M reads and 4 M multiply-adds.
+    // dm[j][v] = C[4 * (lane / 16) + v][4 * cg + j], summed over the wave's k rows.
+    v4f dm[4];
+    if constexpr (MFMA) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) dm[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        // A lane past the last column reads the strip's first columns instead and a lane whose row m does
+        // not exist reads row 0: what they compute lands in columns / rows that are never stored, and the
+        // loads of a full batch need no predicate.
+        const float *bq = col < N ? bp : B + n0;
+        const float *xrow = xs + (cg < MR ? cg : 0) * k_per_split;
+        if (pre_all) {
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const float xa = xrow[k + u * KGROUPS];
+#pragma unroll
+                for (int j = 0; j < 4; j++) dm[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa, w0[u][j], dm[j], 0, 0, 0);
+            }
+            k += UNROLL * KGROUPS;
+        }
+        // every lane makes the same number of rounds: k - kg is the same for the whole workgroup
+        int64_t kb = k - kg;
+        for (; kb + UNROLL * KGROUPS <= klen; kb += UNROLL * KGROUPS) {
+            v4f w[UNROLL];
+            float xa[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                w[u] = *reinterpret_cast<const v4f *>(bq + (k_begin + kb + u * KGROUPS + kg) * ldb);
+                xa[u] = xrow[kb + u * KGROUPS + kg];
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) dm[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[u], w[u][j], dm[j], 0, 0, 0);
+        }
+        // the last, partial batch: a lane whose row lies past the split contributes zeros
+        for (; kb < klen; kb += KGROUPS) {
+            const int64_t row = kb + kg;
+            const bool in = row < klen;
+            const v4f w = in ? *reinterpret_cast<const v4f *>(bq + (k_begin + row) * ldb) : v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            const float xa = in ? xrow[row] : 0.0f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) dm[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa, w[j], dm[j], 0, 0, 0);
+        }
+    } else if (VEC) {
         if (col < N) {      // N % 4 == 0: a float4 is entirely inside or outside
             if (pre) {
 #pragma unroll
@@ -196,9 +250,18 @@ k_skinny(const float *__restrict__ A, int64_t lda, const float *__restrict__ B, 
     // l^16, l^32, l^48 hold the same columns) are first added with the row-swap instructions, so
     // that one partial per wave goes through LDS and the buffer stays small enough for three
     // workgroups per CU; up to M = 8 every lane group writes its own partial (measured faster there).
-    constexpr bool PRE = MR > 8;
+    constexpr bool PRE = MR > 8 || MFMA;
     constexpr int NPART = PRE ? 4 : KGROUPS;
     float *red = sm + (int64_t)MR * k_per_split;
+    if constexpr (MFMA) {
+        // the wave's sums are complete in dm: one partial tile per wave, rows 4 * (lane / 16) + v
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int m = 4 * ((tid & 63) >> 4) + v;
+            if (m < MR)
+                *reinterpret_cast<v4f *>(red + ((tid >> 6) * MR + m) * COLS + 4 * cg) = v4f{dm[0][v], dm[1][v], dm[2][v], dm[3][v]};
+        }
+    } else
 #pragma unroll
     for (int m = 0; m < MR; m++) {
         if (PRE) {
@@ -392,7 +455,8 @@ int plan_skinny(int64_t M, int64_t N, int64_t K, const float *B, int64_t ldb, Sk
     int64_t kps = (K + splits - 1) / splits;
     kps = (kps + KGROUPS - 1) / KGROUPS * KGROUPS;
     // the activations of one split must fit LDS next to the reduction buffer
-    p.red_floats = (int64_t)(M > 8 ? 4 : KGROUPS) * M * COLS;   // partials per workgroup, as in the kernel
+    p.vec = (N % 4 == 0) && (ldb % 4 == 0) && ((uintptr_t)B % 16 == 0);
+    p.red_floats = (int64_t)(M > 8 || (p.vec && M >= kMfmaFromM) ? 4 : KGROUPS) * M * COLS;   // partials per workgroup, as in the kernel
     // ... within 52 KiB, so that three workgroups share a CU whatever M is (4096 x 11008 at M = 16: 95 us
     // with one 96 KiB workgroup per CU, 60 us this way)
     const int64_t max_kps = ((int64_t)(52 * 1024 / 4) - p.red_floats) / M / KGROUPS * KGROUPS;
@@ -404,7 +468,6 @@ int plan_skinny(int64_t M, int64_t N, int64_t K, const float *B, int64_t ldb, Sk
     if (splits > 65535) return fail(AXHIP_ERR_SHAPE, "sgemm_skinny: K=%lld too large", (long long)K);
     p.splits = splits;
     p.kps = kps;
-    p.vec = (N % 4 == 0) && (ldb % 4 == 0) && ((uintptr_t)B % 16 == 0);
     p.smem = (size_t)(M * kps + p.red_floats) * sizeof(float);
     p.partial_bytes = splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
     return AXHIP_OK;
