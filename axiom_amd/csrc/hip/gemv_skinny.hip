@@ -7,8 +7,9 @@
 // a k row are wave-uniform only per lane group, so they come from LDS (staged once per
 // workgroup); the first batch of weight loads is issued before that staging so HBM latency
 // overlaps it.  The 16 lane groups' sums are joined through LDS in a fixed order; from M = 9 on the
-// four lane groups of a wave are first added inside the wave (row swaps), which keeps the LDS
-// buffer at four partial tiles whatever M is.  When K is split over
+// products run on the matrix cores (v_mfma_f32_16x16x4_f32, which sums a wave's four k rows itself;
+// rows off the 16-byte grid: vector ALU, the four lane groups of a wave added with row swaps), which
+// keeps the LDS buffer at four partial tiles whatever M is.  When K is split over
 // several workgroups each writes its partial tile to a workspace and bumps a per-strip
 // counter; the workgroup that arrives last adds the partials in split order (not arrival
 // order) and applies bias and activation.  The sum order is fixed, so results are
