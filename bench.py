@@ -292,6 +292,30 @@ def secondary(hip):
     res["skinny_layer_8192x8192"] = big
     del big_sets
 
+    # what a skinny launch costs before and beyond its bytes: time against K at N = 4096, M = 1 (weights from
+    # HBM, rotating sets of at least 600 MB), least-squares line  time = fixed + bytes / rate
+    pts = []
+    for K in (512, 1024, 2048, 4096, 8192, 16384):
+        nset = max(3, int(600e6 / (K * 4096 * 4)) + 1)
+        base = rng.uniform(-0.03, 0.03, (K, 4096)).astype(np.float32)      # the same values in every set: only the addresses differ
+        wsets = [hip.array(base) for _ in range(nset)]
+        xin, yo_ = hip.array(rng.uniform(0, 1, (1, K)).astype(np.float32)), hip.empty((1, 4096))
+        it = [0]
+
+        def line_step():
+            w_ = wsets[it[0] % nset]
+            it[0] += 1
+            hip.check(hip.L.axhip_sgemm(0, 0, 1, 4096, K, 1.0, xin.ptr, K, w_.ptr, 4096, 0.0, yo_.ptr, 4096, zeros.ptr, 1))
+
+        _, ms = time_calls(hip, line_step, seconds=0.15)
+        pts.append((K * 4096 * 4, ms * 1e3))
+        del wsets
+    xs_, ys_ = np.array([p[0] for p in pts], np.float64), np.array([p[1] for p in pts], np.float64)
+    slope, fixed = np.polyfit(xs_, ys_, 1)
+    res["skinny_time_vs_bytes_M1_N4096"] = {
+        "points_MB_us": [[b / 1e6, t] for b, t in pts], "fixed_us": float(fixed), "marginal_GB/s": float(1e-3 / slope),
+        "marginal_frac_of_hbm_peak": float(1e-3 / slope / PEAK_HBM_GBS), "launch_floor_us": None}
+
     # config 4b: strided-batched attention-shaped products, 512 heads of [512,64]
     Bn, S, D = 512, 512, 64
     q = hip.array(rng.normal(0, 1, (Bn, S, D)).astype(np.float32))
@@ -362,6 +386,7 @@ def secondary(hip):
     tiny = hip.empty((64,))
     _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_fill_f32(tiny.ptr, 1.0, 64)))
     res["launch_floor_us"] = ms * 1e3
+    res["skinny_time_vs_bytes_M1_N4096"]["launch_floor_us"] = ms * 1e3
     del tiny
 
     # the seven shapes of the reference's benchmarks/bench_qgemm.c:76-82 (fp32 GEMM against W8A32 on the
