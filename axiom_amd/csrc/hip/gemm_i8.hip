@@ -543,7 +543,7 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 // waves on every SIMD with no more global traffic, so one wave's waits for LDS and for the slab
 // barrier are covered by the other's MFMAs: for a launch of at most one small tile per CU, whose
 // time is the chain of those waits rather than memory or matrix-core throughput.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int ACT, bool EDGE = false, int WAVES_K = 1>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int ACT, bool EDGE = false, int WAVES_K = 1, int SPB = 1>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64)
 k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
                  int64_t K, float x_scale, const float *__restrict__ w_scales,
@@ -553,17 +553,21 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     constexpr int NWO = WAVES_M * WAVES_N, NW = NWO * WAVES_K, BKB = 128;      // waves that own outputs / all waves
     constexpr int KSTEPS = 4 / WAVES_K;                                        // k-steps of a slab per wave
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
-    constexpr int XS = BM * BKB, WS = BN * BKB;          // bytes of one stage of each operand
-    constexpr int W_BASE = NST * XS;
+    // SPB = 2: a stage holds two slabs and the loop synchronises once per two (half the barriers and
+    // waits, for tiles whose slab is only a few dozen MFMA cycles); K is then a multiple of 256, no
+    // EDGE and no split.  XS / WS stay the bytes of ONE slab; a stage is SPB of them.
+    constexpr int XS = BM * BKB, WS = BN * BKB;          // bytes of one slab of each operand
+    constexpr int W_BASE = NST * SPB * XS;
     constexpr int IPW_X = BM / 8 / NW, IPW_W = BN / 8 / NW;   // load instructions per wave and slab
     constexpr int NREADS = TM + TN;
-    constexpr int VM_KEEP = (NST - 2) * (IPW_X + IPW_W);
+    constexpr int VM_KEEP = (NST - 2) * SPB * (IPW_X + IPW_W);
     static_assert(IPW_X * 8 * NW == BM && IPW_W * 8 * NW == BN, "slab must divide over the waves");
     static_assert(NST >= 2 && NST <= 4 && VM_KEEP < 64, "stage count");
-    static_assert((NST - 1) * XS + (TM - 1) * 4096 < 65536 && (NST - 1) * WS + (TN - 1) * 4096 < 65536,
+    static_assert(SPB == 1 || (SPB == 2 && !EDGE), "one or two slabs per stage");
+    static_assert((NST * SPB - 1) * XS + (TM - 1) * 4096 < 65536 && (NST * SPB - 1) * WS + (TN - 1) * 4096 < 65536,
                   "ds_read immediates are 16 bits");
     static_assert(WAVES_K == 1 || WAVES_K == 2, "one or two wave sets over k");
-    static_assert(NWO * 4096 + (WAVES_K - 1) * NWO * TM * TN * 4096 <= NST * XS, "write-back turn area and k hand-over");
+    static_assert(NWO * 4096 + (WAVES_K - 1) * NWO * TM * TN * 4096 <= NST * SPB * XS, "write-back turn area and k hand-over");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -615,7 +619,7 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     }
 
     typedef float v4f_t __attribute__((ext_vector_type(4)));
-    float *lds_scale = reinterpret_cast<float *>(lds + NST * (XS + WS)), *lds_bias = lds_scale + BN;
+    float *lds_scale = reinterpret_cast<float *>(lds + NST * SPB * (XS + WS)), *lds_bias = lds_scale + BN;
     if (out) {
         for (int c = tid; c < BN; c += NW * 64) {
             const bool live = c < nrows;
@@ -633,7 +637,7 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
     v4i fx[2][TM], fw[2][TN];
 
-#define AXI8G_ISSUE(ST)                                                                          \
+#define AXI8G_ISSUE1(ST)                                                                         \
     do {                                                                                         \
         --left;                                                                                  \
         if (EDGE && left == 0 && ktail < BKB) {                                                  \
@@ -656,6 +660,12 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         gx += BKB;                                                                               \
         gw += BKB;                                                                               \
     } while (0)
+// a stage: SPB slabs into consecutive slab places
+#define AXI8G_ISSUE(ST)                                                                          \
+    do {                                                                                         \
+        AXI8G_ISSUE1((ST) * SPB);                                                                \
+        if constexpr (SPB == 2) AXI8G_ISSUE1((ST) * SPB + 1);                                    \
+    } while (0)
 #define AXI8G_FRAGS(buf, ST, ks)                                                                 \
     do {                                                                                         \
         _Pragma("unroll") for (int t = 0; t < TM; t++)                                           \
@@ -673,33 +683,39 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         __builtin_amdgcn_sched_barrier(0);                                                       \
     } while (0)
     // one slab out of stage ST; `more`: slab s+NST-1 exists and is fetched into the stage read last
-#define AXI8G_SLAB(ST, more)                                                                     \
+#define AXI8G_COMPUTE(SS)                                                                        \
     do {                                                                                         \
-        if (more) AXI8G_ISSUE(((ST) + NST - 1) % NST);                                           \
-        AXI8G_FRAGS(0, ST, 0);                                                                   \
-        AXI8G_FRAGS(1, ST, 1);                                                                   \
+        AXI8G_FRAGS(0, SS, 0);                                                                   \
+        AXI8G_FRAGS(1, SS, 1);                                                                   \
         AXI8_LGKM(NREADS);                                                                       \
         AXI8G_MFMAS(0);                                                                          \
         if constexpr (KSTEPS == 4) {                                                             \
-            AXI8G_FRAGS(0, ST, 2);                                                               \
+            AXI8G_FRAGS(0, SS, 2);                                                               \
             AXI8_LGKM(NREADS);                                                                   \
             AXI8G_MFMAS(1);                                                                      \
-            AXI8G_FRAGS(1, ST, 3);                                                               \
+            AXI8G_FRAGS(1, SS, 3);                                                               \
             AXI8_LGKM(NREADS);                                                                   \
             AXI8G_MFMAS(0);                                                                      \
         }                                                                                        \
         AXI8_LGKM(0);                                                                            \
         AXI8G_MFMAS(1);                                                                          \
+    } while (0)
+#define AXI8G_SLAB(ST, more)                                                                     \
+    do {                                                                                         \
+        if (more) AXI8G_ISSUE(((ST) + NST - 1) % NST);                                           \
+        AXI8G_COMPUTE((ST) * SPB);                                                               \
+        if constexpr (SPB == 2) AXI8G_COMPUTE((ST) * SPB + 1);                                   \
         if (VM_KEEP > 0 && (more)) AXI8_VM(VM_KEEP); else AXI8_VM(0);                            \
         __builtin_amdgcn_s_barrier();                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     } while (0)
 
     // prologue: the first NST-1 slabs are requested; compute starts as soon as the first has landed
+    const int rounds = slabs / SPB;              // stages' worth of slabs (SPB == 2: the host guarantees an even count)
     AXI8G_ISSUE(0);
-    if constexpr (NST > 2) { if (slabs > 1) AXI8G_ISSUE(1); }
-    if constexpr (NST > 3) { if (slabs > 2) AXI8G_ISSUE(2); }
-    if (VM_KEEP > 0 && slabs >= NST - 1) AXI8_VM(VM_KEEP); else AXI8_VM(0);
+    if constexpr (NST > 2) { if (rounds > 1) AXI8G_ISSUE(1); }
+    if constexpr (NST > 3) { if (rounds > 2) AXI8G_ISSUE(2); }
+    if (VM_KEEP > 0 && rounds >= NST - 1) AXI8_VM(VM_KEEP); else AXI8_VM(0);
     if constexpr (EDGE) AXI8_LGKM(0);            // zeros written for a K tail that is already in the first slabs
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
@@ -707,18 +723,20 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
     // left to fetch by then): an exit between two slabs of the loop body makes the compiler copy the
     // accumulators from one register set to another every round
     int s = 0;
-    for (; s + NST <= slabs; s += NST) {
-        AXI8G_SLAB(0, s + NST - 1 < slabs);
-        AXI8G_SLAB(1, s + NST < slabs);
-        if constexpr (NST > 2) AXI8G_SLAB(2, s + NST + 1 < slabs);
-        if constexpr (NST > 3) AXI8G_SLAB(3, s + NST + 2 < slabs);
+    for (; s + NST <= rounds; s += NST) {
+        AXI8G_SLAB(0, s + NST - 1 < rounds);
+        AXI8G_SLAB(1, s + NST < rounds);
+        if constexpr (NST > 2) AXI8G_SLAB(2, s + NST + 1 < rounds);
+        if constexpr (NST > 3) AXI8G_SLAB(3, s + NST + 2 < rounds);
     }
-    if (s < slabs) AXI8G_SLAB(0, false);
-    if (s + 1 < slabs) AXI8G_SLAB(1, false);
-    if constexpr (NST > 3) { if (s + 2 < slabs) AXI8G_SLAB(2, false); }
+    if (s < rounds) AXI8G_SLAB(0, false);
+    if (s + 1 < rounds) AXI8G_SLAB(1, false);
+    if constexpr (NST > 3) { if (s + 2 < rounds) AXI8G_SLAB(2, false); }
+#undef AXI8G_ISSUE1
 #undef AXI8G_ISSUE
 #undef AXI8G_FRAGS
 #undef AXI8G_MFMAS
+#undef AXI8G_COMPUTE
 #undef AXI8G_SLAB
 
     if constexpr (WAVES_K == 2) {
@@ -861,16 +879,16 @@ int pick_splits(int64_t tiles, int64_t slabs) {
     return (int)((slabs + per - 1) / per);          // drop ranges that would be empty
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool EDGE = false, int WAVES_K = 1>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool EDGE = false, int WAVES_K = 1, int SPB = 1>
 int launch_dma(const char *name, const char *split_name, const int8_t *x, float x_scale, const int8_t *w,
                const float *w_scales, const float *bias, int act, float *out, int32_t *acc_out, int64_t M, int64_t N,
                int64_t K, int64_t ldc) {
-    constexpr int smem = NST * (BM + BN) * 128 + 2 * BN * 4 + 16;      // stages, scale and bias rows, the split join's flag
+    constexpr int smem = NST * SPB * (BM + BN) * 128 + 2 * BN * 4 + 16;      // stages, scale and bias rows, the split join's flag
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
                            const float *, float *, int32_t *, int64_t, int, int32_t *, int *);
-    static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE, WAVES_K>,
-                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU, EDGE, WAVES_K>,
-                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE, WAVES_K>};
+    static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE, WAVES_K, SPB>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU, EDGE, WAVES_K, SPB>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE, WAVES_K, SPB>};
     static bool attr_set = false;
     if (!attr_set) {
         for (kern_t kf : kerns)
@@ -881,7 +899,7 @@ int launch_dma(const char *name, const char *split_name, const int8_t *x, float 
     }
     const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     if (tiles > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: too many tiles");
-    const int splits = pick_splits(tiles, (K + 127) / 128);
+    const int splits = SPB == 2 ? 1 : pick_splits(tiles, (K + 127) / 128);     // two slabs per stage: the caller checked that no split is wanted
     int32_t *partials = nullptr;
     int *counters = nullptr;
     if (splits > 1) {
@@ -1011,13 +1029,19 @@ int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_
         if (fits128 && (force == 128 || (force == 0 && (M / 128) * (N / 128) >= 256)))
             return launch_dma<128, 128, 2, 2, 3>("qgemm_w8a8_128x128_dma", "qgemm_w8a8_128x128_dma_splitk", x, x_scale, w,
                                                  w_scales, bias, act, out, acc_out, M, N, K, ldc);
-        // at most one 64x64 tile per CU: the whole LDS goes to slabs in flight (M = 256, N = K = 4096: 8 stages
-        // xx us against 9.6 with four), since a lone workgroup's loads are bound by latency, not by the CU's fill rate
         // at most one 64x64 tile per CU: two wave sets share each slab's k-steps (M = 256, N = K = 4096: 9.8 us
-        // against 10.5; 256 x 2048 x 8192: 14.8 against 17.7)
-        if (force == 642 || (force == 0 && (M / 64) * (N / 64) <= cu_count()))
+        // against 10.5; 256 x 2048 x 8192: 14.8 against 17.7).  Such a launch is bound by what one CU can pull
+        // out of L2: 512 KiB of operand rows per workgroup at the 115 GB/s a lone workgroup reaches on L2 hits
+        // is 4.5 us, and more stages in flight (six, eight) change nothing.
+        if (force == 642 || (force == 0 && (M / 64) * (N / 64) <= cu_count())) {
+            // a slab of such a tile is 64 MFMA cycles per wave: with K on the 256 grid and no split, two slabs
+            // per stage and barrier (three stages of 32 KiB; M = 256, N = K = 4096: 8.6 us against 8.9)
+            if (K % 256 == 0 && K >= 1024 && pick_splits((M / 64) * (N / 64), K / 128) == 1)
+                return launch_dma<64, 64, 2, 2, 3, false, 2, 2>("qgemm_w8a8_64x64k2_dma", "qgemm_w8a8_64x64k2_dma_splitk", x, x_scale,
+                                                                w, w_scales, bias, act, out, acc_out, M, N, K, ldc);
             return launch_dma<64, 64, 2, 2, 4, false, 2>("qgemm_w8a8_64x64k2_dma", "qgemm_w8a8_64x64k2_dma_splitk", x, x_scale, w,
                                                          w_scales, bias, act, out, acc_out, M, N, K, ldc);
+        }
         return launch_dma<64, 64, 2, 2, 4>("qgemm_w8a8_64x64_dma", "qgemm_w8a8_64x64_dma_splitk", x, x_scale, w, w_scales,
                                            bias, act, out, acc_out, M, N, K, ldc);
     }
