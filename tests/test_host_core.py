@@ -168,3 +168,41 @@ def test_error_convention_and_no_cpu_compute(ax):
         L.ax_set_default_device(0)
         ax.free(b2, out)
     ax.free(a, b)
+
+
+def test_backend_refuses_overlapping_rows_without_touching_the_device(ax):
+    """The backend's matrix view of a tensor (hip_backend.c, as_matrix) refuses a 2-D view whose rows overlap or
+    repeat (row stride below the row length: an expanded row, say) instead of reading it as a dense matrix.  The
+    check comes before any device call, so it is exercised here with host tensors relabelled as device ones."""
+    L = ax.L
+    layout = json.load(open(os.path.join(ROOT, "tests", "golden", "abi_layout.json")))
+    plugin = C.CDLL(os.path.join(ROOT, "axiom_amd", "lib", "libax_hip_plugin.so"))
+    table = C.addressof(C.c_char.in_dll(plugin, "ax_hip_ops"))
+    from axiom_amd.axiom import TP
+    gemm = C.CFUNCTYPE(C.c_int, TP, TP, TP)(C.c_void_p.from_address(table + layout["struct ax_backend_ops.gemm"]).value)
+    L.ax_set_default_device(0)
+    sh, nd = ax.shape_arg((4, 8))
+    a, out = L.ax_tensor_zeros(sh, nd, 0), L.ax_tensor_zeros(sh, nd, 0)
+    sh2, nd2 = ax.shape_arg((8, 8))
+    b = L.ax_tensor_zeros(sh2, nd2, 0)
+    AX_DEVICE_HIP = 2
+    saved = [t.contents.storage.contents.device for t in (a, b, out)]
+    try:
+        for t in (a, b, out):
+            t.contents.storage.contents.device = AX_DEVICE_HIP
+        a.contents.strides[0] = 0                    # four copies of one row
+        L.ax_err_clear()
+        assert gemm(a, b, out) == 3                  # AX_ERR_SHAPE_MISMATCH
+        assert "overlap" in ax.err()[1]
+        a.contents.strides[0] = 4                    # rows of 8 that start 4 apart
+        assert gemm(a, b, out) == 3
+        a.contents.strides[0] = 8
+        out.contents.strides[0] = 7
+        assert gemm(a, b, out) == 3 and "out" in ax.err()[1]
+    finally:
+        a.contents.strides[0] = 8
+        out.contents.strides[0] = 8
+        for t, d in zip((a, b, out), saved):
+            t.contents.storage.contents.device = d
+        L.ax_err_clear()
+        ax.free(a, b, out)
