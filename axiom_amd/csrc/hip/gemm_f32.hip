@@ -1127,7 +1127,7 @@ int try_nn_stream(const SgemmArgs &g, int64_t batch) {
 
 // Chooses the largest tile that still leaves about eight waves per CU; returns -1 when the
 // shape does not qualify for the fast path (the caller then uses the register-staged kernel).
-// names: 128x256, 64x64, 64x64 with the k split.
+// names: 128x128, 64x64, 64x64 with the k split.
 template <bool A_KC, bool B_KC>
 int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
     const bool ok = g.K % 4 == 0 && g.K > 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
@@ -1142,22 +1142,24 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
         return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 1, true>(edge_names[0], g, batch);
     }
     auto count = [&](int64_t bm, int64_t bn) { return (g.M / bm) * (g.N / bn) * batch; };
-    // Sustained timings over the benchmark shapes: 128x256 (8 waves, one workgroup per CU) wins
-    // once it fills the chip; below that 64x64 tiles with the k split beat 128x128 and 128x64
-    // everywhere, and two stages are as good as three or four.  With only a few slabs per tile
-    // (K <= 128) a workgroup's life is mostly its loads and its write-back: plain 64x64 tiles,
-    // several workgroups per CU.
+    // Sustained timings over the benchmark shapes: 128x128 with eight waves (2 x 4, wave tile 64x32;
+    // 64 KiB of LDS, so two workgroups share a CU and one's first loads and write-back run under the
+    // other's MFMAs) wins once there is a tile for every CU: 8192^3 151 TFLOP/s against 145 on 128x256
+    // tiles (one workgroup per CU) and 4096^3 148 against 143; the four-wave form of the same tile and
+    // 128x64 are behind both.  Below that 64x64 tiles with the k split are best everywhere, and two
+    // stages are as good as three or four.  With only a few slabs per tile (K <= 128) a workgroup's
+    // life is mostly its loads and its write-back: plain 64x64 tiles, several workgroups per CU.
     const int force = tuning().f32_tile;         // 0 = by shape; 128, 64 or 642 (64x64 with the k split) where the shape permits
-    if (force == 128 && g.M % 128 == 0 && g.N % 256 == 0 && g.K >= 64)
-        return launch_dma<128, 256, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
+    if (force == 128 && g.M % 128 == 0 && g.N % 128 == 0 && g.K >= 64)
+        return launch_dma<128, 128, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
     if (force == 642 && g.K >= 64) return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[2], g, batch);
     if (force == 64) return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
     if (g.K > 128) {
-        // ... provided its rounds of one tile per CU come out nearly full: 384 tiles are a full round
-        // and a half-empty one (3072x4096x2048: 106 TFLOP/s, against 130 on 64x64 tiles)
-        const int64_t big = count(128, 256), cus = cu_count(), rounds = (big + cus - 1) / cus;
-        if (g.M % 128 == 0 && g.N % 256 == 0 && big >= 256 && big * 10 >= rounds * cus * 9)
-            return launch_dma<128, 256, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
+        // ... provided the tiles come out at nearly the same number for every CU: 384 tiles are one
+        // each and a second one for half the CUs, which then take twice as long
+        const int64_t big = count(128, 128), cus = cu_count(), rounds = (big + cus - 1) / cus;
+        if (g.M % 128 == 0 && g.N % 128 == 0 && big >= cus && big * 10 >= rounds * cus * 9)
+            return launch_dma<128, 128, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
         return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[2], g, batch);
     }
     return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
@@ -1166,7 +1168,7 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
 // The same fast path with int8 weights as the B operand (W8A32: A fp32 [M,K], B int8 [N,K], the
 // per-column scale applied in the write-back).  K must be a multiple of 32 (whole slabs, rows of B on
 // 16-byte boundaries); M and N may be off the tile grid.  Returns -1 when the shape does not qualify.
-const char *const kI8DmaNames[3] = {"qgemm_w8a32_mfma_128x256_dma", "qgemm_w8a32_mfma_64x64_dma", "qgemm_w8a32_mfma_64x64k2_dma"};
+const char *const kI8DmaNames[3] = {"qgemm_w8a32_mfma_128x128_dma", "qgemm_w8a32_mfma_64x64_dma", "qgemm_w8a32_mfma_64x64k2_dma"};
 int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
     const bool ok = g.K % 32 == 0 && g.K > 0 && ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) &&
                     ((uintptr_t)g.C % 16 == 0) && ((uintptr_t)g.bias % 16 == 0) && ((uintptr_t)g.col_scale % 16 == 0) &&
@@ -1179,9 +1181,9 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
         return launch_dma<64, 64, 2, 2, 2, true, true, 1, 1, true, int8_t>(names[1], g, batch);
     }
     if (g.K > 128) {
-        const int64_t big = (g.M / 128) * (g.N / 256) * batch, cus = cu_count(), rounds = (big + cus - 1) / cus;
-        if (g.M % 128 == 0 && g.N % 256 == 0 && big >= 256 && big * 10 >= rounds * cus * 9)
-            return launch_dma<128, 256, 2, 4, 2, true, true, 1, 1, false, int8_t>(names[0], g, batch);
+        const int64_t big = (g.M / 128) * (g.N / 128) * batch, cus = cu_count(), rounds = (big + cus - 1) / cus;
+        if (g.M % 128 == 0 && g.N % 128 == 0 && big >= cus && big * 10 >= rounds * cus * 9)
+            return launch_dma<128, 128, 2, 4, 2, true, true, 1, 1, false, int8_t>(names[0], g, batch);
         return launch_dma<64, 64, 2, 2, 2, true, true, 1, 2, false, int8_t>(names[2], g, batch);
     }
     return launch_dma<64, 64, 2, 2, 2, true, true, 1, 1, false, int8_t>(names[1], g, batch);
@@ -1311,9 +1313,9 @@ int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     static const char *const nn[3] = {"sgemm_nn_128x128", "sgemm_nn_64x64", "sgemm_nn_64x64_guarded"};
     static const char *const nt[3] = {"sgemm_nt_128x128", "sgemm_nt_64x64", "sgemm_nt_64x64_guarded"};
     static const char *const tn[3] = {"sgemm_tn_128x128", "sgemm_tn_64x64", "sgemm_tn_64x64_guarded"};
-    static const char *const nn_d[3] = {"sgemm_nn_128x256_dma", "sgemm_nn_64x64_dma", "sgemm_nn_64x64k2_dma"};
-    static const char *const nt_d[3] = {"sgemm_nt_128x256_dma", "sgemm_nt_64x64_dma", "sgemm_nt_64x64k2_dma"};
-    static const char *const tn_d[3] = {"sgemm_tn_128x256_dma", "sgemm_tn_64x64_dma", "sgemm_tn_64x64k2_dma"};
+    static const char *const nn_d[3] = {"sgemm_nn_128x128_dma", "sgemm_nn_64x64_dma", "sgemm_nn_64x64k2_dma"};
+    static const char *const nt_d[3] = {"sgemm_nt_128x128_dma", "sgemm_nt_64x64_dma", "sgemm_nt_64x64k2_dma"};
+    static const char *const tn_d[3] = {"sgemm_tn_128x128_dma", "sgemm_tn_64x64_dma", "sgemm_tn_64x64k2_dma"};
     int rc = -1;
     if (!transa && transb) rc = try_nt_rows(g, batch);
     if (!transa && !transb) rc = try_nn_stream(g, batch);
@@ -1329,7 +1331,7 @@ int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
 }
 
 // A large fp32 shape off the tile grid runs on 64x64 tiles with guarded edges (4000^3: 125
-// TFLOP/s against 141 for 128x256 tiles on the grid).  When it is large enough for 128x256
+// TFLOP/s against 141 for the large tiles on the grid).  When it is large enough for 128x128
 // tiles, its interior on that grid goes to them and only the right and bottom fringes to the
 // edge form; every block is a sub-matrix reached by pointer offsets.  Returns -1 when the shape
 // is left alone.
@@ -1338,8 +1340,8 @@ int try_interior_and_fringes(const SgemmArgs &g, int transa, int transb) {
     if ((((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.C | (uintptr_t)g.bias) & 15) != 0 || g.lda % 4 != 0 ||
         g.ldb % 4 != 0 || g.ldc % 4 != 0)
         return -1;                                           // the interior would not qualify for the fast kernels either
-    if ((g.M / 128) * (g.N / 256) < 256) return -1;
-    const int64_t Mi = g.M / 128 * 128, Ni = g.N / 256 * 256;
+    if ((g.M / 128) * (g.N / 128) < 2 * (int64_t)cu_count()) return -1;
+    const int64_t Mi = g.M / 128 * 128, Ni = g.N / 128 * 128;
     if (Mi == g.M && Ni == g.N) return -1;
     const float *A = static_cast<const float *>(g.A), *B = static_cast<const float *>(g.B);
     // a fringe is a strip of few tiles with the whole K: the split-K route when it qualifies
@@ -1381,8 +1383,8 @@ int try_k_tail(const SgemmArgs &g, int transa, int transb) {
     const int64_t Km = g.K / 32 * 32;
     if ((transa && transb) || Km == g.K || Km < 256) return -1;
     // K a multiple of 4 runs in one pass on the 64x64 tiles with guarded edges, which take a K tail
-    // themselves; two passes are for the other K and for shapes whose main part earns 128x256 tiles
-    if (g.K % 4 == 0 && (g.M / 128) * (g.N / 256) < 256) return -1;
+    // themselves; two passes are for the other K and for shapes whose main part earns 128x128 tiles
+    if (g.K % 4 == 0 && (g.M / 128) * (g.N / 128) < 2 * (int64_t)cu_count()) return -1;
     const float *A = static_cast<const float *>(g.A), *B = static_cast<const float *>(g.B);
     SgemmArgs p = g;
     p.K = Km;

@@ -50,7 +50,7 @@ def test_tuning_variables_parse(monkeypatch):
     cases = {"AX_HIP_I8_TILE": [("64x64", 64), ("64x64k2", 642), ("128x128", 128), ("256x256", 256), ("256", 256),
                                 ("32x32", 0), ("", 0), ("tile", 0)],
              "AX_HIP_I8_SPLITK": [("1", 1), ("16", 16), ("17", 0), ("0", 0), ("-3", 0), ("4x", 0)],
-             "AX_HIP_F32_TILE": [("64x64", 64), ("64x64k2", 642), ("128x256", 128), ("256x256", 0)],
+             "AX_HIP_F32_TILE": [("64x64", 64), ("64x64k2", 642), ("128x128", 128), ("128x256", 128), ("256x256", 0)],
              "AX_HIP_F32_SPLITK": [("1", 1), ("4096", 4096), ("4097", 0)],
              "AX_HIP_SKINNY_BLOCKS": [("512", 512), ("65535", 65535), ("65536", 0), ("many", 0)]}
     for name, pairs in cases.items():

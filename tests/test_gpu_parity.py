@@ -133,7 +133,7 @@ def test_w8a8_persistent_tiles_properties(hip, oracle, M, N, K):
 F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), (64, 64, 32),
               (128, 128, 64), (130, 260, 700), (256, 384, 512), (33, 40, 100), (96, 96, 96),
               (2048, 1024, 256),
-              # shapes that take the 128x256 tile, and ones just short of it in N or in tile count
+              # shapes that take the 128x128 eight-wave tile, and ones just short of it in N or in tile count
               (2048, 4096, 64), (4096, 2176, 64), (4096, 1088, 32), (128, 64, 4096),
               # few output tiles and a long K: the split-K route (bench_qgemm.c shapes among them)
               (32, 768, 768), (64, 1024, 4096), (128, 4096, 1024), (9, 100, 512), (16, 16, 8192), (70, 130, 1536),
@@ -363,14 +363,14 @@ def test_forced_tiles_and_splits_keep_parity(hip, oracle):
         assert {"qgemm_w8a8_64x64_dma", "qgemm_w8a8_64x64_dma_splitk", "qgemm_w8a8_64x64k2_dma", "qgemm_w8a8_64x64k2_dma_splitk",
                 "qgemm_w8a8_128x128_dma_splitk", "qgemm_w8a8_256x256_dma"} <= seen, seen
         seen = set()
-        for tile, split in (("64x64", "1"), ("64x64k2", "1"), ("128x256", "1"), ("", "4"), ("64x64", "8")):
+        for tile, split in (("64x64", "1"), ("64x64k2", "1"), ("128x128", "1"), ("", "4"), ("64x64", "8")):
             os.environ["AX_HIP_F32_TILE"], os.environ["AX_HIP_F32_SPLITK"] = tile, split
             hip.L.axhip_tuning_reload()
             say("forced f32", tile, split)
             got = hip.sgemm(da, dbm).numpy()
             seen.add(hip.last_kernel())
             check_fp32(oracle, got, a, b, ref=ref)
-        assert {"sgemm_nn_64x64_dma", "sgemm_nn_64x64k2_dma", "sgemm_nn_128x256_dma", "sgemm_splitk"} <= seen, seen
+        assert {"sgemm_nn_64x64_dma", "sgemm_nn_64x64k2_dma", "sgemm_nn_128x128_dma", "sgemm_splitk"} <= seen, seen
         for blocks in ("8", "64", "4000"):
             os.environ["AX_HIP_SKINNY_BLOCKS"] = blocks
             hip.L.axhip_tuning_reload()
