@@ -168,6 +168,17 @@ def secondary(hip):
                              "kernel": hip.last_kernel()}
     result_line("axhip", "f32_nn_1024x1024x1024", "gflops", tf * 1e3)
 
+    # the same product at the sizes where the matrix cores, not the launch, set the time
+    for n_ in (4096, 8192):
+        a, b = f32((n_, n_), (n_, n_))
+        c = hip.empty((n_, n_))
+        _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm(
+            0, 0, n_, n_, n_, 1.0, a.ptr, n_, b.ptr, n_, 0.0, c.ptr, n_, None, 0)), seconds=0.4)
+        tf = 2 * n_ ** 3 / ms / 1e9
+        res[f"fp32_gemm_{n_}"] = {"us": ms * 1e3, "TFLOP/s": tf, "frac_of_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS,
+                                  "kernel": hip.last_kernel()}
+    del a, b, c
+
     # config 3: FFN block 2048 x 1024 x 4096, bias + GELU fused into GEMM1, bias into GEMM2
     x, w1 = f32((2048, 1024), (1024, 4096))
     w2 = hip.array(rng.normal(0, 0.02, (4096, 1024)).astype(np.float32))
