@@ -1019,8 +1019,19 @@ int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_
     // the persistent 256x256 kernel from about 80 tiles on (81 tiles, 2304^2 x 8192: 72 us against 82 on
     // 128x128 tiles; 64 tiles, 2048^2 x 4096: 40 against 26)
     if (aligned && vec_out && M % 256 == 0 && N % 256 == 0 && K < (int64_t(1) << 24) &&   // per-lane 32-bit byte offsets span 256 rows
-        (tuning().i8_tile == 256 || (tuning().i8_tile == 0 && (M / 256) * (N / 256) >= 80)))
+        (tuning().i8_tile == 256 || (tuning().i8_tile == 0 && (M / 256) * (N / 256) >= 80))) {
+        // When the 256x256 tiles leave CUs idle or make a short last round, 256x128 tiles (eight waves, one
+        // workgroup per CU) spread the work better: a half tile costs about 0.6 of a whole one, so they win
+        // when their rounds are fewer than 1.6 times as many and K is long (same box: 2048 x 4096 x 4096, 128
+        // whole tiles, 43.1 -> 41.0 us; 2048 x 10752 x 4096, 344: 111.5 -> 105.3; 2304^2 x 8192, 81: 72.2 -> 56.4;
+        // but 2048 x 4096 x 1024 17.4 against 20.1 and 4096^3, 256 tiles, 63.2 against 71.8: those stay).
+        const int64_t whole = (M / 256) * (N / 256), cus = cu_count();
+        const int64_t rounds_whole = (whole + cus - 1) / cus, rounds_half = (2 * whole + cus - 1) / cus;
+        if (tuning().i8_tile == 0 && K % 128 == 0 && K >= 2048 && rounds_half * 60 < rounds_whole * 95)
+            return launch_dma<256, 128, 4, 2, 2>("qgemm_w8a8_256x128_dma", "qgemm_w8a8_256x128_dma_splitk", x, x_scale, w, w_scales,
+                                                 bias, act, out, acc_out, M, N, K, ldc);
         return launch_256(x, x_scale, w, w_scales, bias, act, out, acc_out, M, N, K, ldc);
+    }
     // aligned but too few 256x256 tiles: direct-to-LDS kernel over smaller tiles
     const int force = tuning().i8_tile;             // 0 = by shape, else 64 / 128 where the shape permits
     if (aligned && vec_out && K % 128 == 0 && M % 64 == 0 && N % 64 == 0 && K < (int64_t(1) << 24)) {

@@ -93,11 +93,13 @@ def test_w8a8_extreme_values_and_golden(hip, oracle, golden):
         assert np.array_equal(acc.numpy().astype(np.float64), golden[f"acc_K{K}"].astype(np.float64))
 
 
-@pytest.mark.parametrize("M,N,K", [(8192, 8192, 8192), (4096, 8192, 384), (4096, 8192, 512), (2048, 4096, 128)])
+@pytest.mark.parametrize("M,N,K", [(8192, 8192, 8192), (4096, 8192, 384), (4096, 8192, 512), (2048, 4096, 128),
+                                   (2048, 4096, 2048), (2048, 11008 // 256 * 256, 2048)])
 def test_w8a8_persistent_tiles_properties(hip, oracle, M, N, K):
     """Shapes served by the persistent 256x256 kernel, several tiles per workgroup, with an even
     slab count (next tile's first slab fetched under the write-back), an odd one, and one slab;
-    the first is the full size of the headline config.  Exact row/column checksums and 4096
+    the first is the full size of the headline config.  The last two have whole tiles for half the
+    CUs / a short last round and a long K: they run on 256x128 tiles.  Exact row/column checksums and 4096
     sampled entries of the accumulators; the fp32 output of the out-only call (the form the
     benchmark times) against the epilogue applied to those accumulators."""
     oracle.seed(M + N + K)
@@ -109,7 +111,7 @@ def test_w8a8_persistent_tiles_properties(hip, oracle, M, N, K):
     say("w8a8 persistent", M, N, K)
     out, acc = hip.qgemm_w8a8(dx, xs, dw, dws, db, 0)
     say("  kernel", hip.last_kernel())
-    assert hip.last_kernel() == "qgemm_w8a8_256x256_dma"
+    assert hip.last_kernel() == ("qgemm_w8a8_256x128_dma" if K == 2048 else "qgemm_w8a8_256x256_dma")
     a = acc.numpy()
     xi, wi = x.astype(np.int64), w.astype(np.int64)
     assert np.array_equal(a.astype(np.int64).sum(axis=0), wi @ xi.sum(axis=0))   # column sums
