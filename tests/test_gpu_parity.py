@@ -137,6 +137,8 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               (2048, 1024, 256),
               # shapes that take the 128x128 eight-wave tile, and ones just short of it in N or in tile count
               (2048, 4096, 64), (4096, 2176, 64), (4096, 1088, 32), (128, 64, 4096),
+              # 64x64 tile counts with a nearly empty last round of one tile per CU: 32x64 tiles (NN and NT)
+              (1152, 1152, 192), (1280, 960, 256),
               # few output tiles and a long K: the split-K route (bench_qgemm.c shapes among them)
               (32, 768, 768), (64, 1024, 4096), (128, 4096, 1024), (9, 100, 512), (16, 16, 8192), (70, 130, 1536),
               # off the tile grid with a large interior: fast kernels inside, guarded kernel on the fringes
