@@ -36,7 +36,7 @@ int skinny_setup();
 // Tile-selection overrides from the environment (0 = choose by shape), read at axhip_init and by
 // axhip_tuning_reload; what each one forces is described next to axhip_tuning_reload in axhip.h.
 struct Tuning {
-    int i8_tile;         // AX_HIP_I8_TILE: 64 (64x64), 642 (64x64 with the k-steps split over two wave sets), 128 or 256
+    int i8_tile;         // AX_HIP_I8_TILE: 64 (64x64), 642 (64x64 with the k-steps split over two wave sets), 1264 (128x64), 128 or 256
     int i8_splitk;       // AX_HIP_I8_SPLITK: 1..16
     int f32_tile;        // AX_HIP_F32_TILE: 64 (64x64), 642 (64x64 with the k split over two wave sets), 128 (128x128, eight waves)
     int f32_splitk;      // AX_HIP_F32_SPLITK: 1 = never split K, 2.. = that many ranges where the route applies

@@ -1038,6 +1038,20 @@ int qgemm_block(const int8_t *x, float x_scale, const int8_t *w, const float *w_
         // 128x128 tiles once there is one for every CU (2048^2 x 4096: 26.2 us against 30.7 on 64x64); eight waves
         // (2 x 4, wave tile 64x32), two on every SIMD: 25.0 -> 24.2 us against four waves of 64x64
         const bool fits128 = M % 128 == 0 && N % 128 == 0;
+        // Between one 64x64 tile per CU and a 128x128 tile per CU, 128x64 tiles on eight waves (4 x 2, wave tile
+        // 32x32; 72 KiB of stages, two workgroups per CU): a quarter less operand traffic into LDS per output
+        // than 64x64 (same box: 512 x 4096 x 4096 17.5 -> 14.8 us, 896 x 4096 x 4096 28.8 -> 23.4,
+        // 512 x 4096 x 11008 39.2 -> 33.3, 256 x 6144 x 4096 14.1 -> 12.5).  One row of tiles (M = 128) stays on
+        // 64x64, whose 512 workgroups keep more of W's only pass in flight (128 x 16384 x 4096: 17.6 against 20.0).
+        // With 256 to 511 128x128 tiles they also win for K of 2048 to 4096 (2048^3 21.8 -> 17.6,
+        // 1024 x 4096 x 4096 29.6 -> 25.3, 1536 x 3072 x 3072 29.2 -> 26.0), not for shorter or longer K
+        // (1024 x 4096 x 1024 13.0 against 14.7; 2048^2 x 8192 40.6 against 47.4).
+        const int64_t t64 = (M / 64) * (N / 64), t128 = (M / 128) * (N / 128);
+        const bool mid_k = K >= 2048 && K <= 4096;
+        if (M % 128 == 0 && (force == 1264 || (force == 0 && M >= 256 && t64 > cu_count() &&
+                                               (!fits128 || t128 < 256 || (t128 < 512 && mid_k)))))
+            return launch_dma<128, 64, 4, 2, 3>("qgemm_w8a8_128x64_dma", "qgemm_w8a8_128x64_dma_splitk", x, x_scale, w,
+                                                w_scales, bias, act, out, acc_out, M, N, K, ldc);
         if (fits128 && (force == 128 || (force == 0 && (M / 128) * (N / 128) >= 256)))
             return launch_dma<128, 128, 2, 4, 3>("qgemm_w8a8_128x128_dma", "qgemm_w8a8_128x128_dma_splitk", x, x_scale, w,
                                                  w_scales, bias, act, out, acc_out, M, N, K, ldc);

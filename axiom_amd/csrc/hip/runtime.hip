@@ -46,6 +46,7 @@ int parse_tile(const char *name, const int *allowed, int n_allowed) {
     long t = strtol(v, &end, 10);
     if (end == v) return 0;
     if (strstr(v, "k2")) t = t * 10 + 2;
+    if (t == 128 && !strcmp(end, "x64")) t = 1264;
     for (int i = 0; i < n_allowed; i++)
         if (allowed[i] == t) return (int)t;
     return 0;
@@ -191,8 +192,8 @@ int axhip_device_count(void) {
 }
 
 int axhip_tuning_reload(void) {
-    static const int i8_tiles[] = {64, 642, 128, 256}, f32_tiles[] = {64, 642, 128};
-    g_tuning.i8_tile = parse_tile("AX_HIP_I8_TILE", i8_tiles, 4);
+    static const int i8_tiles[] = {64, 642, 128, 1264, 256}, f32_tiles[] = {64, 642, 128};
+    g_tuning.i8_tile = parse_tile("AX_HIP_I8_TILE", i8_tiles, 5);
     g_tuning.i8_splitk = parse_count("AX_HIP_I8_SPLITK", 1, 16);
     g_tuning.f32_tile = parse_tile("AX_HIP_F32_TILE", f32_tiles, 3);
     g_tuning.f32_splitk = parse_count("AX_HIP_F32_SPLITK", 1, 4096);

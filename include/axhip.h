@@ -52,14 +52,14 @@ const char *axhip_device_name(void);          /* gcnArchName of device 0, "" wit
  * Read from the environment by axhip_init and again by axhip_tuning_reload (which needs no GPU and
  * returns how many variables were recognised); unset, empty or invalid values mean "choose by shape".
  * A forced choice applies only where the shape permits that kernel; results do not depend on it.
- *   AX_HIP_I8_TILE       64x64 | 64x64k2 | 128x128 | 256x256   W8A8 tile (256x256: M, N multiples of 256; k2: two
- *                        wave sets split each K slab)
+ *   AX_HIP_I8_TILE       64x64 | 64x64k2 | 128x64 | 128x128 | 256x256   W8A8 tile (256x256: M, N multiples of 256;
+ *                        k2: two wave sets split each K slab)
  *   AX_HIP_I8_SPLITK     1..16      workgroups over K per W8A8 tile of 64x64 / 128x128 (1: never split)
  *   AX_HIP_F32_TILE      64x64 | 64x64k2 | 128x128   fp32 tile on the aligned fast path (k2: two wave sets split each K slab)
  *   AX_HIP_F32_SPLITK    1..4096    K ranges of the fp32 few-tile route (1: never split)
  *   AX_HIP_SKINNY_BLOCKS 1..65535   workgroups the skinny-M route aims for
  * axhip_tuning_get returns the value in effect (0: automatic; tiles as their first number, 64x64k2 as
- * 642), or -1 for an unknown name. */
+ * 642, 128x64 as 1264), or -1 for an unknown name. */
 int axhip_tuning_reload(void);
 int axhip_tuning_get(const char *name);
 

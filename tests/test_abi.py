@@ -47,7 +47,7 @@ def test_tuning_variables_parse(monkeypatch):
         monkeypatch.delenv(n, raising=False)
     assert h.L.axhip_tuning_reload() == 0
     assert [h.L.axhip_tuning_get(n.encode()) for n in names] == [0] * 5
-    cases = {"AX_HIP_I8_TILE": [("64x64", 64), ("64x64k2", 642), ("128x128", 128), ("256x256", 256), ("256", 256),
+    cases = {"AX_HIP_I8_TILE": [("64x64", 64), ("64x64k2", 642), ("128x128", 128), ("128x64", 1264), ("256x256", 256), ("256", 256),
                                 ("32x32", 0), ("", 0), ("tile", 0)],
              "AX_HIP_I8_SPLITK": [("1", 1), ("16", 16), ("17", 0), ("0", 0), ("-3", 0), ("4x", 0)],
              "AX_HIP_F32_TILE": [("64x64", 64), ("64x64k2", 642), ("128x128", 128), ("128x256", 128), ("256x256", 0)],

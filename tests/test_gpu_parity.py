@@ -48,7 +48,9 @@ INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300
                (64, 128, 1040), (128, 128, 112),
                # few tiles against a long K: workgroups split K and the last one of a tile adds the int32 partials
                (64, 1024, 4096), (64, 64, 8192), (256, 2048, 8192), (512, 1024, 4096), (100, 4096, 4096), (70, 200, 2064),
-               (128, 128, 2048)]
+               (128, 128, 2048),
+               # more than one 64x64 tile per CU, fewer than one 128x128 tile per CU: 128x64 tiles on eight waves
+               (512, 4096, 512), (384, 2752, 256), (256, 6144, 1152), (2048, 2048, 2048)]
 
 
 @pytest.mark.parametrize("M,N,K", INT8_SHAPES)
@@ -356,7 +358,7 @@ def test_forced_tiles_and_splits_keep_parity(hip, oracle):
     seen = set()
     try:
         for tile, split in (("64x64", "1"), ("64x64", "4"), ("64x64k2", "1"), ("64x64k2", "3"), ("128x128", "2"),
-                            ("256x256", "1"), ("", "16"), ("bogus", "99")):
+                            ("128x64", "1"), ("128x64", "3"), ("256x256", "1"), ("", "16"), ("bogus", "99")):
             os.environ["AX_HIP_I8_TILE"], os.environ["AX_HIP_I8_SPLITK"] = tile, split
             hip.L.axhip_tuning_reload()
             say("forced i8", tile, split)
@@ -365,7 +367,8 @@ def test_forced_tiles_and_splits_keep_parity(hip, oracle):
             assert np.array_equal(acc.numpy(), want_acc), (tile, split, hip.last_kernel())
             assert np.array_equal(out.numpy(), want_out), (tile, split, hip.last_kernel())
         assert {"qgemm_w8a8_64x64_dma", "qgemm_w8a8_64x64_dma_splitk", "qgemm_w8a8_64x64k2_dma", "qgemm_w8a8_64x64k2_dma_splitk",
-                "qgemm_w8a8_128x128_dma_splitk", "qgemm_w8a8_256x256_dma"} <= seen, seen
+                "qgemm_w8a8_128x128_dma_splitk", "qgemm_w8a8_128x64_dma", "qgemm_w8a8_128x64_dma_splitk",
+                "qgemm_w8a8_256x256_dma"} <= seen, seen
         seen = set()
         for tile, split in (("64x64", "1"), ("64x64k2", "1"), ("128x128", "1"), ("", "4"), ("64x64", "8")):
             os.environ["AX_HIP_F32_TILE"], os.environ["AX_HIP_F32_SPLITK"] = tile, split
