@@ -1193,6 +1193,11 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
         const int64_t big = (g.M / 128) * (g.N / 128) * batch, cus = cu_count(), rounds = (big + cus - 1) / cus;
         if (g.M % 128 == 0 && g.N % 128 == 0 && big >= cus && big * 10 >= rounds * cus * 9)
             return launch_dma<128, 128, 2, 4, 2, true, true, 1, 1, false, int8_t>(names[0], g, batch);
+        // the last round of one 64x64 tile per CU mostly empty: 32x64 tiles, as for fp32 operands
+        const int64_t whole = (g.M / 64) * (g.N / 64) * batch, rounds_whole = (whole + cus - 1) / cus,
+                      rounds_half = (2 * whole + cus - 1) / cus;
+        if (tuning().f32_tile == 0 && rounds_half * 55 <= rounds_whole * 95)
+            return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
         return launch_dma<64, 64, 2, 2, 2, true, true, 1, 2, false, int8_t>(names[2], g, batch);
     }
     return launch_dma<64, 64, 2, 2, 2, true, true, 1, 1, false, int8_t>(names[1], g, batch);
@@ -1274,9 +1279,29 @@ int64_t split_count(int64_t M, int64_t N, int64_t K) {
     return (below * 2 < want && above) ? above : below;
 }
 
+// With rows of A K-contiguous, a shape on the tile grid with few 64x64 tiles runs on 32x64 tiles with
+// the k split (twice the workgroups, eight waves each), and that one launch costs 3.4 us plus 2.3 us
+// per 256 of K up to K = 1536 whatever the tile count (K = 256: 5.7 us, 512: 8.0, 768: 10.3, 1024: 12.7,
+// 1536: 17.5; from 2048 on the rows of A are 8 KiB apart and it takes 29).  The two launches of the split
+// route take 7.8 to 10.5 us at K = 256, 9.3 to 12.2 at 512, 11.1 at 768, 11.8 to 12.3 at K = 1024 up to 64
+// tiles and 15.9 with 128 (1024 x 512 x 1024), 20 at K = 1536 with 128 tiles; a dozen tiles split many
+// ways take 8.1 at K = 768.  So the split is left out up to K = 512, up to K = 768 from 48 tiles on, and
+// up to K = 1536 for more than 64 tiles.  The same holds with int8 weights as B (128 x 4096 x 1024:
+// 18.3 -> 15.3 us).
+bool one_launch_on_half_tiles(const SgemmArgs &g, int transa) {
+    if (transa || tuning().f32_splitk != 0 || tuning().f32_tile != 0) return false;
+    if (g.M % 64 != 0 || g.N % 64 != 0 || g.K % 32 != 0) return false;
+    if ((((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.C | (uintptr_t)g.bias | (uintptr_t)g.col_scale) & 15) != 0 ||
+        g.lda % 4 != 0 || g.ldb % 16 != 0 || g.ldc % 4 != 0)
+        return false;                                        // the fast kernels would not take it
+    const int64_t tiles = (g.M / 64) * (g.N / 64);
+    return g.K <= 512 || (g.K <= 768 && tiles >= 48) || (g.K <= 1536 && tiles > 64);
+}
+
 // returns -1 when the shape is left to the ordinary path
 template <typename BSRC>
 int try_split_k(const SgemmArgs &g, int transa, int transb, const char *name, const char *const i8_names[3]) {
+    if (one_launch_on_half_tiles(g, transa)) return -1;
     const int64_t splits = split_count(g.M, g.N, g.K);
     if (splits < 2 || splits > 65535) return -1;
     const int64_t kr = g.K / splits;

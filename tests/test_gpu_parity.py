@@ -143,6 +143,8 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               (1152, 1152, 192), (1280, 960, 256),
               # few output tiles and a long K: the split-K route (bench_qgemm.c shapes among them)
               (32, 768, 768), (64, 1024, 4096), (128, 4096, 1024), (9, 100, 512), (16, 16, 8192), (70, 130, 1536),
+              # few tiles and K short enough that one launch on 32x64 tiles beats the split, and their neighbours that split
+              (1024, 256, 256), (64, 4096, 512), (256, 768, 768), (64, 768, 768), (1024, 512, 1536), (256, 1024, 1024),
               # off the tile grid with a large interior: fast kernels inside, guarded kernel on the fringes
               (1032, 1100, 96), (2100, 4200, 64), (1024, 1092, 160),
               (130, 257, 1027), (67, 1001, 129),                  # rows off the 16-byte grid in every form
@@ -661,6 +663,7 @@ W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 
                 (1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024),
                 (64, 1024, 4096), (1, 4096, 4096), (5, 33, 100),
                 (2, 130, 256), (6, 67, 1040), (7, 5, 2064),
+                (128, 1024, 512), (1024, 512, 1024), (256, 768, 768), (64, 768, 768),   # one launch on 32x64 tiles / split
                 (32, 128, 517), (70, 260, 1031), (3, 64, 1037)]   # rows at odd byte offsets       # every row count of the wave-per-rows form
 
 
