@@ -43,6 +43,7 @@ INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300
                # M or N off the 64 grid with K on the 128 grid: the direct-to-LDS kernel with clamped edge tiles
                (100, 4096, 512), (130, 260, 256), (2000, 2000, 128), (63, 60, 128), (9, 4, 128), (500, 1000, 1024),
                (65, 64, 256), (64, 68, 384), (2900, 3000, 128),
+               (500, 4096, 512), (900, 1004, 384), (260, 6148, 256),   # 128x64 tiles with clamped edges, and M = 260 that stays on 64x64
                # K a multiple of 16 off the 128 grid: the last slab's tail is zero-filled in LDS
                (100, 4096, 784), (64, 64, 16), (130, 260, 144), (256, 4096, 784), (2900, 3000, 400), (9, 4, 48),
                (64, 128, 1040), (128, 128, 112),
