@@ -202,6 +202,13 @@ int axhip_tuning_reload(void) {
            (g_tuning.skinny_blocks != 0);
 }
 
+int axhip_workspace_reserve(size_t bytes, size_t *have) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (bytes > 0 && !axhip::workspace(bytes)) return AXHIP_ERR_ALLOC;
+    if (have) *have = g_ws_bytes;
+    return AXHIP_OK;
+}
+
 int axhip_tuning_get(const char *name) {
     if (!name) return -1;
     if (!strcmp(name, "AX_HIP_I8_TILE")) return g_tuning.i8_tile;

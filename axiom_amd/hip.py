@@ -22,6 +22,7 @@ SIGNATURES = {
     "axhip_device_name": (C.c_char_p, []),
     "axhip_tuning_reload": (C.c_int, []),
     "axhip_tuning_get": (C.c_int, [C.c_char_p]),
+    "axhip_workspace_reserve": (C.c_int, [C.c_size_t, C.POINTER(C.c_size_t)]),
     "axhip_malloc": (vp, [C.c_size_t]),
     "axhip_malloc_uninit": (vp, [C.c_size_t]),
     "axhip_free": (None, [vp]),

@@ -86,6 +86,15 @@ void  axhip_free(void *device_ptr);             /* NULL, foreign and already-fre
 void  axhip_alloc_stats(int64_t *allocs, int64_t *frees, int64_t *bytes_alloc, int64_t *bytes_free,
                         int64_t *driver_allocs, int64_t *bytes_cached);
 void  axhip_reset_alloc_stats(void);
+/* The shared device workspace (split-K partial sums, reduction partials, padded operand copies) is 64 MiB
+ * from axhip_init on and grows when a call needs more; growing waits for the device, frees the old block and asks the
+ * driver for a new one, which costs the first call at a larger shape some tens of microseconds that later
+ * calls do not pay.  axhip_workspace_reserve grows it ahead of time (at model load, before a timed or
+ * latency-bound loop) to at least `bytes` and reports the size it then has in *have (may be NULL); bytes = 0
+ * only reports.  It never shrinks.  No counterpart in the reference, whose CUDA backend grows its score
+ * buffer on demand in the same way (cuda/ops_attention.cu:305-318) and offers no call to do it ahead of
+ * time.  Same threading rule as the compute entry points. */
+int   axhip_workspace_reserve(size_t bytes, size_t *have);
 int   axhip_memset(void *device_ptr, int byte_value, size_t bytes);
 int   axhip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes);
 int   axhip_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes);   /* blocking */

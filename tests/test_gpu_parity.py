@@ -1401,3 +1401,26 @@ def test_allocation_pool(hip):
     hip.L.axhip_alloc_stats(*[C.byref(v) for v in st])
     allocs, frees, b_alloc, b_free, driver, cached = (v.value for v in st)
     assert allocs == 3 and frees == 3 and b_alloc == b_free == 3 * 16384 and driver <= 2 and cached >= 2 * 16384
+
+
+def test_workspace_reserve_grows_once_and_never_shrinks(hip, oracle):
+    """axhip_workspace_reserve sizes the shared workspace ahead of time: the size only grows, a split-K product
+    that fits runs in the reserved block (same size afterwards) and still meets the fp32 gate."""
+    import ctypes as C
+    have = C.c_size_t(0)
+    hip.check(hip.L.axhip_workspace_reserve(0, C.byref(have)))
+    start = have.value
+    want = max(start, 8 << 20) + (24 << 20)
+    hip.check(hip.L.axhip_workspace_reserve(want, C.byref(have)))
+    assert have.value >= want
+    grown = have.value
+    hip.check(hip.L.axhip_workspace_reserve(1 << 20, C.byref(have)))
+    assert have.value == grown
+    hip.check(hip.L.axhip_workspace_reserve(0, None))
+    oracle.seed(5)
+    a, b = oracle.uniform((64, 4096), -1, 1), oracle.uniform((4096, 1024), -1, 1)
+    got = hip.sgemm(hip.array(a), hip.array(b)).numpy()
+    assert hip.last_kernel() == "sgemm_splitk"
+    check_fp32(oracle, got, a, b)
+    hip.check(hip.L.axhip_workspace_reserve(0, C.byref(have)))
+    assert have.value == grown
