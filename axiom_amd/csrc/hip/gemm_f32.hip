@@ -1125,6 +1125,13 @@ int try_nn_stream(const SgemmArgs &g, int64_t batch) {
     return check_launch("sgemm_nn_stream128x64_dma");
 }
 
+// Up to 160 rows (K-contiguous) whose count of 32-row blocks is odd (1..32, 65..96, 129..160) run on 32x64 tiles
+// instead of 64x64 tiles whose last row block is at least half padding (same box, 32 x 11008 x 4096: 71.9 ->
+// 57.1 us and 32.4 with the K split that the smaller tiles then earn, with int8 weights 84.9 -> 32.9;
+// 160 x 11008 x 4096: 181.6 -> 143.7).  A 32x64 tile costs about 0.55 of a 64x64 one, so from 224 rows on the
+// padded row block is the cheaper choice again (224 x 11008 x 4096: 182.6 against 198.4).
+inline bool half_row_tiles(int64_t M) { return M <= 160 && ((M + 31) / 32) % 2 == 1; }
+
 // Chooses the largest tile that still leaves about eight waves per CU; returns -1 when the
 // shape does not qualify for the fast path (the caller then uses the register-staged kernel).
 // names: 128x128, 64x64, 64x64 with the k split.
@@ -1136,6 +1143,13 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
                     g.stride_c % 4 == 0 && g.lda < (1 << 20) && g.ldb < (1 << 20) && batch <= 65535 &&
                     g.N % 4 == 0 && (A_KC || g.M % 4 == 0) && ((g.M + 63) / 64) * ((g.N + 63) / 64) <= 0x7fffffff;
     if (!ok) return -1;
+    if constexpr (A_KC) {
+        if (half_row_tiles(g.M) && g.K >= 64 && tuning().f32_tile == 0) {
+            if (g.M % 32 == 0 && g.N % 64 == 0 && g.K % 32 == 0)
+                return launch_dma<32, 64, 1, 2, 2, A_KC, B_KC, 1, 2>(B_KC ? "sgemm_nt_32x64k2_dma" : "sgemm_nn_32x64k2_dma", g, batch);
+            return launch_dma<32, 64, 1, 2, 2, A_KC, B_KC, 1, 2, true>("sgemm_32x64k2_dma_edge", g, batch);
+        }
+    }
     if (g.M % 64 != 0 || g.N % 64 != 0 || g.K % 32 != 0) {  // off the tile grid: 64x64 tiles with guarded edges
         static const char *const edge_names[2] = {"sgemm_64x64_dma_edge", "sgemm_64x64k2_dma_edge"};
         if (g.K > 128) return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2, true>(edge_names[1], g, batch);
@@ -1185,6 +1199,11 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
                     g.stride_c % 4 == 0 && g.lda < (1 << 20) && g.ldb < (1 << 22) && batch <= 65535 && g.N % 4 == 0 &&
                     ((g.M + 63) / 64) * ((g.N + 63) / 64) <= 0x7fffffff;
     if (!ok) return -1;
+    if (half_row_tiles(g.M) && g.K >= 64 && tuning().f32_tile == 0) {   // as for fp32 operands
+        if (g.M % 32 == 0 && g.N % 64 == 0)
+            return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
+        return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, true, int8_t>("qgemm_w8a32_mfma_32x64k2_dma_edge", g, batch);
+    }
     if (g.M % 64 != 0 || g.N % 64 != 0) {
         if (g.K > 128) return launch_dma<64, 64, 2, 2, 2, true, true, 1, 2, true, int8_t>(names[2], g, batch);
         return launch_dma<64, 64, 2, 2, 2, true, true, 1, 1, true, int8_t>(names[1], g, batch);
@@ -1255,15 +1274,17 @@ k_splitk_finish(const float *__restrict__ part, int splits, int64_t M, int64_t N
 int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch);
 
 // how many K ranges to use (1: none).  Every range must be a whole number of 32-wide slabs.
-int64_t split_count(int64_t M, int64_t N, int64_t K) {
-    const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
+int64_t split_count(int64_t M, int64_t N, int64_t K, bool a_rows_k_contiguous) {
+    // whole 32x64 tiles count as 0.55 of a tile each
+    const bool halves = a_rows_k_contiguous && tuning().f32_tile == 0 && half_row_tiles(M);
+    const int64_t tiles = halves ? (((M + 31) / 32) * ((N + 63) / 64) * 11 + 19) / 20 : ((M + 63) / 64) * ((N + 63) / 64);
     const int64_t cus = cu_count();
     if (tiles * 2 > cus || K < 256 || K % 32 != 0) return 1;
     // One workgroup per CU measured best for tiles on the 64 grid (32x768x768: 10.5 us against 27
     // unsplit; 64x1024x4096: 12 against 70; 128x4096x1024: 16.5 against 20; more ranges only add
     // partial sums to move); strips off the grid, part of whose tiles is padding, gain from two
     // (4x4100x4096: 38 -> 30 us; 9x8000x8192: 78 -> 69).
-    const bool ragged = M % 64 != 0 || N % 64 != 0;
+    const bool ragged = halves || M % 64 != 0 || N % 64 != 0;     // small workgroups, too: two per CU (96 x 4096 x 4096: 33.9 us against 40.4)
     int64_t want = ((ragged ? 2 : 1) * cus + tiles - 1) / tiles;
     if (tuning().f32_splitk == 1) return 1;
     if (tuning().f32_splitk > 1) want = tuning().f32_splitk;
@@ -1302,7 +1323,7 @@ bool one_launch_on_half_tiles(const SgemmArgs &g, int transa) {
 template <typename BSRC>
 int try_split_k(const SgemmArgs &g, int transa, int transb, const char *name, const char *const i8_names[3]) {
     if (one_launch_on_half_tiles(g, transa)) return -1;
-    const int64_t splits = split_count(g.M, g.N, g.K);
+    const int64_t splits = split_count(g.M, g.N, g.K, !transa);
     if (splits < 2 || splits > 65535) return -1;
     const int64_t kr = g.K / splits;
     float *part = static_cast<float *>(workspace((size_t)splits * g.M * g.N * sizeof(float)));

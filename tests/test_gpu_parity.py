@@ -146,6 +146,9 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               (32, 768, 768), (64, 1024, 4096), (128, 4096, 1024), (9, 100, 512), (16, 16, 8192), (70, 130, 1536),
               # few tiles and K short enough that one launch on 32x64 tiles beats the split, and their neighbours that split
               (1024, 256, 256), (64, 4096, 512), (256, 768, 768), (64, 768, 768), (1024, 512, 1536), (256, 1024, 1024),
+              # up to 160 rows with an odd count of 32-row blocks: 32x64 tiles (whole and with clamped edges), alone and under the K split
+              (32, 2048, 128), (96, 4096, 1024), (160, 3072, 768), (20, 2048, 512), (80, 1088, 256), (150, 260, 160), (130, 4096, 96),
+              (24, 11008, 512),
               # off the tile grid with a large interior: fast kernels inside, guarded kernel on the fringes
               (1032, 1100, 96), (2100, 4200, 64), (1024, 1092, 160),
               (130, 257, 1027), (67, 1001, 129),                  # rows off the 16-byte grid in every form
@@ -665,6 +668,7 @@ W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 
                 (64, 1024, 4096), (1, 4096, 4096), (5, 33, 100),
                 (2, 130, 256), (6, 67, 1040), (7, 5, 2064),
                 (128, 1024, 512), (1024, 512, 1024), (256, 768, 768), (64, 768, 768),   # one launch on 32x64 tiles / split
+                (20, 1024, 512), (150, 260, 160), (96, 2048, 1024), (160, 3072, 768),   # 32x64 tiles, whole and with clamped edges
                 (32, 128, 517), (70, 260, 1031), (3, 64, 1037)]   # rows at odd byte offsets       # every row count of the wave-per-rows form
 
 
