@@ -1174,15 +1174,26 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
         const int64_t big = count(128, 128), cus = cu_count(), rounds = (big + cus - 1) / cus;
         if (g.M % 128 == 0 && g.N % 128 == 0 && big >= cus && big * 10 >= rounds * cus * 9)
             return launch_dma<128, 128, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
+        // One round of tiles over a long K with operands too large for the L2s: every workgroup's life is one
+        // stream from memory with nothing else on its CU to cover the latency, and a third stage keeps more of it
+        // in flight (operands in HBM: 256 x 4096 x 4096 84.0 -> 71.6 us, 512 x 2048 x 4096 86.0 -> 71.3; the same
+        // operands in the Infinity Cache: 68.4 -> 70.5, 68.2 -> 70.1; 128 x 4096 x 2048 on 32x64 tiles 29.2 -> 23.2).
+        // With two rounds or more the other workgroup of a CU covers it and two stages stay (within 1.5 % either way).
+        // The K ranges of a split count like tiles (128 x 4096 x 4096 in two ranges, from HBM: 48.5 us with two stages).
+        const bool streams = count(64, 64) <= cus && g.K >= 2048 && (g.M + g.N) * g.K * 4 * batch >= (int64_t(24) << 20);
         // 64x64 tiles whose count leaves the last round of one tile per CU mostly empty (300 tiles: a full
         // round and 44 CUs' worth) run as 32x64 tiles instead when that evens the rounds out: a half tile
         // costs about 0.55 of a whole one (1280 x 960 x 2048: 63.8 -> 53.1 us; 1152^3: 38.2 -> 31.8; 896 x
         // 1280 x 4096: 123 -> 102).  Rows of A must be K-contiguous for a 32-row tile (NN and NT).
         if constexpr (A_KC) {
             const int64_t whole = count(64, 64), rounds_whole = (whole + cus - 1) / cus, rounds_half = (2 * whole + cus - 1) / cus;
-            if (rounds_half * 55 <= rounds_whole * 95)
+            if (rounds_half * 55 <= rounds_whole * 95) {
+                if (streams)
+                    return launch_dma<32, 64, 1, 2, 3, A_KC, B_KC, 1, 2>(B_KC ? "sgemm_nt_32x64k2_dma" : "sgemm_nn_32x64k2_dma", g, batch);
                 return launch_dma<32, 64, 1, 2, 2, A_KC, B_KC, 1, 2>(B_KC ? "sgemm_nt_32x64k2_dma" : "sgemm_nn_32x64k2_dma", g, batch);
+            }
         }
+        if (streams) return launch_dma<64, 64, 2, 2, 3, A_KC, B_KC, 1, 2>(names[2], g, batch);
         return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[2], g, batch);
     }
     return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1>(names[1], g, batch);
@@ -1279,14 +1290,22 @@ int64_t split_count(int64_t M, int64_t N, int64_t K, bool a_rows_k_contiguous) {
     const bool halves = a_rows_k_contiguous && tuning().f32_tile == 0 && half_row_tiles(M);
     const int64_t tiles = halves ? (((M + 31) / 32) * ((N + 63) / 64) * 11 + 19) / 20 : ((M + 63) / 64) * ((N + 63) / 64);
     const int64_t cus = cu_count();
-    if (tiles * 2 > cus || K < 256 || K % 32 != 0) return 1;
+    if (tuning().f32_splitk == 1 || K < 256 || K % 32 != 0) return 1;
+    if (tiles * 2 > cus) {
+        // More than half the CUs have a tile: a split pays only when a fifth of them would sit idle through a long
+        // K (192 tiles, K = 4096: 68 -> 55..57 us with the operands in the Infinity Cache, 84..88 -> 58..61 from
+        // HBM; with 256 tiles it loses 3 % cached and gains no more than a third stage does).
+        if (tiles * 5 > cus * 4 || K < 4096 || halves || tuning().f32_splitk != 0) return 1;
+        for (int64_t s = 4; s >= 2; s--)
+            if (K % (s * 32) == 0) return s;
+        return 1;
+    }
     // One workgroup per CU measured best for tiles on the 64 grid (32x768x768: 10.5 us against 27
     // unsplit; 64x1024x4096: 12 against 70; 128x4096x1024: 16.5 against 20; more ranges only add
     // partial sums to move); strips off the grid, part of whose tiles is padding, gain from two
     // (4x4100x4096: 38 -> 30 us; 9x8000x8192: 78 -> 69).
     const bool ragged = halves || M % 64 != 0 || N % 64 != 0;     // small workgroups, too: two per CU (96 x 4096 x 4096: 33.9 us against 40.4)
     int64_t want = ((ragged ? 2 : 1) * cus + tiles - 1) / tiles;
-    if (tuning().f32_splitk == 1) return 1;
     if (tuning().f32_splitk > 1) want = tuning().f32_splitk;
     const int64_t most = K / 64;                             // ranges of at least 64
     if (want > most) want = most;

@@ -149,6 +149,8 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               # up to 160 rows with an odd count of 32-row blocks: 32x64 tiles (whole and with clamped edges), alone and under the K split
               (32, 2048, 128), (96, 4096, 1024), (160, 3072, 768), (20, 2048, 512), (80, 1088, 256), (150, 260, 160), (130, 4096, 96),
               (24, 11008, 512),
+              # one round of tiles over a long K: three stages (operands past the L2s), and the K split when a fifth of the CUs would idle
+              (256, 3072, 2048), (192, 2816, 4096),
               # off the tile grid with a large interior: fast kernels inside, guarded kernel on the fringes
               (1032, 1100, 96), (2100, 4200, 64), (1024, 1092, 160),
               (130, 257, 1027), (67, 1001, 129),                  # rows off the 16-byte grid in every form
