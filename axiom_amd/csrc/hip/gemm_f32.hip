@@ -1174,13 +1174,15 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
         const int64_t big = count(128, 128), cus = cu_count(), rounds = (big + cus - 1) / cus;
         if (g.M % 128 == 0 && g.N % 128 == 0 && big >= cus && big * 10 >= rounds * cus * 9)
             return launch_dma<128, 128, 2, 4, 2, A_KC, B_KC, 1>(names[0], g, batch);
-        // One round of tiles over a long K with operands too large for the L2s: every workgroup's life is one
-        // stream from memory with nothing else on its CU to cover the latency, and a third stage keeps more of it
-        // in flight (operands in HBM: 256 x 4096 x 4096 84.0 -> 71.6 us, 512 x 2048 x 4096 86.0 -> 71.3; the same
-        // operands in the Infinity Cache: 68.4 -> 70.5, 68.2 -> 70.1; 128 x 4096 x 2048 on 32x64 tiles 29.2 -> 23.2).
-        // With two rounds or more the other workgroup of a CU covers it and two stages stay (within 1.5 % either way).
-        // The K ranges of a split count like tiles (128 x 4096 x 4096 in two ranges, from HBM: 48.5 us with two stages).
-        const bool streams = count(64, 64) <= cus && g.K >= 2048 && (g.M + g.N) * g.K * 4 * batch >= (int64_t(24) << 20);
+        // One round of tiles with operands too large to be met in the L2s: every workgroup's life is one stream
+        // from memory with nothing else on its CU to cover the latency, and a third stage keeps more of it in
+        // flight.  Operands in HBM (rotating sets): 256 x 4096 x 4096 84.0 -> 71.6 us, 512 x 2048 x 4096 86.0 -> 71.3,
+        // 128 x 4096 x 1024 on 32x64 tiles 22.6 -> 14.3, 128 x 4096 x 768 18.1 -> 12.0, 256 x 4096 x 1024 24.1 -> 21.1;
+        // the same operands in the Infinity Cache: 68.4 -> 70.5, 68.2 -> 70.1, 12.8 -> 13.3, 10.3 -> 10.8, 19.8 -> 20.5.
+        // With two rounds or more the other workgroup of a CU covers the latency and two stages stay (within 1.5 %
+        // either way).  The K ranges of a split count like tiles (128 x 4096 x 4096 in two ranges, from HBM:
+        // 48.6 -> 41.6 us).  Operands of at most 8 MiB together, a quarter of the L2s, keep two stages.
+        const bool streams = count(64, 64) <= cus && g.K >= 512 && (g.M + g.N) * g.K * 4 * batch > (int64_t(8) << 20);
         // 64x64 tiles whose count leaves the last round of one tile per CU mostly empty (300 tiles: a full
         // round and 44 CUs' worth) run as 32x64 tiles instead when that evens the rounds out: a half tile
         // costs about 0.55 of a whole one (1280 x 960 x 2048: 63.8 -> 53.1 us; 1152^3: 38.2 -> 31.8; 896 x

@@ -230,7 +230,33 @@ def secondary(hip):
                                        "GB/s": nbytes / ms / 1e6,
                                        "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS,
                                        "kernel": hip.last_kernel()}
-    del xi, wi, oi
+    # the same with 36 weight matrices in rotation (604 MB), so that every launch meets its weights in HBM
+    # rather than in the 256 MB Infinity Cache, as a layer of a large model does
+    wsets = [wi] + [hip.array(rand_i8(rng, (4096, 4096))) for _ in range(35)]
+    turn = [0]
+
+    def config2_rotating():
+        turn[0] = (turn[0] + 1) % len(wsets)
+        hip.check(hip.L.axhip_qgemm_w8a8(xi.ptr, 0.01, wsets[turn[0]].ptr, ws.ptr, bi.ptr, 0, oi.ptr, None, 256, 4096, 4096))
+    _, ms = time_calls(hip, config2_rotating)
+    res["int8_qgemm_256x4096x4096"]["weights_from_hbm_us"] = ms * 1e3
+    del xi, wi, oi, wsets
+
+    # one round of fp32 tiles over a long K (256 tiles, K = 4096), operands cached and in rotation (9 x 67 MB)
+    a1 = hip.array(rng.normal(0, 1, (256, 4096)).astype(np.float32))
+    bsets = [hip.array(rng.normal(0, 0.02, (4096, 4096)).astype(np.float32)) for _ in range(9)]
+    c1 = hip.empty((256, 4096))
+    _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm(0, 0, 256, 4096, 4096, 1.0, a1.ptr, 4096, bsets[0].ptr, 4096, 0.0,
+                                                                c1.ptr, 4096, None, 0)))
+
+    def one_round_rotating():
+        turn[0] = (turn[0] + 1) % len(bsets)
+        hip.check(hip.L.axhip_sgemm(0, 0, 256, 4096, 4096, 1.0, a1.ptr, 4096, bsets[turn[0]].ptr, 4096, 0.0, c1.ptr, 4096, None, 0))
+    _, ms2 = time_calls(hip, one_round_rotating)
+    fl = 2 * 256 * 4096 * 4096
+    res["fp32_gemm_256x4096x4096"] = {"us": ms * 1e3, "TFLOP/s": fl / ms / 1e9, "weights_from_hbm_us": ms2 * 1e3,
+                                      "weights_from_hbm_TFLOP/s": fl / ms2 / 1e9, "kernel": hip.last_kernel()}
+    del a1, bsets, c1
 
     # config 1: bs=1 MLP 784 -> 4096 -> 4096 -> 10 through the skinny-M route, M in {1,2,4,8}.
     # 8 rotating weight sets (641 MB) so every pass streams from HBM, not the 256 MB Infinity Cache.
@@ -418,6 +444,25 @@ def secondary(hip):
                                                                          M, N, K)))
         qshapes[f"{M}x{N}x{K}"] = {"fp32_us": t_fp * 1e3, "w8a32_us": t_q * 1e3, "w8a8_us": t_8 * 1e3,
                                    "w8a32_speedup_over_fp32": t_fp / t_q, "w8a8_kernel": hip.last_kernel()}
+        # the same two with the weights in rotation (about 600 MB of each kind), i.e. read from HBM on every call as the
+        # reference's CPU benchmark reads them from DRAM: the case a quarter of the weight bytes is for
+        nset = max(2, min(64, int(600e6 // (4 * N * K))))
+        wts = [wt] + [hip.array(rng.uniform(-1, 1, (K, N)).astype(np.float32)) for _ in range(nset - 1)]
+        wqs = [wq] + [hip.array(rand_i8(rng, (N, K))) for _ in range(4 * nset - 1)]
+        turn = [0, 0]
+
+        def fp_rot():
+            turn[0] = (turn[0] + 1) % len(wts)
+            hip.check(hip.L.axhip_sgemm(0, 0, M, N, K, 1.0, a.ptr, K, wts[turn[0]].ptr, N, 0.0, out.ptr, N, None, 0))
+
+        def q_rot():
+            turn[1] = (turn[1] + 1) % len(wqs)
+            hip.check(hip.L.axhip_qgemm_w8a32(a.ptr, wqs[turn[1]].ptr, ws.ptr, out.ptr, M, N, K))
+        _, t_fp = time_calls(hip, fp_rot, seconds=0.2)
+        _, t_q = time_calls(hip, q_rot, seconds=0.2)
+        qshapes[f"{M}x{N}x{K}"].update({"fp32_weights_from_hbm_us": t_fp * 1e3, "w8a32_weights_from_hbm_us": t_q * 1e3,
+                                        "w8a32_speedup_weights_from_hbm": t_fp / t_q})
+        del wts, wqs
     res["bench_qgemm_shapes"] = qshapes
 
     # config 1 again, end to end through the public API the reference's users call: ax_layer_forward of a
