@@ -1,10 +1,17 @@
 // W8A32: out[m,n] = w_scales[n] * sum_k a[m,k] * (float)w[n,k], fp32 accumulation.
 //
-// M <= 8 (the bandwidth-bound inference case): one wave owns 4 weight rows.  Lanes walk K in
-// 16-element steps (a wave-wide load covers 1 KiB of one row), each lane keeps the activations of
-// its k positions in registers across the 4 rows, and the 4*M partial sums are reduced over
-// the wave together, in a fixed tree order, ending one per lane for the write-back.  Larger M goes through the fp32
-// matrix-core GEMM with the int8 operand converted while it is staged in LDS.
+// M <= 6 (the bandwidth-bound inference case) streams the weights once.  A workgroup of four waves owns
+// 4 * R consecutive weight rows, a wave R of them over all of K.  K is walked in windows of 1024: a
+// wave-wide 16-byte load covers 1 KiB of one row, lane l the k values 16 l .. 16 l + 15 of the window.
+// The activations of a slice of K sit in LDS, laid out so that the four 16-byte reads a lane makes per
+// window and activation row are consecutive across lanes; a lane turns its 16 weight bytes of each of the
+// R rows into floats and multiplies them into R * M running sums.  Weights of the next U windows
+// (R * U = 8 loads of 16 bytes per lane) are requested before the current ones are used, and the first
+// batch before the activations are staged, so 16 KiB per wave are in flight throughout.  The R * M sums
+// are added over the wave together in a fixed tree order and end one per lane for the write-back.
+// Rows at any byte alignment and any K: whole 16-byte steps are fetched with one load wherever the row
+// starts (global memory takes unaligned vector loads), the last partial step byte by byte.
+// Larger M goes through the fp32 matrix-core GEMM with the int8 operand converted while it is staged.
 #include "common.h"
 
 namespace axhip {
@@ -15,83 +22,201 @@ int sgemm_i8w(int64_t M, int64_t N, int64_t K, const float *a, const int8_t *w,
 namespace {
 using namespace axhip;
 
-constexpr int ROWS = 4;   // weight rows per wave
+// windows requested together: 8 loads per lane in all, less where M activation rows leave no room for more in LDS
+template <int MR, int R> constexpr int windows_per_step() {
+    constexpr int most = MR <= 2 ? 8 : MR <= 4 ? 4 : 2;
+    return 8 / R < most ? 8 / R : most;
+}
 
-template <int MR>
-__global__ void __launch_bounds__(64)
-k_w8a32_gemv(const float *__restrict__ a, const int8_t *__restrict__ w,
-             const float *__restrict__ w_scales, float *__restrict__ out, int64_t N, int64_t K) {
-    const int lane = threadIdx.x;
-    const int64_t n0 = (int64_t)blockIdx.x * ROWS;
-    float acc[ROWS][MR];
+template <int R, int U>
+__device__ __forceinline__ void w8a32_request(v4i (&dst)[R][U], const int8_t *w, int64_t first_row, int64_t N, int64_t k0, int lane,
+                                              int64_t K) {
 #pragma unroll
-    for (int r = 0; r < ROWS; r++)
+    for (int u = 0; u < U; u++) {
+        const int64_t k = k0 + (int64_t)u * 1024 + lane * 16;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int64_t n = first_row + r < N ? first_row + r : N - 1;     // rows past N repeat the last one, unstored
+            const int8_t *row = w + n * K;
+            v4i p = {0, 0, 0, 0};
+            if (k + 16 <= K) {
+                __builtin_memcpy(&p, row + k, 16);
+            } else if (k < K) {
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    if (k + e < K) p[e >> 2] |= (int)(unsigned char)row[k + e] << (8 * (e & 3));
+            }
+            dst[r][u] = p;
+        }
+    }
+}
+
+template <int MR, int R, int U>
+__device__ __forceinline__ void w8a32_multiply(const v4i (&src)[R][U], float (&acc)[R][MR], const v4f *xs, int quads_per_row,
+                                               int window0, int lane) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        v4f xa[MR][4];
+#pragma unroll
+        for (int m = 0; m < MR; m++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) xa[m][q] = xs[m * quads_per_row + ((window0 + u) * 4 + q) * 64 + lane];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int word = src[r][u][q];
+                const float f0 = (float)(signed char)(word & 0xff), f1 = (float)(signed char)((word >> 8) & 0xff),
+                            f2 = (float)(signed char)((word >> 16) & 0xff), f3 = (float)(signed char)((word >> 24) & 0xff);
+#pragma unroll
+                for (int m = 0; m < MR; m++) {
+                    float s = acc[r][m];
+                    s = __builtin_fmaf(xa[m][q].x, f0, s);
+                    s = __builtin_fmaf(xa[m][q].y, f1, s);
+                    s = __builtin_fmaf(xa[m][q].z, f2, s);
+                    s = __builtin_fmaf(xa[m][q].w, f3, s);
+                    acc[r][m] = s;
+                }
+            }
+    }
+}
+
+// slice: k values of the activations held in LDS at a time, a multiple of U * 1024.  groups: row groups of 4 * R
+// rows a workgroup walks one after the other (more than one only when a single slice holds all of K, so the
+// activations are staged once); the weight requests run ahead across group boundaries.
+template <int MR, int R>
+__global__ void __launch_bounds__(256)
+k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const float *__restrict__ w_scales,
+             float *__restrict__ out, int64_t N, int64_t K, int slice, int groups) {
+    constexpr int U = windows_per_step<MR, R>();
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    v4f *xs = reinterpret_cast<v4f *>(lds_raw);                 // [MR][slice / 4], permuted inside each window
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t base = (int64_t)blockIdx.x * groups * (4 * R) + wave * R;      // this wave's rows of group g: base + g * 4 R
+    float acc[R][MR];
+#pragma unroll
+    for (int r = 0; r < R; r++)
 #pragma unroll
         for (int m = 0; m < MR; m++) acc[r][m] = 0.0f;
 
-    for (int64_t k = (int64_t)lane * 16; k < K; k += 64 * 16) {
-        // A step wholly inside the row is fetched with 16-byte loads at whatever alignment K and
-        // the base pointers leave (global memory takes unaligned vector loads); only the last,
-        // partial step of a row goes element by element.
-        const bool whole = k + 16 <= K;
-        float xa[MR][16];
-        if (whole) {
-#pragma unroll
-            for (int m = 0; m < MR; m++)
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    v4f t;
-                    __builtin_memcpy(&t, a + m * K + k + 4 * q, 16);
-                    xa[m][4 * q] = t.x; xa[m][4 * q + 1] = t.y; xa[m][4 * q + 2] = t.z; xa[m][4 * q + 3] = t.w;
-                }
-        } else {
-#pragma unroll
-            for (int m = 0; m < MR; m++)
-#pragma unroll
-                for (int e = 0; e < 16; e++) xa[m][e] = (k + e < K) ? a[m * K + k + e] : 0.0f;
-        }
-#pragma unroll
-        for (int r = 0; r < ROWS; r++) {
-            const int64_t n = n0 + r;
-            if (n >= N) break;
-            float wf[16];
-            if (whole) {
-                v4i p;
-                __builtin_memcpy(&p, w + n * K + k, 16);
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const int word = p[q];
-                    wf[4 * q] = (float)(signed char)(word & 0xff);
-                    wf[4 * q + 1] = (float)(signed char)((word >> 8) & 0xff);
-                    wf[4 * q + 2] = (float)(signed char)((word >> 16) & 0xff);
-                    wf[4 * q + 3] = (float)(signed char)((word >> 24) & 0xff);
-                }
+    const int quads = slice / 4, steps_per_slice = slice / (U * 1024);
+    const int steps = (int)((K + U * 1024 - 1) / (U * 1024));
+    // activations of slice s -> LDS: 16-byte piece q of lane l's 16 values of window v at quad (4 v + q) * 64 + l
+    auto stage = [&](int64_t s) {
+        for (int f = tid; f < MR * quads; f += 256) {
+            const int m = f / quads, fr = f - m * quads;
+            const int v = fr >> 8, q = (fr >> 6) & 3, l = fr & 63;
+            const int64_t k = s * slice + v * 1024 + l * 16 + q * 4;
+            v4f t = {0.f, 0.f, 0.f, 0.f};
+            if (k + 4 <= K) {
+                __builtin_memcpy(&t, a + m * K + k, 16);
             } else {
 #pragma unroll
-                for (int e = 0; e < 16; e++) wf[e] = (k + e < K) ? (float)w[n * K + k + e] : 0.0f;
+                for (int e = 0; e < 4; e++)
+                    if (k + e < K) t[e] = a[m * K + k + e];
             }
-#pragma unroll
-            for (int m = 0; m < MR; m++)
-#pragma unroll
-                for (int e = 0; e < 16; e++) acc[r][m] = __builtin_fmaf(xa[m][e], wf[e], acc[r][m]);
+            xs[f] = t;
         }
-    }
-    constexpr int NV = ROWS * MR <= 4 ? 4 : ROWS * MR <= 8 ? 8 : ROWS * MR <= 16 ? 16 : 32;
-    float v[NV];
+    };
+    // the sums of a finished group: added over the wave in a fixed tree, one result per lane, scaled and stored
+    auto finish = [&](int64_t first_row) {
+        constexpr int NV = R * MR <= 1 ? 1 : R * MR <= 2 ? 2 : R * MR <= 4 ? 4 : R * MR <= 8 ? 8 : R * MR <= 16 ? 16 : 32;
+        float v[NV];
 #pragma unroll
-    for (int i = 0; i < NV; i++) v[i] = i < ROWS * MR ? acc[i / MR][i % MR] : 0.0f;
-    wave_sum_spread(v, lane);
-    const int idx = lane / (64 / NV), r = idx / MR, m = idx % MR;
-    if (lane % (64 / NV) != 0 || idx >= ROWS * MR || n0 + r >= N) return;
-    out[m * N + n0 + r] = v[0] * w_scales[n0 + r];
+        for (int i = 0; i < NV; i++) v[i] = i < R * MR ? acc[i / MR][i % MR] : 0.0f;
+        wave_sum_spread(v, lane);
+        const int idx = lane / (64 / NV), r = idx / MR, m = idx % MR;
+        if (lane % (64 / NV) == 0 && idx < R * MR && first_row + r < N) out[m * N + first_row + r] = v[0] * w_scales[first_row + r];
+#pragma unroll
+        for (int rr = 0; rr < R; rr++)
+#pragma unroll
+            for (int mm = 0; mm < MR; mm++) acc[rr][mm] = 0.0f;
+    };
+    v4i wa[R][U], wb[R][U];
+    w8a32_request<R, U>(wa, w, base, N, 0, lane, K);            // before the activations: the latency of both overlaps
+    // One flat walk over (group, step): every quantity below is uniform over the workgroup.  Two steps per
+    // round so that the two weight buffers keep their names.
+    int g = 0, it = 0, in_slice = steps_per_slice;              // "slice full" forces the first staging
+    int64_t s = 0;
+    const int total = groups * steps;
+    auto enter = [&]() {                                        // the slice of step `it` is in LDS
+        if (in_slice == steps_per_slice && (groups == 1 || (g == 0 && it == 0))) {
+            __syncthreads();
+            stage(s++);
+            __syncthreads();
+            in_slice = 0;
+        }
+    };
+    auto advance = [&]() {                                      // after a step: the group ends with its last one
+        ++it;
+        ++in_slice;
+        if (it == steps) {
+            finish(base + (int64_t)g * (4 * R));
+            it = 0;
+            ++g;
+            if (groups > 1) in_slice = 0;                       // one slice holds all of K: start over in it
+            else { in_slice = steps_per_slice; s = 0; }
+        }
+    };
+    for (int t = 0; t < total;) {
+        enter();
+        if (t + 1 < total) {
+            const bool wrap = it + 1 == steps;
+            w8a32_request<R, U>(wb, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * U * 1024, lane, K);
+        }
+        w8a32_multiply<MR, R, U>(wa, acc, xs, quads, in_slice * U, lane);
+        advance();
+        if (++t >= total) break;
+        enter();
+        if (t + 1 < total) {
+            const bool wrap = it + 1 == steps;
+            w8a32_request<R, U>(wa, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * U * 1024, lane, K);
+        }
+        w8a32_multiply<MR, R, U>(wb, acc, xs, quads, in_slice * U, lane);
+        advance();
+        ++t;
+    }
 }
 
-template <int MR>
-int launch_gemv(const float *a, const int8_t *w, const float *s, float *out, int64_t N, int64_t K) {
-    dim3 grid((unsigned)((N + ROWS - 1) / ROWS));
-    hipLaunchKernelGGL(k_w8a32_gemv<MR>, grid, dim3(64), 0, kStream, a, w, s, out, N, K);
+template <int MR, int R>
+int launch_rows(const float *a, const int8_t *w, const float *s, float *out, int64_t N, int64_t K) {
+    constexpr int U = windows_per_step<MR, R>();
+    // up to 64 KiB of activations at a time (two workgroups share a CU), no more than K needs
+    int64_t slice = (16384 / MR) / (U * 1024) * (U * 1024);
+    const int64_t need = (K + U * 1024 - 1) / (U * 1024) * (U * 1024);
+    if (slice > need) slice = need;
+    // With all of K in one slice a workgroup stages the activations once and walks several row groups, as
+    // many as still leave two workgroups for every CU (M = 1: 32000 x 4096 30.1 -> 25.3 us, 16384 x 4096
+    // 17.8 -> 15.2 against one group each; with short rows one group each stays ahead, 50000 x 2048: 18.5 against 20.9).
+    int64_t groups = 1;
+    if (slice == need) {
+        groups = N / (4 * R * 2 * (int64_t)cu_count());
+        if (groups < 1) groups = 1;
+        if (groups > 64) groups = 64;
+    }
+    const size_t smem = (size_t)MR * slice * sizeof(float);
+    auto kern = k_w8a32_rows<MR, R>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 65536),
+                      "hipFuncSetAttribute");
+        attr_set = true;
+    }
+    const int64_t rows_per_block = 4 * R * groups, blocks = (N + rows_per_block - 1) / rows_per_block;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), smem, kStream, a, w, s, out, N, K, (int)slice, (int)groups);
     return check_launch("qgemm_w8a32_gemv");
 }
+
+// Rows per wave: as many as still leave two workgroups for every CU (fewer, fuller workgroups measured slower at
+// every M: 8 x 4096 x 4096 on four rows per wave and one workgroup per CU 20.6 us against 13.6).
+template <int MR>
+int launch_gemv(const float *a, const int8_t *w, const float *s, float *out, int64_t N, int64_t K) {
+    const int64_t cus = cu_count();
+    if (N >= 32 * cus) return launch_rows<MR, 4>(a, w, s, out, N, K);
+    if (N >= 16 * cus) return launch_rows<MR, 2>(a, w, s, out, N, K);
+    return launch_rows<MR, 1>(a, w, s, out, N, K);
+}
+
 }  // namespace
 
 extern "C" int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w_scales, float *out,
@@ -100,8 +225,11 @@ extern "C" int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w
     if (!a || !w || !w_scales || !out) return fail(AXHIP_ERR_NULL_ARG, "qgemm_w8a32: NULL");
     if (M < 0 || N < 0 || K < 0) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a32: negative dimension");
     if (M == 0 || N == 0) return AXHIP_OK;
-    if (M > 8) return axhip::sgemm_i8w(M, N, K, a, w, w_scales, out);
-    if ((N + ROWS - 1) / ROWS > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a32: N too large");
+    // The weight-streaming form pays M multiply-adds per weight byte on the vector ALU (4096 x 4096: 4.4 us at
+    // M = 1, +1.4 us per further row); from M = 7 on the matrix-core tiles are level or ahead (M = 8:
+    // 11008 x 4096 43.0 against 30.8 us, 4096 x 11008 52.8 against 31.2, 4096 x 4096 13.9 against 15.3).
+    if (M > 6) return axhip::sgemm_i8w(M, N, K, a, w, w_scales, out);
+    if ((N + 3) / 4 > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a32: N too large");
     note_kernel("qgemm_w8a32_gemv");
     switch (M) {
         case 1: return launch_gemv<1>(a, w, w_scales, out, N, K);
@@ -109,8 +237,6 @@ extern "C" int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w
         case 3: return launch_gemv<3>(a, w, w_scales, out, N, K);
         case 4: return launch_gemv<4>(a, w, w_scales, out, N, K);
         case 5: return launch_gemv<5>(a, w, w_scales, out, N, K);
-        case 6: return launch_gemv<6>(a, w, w_scales, out, N, K);
-        case 7: return launch_gemv<7>(a, w, w_scales, out, N, K);
-        default: return launch_gemv<8>(a, w, w_scales, out, N, K);
+        default: return launch_gemv<6>(a, w, w_scales, out, N, K);
     }
 }

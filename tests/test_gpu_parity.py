@@ -401,7 +401,7 @@ def test_forced_tiles_and_splits_keep_parity(hip, oracle):
 
 
 def test_w8a32_dispatch_sweep(hip, oracle):
-    """80 seeded W8A32 shapes from the boundary dimensions: the row-per-wave form (M <= 8), the matrix-core form,
+    """80 seeded W8A32 shapes from the boundary dimensions: the weight-streaming form (M <= 6), the matrix-core form,
     its split over K and its K tail all obey the fp64 bound of a correct fp32 accumulation."""
     rng = np.random.default_rng(20243)
     seen = set()
@@ -671,7 +671,11 @@ W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 
                 (2, 130, 256), (6, 67, 1040), (7, 5, 2064),
                 (128, 1024, 512), (1024, 512, 1024), (256, 768, 768), (64, 768, 768),   # one launch on 32x64 tiles / split
                 (20, 1024, 512), (150, 260, 160), (96, 2048, 1024), (160, 3072, 768),   # 32x64 tiles, whole and with clamped edges
-                (32, 128, 517), (70, 260, 1031), (3, 64, 1037)]   # rows at odd byte offsets       # every row count of the wave-per-rows form
+                # the weight-streaming form: several row groups on one staging, 1 / 2 / 4 rows per wave, several slices of K,
+                # a last window that ends inside a 16-byte step, rows that run past N
+                (1, 20000, 520), (2, 16400, 300), (3, 8200, 1031), (6, 4100, 8192), (5, 4099, 2050), (4, 9000, 4100),
+                (6, 33, 10000), (1, 70, 20000),
+                (32, 128, 517), (70, 260, 1031), (3, 64, 1037)]   # rows at odd byte offsets
 
 
 @pytest.mark.parametrize("M,N,K", W8A32_SHAPES)
