@@ -31,9 +31,9 @@ def check_fp32(oracle, got, a, b, transb=False, ref=None):
 INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300), (33, 64, 1000),
                (128, 128, 256), (128, 256, 128), (256, 512, 384), (384, 128, 4096),
                (2048, 4096, 512), (256, 4096, 4096),
-               # M <= 8 with whole 16-byte steps of K: the wave-per-rows dot-product route
+               # M <= 4 with whole 16-byte steps of K: the wave-per-rows dot-product route (and M = 5..8, on the tiles since)
                (1, 768, 3072), (1, 4096, 4096), (8, 768, 768), (3, 5, 16), (7, 1001, 1040), (2, 3, 4112),
-               (4, 33, 64), (5, 9, 48), (6, 130, 256),
+               (4, 33, 64), (5, 9, 48), (6, 130, 256), (4, 11008, 512), (3, 4100, 2064),
                # off the 256 grid with a large interior: persistent kernel inside, smaller tiles on the fringes
                (2112, 4128, 256), (4100, 2304, 128), (2048, 4100, 128),
                # rows that start at odd byte offsets (K % 16 != 0)
@@ -85,7 +85,7 @@ def test_w8a8_extreme_values_and_golden(hip, oracle, golden):
     w = np.full((128, 8192), -127, np.int8)
     _, acc = hip.qgemm_w8a8(hip.array(x), 1.0, hip.array(w), None, want_out=False)
     assert (acc.numpy() == 127 * 127 * 8192).all()
-    xg = hip.array(x[:8].copy())                          # same through the M <= 8 route
+    xg = hip.array(x[:4].copy())                          # same through the M <= 4 route
     wg = hip.array(np.full((128, 8192), -128, np.int8))
     _, acc = hip.qgemm_w8a8(xg, 1.0, wg, None, want_out=False)
     assert hip.last_kernel() == "qgemm_w8a8_gemv" and (acc.numpy() == 127 * 128 * 8192).all()
