@@ -1,6 +1,6 @@
 // W8A32: out[m,n] = w_scales[n] * sum_k a[m,k] * (float)w[n,k], fp32 accumulation.
 //
-// M <= 6 (the bandwidth-bound inference case) streams the weights once.  A workgroup of four waves owns
+// M = 2..6 (the bandwidth-bound inference case) streams the weights once.  A workgroup of four waves owns
 // 4 * R consecutive weight rows, a wave R of them over all of K.  K is walked in windows of 1024: a
 // wave-wide 16-byte load covers 1 KiB of one row, lane l the k values 16 l .. 16 l + 15 of the window.
 // The activations of a slice of K sit in LDS, laid out so that the four 16-byte reads a lane makes per
@@ -11,7 +11,8 @@
 // are added over the wave together in a fixed tree order and end one per lane for the write-back.
 // Rows at any byte alignment and any K: whole 16-byte steps are fetched with one load wherever the row
 // starts (global memory takes unaligned vector loads), the last partial step byte by byte.
-// Larger M goes through the fp32 matrix-core GEMM with the int8 operand converted while it is staged.
+// M = 1 has a form of its own without LDS (below).  Larger M goes through the fp32 matrix-core GEMM with the
+// int8 operand converted while it is staged.
 #include "common.h"
 
 namespace axhip {
@@ -30,9 +31,10 @@ template <int MR, int R> constexpr int windows_per_step() {
 
 template <int R, int U>
 __device__ __forceinline__ void w8a32_request(v4i (&dst)[R][U], const int8_t *w, int64_t first_row, int64_t N, int64_t k0, int lane,
-                                              int64_t K) {
+                                              int64_t K, int used) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
+        if (u >= used) break;                                   // uniform: a short K fills fewer windows per step
         const int64_t k = k0 + (int64_t)u * 1024 + lane * 16;
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -53,9 +55,10 @@ __device__ __forceinline__ void w8a32_request(v4i (&dst)[R][U], const int8_t *w,
 
 template <int MR, int R, int U>
 __device__ __forceinline__ void w8a32_multiply(const v4i (&src)[R][U], float (&acc)[R][MR], const v4f *xs, int quads_per_row,
-                                               int window0, int lane) {
+                                               int window0, int lane, int used) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
+        if (u >= used) break;
         v4f xa[MR][4];
 #pragma unroll
         for (int m = 0; m < MR; m++)
@@ -81,13 +84,13 @@ __device__ __forceinline__ void w8a32_multiply(const v4i (&src)[R][U], float (&a
     }
 }
 
-// slice: k values of the activations held in LDS at a time, a multiple of U * 1024.  groups: row groups of 4 * R
+// slice: k values of the activations held in LDS at a time, a multiple of used * 1024.  groups: row groups of 4 * R
 // rows a workgroup walks one after the other (more than one only when a single slice holds all of K, so the
 // activations are staged once); the weight requests run ahead across group boundaries.
 template <int MR, int R>
 __global__ void __launch_bounds__(256)
 k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const float *__restrict__ w_scales,
-             float *__restrict__ out, int64_t N, int64_t K, int slice, int groups) {
+             float *__restrict__ out, int64_t N, int64_t K, int slice, int groups, int used) {
     constexpr int U = windows_per_step<MR, R>();
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     v4f *xs = reinterpret_cast<v4f *>(lds_raw);                 // [MR][slice / 4], permuted inside each window
@@ -99,8 +102,9 @@ k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const fl
 #pragma unroll
         for (int m = 0; m < MR; m++) acc[r][m] = 0.0f;
 
-    const int quads = slice / 4, steps_per_slice = slice / (U * 1024);
-    const int steps = (int)((K + U * 1024 - 1) / (U * 1024));
+    const int span = used * 1024;                               // k values of a step: `used` <= U windows
+    const int quads = slice / 4, steps_per_slice = slice / span;
+    const int steps = (int)((K + span - 1) / span);
     // activations of slice s -> LDS: 16-byte piece q of lane l's 16 values of window v at quad (4 v + q) * 64 + l
     auto stage = [&](int64_t s) {
         for (int f = tid; f < MR * quads; f += 256) {
@@ -133,7 +137,7 @@ k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const fl
             for (int mm = 0; mm < MR; mm++) acc[rr][mm] = 0.0f;
     };
     v4i wa[R][U], wb[R][U];
-    w8a32_request<R, U>(wa, w, base, N, 0, lane, K);            // before the activations: the latency of both overlaps
+    w8a32_request<R, U>(wa, w, base, N, 0, lane, K, used);      // before the activations: the latency of both overlaps
     // One flat walk over (group, step): every quantity below is uniform over the workgroup.  Two steps per
     // round so that the two weight buffers keep their names.
     int g = 0, it = 0, in_slice = steps_per_slice;              // "slice full" forces the first staging
@@ -162,28 +166,150 @@ k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const fl
         enter();
         if (t + 1 < total) {
             const bool wrap = it + 1 == steps;
-            w8a32_request<R, U>(wb, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * U * 1024, lane, K);
+            w8a32_request<R, U>(wb, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K, used);
         }
-        w8a32_multiply<MR, R, U>(wa, acc, xs, quads, in_slice * U, lane);
+        w8a32_multiply<MR, R, U>(wa, acc, xs, quads, in_slice * used, lane, used);
         advance();
         if (++t >= total) break;
         enter();
         if (t + 1 < total) {
             const bool wrap = it + 1 == steps;
-            w8a32_request<R, U>(wa, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * U * 1024, lane, K);
+            w8a32_request<R, U>(wa, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K, used);
         }
-        w8a32_multiply<MR, R, U>(wb, acc, xs, quads, in_slice * U, lane);
+        w8a32_multiply<MR, R, U>(wb, acc, xs, quads, in_slice * used, lane, used);
         advance();
         ++t;
     }
 }
 
+// ---- M = 1 ------------------------------------------------------------------------------------------
+// One activation row needs no LDS: a lane's 16 activations of a window are 64 bytes that every wave of the
+// chip reads from cache, so they travel with the weight requests (two buffers of R * U weight loads and 4 U
+// activation loads per lane) and no workgroup waits for a staging pass before its stream starts (same box, LDS form
+// -> this one, cached / weights from HBM: 4096 x 4096 5.0 / 7.2 -> 4.6 / 5.9 us, 8192 x 8192 16.2 / 18.1 -> 13.2 / 15.9,
+// 32000 x 4096 24.7 / 29.6 -> 22.7 / 28.0, 4096 x 11008 14.7 / 18.3 -> 11.9 / 15.2).  Otherwise the walk of the form above.
+template <int R, int U>
+struct W8a32Row1Buf {
+    v4i w[R][U];
+    v4f x[U][4];
+};
+
+template <int R, int U>
+__device__ __forceinline__ void w8a32_row1_request(W8a32Row1Buf<R, U> &b, const float *a, const int8_t *w, int64_t first_row, int64_t N,
+                                                   int64_t k0, int lane, int64_t K, int used) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        if (u >= used) break;
+        const int64_t k = k0 + (int64_t)u * 1024 + lane * 16;
+#pragma unroll
+        for (int q = 0; q < 4; q++) b.x[u][q] = v4f{0.f, 0.f, 0.f, 0.f};
+        if (k + 16 <= K) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) __builtin_memcpy(&b.x[u][q], a + k + 4 * q, 16);
+        } else if (k < K) {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (k + 4 * q + e < K) b.x[u][q][e] = a[k + 4 * q + e];
+        }
+    }
+    w8a32_request<R, U>(b.w, w, first_row, N, k0, lane, K, used);
+}
+
+template <int R, int U>
+__device__ __forceinline__ void w8a32_row1_multiply(const W8a32Row1Buf<R, U> &b, float (&acc)[R], int used) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        if (u >= used) break;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int word = b.w[r][u][q];
+                float s = acc[r];
+                s = __builtin_fmaf(b.x[u][q].x, (float)(signed char)(word & 0xff), s);
+                s = __builtin_fmaf(b.x[u][q].y, (float)(signed char)((word >> 8) & 0xff), s);
+                s = __builtin_fmaf(b.x[u][q].z, (float)(signed char)((word >> 16) & 0xff), s);
+                s = __builtin_fmaf(b.x[u][q].w, (float)(signed char)((word >> 24) & 0xff), s);
+                acc[r] = s;
+            }
+    }
+}
+
+template <int R, int U>
+__global__ void __launch_bounds__(256)
+k_w8a32_row1(const float *__restrict__ a, const int8_t *__restrict__ w, const float *__restrict__ w_scales,
+             float *__restrict__ out, int64_t N, int64_t K, int groups, int used) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t base = (int64_t)blockIdx.x * groups * (4 * R) + wave * R;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    const int span = used * 1024;
+    const int steps = (int)((K + span - 1) / span), total = groups * steps;
+    W8a32Row1Buf<R, U> ba, bb;
+    w8a32_row1_request<R, U>(ba, a, w, base, N, 0, lane, K, used);
+    int g = 0, it = 0;
+    auto finish = [&]() {                                       // the group's R sums: over the wave, scaled, stored
+        constexpr int NV = R;                                   // 1, 2 or 4
+        float v[NV];
+#pragma unroll
+        for (int i = 0; i < NV; i++) v[i] = acc[i];
+        wave_sum_spread(v, lane);
+        const int r = lane / (64 / NV);
+        const int64_t n = base + (int64_t)g * (4 * R) + r;
+        if (lane % (64 / NV) == 0 && n < N) out[n] = v[0] * w_scales[n];
+#pragma unroll
+        for (int i = 0; i < R; i++) acc[i] = 0.0f;
+    };
+    auto next_request = [&](W8a32Row1Buf<R, U> &b) {            // operands of the step after (g, it)
+        const bool wrap = it + 1 == steps;
+        w8a32_row1_request<R, U>(b, a, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K, used);
+    };
+    auto advance = [&]() {
+        if (++it == steps) {
+            finish();
+            it = 0;
+            ++g;
+        }
+    };
+    for (int t = 0; t < total;) {
+        if (t + 1 < total) next_request(bb);
+        w8a32_row1_multiply<R, U>(ba, acc, used);
+        advance();
+        if (++t >= total) break;
+        if (t + 1 < total) next_request(ba);
+        w8a32_row1_multiply<R, U>(bb, acc, used);
+        advance();
+        ++t;
+    }
+}
+
+template <int R, int U>
+int launch_row1(const float *a, const int8_t *w, const float *s, float *out, int64_t N, int64_t K) {
+    const int64_t windows = (K + 1023) / 1024;
+    int used = U;
+    while (used > 1 && used / 2 >= windows) used /= 2;
+    int64_t groups = N / (4 * R * 2 * (int64_t)cu_count());     // as many as still leave two workgroups for every CU
+    if (groups < 1) groups = 1;
+    if (groups > 64) groups = 64;
+    const int64_t rows_per_block = 4 * R * groups, blocks = (N + rows_per_block - 1) / rows_per_block;
+    hipLaunchKernelGGL((k_w8a32_row1<R, U>), dim3((unsigned)blocks), dim3(256), 0, kStream, a, w, s, out, N, K, (int)groups, used);
+    return check_launch("qgemm_w8a32_gemv");
+}
+
 template <int MR, int R>
 int launch_rows(const float *a, const int8_t *w, const float *s, float *out, int64_t N, int64_t K) {
     constexpr int U = windows_per_step<MR, R>();
+    // windows of 1024 k a step takes: all U the registers allow, fewer when K does not fill them
+    const int64_t windows = (K + 1023) / 1024;
+    int used = U;
+    while (used > 1 && used / 2 >= windows) used /= 2;
+    const int64_t span = (int64_t)used * 1024;
     // up to 64 KiB of activations at a time (two workgroups share a CU), no more than K needs
-    int64_t slice = (16384 / MR) / (U * 1024) * (U * 1024);
-    const int64_t need = (K + U * 1024 - 1) / (U * 1024) * (U * 1024);
+    int64_t slice = (16384 / MR) / span * span;
+    const int64_t need = (K + span - 1) / span * span;
     if (slice > need) slice = need;
     // With all of K in one slice a workgroup stages the activations once and walks several row groups, as
     // many as still leave two workgroups for every CU (M = 1: 32000 x 4096 30.1 -> 25.3 us, 16384 x 4096
@@ -203,7 +329,7 @@ int launch_rows(const float *a, const int8_t *w, const float *s, float *out, int
         attr_set = true;
     }
     const int64_t rows_per_block = 4 * R * groups, blocks = (N + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), smem, kStream, a, w, s, out, N, K, (int)slice, (int)groups);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), smem, kStream, a, w, s, out, N, K, (int)slice, (int)groups, used);
     return check_launch("qgemm_w8a32_gemv");
 }
 
@@ -212,7 +338,15 @@ int launch_rows(const float *a, const int8_t *w, const float *s, float *out, int
 template <int MR>
 int launch_gemv(const float *a, const int8_t *w, const float *s, float *out, int64_t N, int64_t K) {
     const int64_t cus = cu_count();
-    if (N >= 32 * cus) return launch_rows<MR, 4>(a, w, s, out, N, K);
+    if constexpr (MR == 1) {
+        // rows per wave x windows per request, by sweep (cached / weights from HBM, us): 32000 x 4096 on 4 x 1 22.7 / 28.0
+        // (2 x 2: 30.0 / 39.6), 8192 x 8192 13.2 / 15.9, 4096 x 4096 on 2 x 4 4.6 / 5.9 (4 x 2: 4.8 / 8.0), 4096 x 11008 11.9 / 15.2
+        if (N >= 32 * cus) return launch_row1<4, 1>(a, w, s, out, N, K);
+        if (N >= 16 * cus) return launch_row1<2, 4>(a, w, s, out, N, K);
+        if (N >= 8 * cus) return launch_row1<2, 2>(a, w, s, out, N, K);
+        return launch_row1<1, 2>(a, w, s, out, N, K);
+    }
+    if (N >= 64 * cus) return launch_rows<MR, 4>(a, w, s, out, N, K);
     if (N >= 16 * cus) return launch_rows<MR, 2>(a, w, s, out, N, K);
     return launch_rows<MR, 1>(a, w, s, out, N, K);
 }
