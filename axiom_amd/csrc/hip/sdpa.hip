@@ -82,7 +82,7 @@ template <int DK, bool CAUSAL, bool RAG, bool PAD>
 __global__ void __launch_bounds__(256)
 k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__restrict__ V,
        float *__restrict__ O, float *__restrict__ L, int64_t BH, int64_t S, float scale_log2e,
-       int64_t H, int64_t ld, int64_t ldo, int dkr) {
+       int64_t H, int64_t ld, int64_t ldo, int dkr, int pair_tiles) {
     using G = SdGeom<DK>;
     constexpr int KB = DK / 8;                   // 8-wide k-blocks of the score product
     constexpr int DT = DK / 32;                  // 32-wide column tiles of the output
@@ -96,12 +96,15 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
     // heads form a group: workgroup r of a group works on head r % 8 (every query tile of a
     // head then runs on the same XCD and shares its L2 copy of K and V) and on unit r / 8.
     // A unit is one query tile, or, causal, the pair of tiles p and nq-1-p, which together
-    // visit nq+1 key blocks whatever p is (the middle tile of an odd nq stands alone).
-    const int64_t units = CAUSAL ? (nq + 1) / 2 : nq;
+    // visit nq+1 key blocks whatever p is (the middle tile of an odd nq stands alone).  A launch
+    // with no more single tiles than CUs keeps them single (pair_tiles = 0): pairing would only
+    // halve the CUs at work (64 heads of 256 rows: 33.3 us paired, 22.7 single, 20.7 unmasked).
+    const bool paired = CAUSAL && pair_tiles;
+    const int64_t units = paired ? (nq + 1) / 2 : nq;
     const int64_t lin = blockIdx.x, group = lin / (8 * units), left = BH - group * 8;
     const int64_t r = lin - group * 8 * units, hpg = left < 8 ? left : 8;
     const int64_t head = group * 8 + r % hpg, unit = r / hpg;
-    const int passes = (CAUSAL && unit != nq - 1 - unit) ? 2 : 1;
+    const int passes = (paired && unit != nq - 1 - unit) ? 2 : 1;
     // head b * H + h starts at row b * S, column h * DK of matrices with row pitch ld (Q, K, V)
     // and ldo (O): H = 1, ld = DK is one matrix per head; H heads side by side in rows of
     // ld >= H * DK floats is the layout a fused projection writes and the output projection reads
@@ -144,7 +147,7 @@ k_sdpa(const float *__restrict__ Q, const float *__restrict__ K, const float *__
     };
 
     for (int pass = 0; pass < passes; pass++) {
-        const int64_t q0 = (CAUSAL && pass == 0 ? nq - 1 - unit : unit) * SD_BQ;
+        const int64_t q0 = (paired && pass == 0 ? nq - 1 - unit : unit) * SD_BQ;
         if (pass) __syncthreads();                   // the first tile's last key block has been read
         // ---- Q tile (128 rows) through the V area, then into registers; the first key block's
         // K rows stream into their own stage at the same time, so a workgroup pays one load
@@ -365,11 +368,14 @@ int launch_sdpa_p(const float *Q, const float *K, const float *V, float *O, floa
     }
     const float sl2 = scale * 1.4426950408889634f;
     const int64_t nq = (S + SD_BQ - 1) / SD_BQ;
-    dim3 grid((unsigned)((causal ? (nq + 1) / 2 : nq) * BH));
+    // causal tiles p and nq-1-p in one workgroup once there are more tiles than CUs; with a CU for every tile the
+    // longest tile sets the time either way and pairing only halves the CUs at work
+    const int pair = causal && nq * BH > (int64_t)cu_count();
+    dim3 grid((unsigned)((pair ? (nq + 1) / 2 : nq) * BH));
     const bool rag = S % SD_BQ != 0;
 #define AXS_GO(C, R)                                                                                              \
     hipLaunchKernelGGL((k_sdpa<DK, C, R, PAD>), grid, dim3(256), G::SMEM, kStream, Q, K, V, O, L, BH, S, sl2, H, ld, \
-                       ldo, dkr)
+                       ldo, dkr, pair)
     if (causal && rag) AXS_GO(true, true);
     else if (causal) AXS_GO(true, false);
     else if (rag) AXS_GO(false, true);
