@@ -11,7 +11,7 @@
 // are added over the wave together in a fixed tree order and end one per lane for the write-back.
 // Rows at any byte alignment and any K: whole 16-byte steps are fetched with one load wherever the row
 // starts (global memory takes unaligned vector loads), the last partial step byte by byte.
-// M = 1 has a form of its own without LDS (below).  Larger M goes through the fp32 matrix-core GEMM with the
+// M = 1, and up to four rows against fewer than 16384 weight rows, take a form without LDS (below).  Larger M goes through the fp32 matrix-core GEMM with the
 // int8 operand converted while it is staged.
 #include "common.h"
 
@@ -182,43 +182,46 @@ k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const fl
     }
 }
 
-// ---- M = 1 ------------------------------------------------------------------------------------------
+// ---- M = 1 (and up to four rows against fewer than 16384 weight rows) ------------------------------
 // One activation row needs no LDS: a lane's 16 activations of a window are 64 bytes that every wave of the
 // chip reads from cache, so they travel with the weight requests (two buffers of R * U weight loads and 4 U
 // activation loads per lane) and no workgroup waits for a staging pass before its stream starts (same box, LDS form
 // -> this one, cached / weights from HBM: 4096 x 4096 5.0 / 7.2 -> 4.6 / 5.9 us, 8192 x 8192 16.2 / 18.1 -> 13.2 / 15.9,
 // 32000 x 4096 24.7 / 29.6 -> 22.7 / 28.0, 4096 x 11008 14.7 / 18.3 -> 11.9 / 15.2).  Otherwise the walk of the form above.
-template <int R, int U>
-struct W8a32Row1Buf {
+template <int MR, int R, int U>
+struct W8a32DirectBuf {
     v4i w[R][U];
-    v4f x[U][4];
+    v4f x[MR][U][4];
 };
 
-template <int R, int U>
-__device__ __forceinline__ void w8a32_row1_request(W8a32Row1Buf<R, U> &b, const float *a, const int8_t *w, int64_t first_row, int64_t N,
-                                                   int64_t k0, int lane, int64_t K, int used) {
+template <int MR, int R, int U>
+__device__ __forceinline__ void w8a32_direct_request(W8a32DirectBuf<MR, R, U> &b, const float *a, const int8_t *w, int64_t first_row,
+                                                     int64_t N, int64_t k0, int lane, int64_t K, int used) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
         if (u >= used) break;
         const int64_t k = k0 + (int64_t)u * 1024 + lane * 16;
 #pragma unroll
-        for (int q = 0; q < 4; q++) b.x[u][q] = v4f{0.f, 0.f, 0.f, 0.f};
-        if (k + 16 <= K) {
+        for (int m = 0; m < MR; m++) {
 #pragma unroll
-            for (int q = 0; q < 4; q++) __builtin_memcpy(&b.x[u][q], a + k + 4 * q, 16);
-        } else if (k < K) {
+            for (int q = 0; q < 4; q++) b.x[m][u][q] = v4f{0.f, 0.f, 0.f, 0.f};
+            if (k + 16 <= K) {
 #pragma unroll
-            for (int q = 0; q < 4; q++)
+                for (int q = 0; q < 4; q++) __builtin_memcpy(&b.x[m][u][q], a + m * K + k + 4 * q, 16);
+            } else if (k < K) {
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (k + 4 * q + e < K) b.x[u][q][e] = a[k + 4 * q + e];
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (k + 4 * q + e < K) b.x[m][u][q][e] = a[m * K + k + 4 * q + e];
+            }
         }
     }
     w8a32_request<R, U>(b.w, w, first_row, N, k0, lane, K, used);
 }
 
-template <int R, int U>
-__device__ __forceinline__ void w8a32_row1_multiply(const W8a32Row1Buf<R, U> &b, float (&acc)[R], int used) {
+template <int MR, int R, int U>
+__device__ __forceinline__ void w8a32_direct_multiply(const W8a32DirectBuf<MR, R, U> &b, float (&acc)[R][MR], int used) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
         if (u >= used) break;
@@ -227,45 +230,56 @@ __device__ __forceinline__ void w8a32_row1_multiply(const W8a32Row1Buf<R, U> &b,
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const int word = b.w[r][u][q];
-                float s = acc[r];
-                s = __builtin_fmaf(b.x[u][q].x, (float)(signed char)(word & 0xff), s);
-                s = __builtin_fmaf(b.x[u][q].y, (float)(signed char)((word >> 8) & 0xff), s);
-                s = __builtin_fmaf(b.x[u][q].z, (float)(signed char)((word >> 16) & 0xff), s);
-                s = __builtin_fmaf(b.x[u][q].w, (float)(signed char)((word >> 24) & 0xff), s);
-                acc[r] = s;
+                const float f0 = (float)(signed char)(word & 0xff), f1 = (float)(signed char)((word >> 8) & 0xff),
+                            f2 = (float)(signed char)((word >> 16) & 0xff), f3 = (float)(signed char)((word >> 24) & 0xff);
+#pragma unroll
+                for (int m = 0; m < MR; m++) {
+                    float s = acc[r][m];
+                    s = __builtin_fmaf(b.x[m][u][q].x, f0, s);
+                    s = __builtin_fmaf(b.x[m][u][q].y, f1, s);
+                    s = __builtin_fmaf(b.x[m][u][q].z, f2, s);
+                    s = __builtin_fmaf(b.x[m][u][q].w, f3, s);
+                    acc[r][m] = s;
+                }
             }
     }
 }
 
-template <int R, int U>
+template <int MR, int R, int U>
 __global__ void __launch_bounds__(256)
-k_w8a32_row1(const float *__restrict__ a, const int8_t *__restrict__ w, const float *__restrict__ w_scales,
-             float *__restrict__ out, int64_t N, int64_t K, int groups, int used) {
+k_w8a32_direct(const float *__restrict__ a, const int8_t *__restrict__ w, const float *__restrict__ w_scales,
+               float *__restrict__ out, int64_t N, int64_t K, int groups, int used) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t base = (int64_t)blockIdx.x * groups * (4 * R) + wave * R;
-    float acc[R];
+    float acc[R][MR];
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int m = 0; m < MR; m++) acc[r][m] = 0.0f;
     const int span = used * 1024;
     const int steps = (int)((K + span - 1) / span), total = groups * steps;
-    W8a32Row1Buf<R, U> ba, bb;
-    w8a32_row1_request<R, U>(ba, a, w, base, N, 0, lane, K, used);
+    W8a32DirectBuf<MR, R, U> ba, bb;
+    w8a32_direct_request<MR, R, U>(ba, a, w, base, N, 0, lane, K, used);
     int g = 0, it = 0;
-    auto finish = [&]() {                                       // the group's R sums: over the wave, scaled, stored
-        constexpr int NV = R;                                   // 1, 2 or 4
+    auto finish = [&]() {                                       // the group's R * MR sums: over the wave, scaled, stored
+        constexpr int NV = R * MR <= 1 ? 1 : R * MR <= 2 ? 2 : R * MR <= 4 ? 4 : R * MR <= 8 ? 8 : 16;
+        static_assert(R * MR <= 16, "sums per wave");
         float v[NV];
 #pragma unroll
-        for (int i = 0; i < NV; i++) v[i] = acc[i];
+        for (int i = 0; i < NV; i++) v[i] = i < R * MR ? acc[i / MR][i % MR] : 0.0f;
         wave_sum_spread(v, lane);
-        const int r = lane / (64 / NV);
+        const int idx = lane / (64 / NV), r = idx / MR, m = idx % MR;
         const int64_t n = base + (int64_t)g * (4 * R) + r;
-        if (lane % (64 / NV) == 0 && n < N) out[n] = v[0] * w_scales[n];
+        if (lane % (64 / NV) == 0 && idx < R * MR && n < N) out[m * N + n] = v[0] * w_scales[n];
 #pragma unroll
-        for (int i = 0; i < R; i++) acc[i] = 0.0f;
+        for (int rr = 0; rr < R; rr++)
+#pragma unroll
+            for (int mm = 0; mm < MR; mm++) acc[rr][mm] = 0.0f;
     };
-    auto next_request = [&](W8a32Row1Buf<R, U> &b) {            // operands of the step after (g, it)
+    auto next_request = [&](W8a32DirectBuf<MR, R, U> &b) {      // operands of the step after (g, it)
         const bool wrap = it + 1 == steps;
-        w8a32_row1_request<R, U>(b, a, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K, used);
+        w8a32_direct_request<MR, R, U>(b, a, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K,
+                                       used);
     };
     auto advance = [&]() {
         if (++it == steps) {
@@ -276,18 +290,18 @@ k_w8a32_row1(const float *__restrict__ a, const int8_t *__restrict__ w, const fl
     };
     for (int t = 0; t < total;) {
         if (t + 1 < total) next_request(bb);
-        w8a32_row1_multiply<R, U>(ba, acc, used);
+        w8a32_direct_multiply<MR, R, U>(ba, acc, used);
         advance();
         if (++t >= total) break;
         if (t + 1 < total) next_request(ba);
-        w8a32_row1_multiply<R, U>(bb, acc, used);
+        w8a32_direct_multiply<MR, R, U>(bb, acc, used);
         advance();
         ++t;
     }
 }
 
-template <int R, int U>
-int launch_row1(const float *a, const int8_t *w, const float *s, float *out, int64_t N, int64_t K) {
+template <int MR, int R, int U>
+int launch_direct(const float *a, const int8_t *w, const float *s, float *out, int64_t N, int64_t K) {
     const int64_t windows = (K + 1023) / 1024;
     int used = U;
     while (used > 1 && used / 2 >= windows) used /= 2;
@@ -295,7 +309,7 @@ int launch_row1(const float *a, const int8_t *w, const float *s, float *out, int
     if (groups < 1) groups = 1;
     if (groups > 64) groups = 64;
     const int64_t rows_per_block = 4 * R * groups, blocks = (N + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL((k_w8a32_row1<R, U>), dim3((unsigned)blocks), dim3(256), 0, kStream, a, w, s, out, N, K, (int)groups, used);
+    hipLaunchKernelGGL((k_w8a32_direct<MR, R, U>), dim3((unsigned)blocks), dim3(256), 0, kStream, a, w, s, out, N, K, (int)groups, used);
     return check_launch("qgemm_w8a32_gemv");
 }
 
@@ -341,10 +355,19 @@ int launch_gemv(const float *a, const int8_t *w, const float *s, float *out, int
     if constexpr (MR == 1) {
         // rows per wave x windows per request, by sweep (cached / weights from HBM, us): 32000 x 4096 on 4 x 1 22.7 / 28.0
         // (2 x 2: 30.0 / 39.6), 8192 x 8192 13.2 / 15.9, 4096 x 4096 on 2 x 4 4.6 / 5.9 (4 x 2: 4.8 / 8.0), 4096 x 11008 11.9 / 15.2
-        if (N >= 32 * cus) return launch_row1<4, 1>(a, w, s, out, N, K);
-        if (N >= 16 * cus) return launch_row1<2, 4>(a, w, s, out, N, K);
-        if (N >= 8 * cus) return launch_row1<2, 2>(a, w, s, out, N, K);
-        return launch_row1<1, 2>(a, w, s, out, N, K);
+        if (N >= 32 * cus) return launch_direct<1, 4, 1>(a, w, s, out, N, K);
+        if (N >= 16 * cus) return launch_direct<1, 2, 4>(a, w, s, out, N, K);
+        if (N >= 8 * cus) return launch_direct<1, 2, 2>(a, w, s, out, N, K);
+        return launch_direct<1, 1, 2>(a, w, s, out, N, K);
+    }
+    if constexpr (MR >= 2 && MR <= 4) {
+        // up to four rows the same form without LDS is level or ahead below N = 16384 (cached / from HBM, M = 4:
+        // 11008 x 4096 23.3 / 25.0 -> 19.2 / 20.8 us, 4096 x 11008 31.1 / 34.2 -> 23.5 / 25.4, 4096 x 4096 9.0 / 11.3 ->
+        // 9.0 / 10.3); beyond, the staged form keeps the lead (32000 x 4096: 46.0 / 51.1 against 51.1 / 56.2)
+        if (N < 64 * cus) {
+            if (MR == 2 && N < 32 * cus) return launch_direct<MR, 2, 1>(a, w, s, out, N, K);
+            return launch_direct<MR, 4, 1>(a, w, s, out, N, K);
+        }
     }
     if (N >= 64 * cus) return launch_rows<MR, 4>(a, w, s, out, N, K);
     if (N >= 16 * cus) return launch_rows<MR, 2>(a, w, s, out, N, K);
