@@ -549,7 +549,7 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
                  int64_t K, float x_scale, const float *__restrict__ w_scales,
                  const float *__restrict__ bias, float *__restrict__ out,
                  int32_t *__restrict__ acc_out, int64_t ldc, int splits, int32_t *partials,
-                 int *__restrict__ counters) {
+                 int *__restrict__ counters, int phases) {
     constexpr int NWO = WAVES_M * WAVES_N, NW = NWO * WAVES_K, BKB = 128;      // waves that own outputs / all waves
     constexpr int KSTEPS = 4 / WAVES_K;                                        // k-steps of a slab per wave
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
@@ -605,7 +605,13 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         vw[j] = (unsigned)((row < nrows ? row : nrows - 1) * K + (((lane & 7) ^ ((row >> 1) & 7)) << 4));
         tw[j] = (((lane & 7) ^ ((row >> 1) & 7)) << 4) < ktail;
     }
-    const int8_t *gx = X + m0 * K + (int64_t)slab0 * BKB, *gw = W + n0 * K + (int64_t)slab0 * BKB;
+    // phases > 1 (K on the slab grid): the workgroups that share a block of W rows (same tn) or of X rows (same
+    // tm) start their walk over K at different slabs and wrap around, so they miss on different lines at any
+    // moment and find the others' lines in L2 later.  Integer sums are exact in any order.
+    int first = 0;
+    if (phases > 1 && slabs >= phases) first = ((tm * 7 + tn * 3) % phases) * (slabs / phases);
+    int wrap_in = slabs - first;                                               // slabs to request before the walk wraps to this range's start
+    const int8_t *gx = X + m0 * K + (int64_t)(slab0 + first) * BKB, *gw = W + n0 * K + (int64_t)(slab0 + first) * BKB;
     const unsigned lds0 = (unsigned)(uintptr_t)lds, lds_w = lds0 + wave * 1024;
 
     const int frow = lane & 31, fhalf = lane >> 5;
@@ -659,6 +665,10 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         }                                                                                        \
         gx += BKB;                                                                               \
         gw += BKB;                                                                               \
+        if (--wrap_in == 0) {                                                                    \
+            gx -= (int64_t)slabs * BKB;                                                          \
+            gw -= (int64_t)slabs * BKB;                                                          \
+        }                                                                                        \
     } while (0)
 // a stage: SPB slabs into consecutive slab places
 #define AXI8G_ISSUE(ST)                                                                          \
@@ -885,7 +895,7 @@ int launch_dma(const char *name, const char *split_name, const int8_t *x, float 
                int64_t K, int64_t ldc) {
     constexpr int smem = NST * SPB * (BM + BN) * 128 + 2 * BN * 4 + 16;      // stages, scale and bias rows, the split join's flag
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
-                           const float *, float *, int32_t *, int64_t, int, int32_t *, int *);
+                           const float *, float *, int32_t *, int64_t, int, int32_t *, int *, int);
     static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE, WAVES_K, SPB>,
                                     k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU, EDGE, WAVES_K, SPB>,
                                     k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE, WAVES_K, SPB>};
@@ -907,9 +917,16 @@ int launch_dma(const char *name, const char *split_name, const int8_t *x, float 
         counters = strip_counters((size_t)tiles);
         if (!partials || !counters) return AXHIP_ERR_ALLOC;
     }
+    // Staggered walks over K (kernel comment) pay when the weights come from HBM: a CU sustains only about 31 GB/s
+    // of misses, so workgroups that miss on the same lines together divide the rate at which new bytes arrive
+    // (M = 256, N = K = 4096, weights in rotation: 13.0 -> 10.8 us; the same weights cached: 8.5 -> 8.7).  They need
+    // an XCD's share of the operands to stay in its 4 MiB of L2 until the last sharer has passed, or every line
+    // is fetched once per sharer (512 x 4096 x 11008: 31.6 -> 52.2 us): one round of tiles, all of X and an eighth
+    // of W within 3 MiB.
+    const int phases = (K % 128 == 0 && tiles <= cu_count() && (M + N / 8) * K <= (int64_t(3) << 20)) ? 4 : 0;
     note_kernel(splits > 1 ? split_name : name);
     hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles, (unsigned)splits), dim3(WAVES_M * WAVES_N * WAVES_K * 64), smem, kStream,
-                       x, w, M, N, K, x_scale, w_scales, bias, out, acc_out, ldc, splits, partials, counters);
+                       x, w, M, N, K, x_scale, w_scales, bias, out, acc_out, ldc, splits, partials, counters, phases);
     return check_launch(name);
 }
 
