@@ -513,13 +513,19 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         }                                                                                        \
     } while (0)
 
+// int8 B: the four conversions of a k-block come first, so that its products issue back to back (a conversion
+// between two products that add into the same accumulator costs the pair its hand-over)
 #define AXF_MFMAS(BUF)                                                                           \
     do {                                                                                         \
         __builtin_amdgcn_sched_barrier(0);                                                       \
+        float bq[TN][4];                                                                         \
+        _Pragma("unroll") for (int j = 0; j < TN; j++)                                           \
+            _Pragma("unroll") for (int e = 0; e < 4; e++) bq[j][e] = fb[BUF][j].get(e);          \
+        if constexpr (B_I8) __builtin_amdgcn_sched_barrier(0);                                   \
         _Pragma("unroll") for (int e = 0; e < 4; e++)                                            \
             _Pragma("unroll") for (int i = 0; i < TM; i++)                                       \
                 _Pragma("unroll") for (int j = 0; j < TN; j++)                                   \
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[BUF][j].get(e),          \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bq[j][e],                   \
                                                                      fa[BUF][i].get(e), acc[i][j], 0, 0, 0); \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     } while (0)
