@@ -34,6 +34,8 @@ INT8_SHAPES = [(1, 1, 1), (3, 17, 45), (5, 7, 16), (64, 64, 128), (100, 200, 300
                # M <= 4 with whole 16-byte steps of K: the wave-per-rows dot-product route (and M = 5..8, on the tiles since)
                (1, 768, 3072), (1, 4096, 4096), (8, 768, 768), (3, 5, 16), (7, 1001, 1040), (2, 3, 4112),
                (4, 33, 64), (5, 9, 48), (6, 130, 256), (4, 11008, 512), (3, 4100, 2064),
+               # staggered walks over K: a start slab that is odd with two slabs per stage, and with the K split
+               (256, 4096, 1536), (128, 2048, 2560),
                # off the 256 grid with a large interior: persistent kernel inside, smaller tiles on the fringes
                (2112, 4128, 256), (4100, 2304, 128), (2048, 4100, 128),
                # rows that start at odd byte offsets (K % 16 != 0)
