@@ -322,10 +322,10 @@ struct DmaOperand {
 
 // An int8 operand stored [rows, K] (K contiguous; the weights of the W8A32 product): a slab is 32 bytes
 // per row, one load instruction carries 32 rows (lane l -> row l >> 1, 16-byte half l & 1), and only the
-// first NINSTR waves have one to issue.  A fragment is one ds_read_b32 — the four k values a lane feeds
-// to the four MFMAs of a k-block — converted to fp32 in registers right before use, so LDS and the
-// loads carry a quarter of the bytes of an fp32 operand.  (Rows 32 bytes apart put the 32 lanes of a
-// read on 8 banks: a 4-way conflict on a read that is a quarter of the other operand's.)
+// first NINSTR waves have one to issue.  A fragment is one ds_read_b32 — a lane's four k values of a
+// k-block — converted to bf16 in registers right before use (bf16_of_i8 below), so LDS and the loads
+// carry a quarter of the bytes of an fp32 operand.  (Rows 32 bytes apart put the 32 lanes of a read on
+// 8 banks: a 4-way conflict on a read that is a quarter of the other operand's.)
 template <int R, int NW>
 struct DmaOperandI8 {
     static constexpr int PITCH = 1024;
@@ -346,8 +346,53 @@ struct DmaOperandI8 {
 
 struct FragI8 {
     int raw;       // k = 4 * (lane >> 5) + e of the k-block in byte e
-    __device__ __forceinline__ float get(int e) const { return (float)(signed char)(raw >> (8 * e)); }
+    __device__ __forceinline__ float get(int e) const { return (float)(signed char)(raw >> (8 * e)); }   // fp32 form, unused by the bf16 products
 };
+
+// fp32 x int8 products on the bf16 matrix core, with fp32 accuracy.  Every int8 value is a bf16 exactly.  An fp32
+// value a is cut into three bf16 terms: hi = a with its low 16 bits cleared, mid = (a - hi) with its low 16 bits
+// cleared, lo = a - hi - mid; both subtractions are exact and lo has at most 8 significant bits, so
+// a = hi + mid + lo exactly, every term times an int8 value is exact in fp32, and only the accumulation rounds —
+// as in the fp32 product, at a sixteenth of its matrix-core time per term.  An infinite a keeps hi = a and
+// mid = lo = 0 (a - hi would be NaN), so infinities and NaNs come out as the fp32 product gives them.
+// Cost per fp32 value: and, subtract, median (the NaN filter), and, subtract, and half of each of three packs:
+// 6.5 vector instructions; per int8 value one conversion and half a pack.
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+struct Bf16x3 {
+    v4i hi, mid, lo;     // 8 k values each: a k-block's four, then the next k-block's four
+};
+__device__ __forceinline__ unsigned top_halves(unsigned second, unsigned first) {   // bf16 of two fp32, by truncation
+    return __builtin_amdgcn_perm(second, first, 0x07060302);
+}
+__device__ __forceinline__ Bf16x3 bf16x3_of(const v4f &p, const v4f &q) {
+    unsigned h[8], m[8], l[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float a = e < 4 ? p[e] : q[e - 4];
+        h[e] = __float_as_uint(a);
+        float r = a - __uint_as_float(h[e] & 0xffff0000u);
+        r = __builtin_amdgcn_fmed3f(r, r, 0.0f);     // NaN (a infinite or NaN) -> 0, anything else unchanged
+        m[e] = __float_as_uint(r);
+        l[e] = __float_as_uint(r - __uint_as_float(m[e] & 0xffff0000u));
+    }
+    Bf16x3 o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        o.hi[e] = (int)top_halves(h[2 * e + 1], h[2 * e]);
+        o.mid[e] = (int)top_halves(m[2 * e + 1], m[2 * e]);
+        o.lo[e] = (int)top_halves(l[2 * e + 1], l[2 * e]);
+    }
+    return o;
+}
+__device__ __forceinline__ v4i bf16_of_i8(int first, int second) {   // two k-blocks of four int8 -> 8 bf16
+    unsigned f[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) f[e] = __float_as_uint((float)(signed char)((e < 4 ? first : second) >> (8 * (e & 3))));
+    v4i o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) o[e] = (int)top_halves(f[2 * e + 1], f[2 * e]);
+    return o;
+}
 
 template <bool KC> struct Frag;
 template <> struct Frag<true> {
@@ -378,14 +423,17 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     static_assert(WAVES_K == 1 || WAVES_K == 2, "k split");
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
     constexpr bool B_I8 = sizeof(BSRC) == 1;     // int8 B, [N, K]: W8A32 (K a multiple of 32, so no K tail)
-    static_assert(!B_I8 || (B_KC && NST == 2 && EPI == 1), "int8 B is K-contiguous, two stages, turned write-back");
+    static_assert(!B_I8 || (B_KC && EPI == 1), "int8 B is K-contiguous, turned write-back");
     using OA = DmaOperand<BM, A_KC, NW>;
     using OB = typename std::conditional<B_I8, DmaOperandI8<BN, NW>, DmaOperand<BN, B_KC, NW>>::type;
     // LDS: NST stages of A, then NST stages of B
     constexpr int B_BASE = NST * OA::BYTES;
     constexpr int NREADS = TM * OA::READS + TN * OB::READS;
     // loads a wave may leave in flight at the end of a slab: everything but the next slab's
-    constexpr int VM_KEEP = (NST - 2) * (OA::IPW + OB::IPW);
+    // int8 B with four stages: the fragments of slab s + 1 are read while slab s is converted and multiplied, so the
+    // loop's barrier must already cover slab s + 2 and one stage less is in flight
+    constexpr bool PIPE = B_I8 && NST == 4;
+    constexpr int VM_KEEP = (NST - (PIPE ? 3 : 2)) * (OA::IPW + OB::IPW);
     static_assert(NST >= 2 && NST <= 4 && VM_KEEP < 64, "stage count");
     static_assert(B_BASE + NST * OB::BYTES <= 160 * 1024, "LDS budget");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -457,8 +505,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    Frag<A_KC> fa[2][TM];
-    typename std::conditional<B_I8, FragI8, Frag<B_KC>>::type fb[2][TN];
+    Frag<A_KC> fa[PIPE ? 8 : B_I8 ? 4 : 2][TM];
+    typename std::conditional<B_I8, FragI8, Frag<B_KC>>::type fb[PIPE ? 8 : B_I8 ? 4 : 2][TN];
 
 // loads of the next unread slab into stage ST
 #define AXF_ISSUE(ST)                                                                            \
@@ -513,42 +561,89 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         }                                                                                        \
     } while (0)
 
-// int8 B: the four conversions of a k-block come first, so that its products issue back to back (a conversion
-// between two products that add into the same accumulator costs the pair its hand-over)
 #define AXF_MFMAS(BUF)                                                                           \
     do {                                                                                         \
         __builtin_amdgcn_sched_barrier(0);                                                       \
-        float bq[TN][4];                                                                         \
-        _Pragma("unroll") for (int j = 0; j < TN; j++)                                           \
-            _Pragma("unroll") for (int e = 0; e < 4; e++) bq[j][e] = fb[BUF][j].get(e);          \
-        if constexpr (B_I8) __builtin_amdgcn_sched_barrier(0);                                   \
         _Pragma("unroll") for (int e = 0; e < 4; e++)                                            \
             _Pragma("unroll") for (int i = 0; i < TM; i++)                                       \
                 _Pragma("unroll") for (int j = 0; j < TN; j++)                                   \
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bq[j][e],                   \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[BUF][j].get(e),          \
                                                                      fa[BUF][i].get(e), acc[i][j], 0, 0, 0); \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     } while (0)
 
+// int8 B: the k-blocks in fragment buffers B0 and B1 (16 k values) as three bf16 products per 32x32 tile.  All
+// conversions come first, so that the products issue back to back (a conversion between two products that add
+// into the same accumulator costs the pair its hand-over); the small terms are added first.
+#define AXF_PAIR(B0, B1)                                                                         \
+    do {                                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+        Bf16x3 ax[TM];                                                                           \
+        v4i bx[TN];                                                                              \
+        _Pragma("unroll") for (int i = 0; i < TM; i++) ax[i] = bf16x3_of(fa[B0][i].q, fa[B1][i].q); \
+        _Pragma("unroll") for (int j = 0; j < TN; j++) bx[j] = bf16_of_i8(fb[B0][j].raw, fb[B1][j].raw); \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+        _Pragma("unroll") for (int t = 0; t < 3; t++)                                            \
+            _Pragma("unroll") for (int i = 0; i < TM; i++)                                       \
+                _Pragma("unroll") for (int j = 0; j < TN; j++)                                   \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                         \
+                        __builtin_bit_cast(v8bf, bx[j]),                                         \
+                        __builtin_bit_cast(v8bf, t == 0 ? ax[i].lo : t == 1 ? ax[i].mid : ax[i].hi), acc[i][j], 0, 0, 0); \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    } while (0)
+
 // one slab out of stage ST; `more`: slab s+NST-1 exists and is fetched into the stage read last
-#define AXF_SLAB(ST, more)                                                                       \
+#define AXF_SLAB(ST, more, next)                                                                 \
     do {                                                                                         \
         if (more) AXF_ISSUE(((ST) + NST - 1) % NST);                                             \
-        AXF_FRAGS(0, ST, 0);                                                                     \
-        AXF_FRAGS(1, ST, 1);                                                                     \
-        AXF_LGKM(NREADS);                                                                        \
-        AXF_MFMAS(0);                                                                            \
-        if constexpr (WAVES_K == 1) {                                                            \
-            AXF_FRAGS(0, ST, 2);                                                                 \
-            AXF_LGKM(NREADS);                                                                    \
-            AXF_MFMAS(1);                                                                        \
-            AXF_FRAGS(1, ST, 3);                                                                 \
+        if constexpr (PIPE) {                                                                    \
+            /* this slab's fragments are in buffers 4 (ST & 1) ..., read a slab ago */            \
+            constexpr int C0 = 4 * ((ST) & 1), N0 = 4 - C0, NS = ((ST) + 1) % NST;               \
+            if (next) {                                                                          \
+                AXF_FRAGS(N0, NS, 0);                                                            \
+                AXF_FRAGS(N0 + 1, NS, 1);                                                        \
+                if constexpr (WAVES_K == 1) {                                                    \
+                    AXF_FRAGS(N0 + 2, NS, 2);                                                    \
+                    AXF_FRAGS(N0 + 3, NS, 3);                                                    \
+                }                                                                                \
+                AXF_LGKM((WAVES_K == 1 ? 4 : 2) * NREADS);                                       \
+            } else AXF_LGKM(0);                                                                  \
+            AXF_PAIR(C0, C0 + 1);                                                                \
+            if constexpr (WAVES_K == 1) AXF_PAIR(C0 + 2, C0 + 3);                                \
+        } else if constexpr (B_I8) {                                                             \
+            AXF_FRAGS(0, ST, 0);                                                                 \
+            AXF_FRAGS(1, ST, 1);                                                                 \
+            if constexpr (WAVES_K == 1) {                                                        \
+                AXF_FRAGS(2, ST, 2);                                                             \
+                AXF_FRAGS(3, ST, 3);                                                             \
+                AXF_LGKM(2 * NREADS);                                                            \
+                AXF_PAIR(0, 1);                                                                  \
+                AXF_LGKM(0);                                                                     \
+                AXF_PAIR(2, 3);                                                                  \
+            } else {                                                                             \
+                AXF_LGKM(0);                                                                     \
+                AXF_PAIR(0, 1);                                                                  \
+            }                                                                                    \
+        } else {                                                                                 \
+            AXF_FRAGS(0, ST, 0);                                                                 \
+            AXF_FRAGS(1, ST, 1);                                                                 \
             AXF_LGKM(NREADS);                                                                    \
             AXF_MFMAS(0);                                                                        \
+            if constexpr (WAVES_K == 1) {                                                        \
+                AXF_FRAGS(0, ST, 2);                                                             \
+                AXF_LGKM(NREADS);                                                                \
+                AXF_MFMAS(1);                                                                    \
+                AXF_FRAGS(1, ST, 3);                                                             \
+                AXF_LGKM(NREADS);                                                                \
+                AXF_MFMAS(0);                                                                    \
+            }                                                                                    \
+            AXF_LGKM(0);                                                                         \
+            AXF_MFMAS(1);                                                                        \
         }                                                                                        \
-        AXF_LGKM(0);                                                                             \
-        AXF_MFMAS(1);                                                                            \
-        if (VM_KEEP > 0 && (more)) AXF_VM(VM_KEEP); else AXF_VM(0);                              \
+        if (VM_KEEP > 0 && (more)) {                                                             \
+            /* a wave past the int8 operand's load instructions has only A's in flight */        \
+            if (B_I8 && wave >= OB::NINSTR) AXF_VM((NST - (PIPE ? 3 : 2)) * OA::IPW); else AXF_VM(VM_KEEP); \
+        } else AXF_VM(0);                                                                        \
         __builtin_amdgcn_s_barrier();                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     } while (0)
@@ -563,41 +658,58 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     AXF_VM(0);
     if constexpr (EDGE) AXF_LGKM(0);             // zeros written for a K tail that is already in the first slabs
     __builtin_amdgcn_s_barrier();
+    if constexpr (PIPE) {
+        AXF_FRAGS(0, 0, 0);
+        AXF_FRAGS(1, 0, 1);
+        if constexpr (WAVES_K == 1) {
+            AXF_FRAGS(2, 0, 2);
+            AXF_FRAGS(3, 0, 3);
+        }
+    }
     // whole rounds of the ring in a loop with one way out, then the slabs % NST that remain (nothing is
     // left to fetch by then): an exit between two slabs of the loop body makes the compiler copy the
     // accumulators from one register set to another every round
     int s = 0;
     for (; s + NST <= slabs; s += NST) {
-        AXF_SLAB(0, ring && s + NST - 1 < slabs);
-        AXF_SLAB(1, s + NST < slabs);
-        if constexpr (NST > 2) AXF_SLAB(2, s + NST + 1 < slabs);
-        if constexpr (NST > 3) AXF_SLAB(3, s + NST + 2 < slabs);
+        AXF_SLAB(0, ring && s + NST - 1 < slabs, s + 1 < slabs);
+        AXF_SLAB(1, s + NST < slabs, s + 2 < slabs);
+        if constexpr (NST > 2) AXF_SLAB(2, s + NST + 1 < slabs, s + 3 < slabs);
+        if constexpr (NST > 3) AXF_SLAB(3, s + NST + 2 < slabs, s + 4 < slabs);
     }
-    if (s < slabs) AXF_SLAB(0, false);
-    if (s + 1 < slabs) AXF_SLAB(1, false);
-    if constexpr (NST > 3) { if (s + 2 < slabs) AXF_SLAB(2, false); }
+    if (s < slabs) AXF_SLAB(0, false, s + 1 < slabs);
+    if (s + 1 < slabs) AXF_SLAB(1, false, s + 2 < slabs);
+    if constexpr (NST > 3) { if (s + 2 < slabs) AXF_SLAB(2, false, false); }
 #undef AXF_ISSUE
 #undef AXF_FRAGS
 #undef AXF_MFMAS
+#undef AXF_PAIR
 #undef AXF_SLAB
 
     if constexpr (WAVES_K == 2) {
-        static_assert(TM == 1 && TN == 1, "the k split is for one 32x32 tile per wave");
-        float *sum = reinterpret_cast<float *>(lds_raw + wmn * 4096);   // the stages are dead now
+        // 4 KiB per 32x32 sub-tile, a wave's sub-tiles side by side (the stages are dead now)
+        float *sum = reinterpret_cast<float *>(lds_raw + wmn * (TM * TN * 4096));
         if (wk == 1) {
 #pragma unroll
-            for (int q = 0; q < 4; q++)
-                *reinterpret_cast<v4f *>(sum + (q * 64 + lane) * 4) =
-                    v4f{acc[0][0][4 * q], acc[0][0][4 * q + 1], acc[0][0][4 * q + 2], acc[0][0][4 * q + 3]};
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        *reinterpret_cast<v4f *>(sum + (i * TN + j) * 1024 + (q * 64 + lane) * 4) =
+                            v4f{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
         }
         __syncthreads();
         if (wk == 1) return;
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const v4f t = *reinterpret_cast<const v4f *>(sum + (q * 64 + lane) * 4);
+        for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) acc[0][0][4 * q + e] += t[e];
-        }
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const v4f t = *reinterpret_cast<const v4f *>(sum + (i * TN + j) * 1024 + (q * 64 + lane) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[i][j][4 * q + e] += t[e];
+                }
     }
 
     // register v of lane l: m = i*32 + (l&31), n = j*32 + 8*(v>>2) + 4*(l>>5) + (v&3)
@@ -632,7 +744,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         // contiguous bytes instead of 32 rows of 32.  Rows of 128 bytes, 16-byte chunk c of row
         // r kept at chunk c ^ ((r>>1)&7): both the write (16 rows, one chunk column) and the
         // read (2 rows, all chunks) of a 16-lane group then touch every bank once.
-        unsigned char *turn = lds_raw + wmn * 4096;
+        unsigned char *turn = lds_raw + wmn * (WAVES_K == 2 ? TM * TN * 4096 : 4096);   // inside the wave's own join area
         const int rrow = lane >> 3, rchunk = lane & 7;
         const int64_t col0 = n0 + wn * WTN + 4 * rchunk;
         float *dst = C + (m0 + wm * WTM + rrow) * g.ldc + col0;
@@ -691,7 +803,8 @@ int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
     using OB = typename std::conditional<sizeof(BSRC) == 1, DmaOperandI8<BN, NW>, DmaOperand<BN, B_KC, NW>>::type;
     constexpr int stage_bytes = NST * (DmaOperand<BM, A_KC, NW>::BYTES + OB::BYTES);
     // the write-back turns 4 KiB per output wave through the dead stages
-    constexpr int smem = stage_bytes > WAVES_M * WAVES_N * 4096 ? stage_bytes : WAVES_M * WAVES_N * 4096;
+    constexpr int after = WAVES_K == 2 ? BM * BN * 4 : WAVES_M * WAVES_N * 4096;   // the join of a k split needs the whole tile
+    constexpr int smem = stage_bytes > after ? stage_bytes : after;
     static bool attr_set = false;
     if (!attr_set) {
         AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -1208,7 +1321,9 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
 }
 
 // The same fast path with int8 weights as the B operand (W8A32: A fp32 [M,K], B int8 [N,K], the
-// per-column scale applied in the write-back).  K must be a multiple of 32 (whole slabs, rows of B on
+// per-column scale applied in the write-back).  The products run on the bf16 matrix core: three exact
+// bf16 terms per fp32 activation (Bf16x3), the int8 weight as one bf16, v_mfma_f32_32x32x16_bf16 with
+// fp32 accumulation — 3/16 of the matrix-core time of the fp32 product at the same accuracy.  K must be a multiple of 32 (whole slabs, rows of B on
 // 16-byte boundaries); M and N may be off the tile grid.  Returns -1 when the shape does not qualify.
 const char *const kI8DmaNames[3] = {"qgemm_w8a32_mfma_128x128_dma", "qgemm_w8a32_mfma_64x64_dma", "qgemm_w8a32_mfma_64x64k2_dma"};
 int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
@@ -1229,8 +1344,22 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
     }
     if (g.K > 128) {
         const int64_t big = (g.M / 128) * (g.N / 128) * batch, cus = cu_count(), rounds = (big + cus - 1) / cus;
+        // The conversions to bf16 run on the vector pipe beside the products, and that pipe needs two waves on a SIMD
+        // to stay busy: take the largest tile that still gives every CU two workgroups (or one of eight waves).  A wave
+        // converts its own rows of A (6.5 instructions a value) and every column of B it multiplies them with (1.5), so
+        // its tile is one 32-row block high and as wide as the tile allows.  (M, N, K, us before -> after:
+        // 4096^3 517 -> 353, 2048 x 4096 x 4096 266 -> 203, 1024 x 4096 x 4096 153 -> 106, 512 x 11008 x 4096 214 -> 153,
+        // 512 x 4096 x 4096 84 -> 65, 2048 x 1024 x 4096 85 -> 62, 256 x 4096 x 4096 54 -> 46, 1024^3 16.1 -> 14.4.)
+        if (tuning().f32_tile == 0) {
+            auto enough = [&](int64_t bm, int64_t bn) { return g.M % bm == 0 && g.N % bn == 0 && (g.M / bm) * (g.N / bn) * batch >= 2 * cus; };
+            if (enough(128, 256)) return launch_dma<128, 256, 4, 1, 2, true, true, 1, 1, false, int8_t>("qgemm_w8a32_mfma_128x256_dma", g, batch);
+            if (enough(128, 128)) return launch_dma<128, 128, 4, 1, 3, true, true, 1, 1, false, int8_t>(names[0], g, batch);
+            if (enough(64, 128)) return launch_dma<64, 128, 2, 1, 2, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_64x128k2_dma", g, batch);
+            if (enough(32, 128)) return launch_dma<32, 128, 1, 2, 4, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x128k2_dma", g, batch);
+            if (enough(32, 64)) return launch_dma<32, 64, 1, 2, 4, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
+        }
         if (g.M % 128 == 0 && g.N % 128 == 0 && big >= cus && big * 10 >= rounds * cus * 9)
-            return launch_dma<128, 128, 2, 4, 2, true, true, 1, 1, false, int8_t>(names[0], g, batch);
+            return launch_dma<128, 128, 4, 1, 3, true, true, 1, 1, false, int8_t>(names[0], g, batch);
         // the last round of one 64x64 tile per CU mostly empty: 32x64 tiles, as for fp32 operands
         const int64_t whole = (g.M / 64) * (g.N / 64) * batch, rounds_whole = (whole + cus - 1) / cus,
                       rounds_half = (2 * whole + cus - 1) / cus;
@@ -1500,7 +1629,8 @@ int run_f32(const SgemmArgs &g, int transa, int transb) {
 }  // namespace
 
 namespace axhip {
-// W8A32 through the matrix cores: B is int8 [N,K], converted to fp32 while it is staged.
+// W8A32 through the matrix cores: B is int8 [N,K].  The direct-to-LDS tiles multiply on the bf16 matrix core
+// (try_dma_i8); shapes they do not take (K off the 32 grid, unaligned rows) convert B to fp32 while it is staged.
 int sgemm_i8w(int64_t M, int64_t N, int64_t K, const float *a, const int8_t *w,
               const float *w_scales, float *out) {
     static const char *const names[3] = {"qgemm_w8a32_mfma_128x128", "qgemm_w8a32_mfma_64x64",

@@ -708,6 +708,80 @@ def test_w8a32_against_oracle(hip, oracle, golden, M, N, K):
     assert diff.max() <= REL_FP32 * max(np.abs(ref).max(), 1e-30)
 
 
+W8A32_TILE_FORMS = [(2048, 8192, 160, "qgemm_w8a32_mfma_128x256_dma"), (2048, 4096, 192, "qgemm_w8a32_mfma_128x128_dma"),
+                    (1024, 4096, 224, "qgemm_w8a32_mfma_64x128k2_dma"), (512, 4096, 288, "qgemm_w8a32_mfma_32x128k2_dma"),
+                    (256, 4096, 160, "qgemm_w8a32_mfma_32x64k2_dma"), (256, 4096, 256, "qgemm_w8a32_mfma_32x64k2_dma"),
+                    (512, 4096, 1056, "qgemm_w8a32_mfma_32x128k2_dma")]
+
+
+@pytest.mark.parametrize("M,N,K,form", W8A32_TILE_FORMS)
+def test_w8a32_tile_forms(hip, M, N, K, form):
+    """The tile forms of the W8A32 product for many output tiles (fp32 activations cut into three bf16 terms, int8 weights
+    as bf16, products on the bf16 matrix core): each obeys the fp64 bound of a correct fp32 accumulation, with slab counts
+    that end the four-stage ring at every position."""
+    say("w8a32 tiles", M, N, K)
+    rng = np.random.default_rng(M + N + K)
+    a = (rng.uniform(-1, 1, (M, K)) * 10.0 ** rng.integers(-3, 4, (M, 1))).astype(np.float32)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    ws = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    got = hip.qgemm_w8a32(hip.array(a), hip.array(w), hip.array(ws)).numpy()
+    assert hip.last_kernel() == form
+    want = (a.astype(np.float64) @ w.astype(np.float64).T) * ws
+    bound = BOUND_FP32 * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64).T) * ws + 1e-30
+    assert (np.abs(got - want) <= bound).all(), float((np.abs(got - want) / bound).max())
+
+
+def test_w8a32_three_bf16_terms_are_exact(hip, oracle):
+    """Activations whose 24 significant bits are all in use, against weight rows with one non-zero: every output is a
+    single product.  With a power of two as the weight the product is exact, so any bit the three-term split lost would
+    show; with 3 or 127 the three exact partial products are rounded as they are added, within one unit in the last place."""
+    M, N, K = 64, 128, 256
+    rng = np.random.default_rng(5)
+    a = rng.uniform(1, 2, (M, K)).astype(np.float32)
+    a = np.nextafter(a, np.float32(3)) * rng.choice([-1, 1], (M, K)).astype(np.float32) * (2.0 ** rng.integers(-60, 60, (M, K))).astype(np.float32)
+    w = np.zeros((N, K), np.int8)
+    cols = rng.integers(0, K, N)
+    vals = rng.choice([1, -1, 2, -64, 127, -128, 3], N)
+    w[np.arange(N), cols] = vals
+    s = np.ones(N, np.float32)
+    got = hip.qgemm_w8a32(hip.array(a), hip.array(w), hip.array(s)).numpy()
+    say("  ", hip.last_kernel())
+    assert hip.last_kernel().startswith("qgemm_w8a32_mfma")
+    want = a[:, cols].astype(np.float64) * vals
+    pow2 = np.isin(vals, [1, -1, 2, -64, -128])
+    assert np.array_equal(got[:, pow2].astype(np.float64), want[:, pow2])
+    assert (np.abs(got - want) <= np.abs(want) * 2.0 ** -23).all()
+
+
+def test_w8a32_non_finite_activations(hip, oracle):
+    """Infinities and NaNs among the activations come out as the reference's fp32 sum gives them (src/core/quantize.c:117-170, a plain fused multiply-add chain):
+    +-inf where one sign of infinity meets non-zero weights, NaN where both signs meet, an infinity meets a zero weight,
+    or a NaN is present; rows without them stay finite."""
+    M, N, K = 40, 192, 320
+    rng = np.random.default_rng(11)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    w[:, 7] = np.where(np.arange(N) % 3 == 0, 0, w[:, 7])           # zero weights under an infinity
+    a[1, 7] = np.inf
+    a[2, 7], a[2, 100] = np.inf, -np.inf
+    a[3, 200] = np.nan
+    a[4, 7] = -np.inf
+    a[5, 300] = np.float32(3.0e38)                                    # finite, overflows in the product
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    for rows in (M, 6):                                               # matrix-core form, weight-streaming form
+        x = a[1:1 + rows] if rows == 6 else a
+        got = hip.qgemm_w8a32(hip.array(x), hip.array(w), hip.array(s)).numpy()
+        say("  ", hip.last_kernel())
+        with np.errstate(all="ignore"):
+            ref = oracle.qgemm_w8a32(x, w, s)
+        assert np.array_equal(np.isnan(got), np.isnan(ref))
+        assert np.array_equal(np.isinf(got), np.isinf(ref))
+        inf = np.isinf(ref)
+        assert np.array_equal(np.sign(got[inf]), np.sign(ref[inf]))
+        fin = np.isfinite(ref)
+        assert np.abs(got[fin] - ref[fin]).max() <= REL_FP32 * np.abs(ref[fin]).max()
+
+
 def test_device_quantizer_bit_exact(hip, oracle, golden):
     for (N, K) in ((8, 8), (128, 128), (64, 1024), (5, 333)):
         w = xorshift32_unit(N * K, 42).reshape(N, K)
