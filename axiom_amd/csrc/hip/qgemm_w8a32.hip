@@ -382,10 +382,13 @@ extern "C" int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w
     if (!a || !w || !w_scales || !out) return fail(AXHIP_ERR_NULL_ARG, "qgemm_w8a32: NULL");
     if (M < 0 || N < 0 || K < 0) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a32: negative dimension");
     if (M == 0 || N == 0) return AXHIP_OK;
-    // The weight-streaming form pays M multiply-adds per weight byte on the vector ALU (4096 x 4096: 4.4 us at
-    // M = 1, +1.4 us per further row); from M = 7 on the matrix-core tiles are level or ahead (M = 8:
-    // 11008 x 4096 43.0 against 30.8 us, 4096 x 11008 52.8 against 31.2, 4096 x 4096 13.9 against 15.3).
-    if (M > 6) return axhip::sgemm_i8w(M, N, K, a, w, w_scales, out);
+    // The weight-streaming form pays M multiply-adds per weight byte on the vector ALU (4096 x 4096: 4.6 us at
+    // M = 1, +1.4 us per further row); from M = 7 on the matrix-core tiles are level or ahead everywhere, and with a
+    // long K already at M = 6, at M = 5 for large weights (us, streaming against tiles — M = 6: 4096 x 4096 11.7 / 11.5,
+    // 1024 x 4096 10.0 / 8.2, 768 x 3072 10.0 / 8.5, 11008 x 4096 35.0 / 21.9; M = 5: 11008 x 4096 31.2 / 21.9 but
+    // 4096 x 4096 10.5 / 11.5; with K = 768 or 1024 the streaming form stays ahead up to M = 6, 4.9-5.7 against 7.8-8.2).
+    const bool tiles_for_rows = K >= 2048 && K % 32 == 0 && (M == 6 || (M == 5 && N * K > (int64_t(1) << 24)));
+    if (M > 6 || tiles_for_rows) return axhip::sgemm_i8w(M, N, K, a, w, w_scales, out);
     if ((N + 3) / 4 > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a32: N too large");
     note_kernel("qgemm_w8a32_gemv");
     switch (M) {

@@ -179,6 +179,24 @@ def secondary(hip):
                                   "kernel": hip.last_kernel()}
     del a, b, c
 
+    # W8A32 with many rows (fp32 activations x int8 weights, fp32 accumulation): the tiles multiply on the bf16 matrix
+    # core with three exact bf16 terms per activation, so the same product takes a fraction of the fp32 GEMM's time
+    for (m_, n_, k_) in ((4096, 4096, 4096), (1024, 4096, 4096)):
+        xa = hip.array(rng.normal(0, 1, (m_, k_)).astype(np.float32))
+        wq = hip.array(rng.integers(-127, 128, (n_, k_), dtype=np.int8))
+        wsc = hip.array(rng.uniform(1e-3, 1e-2, n_).astype(np.float32))
+        wf = hip.array(rng.uniform(-1, 1, (k_, n_)).astype(np.float32))
+        oq = hip.empty((m_, n_))
+        _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_qgemm_w8a32(xa.ptr, wq.ptr, wsc.ptr, oq.ptr, m_, n_, k_)), seconds=0.4)
+        kern = hip.last_kernel()
+        _, ms32 = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm(
+            0, 0, m_, n_, k_, 1.0, xa.ptr, k_, wf.ptr, n_, 0.0, oq.ptr, n_, None, 0)), seconds=0.4)
+        tf = 2 * m_ * n_ * k_ / ms / 1e9
+        res[f"w8a32_gemm_{m_}x{n_}x{k_}"] = {"us": ms * 1e3, "equivalent_TFLOP/s": tf, "fp32_gemm_us": ms32 * 1e3,
+                                             "speedup_over_fp32": ms32 / ms,
+                                             "frac_of_bf16_mfma_peak_at_3_terms": 3 * tf / 2500.0, "kernel": kern}
+        del xa, wq, wsc, wf, oq
+
     # config 3: FFN block 2048 x 1024 x 4096, bias + GELU fused into GEMM1, bias into GEMM2
     x, w1 = f32((2048, 1024), (1024, 4096))
     w2 = hip.array(rng.normal(0, 0.02, (4096, 1024)).astype(np.float32))

@@ -680,8 +680,9 @@ W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 
                 (20, 1024, 512), (150, 260, 160), (96, 2048, 1024), (160, 3072, 768),   # 32x64 tiles, whole and with clamped edges
                 # the weight-streaming form: several row groups on one staging, 1 / 2 / 4 rows per wave, several slices of K,
                 # a last window that ends inside a 16-byte step, rows that run past N
-                (1, 20000, 520), (2, 16400, 300), (3, 8200, 1031), (6, 4100, 8192), (5, 4099, 2050), (4, 9000, 4100),
+                (1, 20000, 520), (2, 16400, 300), (3, 8200, 1031), (6, 4100, 8200), (5, 4099, 2050), (4, 9000, 4100),
                 (6, 33, 10000), (1, 70, 20000),
+                (6, 4100, 8192), (5, 8192, 2048), (6, 64, 2048),   # five or six rows with a long K: the tiles
                 (32, 128, 517), (70, 260, 1031), (3, 64, 1037)]   # rows at odd byte offsets
 
 
