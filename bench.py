@@ -9,7 +9,7 @@ and the skinny-M route's GB/s, each with its own roofline fraction.  RESULT line
 reference's benchmark format (benchmarks/bench_common.h:25-42) go to stderr.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu]
-    python bench.py --counter-probe [headline|skinny|gemm1024|fp32|config2|attention]
+    python bench.py --counter-probe [headline|skinny|gemm1024|fp32|config2|attention|w8a32]
                                         # for hardware-counter runs: a few launches of one case's kernels and 3
                                         # launches of a copy-shaped kernel of known size, no output line
     python bench.py --sustain 8 [--operands zeros]   # back-to-back headline launches, for clock sampling
@@ -565,7 +565,8 @@ def counter_probe(hip, case, repeat=1):
       gemm1024  fp32 1024^3
       fp32      the FFN pair 2048 x 1024 x 4096 (bias + GELU fused into the first GEMM) and back
       config2   W8A8 M = 256, N = K = 4096
-      attention batched Q K^T and P V over 512 heads of [512, 64], then the fused forward"""
+      attention batched Q K^T and P V over 512 heads of [512, 64], then the fused forward
+      w8a32     W8A32 with many rows, 4096^3 and 1024 x 4096 x 4096 (bf16 matrix core, three terms per activation)"""
     rng = np.random.default_rng(0)
     L = hip.L
     reps = 3 * repeat                # `repeat` > 1 (--probe-repeat): long enough for sustained clocks, for kernel traces
@@ -629,6 +630,16 @@ def counter_probe(hip, case, repeat=1):
             k2 = hip.last_kernel()
             hip.check(L.axhip_sdpa_fwd(q.ptr, k.ptr, v.ptr, o.ptr, l.ptr, Bn, S, D, 0.125, 0))
         what = f"{reps} x (QK^T {k1}, PV {k2}, fused {hip.last_kernel()}) over 512 heads of [512, 64]"
+    elif case == "w8a32":
+        what = ""
+        for (M, N, K) in ((4096, 4096, 4096), (1024, 4096, 4096)):
+            xa = hip.array(rng.normal(0, 1, (M, K)).astype(np.float32))
+            wq = hip.array(rand_i8(rng, (N, K)))
+            ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+            out = hip.empty((M, N))
+            for _ in range(reps):
+                hip.check(L.axhip_qgemm_w8a32(xa.ptr, wq.ptr, ws.ptr, out.ptr, M, N, K))
+            what += f"{reps} x qgemm_w8a32 {M}x{N}x{K} ({hip.last_kernel()}) "
     else:
         sys.exit(f"unknown counter-probe case {case!r}")
     hip.sync()
@@ -776,7 +787,7 @@ def main():
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--counter-probe", nargs="?", const="headline", default=None,
-                    choices=["headline", "skinny", "gemm1024", "fp32", "config2", "attention"])
+                    choices=["headline", "skinny", "gemm1024", "fp32", "config2", "attention", "w8a32"])
     ap.add_argument("--probe-repeat", type=int, default=1, help="multiplies the launch counts of --counter-probe")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of back-to-back headline launches")
     ap.add_argument("--operands", choices=["random", "zeros", "fp32", "fp32zeros", "qkt", "qktzeros", "pv", "pvzeros"], default="random")
