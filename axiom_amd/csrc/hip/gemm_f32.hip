@@ -1338,26 +1338,46 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
             return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
         return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, true, int8_t>("qgemm_w8a32_mfma_32x64k2_dma_edge", g, batch);
     }
+    if (g.K > 128 && tuning().f32_tile == 0) {
+        // Many output tiles.  The conversions to bf16 run on the vector pipe beside the products, and that pipe needs two
+        // waves on a SIMD to stay busy.  A wave converts its own rows of A (6.5 instructions a value) and every column of
+        // B it multiplies them with (1.5), so its tile is one 32-row block high and as wide as the tile allows, and the
+        // tile is the largest that still gives the CUs enough workgroups (M, N, K, us before -> after: 4096^3 517 -> 353,
+        // 2048 x 4096 x 4096 266 -> 203, 1024 x 4096 x 4096 153 -> 106, 512 x 11008 x 4096 214 -> 153, 512 x 4096 x 4096
+        // 84 -> 65, 2048 x 1024 x 4096 85 -> 62, 256 x 4096 x 4096 54 -> 46, 1024^3 16.1 -> 14.4).  `eighths` = workgroups
+        // per CU, in eighths, from which a tile shape pays (measured: the 128-row tiles have one wave per SIMD and need
+        // two workgroups per CU, the k-split ones bring two waves themselves).  A shape off the tile grid takes the edge
+        // form when the padding stays under an eighth of the output (1000 x 4096 x 4096 153 -> 111 us, 4000 x 4000 x 4096
+        // 577 -> 355, 300 x 11008 x 4096 146 -> 102, 2000 x 2000 x 2048 79 -> 58).
+        const int64_t cus = cu_count();
+        auto pays = [&](int64_t bm, int64_t bn, int64_t eighths, bool &whole) {
+            const int64_t tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
+            whole = g.M % bm == 0 && g.N % bn == 0;
+            return tm * tn * batch * 8 >= eighths * cus && tm * bm * tn * bn * 8 <= g.M * g.N * 9;
+        };
+        bool whole;
+        if (pays(128, 256, 16, whole))
+            return whole ? launch_dma<128, 256, 4, 1, 2, true, true, 1, 1, false, int8_t>("qgemm_w8a32_mfma_128x256_dma", g, batch)
+                         : launch_dma<128, 256, 4, 1, 2, true, true, 1, 1, true, int8_t>("qgemm_w8a32_mfma_128x256_dma_edge", g, batch);
+        if (pays(128, 128, 16, whole))
+            return whole ? launch_dma<128, 128, 4, 1, 3, true, true, 1, 1, false, int8_t>(names[0], g, batch)
+                         : launch_dma<128, 128, 4, 1, 3, true, true, 1, 1, true, int8_t>("qgemm_w8a32_mfma_128x128_dma_edge", g, batch);
+        if (pays(64, 128, 12, whole))
+            return whole ? launch_dma<64, 128, 2, 1, 2, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_64x128k2_dma", g, batch)
+                         : launch_dma<64, 128, 2, 1, 2, true, true, 1, 2, true, int8_t>("qgemm_w8a32_mfma_64x128k2_dma_edge", g, batch);
+        if (pays(32, 128, 10, whole))
+            return whole ? launch_dma<32, 128, 1, 2, 4, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x128k2_dma", g, batch)
+                         : launch_dma<32, 128, 1, 2, 4, true, true, 1, 2, true, int8_t>("qgemm_w8a32_mfma_32x128k2_dma_edge", g, batch);
+        if (pays(32, 64, 12, whole))
+            return whole ? launch_dma<32, 64, 1, 2, 4, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x64k2_dma", g, batch)
+                         : launch_dma<32, 64, 1, 2, 4, true, true, 1, 2, true, int8_t>("qgemm_w8a32_mfma_32x64k2_dma_edge", g, batch);
+    }
     if (g.M % 64 != 0 || g.N % 64 != 0) {
         if (g.K > 128) return launch_dma<64, 64, 2, 2, 2, true, true, 1, 2, true, int8_t>(names[2], g, batch);
         return launch_dma<64, 64, 2, 2, 2, true, true, 1, 1, true, int8_t>(names[1], g, batch);
     }
     if (g.K > 128) {
         const int64_t big = (g.M / 128) * (g.N / 128) * batch, cus = cu_count(), rounds = (big + cus - 1) / cus;
-        // The conversions to bf16 run on the vector pipe beside the products, and that pipe needs two waves on a SIMD
-        // to stay busy: take the largest tile that still gives every CU two workgroups (or one of eight waves).  A wave
-        // converts its own rows of A (6.5 instructions a value) and every column of B it multiplies them with (1.5), so
-        // its tile is one 32-row block high and as wide as the tile allows.  (M, N, K, us before -> after:
-        // 4096^3 517 -> 353, 2048 x 4096 x 4096 266 -> 203, 1024 x 4096 x 4096 153 -> 106, 512 x 11008 x 4096 214 -> 153,
-        // 512 x 4096 x 4096 84 -> 65, 2048 x 1024 x 4096 85 -> 62, 256 x 4096 x 4096 54 -> 46, 1024^3 16.1 -> 14.4.)
-        if (tuning().f32_tile == 0) {
-            auto enough = [&](int64_t bm, int64_t bn) { return g.M % bm == 0 && g.N % bn == 0 && (g.M / bm) * (g.N / bn) * batch >= 2 * cus; };
-            if (enough(128, 256)) return launch_dma<128, 256, 4, 1, 2, true, true, 1, 1, false, int8_t>("qgemm_w8a32_mfma_128x256_dma", g, batch);
-            if (enough(128, 128)) return launch_dma<128, 128, 4, 1, 3, true, true, 1, 1, false, int8_t>(names[0], g, batch);
-            if (enough(64, 128)) return launch_dma<64, 128, 2, 1, 2, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_64x128k2_dma", g, batch);
-            if (enough(32, 128)) return launch_dma<32, 128, 1, 2, 4, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x128k2_dma", g, batch);
-            if (enough(32, 64)) return launch_dma<32, 64, 1, 2, 4, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
-        }
         if (g.M % 128 == 0 && g.N % 128 == 0 && big >= cus && big * 10 >= rounds * cus * 9)
             return launch_dma<128, 128, 4, 1, 3, true, true, 1, 1, false, int8_t>(names[0], g, batch);
         // the last round of one 64x64 tile per CU mostly empty: 32x64 tiles, as for fp32 operands

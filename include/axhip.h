@@ -170,7 +170,11 @@ int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w, const floa
                      int64_t M, int64_t N, int64_t K);
 
 /* W8A32: out[m,n] = w_scales[n] * sum_k a[m,k] * (float)w[n,k], fp32 accumulation.
- * Device-memory form of ax_qgemm_w8a32 (src/core/quantize.c:100-177). */
+ * Device-memory form of ax_qgemm_w8a32 (src/core/quantize.c:100-177).  Every product
+ * a[m,k] * w[n,k] enters the sum exactly (up to M = 6 as a fused multiply-add; above, as three
+ * bf16 terms of a[m,k] that add up to it exactly, times the int8 weight as a bf16, on the bf16
+ * matrix core); only the order of the fp32 additions differs from the reference's loop.
+ * +-inf and NaN among the activations give what that loop gives. */
 int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w_scales, float *out,
                       int64_t M, int64_t N, int64_t K);
 

@@ -712,7 +712,11 @@ def test_w8a32_against_oracle(hip, oracle, golden, M, N, K):
 W8A32_TILE_FORMS = [(2048, 8192, 160, "qgemm_w8a32_mfma_128x256_dma"), (2048, 4096, 192, "qgemm_w8a32_mfma_128x128_dma"),
                     (1024, 4096, 224, "qgemm_w8a32_mfma_64x128k2_dma"), (512, 4096, 288, "qgemm_w8a32_mfma_32x128k2_dma"),
                     (256, 4096, 160, "qgemm_w8a32_mfma_32x64k2_dma"), (256, 4096, 256, "qgemm_w8a32_mfma_32x64k2_dma"),
-                    (512, 4096, 1056, "qgemm_w8a32_mfma_32x128k2_dma")]
+                    (512, 4096, 1056, "qgemm_w8a32_mfma_32x128k2_dma"),
+                    # off the tile grid: clamped fetches and a guarded write-back
+                    (4000, 4000, 160, "qgemm_w8a32_mfma_128x256_dma_edge"), (2000, 4000, 192, "qgemm_w8a32_mfma_128x128_dma_edge"),
+                    (1000, 4100, 224, "qgemm_w8a32_mfma_64x128k2_dma_edge"), (520, 4096, 288, "qgemm_w8a32_mfma_32x128k2_dma_edge"),
+                    (220, 4100, 160, "qgemm_w8a32_mfma_32x64k2_dma_edge")]
 
 
 @pytest.mark.parametrize("M,N,K,form", W8A32_TILE_FORMS)
@@ -725,8 +729,13 @@ def test_w8a32_tile_forms(hip, M, N, K, form):
     a = (rng.uniform(-1, 1, (M, K)) * 10.0 ** rng.integers(-3, 4, (M, 1))).astype(np.float32)
     w = rng.integers(-127, 128, (N, K), dtype=np.int8)
     ws = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
-    got = hip.qgemm_w8a32(hip.array(a), hip.array(w), hip.array(ws)).numpy()
+    dout = hip.array(np.full((M + 1, N), np.nan, np.float32))          # a row past the output: never written
+    da, dw, ds = hip.array(a), hip.array(w), hip.array(ws)
+    hip.check(hip.L.axhip_qgemm_w8a32(da.ptr, dw.ptr, ds.ptr, dout.ptr, M, N, K))
     assert hip.last_kernel() == form
+    full = dout.numpy()
+    got = full[:M]
+    assert np.isnan(full[M]).all()
     want = (a.astype(np.float64) @ w.astype(np.float64).T) * ws
     bound = BOUND_FP32 * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64).T) * ws + 1e-30
     assert (np.abs(got - want) <= bound).all(), float((np.abs(got - want) / bound).max())
