@@ -712,7 +712,8 @@ def test_w8a32_against_oracle(hip, oracle, golden, M, N, K):
 W8A32_TILE_FORMS = [(2048, 8192, 160, "qgemm_w8a32_mfma_128x256_dma"), (2048, 4096, 192, "qgemm_w8a32_mfma_128x128_dma"),
                     (1024, 4096, 224, "qgemm_w8a32_mfma_64x128k2_dma"), (512, 4096, 288, "qgemm_w8a32_mfma_32x128k2_dma"),
                     (256, 4096, 160, "qgemm_w8a32_mfma_32x64k2_dma"), (256, 4096, 256, "qgemm_w8a32_mfma_32x64k2_dma"),
-                    (512, 4096, 1056, "qgemm_w8a32_mfma_32x128k2_dma"),
+                    (512, 4096, 1056, "qgemm_w8a32_mfma_32x128k2_dma"), (512, 4096, 192, "qgemm_w8a32_mfma_32x128k2_dma"),
+                    (256, 4096, 224, "qgemm_w8a32_mfma_32x64k2_dma"),
                     # off the tile grid: clamped fetches and a guarded write-back
                     (4000, 4000, 160, "qgemm_w8a32_mfma_128x256_dma_edge"), (2000, 4000, 192, "qgemm_w8a32_mfma_128x128_dma_edge"),
                     (1000, 4100, 224, "qgemm_w8a32_mfma_64x128k2_dma_edge"), (520, 4096, 288, "qgemm_w8a32_mfma_32x128k2_dma_edge"),
