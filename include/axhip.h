@@ -174,7 +174,9 @@ int axhip_qgemm_w8a8(const int8_t *x, float x_scale, const int8_t *w, const floa
  * a[m,k] * w[n,k] enters the sum exactly (up to M = 6 as a fused multiply-add; above, as three
  * bf16 terms of a[m,k] that add up to it exactly, times the int8 weight as a bf16, on the bf16
  * matrix core); only the order of the fp32 additions differs from the reference's loop.
- * +-inf and NaN among the activations give what that loop gives. */
+ * +-inf and NaN among the activations give what that loop gives.  The bf16 matrix core flushes
+ * denormal operands: the low-order terms of activations below 2^-110 in magnitude are dropped, an
+ * absolute error of less than K * 2^-118 * w_scales[n] per output on top of the accumulation's. */
 int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w_scales, float *out,
                       int64_t M, int64_t N, int64_t K);
 

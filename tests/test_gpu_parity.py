@@ -764,6 +764,22 @@ def test_w8a32_three_bf16_terms_are_exact(hip, oracle):
     assert (np.abs(got - want) <= np.abs(want) * 2.0 ** -23).all()
 
 
+def test_w8a32_tiny_activations(hip):
+    """The bf16 matrix core flushes denormal operands, so the low-order bf16 terms of activations below 2^-110 are
+    dropped: the result stays within the fp32 bound plus K * 2^-118 per output, whatever the scale of the activations."""
+    M, N, K = 64, 256, 512
+    rng = np.random.default_rng(3)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    s = np.ones(N, np.float32)
+    for scale in (1e-30, 1e-34, 1e-36, 1e-38, 1e-41):
+        a = (rng.uniform(-1, 1, (M, K)) * scale).astype(np.float32)
+        got = hip.qgemm_w8a32(hip.array(a), hip.array(w), hip.array(s)).numpy().astype(np.float64)
+        assert hip.last_kernel().startswith("qgemm_w8a32_mfma")
+        want = a.astype(np.float64) @ w.astype(np.float64).T
+        bound = BOUND_FP32 * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64).T) + K * 2.0 ** -118
+        assert (np.abs(got - want) <= bound).all(), (scale, float((np.abs(got - want) / bound).max()))
+
+
 def test_w8a32_non_finite_activations(hip, oracle):
     """Infinities and NaNs among the activations come out as the reference's fp32 sum gives them (src/core/quantize.c:117-170, a plain fused multiply-add chain):
     +-inf where one sign of infinity meets non-zero weights, NaN where both signs meet, an infinity meets a zero weight,
