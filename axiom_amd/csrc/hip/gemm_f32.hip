@@ -1351,15 +1351,22 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
         // 577 -> 355, 300 x 11008 x 4096 146 -> 102, 2000 x 2000 x 2048 79 -> 58).
         const int64_t cus = cu_count();
         auto pays = [&](int64_t bm, int64_t bn, int64_t eighths, bool &whole) {
-            const int64_t tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
+            const int64_t tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn, tiles = tm * tn * batch;
             whole = g.M % bm == 0 && g.N % bn == 0;
-            return tm * tn * batch * 8 >= eighths * cus && tm * bm * tn * bn * 8 <= g.M * g.N * 9;
+            if (tiles * 8 < eighths * cus || tm * bm * tn * bn * 8 > g.M * g.N * 9) return false;
+            // two of the 128-row workgroups share a CU: a last round of them that is mostly empty costs a whole round
+            // (516 tiles of 128x128 at 768 x 11008 x 4096: 341 us against 310 on 64x64 tiles)
+            if (bm == 128) {
+                const int64_t rounds = (tiles + 2 * cus - 1) / (2 * cus);
+                return tiles * 5 >= rounds * 2 * cus * 4;
+            }
+            return true;
         };
         bool whole;
-        if (pays(128, 256, 16, whole))
+        if (pays(128, 256, 15, whole))
             return whole ? launch_dma<128, 256, 4, 1, 2, true, true, 1, 1, false, int8_t>("qgemm_w8a32_mfma_128x256_dma", g, batch)
                          : launch_dma<128, 256, 4, 1, 2, true, true, 1, 1, true, int8_t>("qgemm_w8a32_mfma_128x256_dma_edge", g, batch);
-        if (pays(128, 128, 16, whole))
+        if (pays(128, 128, 15, whole))
             return whole ? launch_dma<128, 128, 4, 1, 3, true, true, 1, 1, false, int8_t>(names[0], g, batch)
                          : launch_dma<128, 128, 4, 1, 3, true, true, 1, 1, true, int8_t>("qgemm_w8a32_mfma_128x128_dma_edge", g, batch);
         if (pays(64, 128, 12, whole))
