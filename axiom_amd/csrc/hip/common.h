@@ -41,6 +41,7 @@ struct Tuning {
     int f32_tile;        // AX_HIP_F32_TILE: 64 (64x64), 642 (64x64 with the k split over two wave sets), 128 (128x128, eight waves)
     int f32_splitk;      // AX_HIP_F32_SPLITK: 1 = never split K, 2.. = that many ranges where the route applies
     int skinny_blocks;   // AX_HIP_SKINNY_BLOCKS: workgroups the skinny-M route aims for
+    int w8a32_tile;      // AX_HIP_W8A32_TILE: 1 (128x256), 2 (128x128), 3 (64x128), 4 (32x128), 5 (32x64): W8A32 matrix-core tile for K > 128
 };
 const Tuning &tuning();
 

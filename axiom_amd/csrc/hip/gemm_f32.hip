@@ -1333,7 +1333,7 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
                     g.stride_c % 4 == 0 && g.lda < (1 << 20) && g.ldb < (1 << 22) && batch <= 65535 && g.N % 4 == 0 &&
                     ((g.M + 63) / 64) * ((g.N + 63) / 64) <= 0x7fffffff;
     if (!ok) return -1;
-    if (half_row_tiles(g.M) && g.K >= 64 && tuning().f32_tile == 0) {   // as for fp32 operands
+    if (half_row_tiles(g.M) && g.K >= 64 && tuning().f32_tile == 0 && (tuning().w8a32_tile == 0 || g.K <= 128)) {   // as for fp32 operands
         if (g.M % 32 == 0 && g.N % 64 == 0)
             return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
         return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, true, int8_t>("qgemm_w8a32_mfma_32x64k2_dma_edge", g, batch);
@@ -1350,9 +1350,11 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
         // form when the padding stays under an eighth of the output (1000 x 4096 x 4096 153 -> 111 us, 4000 x 4000 x 4096
         // 577 -> 355, 300 x 11008 x 4096 146 -> 102, 2000 x 2000 x 2048 79 -> 58).
         const int64_t cus = cu_count();
+        const int forced = tuning().w8a32_tile;
         auto pays = [&](int64_t bm, int64_t bn, int64_t eighths, bool &whole) {
             const int64_t tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn, tiles = tm * tn * batch;
             whole = g.M % bm == 0 && g.N % bn == 0;
+            if (forced) return forced == (bm == 128 ? (bn == 256 ? 1 : 2) : bm == 64 ? 3 : bn == 128 ? 4 : 5) && tiles <= 0x7fffffff;
             if (tiles * 8 < eighths * cus || tm * bm * tn * bn * 8 > g.M * g.N * 9) return false;
             // two of the 128-row workgroups share a CU: a last round of them that is mostly empty costs a whole round
             // (516 tiles of 128x128 at 768 x 11008 x 4096: 341 us against 310 on 64x64 tiles)

@@ -58,8 +58,10 @@ const char *axhip_device_name(void);          /* gcnArchName of device 0, "" wit
  *   AX_HIP_F32_TILE      64x64 | 64x64k2 | 128x128   fp32 tile on the aligned fast path (k2: two wave sets split each K slab)
  *   AX_HIP_F32_SPLITK    1..4096    K ranges of the fp32 few-tile route (1: never split)
  *   AX_HIP_SKINNY_BLOCKS 1..65535   workgroups the skinny-M route aims for
+ *   AX_HIP_W8A32_TILE    128x256 | 128x128 | 64x128 | 32x128 | 32x64   W8A32 matrix-core tile where K > 128 and a multiple of 32
+ *                        (edge form off the tile grid)
  * axhip_tuning_get returns the value in effect (0: automatic; tiles as their first number, 64x64k2 as
- * 642, 128x64 as 1264), or -1 for an unknown name. */
+ * 642, 128x64 as 1264; AX_HIP_W8A32_TILE as the position in its list, 1..5), or -1 for an unknown name. */
 int axhip_tuning_reload(void);
 int axhip_tuning_get(const char *name);
 

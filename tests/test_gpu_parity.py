@@ -402,6 +402,39 @@ def test_forced_tiles_and_splits_keep_parity(hip, oracle):
         hip.L.axhip_tuning_reload()
 
 
+def test_w8a32_forced_tiles_keep_parity(hip):
+    """AX_HIP_W8A32_TILE picks the matrix-core tile of the W8A32 product, whole or in its edge form; every choice stays
+    inside the fp64 bound of a correct fp32 accumulation."""
+    saved = os.environ.get("AX_HIP_W8A32_TILE")
+    rng = np.random.default_rng(31)
+    cases = []
+    for (M, N, K) in ((256, 512, 320), (200, 260, 160)):
+        a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+        w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+        ws = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        want = (a.astype(np.float64) @ w.astype(np.float64).T) * ws
+        bound = BOUND_FP32 * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64).T) * ws + 1e-30
+        cases.append((M, N, K, hip.array(a), hip.array(w), hip.array(ws), want, bound))
+    try:
+        for tile, form in (("128x256", "qgemm_w8a32_mfma_128x256_dma"), ("128x128", "qgemm_w8a32_mfma_128x128_dma"),
+                           ("64x128", "qgemm_w8a32_mfma_64x128k2_dma"), ("32x128", "qgemm_w8a32_mfma_32x128k2_dma"),
+                           ("32x64", "qgemm_w8a32_mfma_32x64k2_dma")):
+            os.environ["AX_HIP_W8A32_TILE"] = tile
+            assert hip.L.axhip_tuning_reload() == 1
+            for (M, N, K, da, dw, ds, want, bound) in cases:
+                say("forced w8a32", tile, M, N, K)
+                got = hip.qgemm_w8a32(da, dw, ds).numpy()
+                whole = M % int(tile.split("x")[0]) == 0 and N % int(tile.split("x")[1]) == 0
+                assert hip.last_kernel() == form + ("" if whole else "_edge")
+                assert (np.abs(got - want) <= bound).all(), (tile, M, N, K)
+    finally:
+        if saved is None:
+            os.environ.pop("AX_HIP_W8A32_TILE", None)
+        else:
+            os.environ["AX_HIP_W8A32_TILE"] = saved
+        hip.L.axhip_tuning_reload()
+
+
 def test_w8a32_dispatch_sweep(hip, oracle):
     """80 seeded W8A32 shapes from the boundary dimensions: the weight-streaming form (M <= 6), the matrix-core form,
     its split over K and its K tail all obey the fp64 bound of a correct fp32 accumulation."""
