@@ -413,8 +413,10 @@ template <> struct Frag<false> {
 // and guard the write-back; in the last slab, lanes whose k values lie past K write zeros to
 // their LDS place instead of loading, in both operands, so the tail adds exact zeros.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI, int WAVES_K,
-          bool EDGE = false, typename BSRC = float>
+          bool EDGE = false, typename BSRC = float, int SPS = 1>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(SgemmArgs g) {
+    // SPS == 2: a stage holds two slabs (64 k) and the loop's barrier comes once per stage — for tiles whose slab is
+    // only a few MFMAs per wave, where the barrier is a visible share of the slab (K a multiple of 64, no edge form)
     // WAVES_K == 2: a second set of waves shares each tile; set 0 multiplies k-blocks 0 and 1 of
     // every slab, set 1 k-blocks 2 and 3, and the two accumulators are added through LDS at the
     // end.  For 64x64 tiles with one workgroup per CU this puts two waves on every SIMD, so one
@@ -427,15 +429,17 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     using OA = DmaOperand<BM, A_KC, NW>;
     using OB = typename std::conditional<B_I8, DmaOperandI8<BN, NW>, DmaOperand<BN, B_KC, NW>>::type;
     // LDS: NST stages of A, then NST stages of B
-    constexpr int B_BASE = NST * OA::BYTES;
+    static_assert(SPS == 1 || (SPS == 2 && !EDGE && !B_I8), "two slabs per stage: fp32 operands on whole tiles");
+    constexpr int A_STAGE = SPS * OA::BYTES, B_STAGE = SPS * OB::BYTES;
+    constexpr int B_BASE = NST * A_STAGE;
     constexpr int NREADS = TM * OA::READS + TN * OB::READS;
     // loads a wave may leave in flight at the end of a slab: everything but the next slab's
     // int8 B with four stages: the fragments of slab s + 1 are read while slab s is converted and multiplied, so the
     // loop's barrier must already cover slab s + 2 and one stage less is in flight
     constexpr bool PIPE = B_I8 && NST == 4;
-    constexpr int VM_KEEP = (NST - (PIPE ? 3 : 2)) * (OA::IPW + OB::IPW);
+    constexpr int VM_KEEP = (NST - (PIPE ? 3 : 2)) * SPS * (OA::IPW + OB::IPW);
     static_assert(NST >= 2 && NST <= 4 && VM_KEEP < 64, "stage count");
-    static_assert(B_BASE + NST * OB::BYTES <= 160 * 1024, "LDS budget");
+    static_assert(B_BASE + NST * B_STAGE <= 160 * 1024, "LDS budget");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -453,7 +457,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     float *C = g.C + batch * g.stride_c;
     // EDGE also takes a K that ends inside a slab (K a multiple of 4): the last slab's lanes whose four
     // k values lie past K load nothing and write zeros to their LDS place instead
-    const int slabs = EDGE ? (int)((g.K + 31) / 32) : (int)(g.K / 32);
+    const int slabs = EDGE ? (int)((g.K + 31) / 32) : (int)(g.K / (32 * SPS));   // stages to walk
     const int ktail = EDGE ? (int)(g.K - (int64_t)(slabs - 1) * 32) : 32;     // k values in the last slab
     int left = slabs;                                                          // slabs not yet requested
 
@@ -491,9 +495,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         for (int kbi = 0; kbi < 4; kbi++) {
             // with a k split, entries 0 and 1 address this wave set's own two k-blocks
             const int kb = WAVES_K == 2 ? 2 * wk + (kbi & 1) : kbi;
-            ra[st][kbi] = lds0 + st * OA::BYTES + OA::frag_base(wm * WTM, frow, fhalf, kb) +
+            ra[st][kbi] = lds0 + st * A_STAGE + OA::frag_base(wm * WTM, frow, fhalf, kb) +
                           (WAVES_K == 2 && !A_KC ? wk * OA::k_imm(16) : 0);
-            rb[st][kbi] = lds0 + B_BASE + st * OB::BYTES + OB::frag_base(wn * WTN, frow, fhalf, kb) +
+            rb[st][kbi] = lds0 + B_BASE + st * B_STAGE + OB::frag_base(wn * WTN, frow, fhalf, kb) +
                           (WAVES_K == 2 && !B_KC ? wk * OB::k_imm(16) : 0);
         }
 
@@ -514,49 +518,51 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         --left;                                                                                  \
         if (EDGE && left == 0 && ktail < 32) {                                                   \
             _Pragma("unroll") for (int j = 0; j < OA::IPW; j++) {                                \
-                const unsigned at = wave * OA::PITCH + (ST) * OA::BYTES + j * NW * OA::PITCH;    \
+                const unsigned at = wave * OA::PITCH + (ST) * A_STAGE + j * NW * OA::PITCH;      \
                 if (ta[j]) AXF_LOAD_LDS(lds0 + at, va[j], ga);                                   \
                 else *reinterpret_cast<v4f *>(lds_raw + at + lane * 16) = v4f{0.f, 0.f, 0.f, 0.f}; \
             }                                                                                    \
             _Pragma("unroll") for (int j = 0; j < OB::IPW; j++) {                                \
-                const unsigned at = B_BASE + wave * OB::PITCH + (ST) * OB::BYTES + j * NW * OB::PITCH; \
+                const unsigned at = B_BASE + wave * OB::PITCH + (ST) * B_STAGE + j * NW * OB::PITCH; \
                 if (tb[j]) AXF_LOAD_LDS(lds0 + at, vb[j], gb);                                   \
                 else *reinterpret_cast<v4f *>(lds_raw + at + lane * 16) = v4f{0.f, 0.f, 0.f, 0.f}; \
             }                                                                                    \
         } else {                                                                                 \
-            _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                                  \
-                AXF_LOAD_LDS(dma_a + (ST) * OA::BYTES + j * NW * OA::PITCH, va[j], ga);          \
-            _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                                  \
-                if (!B_I8 || j * NW + wave < OB::NINSTR)                                         \
-                    AXF_LOAD_LDS(dma_b + B_BASE + (ST) * OB::BYTES + j * NW * OB::PITCH, vb[j], gb); \
+            _Pragma("unroll") for (int u = 0; u < SPS; u++) {                                    \
+                _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                              \
+                    AXF_LOAD_LDS(dma_a + (ST) * A_STAGE + u * OA::BYTES + j * NW * OA::PITCH, va[j], ga + u * step_a); \
+                _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                              \
+                    if (!B_I8 || j * NW + wave < OB::NINSTR)                                     \
+                        AXF_LOAD_LDS(dma_b + B_BASE + (ST) * B_STAGE + u * OB::BYTES + j * NW * OB::PITCH, vb[j], gb + u * step_b); \
+            }                                                                                    \
         }                                                                                        \
-        ga += step_a;                                                                            \
-        gb += step_b;                                                                            \
+        ga += SPS * step_a;                                                                      \
+        gb += SPS * step_b;                                                                      \
     } while (0)
 
 // fragments of k-block KBI of stage ST
-#define AXF_FRAGS(BUF, ST, KBI)                                                                  \
+#define AXF_FRAGS(BUF, ST, KBI, U)                                                               \
     do {                                                                                         \
         _Pragma("unroll") for (int t = 0; t < TM; t++) {                                         \
             if constexpr (A_KC) {                                                                \
-                AXF_DS128(fa[BUF][t].q, ra[ST][KBI], t * 4096);                                  \
+                AXF_DS128(fa[BUF][t].q, ra[ST][KBI], t * 4096 + (U) * OA::BYTES);                \
             } else {                                                                             \
-                AXF_DS32(fa[BUF][t].s0, ra[ST][0], OA::k_imm((KBI) * 8 + 0) + t * 128);          \
-                AXF_DS32(fa[BUF][t].s1, ra[ST][0], OA::k_imm((KBI) * 8 + 1) + t * 128);          \
-                AXF_DS32(fa[BUF][t].s2, ra[ST][0], OA::k_imm((KBI) * 8 + 2) + t * 128);          \
-                AXF_DS32(fa[BUF][t].s3, ra[ST][0], OA::k_imm((KBI) * 8 + 3) + t * 128);          \
+                AXF_DS32(fa[BUF][t].s0, ra[ST][0], OA::k_imm((KBI) * 8 + 0) + t * 128 + (U) * OA::BYTES); \
+                AXF_DS32(fa[BUF][t].s1, ra[ST][0], OA::k_imm((KBI) * 8 + 1) + t * 128 + (U) * OA::BYTES); \
+                AXF_DS32(fa[BUF][t].s2, ra[ST][0], OA::k_imm((KBI) * 8 + 2) + t * 128 + (U) * OA::BYTES); \
+                AXF_DS32(fa[BUF][t].s3, ra[ST][0], OA::k_imm((KBI) * 8 + 3) + t * 128 + (U) * OA::BYTES); \
             }                                                                                    \
         }                                                                                        \
         _Pragma("unroll") for (int t = 0; t < TN; t++) {                                         \
             if constexpr (B_I8) {                                                                \
                 AXF_DS32(fb[BUF][t].raw, rb[ST][KBI], t * 1024);                                 \
             } else if constexpr (B_KC) {                                                         \
-                AXF_DS128(fb[BUF][t].q, rb[ST][KBI], t * 4096);                                  \
+                AXF_DS128(fb[BUF][t].q, rb[ST][KBI], t * 4096 + (U) * OB::BYTES);                \
             } else {                                                                             \
-                AXF_DS32(fb[BUF][t].s0, rb[ST][0], OB::k_imm((KBI) * 8 + 0) + t * 128);          \
-                AXF_DS32(fb[BUF][t].s1, rb[ST][0], OB::k_imm((KBI) * 8 + 1) + t * 128);          \
-                AXF_DS32(fb[BUF][t].s2, rb[ST][0], OB::k_imm((KBI) * 8 + 2) + t * 128);          \
-                AXF_DS32(fb[BUF][t].s3, rb[ST][0], OB::k_imm((KBI) * 8 + 3) + t * 128);          \
+                AXF_DS32(fb[BUF][t].s0, rb[ST][0], OB::k_imm((KBI) * 8 + 0) + t * 128 + (U) * OB::BYTES); \
+                AXF_DS32(fb[BUF][t].s1, rb[ST][0], OB::k_imm((KBI) * 8 + 1) + t * 128 + (U) * OB::BYTES); \
+                AXF_DS32(fb[BUF][t].s2, rb[ST][0], OB::k_imm((KBI) * 8 + 2) + t * 128 + (U) * OB::BYTES); \
+                AXF_DS32(fb[BUF][t].s3, rb[ST][0], OB::k_imm((KBI) * 8 + 3) + t * 128 + (U) * OB::BYTES); \
             }                                                                                    \
         }                                                                                        \
     } while (0)
@@ -600,22 +606,22 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
             /* this slab's fragments are in buffers 4 (ST & 1) ..., read a slab ago */            \
             constexpr int C0 = 4 * ((ST) & 1), N0 = 4 - C0, NS = ((ST) + 1) % NST;               \
             if (next) {                                                                          \
-                AXF_FRAGS(N0, NS, 0);                                                            \
-                AXF_FRAGS(N0 + 1, NS, 1);                                                        \
+                AXF_FRAGS(N0, NS, 0, 0);                                                         \
+                AXF_FRAGS(N0 + 1, NS, 1, 0);                                                     \
                 if constexpr (WAVES_K == 1) {                                                    \
-                    AXF_FRAGS(N0 + 2, NS, 2);                                                    \
-                    AXF_FRAGS(N0 + 3, NS, 3);                                                    \
+                    AXF_FRAGS(N0 + 2, NS, 2, 0);                                                 \
+                    AXF_FRAGS(N0 + 3, NS, 3, 0);                                                 \
                 }                                                                                \
                 AXF_LGKM((WAVES_K == 1 ? 4 : 2) * NREADS);                                       \
             } else AXF_LGKM(0);                                                                  \
             AXF_PAIR(C0, C0 + 1);                                                                \
             if constexpr (WAVES_K == 1) AXF_PAIR(C0 + 2, C0 + 3);                                \
         } else if constexpr (B_I8) {                                                             \
-            AXF_FRAGS(0, ST, 0);                                                                 \
-            AXF_FRAGS(1, ST, 1);                                                                 \
+            AXF_FRAGS(0, ST, 0, 0);                                                              \
+            AXF_FRAGS(1, ST, 1, 0);                                                              \
             if constexpr (WAVES_K == 1) {                                                        \
-                AXF_FRAGS(2, ST, 2);                                                             \
-                AXF_FRAGS(3, ST, 3);                                                             \
+                AXF_FRAGS(2, ST, 2, 0);                                                          \
+                AXF_FRAGS(3, ST, 3, 0);                                                          \
                 AXF_LGKM(2 * NREADS);                                                            \
                 AXF_PAIR(0, 1);                                                                  \
                 AXF_LGKM(0);                                                                     \
@@ -625,20 +631,22 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
                 AXF_PAIR(0, 1);                                                                  \
             }                                                                                    \
         } else {                                                                                 \
-            AXF_FRAGS(0, ST, 0);                                                                 \
-            AXF_FRAGS(1, ST, 1);                                                                 \
-            AXF_LGKM(NREADS);                                                                    \
-            AXF_MFMAS(0);                                                                        \
-            if constexpr (WAVES_K == 1) {                                                        \
-                AXF_FRAGS(0, ST, 2);                                                             \
-                AXF_LGKM(NREADS);                                                                \
-                AXF_MFMAS(1);                                                                    \
-                AXF_FRAGS(1, ST, 3);                                                             \
+            _Pragma("unroll") for (int u = 0; u < SPS; u++) {                                    \
+                AXF_FRAGS(0, ST, 0, u);                                                          \
+                AXF_FRAGS(1, ST, 1, u);                                                          \
                 AXF_LGKM(NREADS);                                                                \
                 AXF_MFMAS(0);                                                                    \
+                if constexpr (WAVES_K == 1) {                                                    \
+                    AXF_FRAGS(0, ST, 2, u);                                                      \
+                    AXF_LGKM(NREADS);                                                            \
+                    AXF_MFMAS(1);                                                                \
+                    AXF_FRAGS(1, ST, 3, u);                                                      \
+                    AXF_LGKM(NREADS);                                                            \
+                    AXF_MFMAS(0);                                                                \
+                }                                                                                \
+                AXF_LGKM(0);                                                                     \
+                AXF_MFMAS(1);                                                                    \
             }                                                                                    \
-            AXF_LGKM(0);                                                                         \
-            AXF_MFMAS(1);                                                                        \
         }                                                                                        \
         if (VM_KEEP > 0 && (more)) {                                                             \
             /* a wave past the int8 operand's load instructions has only A's in flight */        \
@@ -659,11 +667,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     if constexpr (EDGE) AXF_LGKM(0);             // zeros written for a K tail that is already in the first slabs
     __builtin_amdgcn_s_barrier();
     if constexpr (PIPE) {
-        AXF_FRAGS(0, 0, 0);
-        AXF_FRAGS(1, 0, 1);
+        AXF_FRAGS(0, 0, 0, 0);
+        AXF_FRAGS(1, 0, 1, 0);
         if constexpr (WAVES_K == 1) {
-            AXF_FRAGS(2, 0, 2);
-            AXF_FRAGS(3, 0, 3);
+            AXF_FRAGS(2, 0, 2, 0);
+            AXF_FRAGS(3, 0, 3, 0);
         }
     }
     // whole rounds of the ring in a loop with one way out, then the slabs % NST that remain (nothing is
@@ -795,13 +803,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI = 1, int WAVES_K = 1,
-          bool EDGE = false, typename BSRC = float>
+          bool EDGE = false, typename BSRC = float, int SPS = 1>
 int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
     static_assert(!EDGE || EPI == 1, "the edge form guards the turned write-back only");
-    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K, EDGE, BSRC>;
+    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K, EDGE, BSRC, SPS>;
     constexpr int NW = WAVES_M * WAVES_N * WAVES_K;
     using OB = typename std::conditional<sizeof(BSRC) == 1, DmaOperandI8<BN, NW>, DmaOperand<BN, B_KC, NW>>::type;
-    constexpr int stage_bytes = NST * (DmaOperand<BM, A_KC, NW>::BYTES + OB::BYTES);
+    constexpr int stage_bytes = NST * SPS * (DmaOperand<BM, A_KC, NW>::BYTES + OB::BYTES);
     // the write-back turns 4 KiB per output wave through the dead stages
     constexpr int after = WAVES_K == 2 ? BM * BN * 4 : WAVES_M * WAVES_N * 4096;   // the join of a k split needs the whole tile
     constexpr int smem = stage_bytes > after ? stage_bytes : after;
@@ -1314,6 +1322,12 @@ int try_dma(const char *const names[3], const SgemmArgs &g, int64_t batch) {
                 return launch_dma<32, 64, 1, 2, 2, A_KC, B_KC, 1, 2>(B_KC ? "sgemm_nt_32x64k2_dma" : "sgemm_nn_32x64k2_dma", g, batch);
             }
         }
+        // Two slabs per stage and barrier where K allows (a slab of a 64x64 tile is 8 MFMAs per wave, so the barrier is a
+        // visible share of it), which also keeps as much in flight as the third stage did.  Cached / from HBM:
+        // 256 x 4096 x 4096 70.1 / 72.0 -> 66.8 / 69.9 us, 512 x 2048 x 4096 70.1 / 71.1 -> 66.7 / 68.2, 256 x 4096 x 1024
+        // 20.4 / 20.5 -> 19.6 / 19.9, 1024^3 19.7 / 20.1 -> 19.5 / 19.9, 256 x 11008 x 4096 182 / 194 -> 182 / 188; with three
+        // stages of two slabs 68.3 / 70.1 on the first.
+        if (g.K % 64 == 0) return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2, false, float, 2>(names[2], g, batch);
         if (streams) return launch_dma<64, 64, 2, 2, 3, A_KC, B_KC, 1, 2>(names[2], g, batch);
         return launch_dma<64, 64, 2, 2, 2, A_KC, B_KC, 1, 2>(names[2], g, batch);
     }
