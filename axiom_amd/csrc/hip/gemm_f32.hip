@@ -429,7 +429,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     using OA = DmaOperand<BM, A_KC, NW>;
     using OB = typename std::conditional<B_I8, DmaOperandI8<BN, NW>, DmaOperand<BN, B_KC, NW>>::type;
     // LDS: NST stages of A, then NST stages of B
-    static_assert(SPS == 1 || (SPS == 2 && !EDGE && !B_I8), "two slabs per stage: fp32 operands on whole tiles");
+    static_assert(SPS == 1 || (SPS == 2 && !EDGE), "two slabs per stage: whole tiles");
     constexpr int A_STAGE = SPS * OA::BYTES, B_STAGE = SPS * OB::BYTES;
     constexpr int B_BASE = NST * A_STAGE;
     constexpr int NREADS = TM * OA::READS + TN * OB::READS;
@@ -437,6 +437,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     // int8 B with four stages: the fragments of slab s + 1 are read while slab s is converted and multiplied, so the
     // loop's barrier must already cover slab s + 2 and one stage less is in flight
     constexpr bool PIPE = B_I8 && NST == 4;
+    static_assert(!PIPE || SPS == 1, "fragments read a slab ahead: one slab per stage");
     constexpr int VM_KEEP = (NST - (PIPE ? 3 : 2)) * SPS * (OA::IPW + OB::IPW);
     static_assert(NST >= 2 && NST <= 4 && VM_KEEP < 64, "stage count");
     static_assert(B_BASE + NST * B_STAGE <= 160 * 1024, "LDS budget");
@@ -555,7 +556,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         }                                                                                        \
         _Pragma("unroll") for (int t = 0; t < TN; t++) {                                         \
             if constexpr (B_I8) {                                                                \
-                AXF_DS32(fb[BUF][t].raw, rb[ST][KBI], t * 1024);                                 \
+                AXF_DS32(fb[BUF][t].raw, rb[ST][KBI], t * 1024 + (U) * OB::BYTES);               \
             } else if constexpr (B_KC) {                                                         \
                 AXF_DS128(fb[BUF][t].q, rb[ST][KBI], t * 4096 + (U) * OB::BYTES);                \
             } else {                                                                             \
@@ -617,18 +618,20 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
             AXF_PAIR(C0, C0 + 1);                                                                \
             if constexpr (WAVES_K == 1) AXF_PAIR(C0 + 2, C0 + 3);                                \
         } else if constexpr (B_I8) {                                                             \
-            AXF_FRAGS(0, ST, 0, 0);                                                              \
-            AXF_FRAGS(1, ST, 1, 0);                                                              \
-            if constexpr (WAVES_K == 1) {                                                        \
-                AXF_FRAGS(2, ST, 2, 0);                                                          \
-                AXF_FRAGS(3, ST, 3, 0);                                                          \
-                AXF_LGKM(2 * NREADS);                                                            \
-                AXF_PAIR(0, 1);                                                                  \
-                AXF_LGKM(0);                                                                     \
-                AXF_PAIR(2, 3);                                                                  \
-            } else {                                                                             \
-                AXF_LGKM(0);                                                                     \
-                AXF_PAIR(0, 1);                                                                  \
+            _Pragma("unroll") for (int u = 0; u < SPS; u++) {                                    \
+                AXF_FRAGS(0, ST, 0, u);                                                          \
+                AXF_FRAGS(1, ST, 1, u);                                                          \
+                if constexpr (WAVES_K == 1) {                                                    \
+                    AXF_FRAGS(2, ST, 2, u);                                                      \
+                    AXF_FRAGS(3, ST, 3, u);                                                      \
+                    AXF_LGKM(2 * NREADS);                                                        \
+                    AXF_PAIR(0, 1);                                                              \
+                    AXF_LGKM(0);                                                                 \
+                    AXF_PAIR(2, 3);                                                              \
+                } else {                                                                         \
+                    AXF_LGKM(0);                                                                 \
+                    AXF_PAIR(0, 1);                                                              \
+                }                                                                                \
             }                                                                                    \
         } else {                                                                                 \
             _Pragma("unroll") for (int u = 0; u < SPS; u++) {                                    \
@@ -650,7 +653,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         }                                                                                        \
         if (VM_KEEP > 0 && (more)) {                                                             \
             /* a wave past the int8 operand's load instructions has only A's in flight */        \
-            if (B_I8 && wave >= OB::NINSTR) AXF_VM((NST - (PIPE ? 3 : 2)) * OA::IPW); else AXF_VM(VM_KEEP); \
+            if (B_I8 && wave >= OB::NINSTR) AXF_VM((NST - (PIPE ? 3 : 2)) * SPS * OA::IPW); else AXF_VM(VM_KEEP); \
         } else AXF_VM(0);                                                                        \
         __builtin_amdgcn_s_barrier();                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                       \
@@ -1348,8 +1351,13 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
                     ((g.M + 63) / 64) * ((g.N + 63) / 64) <= 0x7fffffff;
     if (!ok) return -1;
     if (half_row_tiles(g.M) && g.K >= 64 && tuning().f32_tile == 0 && (tuning().w8a32_tile == 0 || g.K <= 128)) {   // as for fp32 operands
-        if (g.M % 32 == 0 && g.N % 64 == 0)
+        if (g.M % 32 == 0 && g.N % 64 == 0) {
+            // two slabs per stage where K allows: level with cached weights, ahead with the weights in HBM
+            // (32 x 4096 x 4096 12.7 / 15.8 -> 13.0 / 14.6 us, 96 x 4096 x 4096 23.6 / 24.8 -> 23.1 / 24.4)
+            if (g.K % 64 == 0)
+                return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, false, int8_t, 2>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
             return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
+        }
         return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, true, int8_t>("qgemm_w8a32_mfma_32x64k2_dma_edge", g, batch);
     }
     if (g.K > 128 && tuning().f32_tile == 0) {
@@ -1406,8 +1414,12 @@ int try_dma_i8(const char *const names[3], const SgemmArgs &g, int64_t batch) {
         // the last round of one 64x64 tile per CU mostly empty: 32x64 tiles, as for fp32 operands
         const int64_t whole = (g.M / 64) * (g.N / 64) * batch, rounds_whole = (whole + cus - 1) / cus,
                       rounds_half = (2 * whole + cus - 1) / cus;
-        if (tuning().f32_tile == 0 && rounds_half * 55 <= rounds_whole * 95)
+        if (tuning().f32_tile == 0 && rounds_half * 55 <= rounds_whole * 95) {
+            // (two slabs per stage, cached / from HBM: 128 x 4096 x 1024 12.9 / 14.5 -> 12.1 / 12.9 us, 128 x 3072 x 768 10.5 / 10.8 -> 9.9 / 10.1)
+            if (g.K % 64 == 0)
+                return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, false, int8_t, 2>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
             return launch_dma<32, 64, 1, 2, 2, true, true, 1, 2, false, int8_t>("qgemm_w8a32_mfma_32x64k2_dma", g, batch);
+        }
         return launch_dma<64, 64, 2, 2, 2, true, true, 1, 2, false, int8_t>(names[2], g, batch);
     }
     return launch_dma<64, 64, 2, 2, 2, true, true, 1, 1, false, int8_t>(names[1], g, batch);
