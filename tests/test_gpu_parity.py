@@ -153,6 +153,8 @@ F32_SHAPES = [(1, 1, 1), (2, 3, 2), (37, 19, 73), (64, 32, 128), (9, 500, 300), 
               (24, 11008, 512),
               # one round of tiles over a long K: three stages (operands past the L2s), and the K split when a fifth of the CUs would idle
               (256, 3072, 2048), (192, 2816, 4096),
+              # 64x64 tiles with the k split: two slabs per stage (K a multiple of 64; an odd and an even count of stages) and one (K = 160)
+              (256, 512, 192), (320, 256, 448), (256, 256, 256), (256, 512, 160),
               # off the tile grid with a large interior: fast kernels inside, guarded kernel on the fringes
               (1032, 1100, 96), (2100, 4200, 64), (1024, 1092, 160),
               (130, 257, 1027), (67, 1001, 129),                  # rows off the 16-byte grid in every form
@@ -716,6 +718,7 @@ W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 
                 (1, 20000, 520), (2, 16400, 300), (3, 8200, 1031), (6, 4100, 8200), (5, 4099, 2050), (4, 9000, 4100),
                 (6, 33, 10000), (1, 70, 20000),
                 (6, 4100, 8192), (5, 8192, 2048), (6, 64, 2048),   # five or six rows with a long K: the tiles
+                (128, 4096, 192), (96, 2048, 320), (128, 3072, 160),   # 32x64 tiles: two slabs per stage (three and five stages), one
                 (32, 128, 517), (70, 260, 1031), (3, 64, 1037)]   # rows at odd byte offsets
 
 
