@@ -438,6 +438,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     // loop's barrier must already cover slab s + 2 and one stage less is in flight
     constexpr bool PIPE = B_I8 && NST == 4;
     static_assert(!PIPE || SPS == 1, "fragments read a slab ahead: one slab per stage");
+    // the wait counts below assume every wave that loads the int8 operand issues the same number of its instructions
+    static_assert(!B_I8 || OB::NINSTR % NW == 0 || OB::NINSTR < NW, "int8 load instructions per wave");
     constexpr int VM_KEEP = (NST - (PIPE ? 3 : 2)) * SPS * (OA::IPW + OB::IPW);
     static_assert(NST >= 2 && NST <= 4 && VM_KEEP < 64, "stage count");
     static_assert(B_BASE + NST * B_STAGE <= 160 * 1024, "LDS budget");
