@@ -13,6 +13,7 @@ reference's benchmark format (benchmarks/bench_common.h:25-42) go to stderr.
                                         # for hardware-counter runs: a few launches of one case's kernels and 3
                                         # launches of a copy-shaped kernel of known size, no output line
     python bench.py --sustain 8 [--operands zeros]   # back-to-back headline launches, for clock sampling
+    python bench.py --hbm-ceiling                    # read / write / copy rates of this GPU on 2 GiB arrays, one JSON line
 """
 import argparse
 import ctypes as C
@@ -651,6 +652,24 @@ def counter_probe(hip, case, repeat=1):
     print(f"counter probe: {what}, then 3 x ReLU (k_unary<0>) over {n} floats", file=sys.stderr, flush=True)
 
 
+def hbm_ceiling(hip):
+    """What this GPU's memory delivers to the library's plainest streaming kernels, on arrays far larger than the 256 MB
+    Infinity Cache (2 GiB each): a read-only pass (sum of all elements), a write-only pass (fill), a copy (ReLU: one read,
+    one write per element).  The figures the bandwidth-bound kernels' fractions of the 8 TB/s datasheet peak are to be
+    read against.  One JSON line."""
+    n = 512 << 20
+    src, dst, one = hip.empty((n,)), hip.empty((n,)), hip.empty((1,))
+    hip.check(hip.L.axhip_fill_f32(src.ptr, 0.25, n))
+    res = {}
+    for name, fn, nbytes in (("read_sum_all", lambda: hip.check(hip.L.axhip_sum_all(src.ptr, n, one.ptr)), 4 * n),
+                             ("write_fill", lambda: hip.check(hip.L.axhip_fill_f32(dst.ptr, 1.0, n)), 4 * n),
+                             ("copy_relu", lambda: hip.check(hip.L.axhip_relu(src.ptr, dst.ptr, n)), 8 * n)):
+        fn()
+        _, ms = time_calls(hip, fn, seconds=0.5)
+        res[name] = {"us": ms * 1e3, "GB/s": nbytes / ms / 1e6, "frac_of_8TBs": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    print(json.dumps({"hbm_ceiling_2GiB_arrays": res, "device": hip.L.axhip_device_name().decode()}), flush=True)
+
+
 def sustain(hip, seconds, operands):
     """One GEMM launched back to back for `seconds`, so that clock and power can be sampled from outside
     (rocm-smi) while it runs: the headline over random int8 operands or all-zero ones (same instruction
@@ -790,6 +809,7 @@ def main():
                     choices=["headline", "skinny", "gemm1024", "fp32", "config2", "attention", "w8a32"])
     ap.add_argument("--probe-repeat", type=int, default=1, help="multiplies the launch counts of --counter-probe")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of back-to-back headline launches")
+    ap.add_argument("--hbm-ceiling", action="store_true", help="read / write / copy rates of this GPU on 2 GiB arrays")
     ap.add_argument("--operands", choices=["random", "zeros", "fp32", "fp32zeros", "qkt", "qktzeros", "pv", "pvzeros"], default="random")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -803,6 +823,9 @@ def main():
         return
     if args.sustain > 0:
         sustain(hip, args.sustain, args.operands)
+        return
+    if args.hbm_ceiling:
+        hbm_ceiling(hip)
         return
 
     h = headline(hip, args.steps, args.warmup)
