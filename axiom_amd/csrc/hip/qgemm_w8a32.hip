@@ -29,7 +29,21 @@ template <int MR, int R> constexpr int windows_per_step() {
     return 8 / R < most ? 8 / R : most;
 }
 
-template <int R, int U>
+// 16 weight bytes at any alignment.  STREAM marks the load non-temporal: every weight byte is read once per launch, and
+// large weights that come from HBM arrive faster that way (M = 1, weights in rotation: 4096 x 11008 16.2 -> 14.7 us,
+// 32000 x 4096 28.2 -> 26.4, 8192 x 8192 16.0 -> 15.3, 11008 x 4096 13.6 -> 13.3; M = 4, 32000 x 4096 50.9 -> 45.8), while
+// one matrix multiplied again and again out of the Infinity Cache loses as much (8192 x 4096, 33.5 MB: 6.5 -> 9.0 us
+// against 11.6 -> 11.5 from HBM).  The launchers set it from 40 MiB of weights on.
+typedef int v4i_any __attribute__((ext_vector_type(4), aligned(1)));
+template <bool STREAM>
+__device__ __forceinline__ v4i load16(const int8_t *p) {
+    if (STREAM) return __builtin_nontemporal_load(reinterpret_cast<const v4i_any *>(p));
+    v4i v;
+    __builtin_memcpy(&v, p, 16);
+    return v;
+}
+
+template <int R, int U, bool STREAM>
 __device__ __forceinline__ void w8a32_request(v4i (&dst)[R][U], const int8_t *w, int64_t first_row, int64_t N, int64_t k0, int lane,
                                               int64_t K, int used) {
 #pragma unroll
@@ -42,7 +56,7 @@ __device__ __forceinline__ void w8a32_request(v4i (&dst)[R][U], const int8_t *w,
             const int8_t *row = w + n * K;
             v4i p = {0, 0, 0, 0};
             if (k + 16 <= K) {
-                __builtin_memcpy(&p, row + k, 16);
+                p = load16<STREAM>(row + k);
             } else if (k < K) {
 #pragma unroll
                 for (int e = 0; e < 16; e++)
@@ -87,7 +101,7 @@ __device__ __forceinline__ void w8a32_multiply(const v4i (&src)[R][U], float (&a
 // slice: k values of the activations held in LDS at a time, a multiple of used * 1024.  groups: row groups of 4 * R
 // rows a workgroup walks one after the other (more than one only when a single slice holds all of K, so the
 // activations are staged once); the weight requests run ahead across group boundaries.
-template <int MR, int R>
+template <int MR, int R, bool STREAM>
 __global__ void __launch_bounds__(256)
 k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const float *__restrict__ w_scales,
              float *__restrict__ out, int64_t N, int64_t K, int slice, int groups, int used) {
@@ -137,7 +151,7 @@ k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const fl
             for (int mm = 0; mm < MR; mm++) acc[rr][mm] = 0.0f;
     };
     v4i wa[R][U], wb[R][U];
-    w8a32_request<R, U>(wa, w, base, N, 0, lane, K, used);      // before the activations: the latency of both overlaps
+    w8a32_request<R, U, STREAM>(wa, w, base, N, 0, lane, K, used);      // before the activations: the latency of both overlaps
     // One flat walk over (group, step): every quantity below is uniform over the workgroup.  Two steps per
     // round so that the two weight buffers keep their names.
     int g = 0, it = 0, in_slice = steps_per_slice;              // "slice full" forces the first staging
@@ -166,7 +180,7 @@ k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const fl
         enter();
         if (t + 1 < total) {
             const bool wrap = it + 1 == steps;
-            w8a32_request<R, U>(wb, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K, used);
+            w8a32_request<R, U, STREAM>(wb, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K, used);
         }
         w8a32_multiply<MR, R, U>(wa, acc, xs, quads, in_slice * used, lane, used);
         advance();
@@ -174,7 +188,7 @@ k_w8a32_rows(const float *__restrict__ a, const int8_t *__restrict__ w, const fl
         enter();
         if (t + 1 < total) {
             const bool wrap = it + 1 == steps;
-            w8a32_request<R, U>(wa, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K, used);
+            w8a32_request<R, U, STREAM>(wa, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K, used);
         }
         w8a32_multiply<MR, R, U>(wb, acc, xs, quads, in_slice * used, lane, used);
         advance();
@@ -194,7 +208,7 @@ struct W8a32DirectBuf {
     v4f x[MR][U][4];
 };
 
-template <int MR, int R, int U>
+template <int MR, int R, int U, bool STREAM>
 __device__ __forceinline__ void w8a32_direct_request(W8a32DirectBuf<MR, R, U> &b, const float *a, const int8_t *w, int64_t first_row,
                                                      int64_t N, int64_t k0, int lane, int64_t K, int used) {
 #pragma unroll
@@ -217,7 +231,7 @@ __device__ __forceinline__ void w8a32_direct_request(W8a32DirectBuf<MR, R, U> &b
             }
         }
     }
-    w8a32_request<R, U>(b.w, w, first_row, N, k0, lane, K, used);
+    w8a32_request<R, U, STREAM>(b.w, w, first_row, N, k0, lane, K, used);
 }
 
 template <int MR, int R, int U>
@@ -245,7 +259,7 @@ __device__ __forceinline__ void w8a32_direct_multiply(const W8a32DirectBuf<MR, R
     }
 }
 
-template <int MR, int R, int U>
+template <int MR, int R, int U, bool STREAM>
 __global__ void __launch_bounds__(256)
 k_w8a32_direct(const float *__restrict__ a, const int8_t *__restrict__ w, const float *__restrict__ w_scales,
                float *__restrict__ out, int64_t N, int64_t K, int groups, int used) {
@@ -259,7 +273,7 @@ k_w8a32_direct(const float *__restrict__ a, const int8_t *__restrict__ w, const 
     const int span = used * 1024;
     const int steps = (int)((K + span - 1) / span), total = groups * steps;
     W8a32DirectBuf<MR, R, U> ba, bb;
-    w8a32_direct_request<MR, R, U>(ba, a, w, base, N, 0, lane, K, used);
+    w8a32_direct_request<MR, R, U, STREAM>(ba, a, w, base, N, 0, lane, K, used);
     int g = 0, it = 0;
     auto finish = [&]() {                                       // the group's R * MR sums: over the wave, scaled, stored
         constexpr int NV = R * MR <= 1 ? 1 : R * MR <= 2 ? 2 : R * MR <= 4 ? 4 : R * MR <= 8 ? 8 : 16;
@@ -278,7 +292,7 @@ k_w8a32_direct(const float *__restrict__ a, const int8_t *__restrict__ w, const 
     };
     auto next_request = [&](W8a32DirectBuf<MR, R, U> &b) {      // operands of the step after (g, it)
         const bool wrap = it + 1 == steps;
-        w8a32_direct_request<MR, R, U>(b, a, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K,
+        w8a32_direct_request<MR, R, U, STREAM>(b, a, w, base + (int64_t)(g + wrap) * (4 * R), N, wrap ? 0 : (int64_t)(it + 1) * span, lane, K,
                                        used);
     };
     auto advance = [&]() {
@@ -309,7 +323,10 @@ int launch_direct(const float *a, const int8_t *w, const float *s, float *out, i
     if (groups < 1) groups = 1;
     if (groups > 64) groups = 64;
     const int64_t rows_per_block = 4 * R * groups, blocks = (N + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL((k_w8a32_direct<MR, R, U>), dim3((unsigned)blocks), dim3(256), 0, kStream, a, w, s, out, N, K, (int)groups, used);
+    if (N * K >= (int64_t(40) << 20))
+        hipLaunchKernelGGL((k_w8a32_direct<MR, R, U, true>), dim3((unsigned)blocks), dim3(256), 0, kStream, a, w, s, out, N, K, (int)groups, used);
+    else
+        hipLaunchKernelGGL((k_w8a32_direct<MR, R, U, false>), dim3((unsigned)blocks), dim3(256), 0, kStream, a, w, s, out, N, K, (int)groups, used);
     return check_launch("qgemm_w8a32_gemv");
 }
 
@@ -335,11 +352,14 @@ int launch_rows(const float *a, const int8_t *w, const float *s, float *out, int
         if (groups > 64) groups = 64;
     }
     const size_t smem = (size_t)MR * slice * sizeof(float);
-    auto kern = k_w8a32_rows<MR, R>;
+    const bool stream = N * K >= (int64_t(40) << 20);
+    auto kern = stream ? k_w8a32_rows<MR, R, true> : k_w8a32_rows<MR, R, false>;
     static bool attr_set = false;
     if (!attr_set) {
-        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 65536),
-                      "hipFuncSetAttribute");
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_w8a32_rows<MR, R, true>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 65536), "hipFuncSetAttribute");
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k_w8a32_rows<MR, R, false>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 65536), "hipFuncSetAttribute");
         attr_set = true;
     }
     const int64_t rows_per_block = 4 * R * groups, blocks = (N + rows_per_block - 1) / rows_per_block;

@@ -800,6 +800,22 @@ def test_w8a32_three_bf16_terms_are_exact(hip, oracle):
     assert (np.abs(got - want) <= np.abs(want) * 2.0 ** -23).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(2, 10300, 4100), (1, 11008, 4096), (5, 10500, 4004), (4, 2000, 21000)])
+def test_w8a32_streaming_loads(hip, M, N, K):
+    """40 MiB of weights and more: the weight-streaming forms read them with non-temporal loads (rows at 4-byte alignment
+    among them).  Same arithmetic, so the same fp64 bound as every other form."""
+    say("w8a32 streaming", M, N, K)
+    rng = np.random.default_rng(M * N + K)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    ws = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    got = hip.qgemm_w8a32(hip.array(a), hip.array(w), hip.array(ws)).numpy()
+    assert hip.last_kernel() == "qgemm_w8a32_gemv"
+    want = (a.astype(np.float64) @ w.astype(np.float64).T) * ws
+    bound = BOUND_FP32 * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64).T) * ws + 1e-30
+    assert (np.abs(got - want) <= bound).all(), float((np.abs(got - want) / bound).max())
+
+
 def test_w8a32_tiny_activations(hip):
     """The bf16 matrix core flushes denormal operands, so the low-order bf16 terms of activations below 2^-110 are
     dropped: the result stays within the fp32 bound plus K * 2^-118 per output, whatever the scale of the activations."""
