@@ -282,6 +282,11 @@ int validate(const char *who, int transa, int transb, int64_t M, int64_t N, int6
 // write-back moves 16 bytes per lane.
 #define AXF_LGKM(n) __builtin_amdgcn_s_waitcnt(0x3F | (3 << 14) | (7 << 4) | (((n) > 15 ? 15 : (n)) << 8))
 #define AXF_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
+// the same for an operand that is read once and is too large to be met again in the caches (non-temporal)
+#define AXF_LOAD_LDS_NT(m0val, voff, base)                                                    \
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m0val), \
+                 "v"(voff), "s"(base)                                                         \
+                 : "memory")
 #define AXF_LOAD_LDS(m0val, voff, base)                                                       \
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0val), \
                  "v"(voff), "s"(base)                                                         \
@@ -1114,7 +1119,8 @@ __global__ void __launch_bounds__(256) k_sgemm_nn_stream(SgemmArgs g, int batch,
 #define AXS_ISSUE()                                                                              \
     do {                                                                                         \
         _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                                      \
-            AXF_LOAD_LDS(dma_a + load_a + j * NW * OA::PITCH, va[j], ga);                        \
+            /* A (the scores of P V, 537 MB at 512 heads) is read once: 157.5 -> 153.3 us */    \
+            AXF_LOAD_LDS_NT(dma_a + load_a + j * NW * OA::PITCH, va[j], ga);                     \
         _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                                      \
             AXF_LOAD_LDS(dma_b + load_b + j * NW * OB::PITCH, vb[j], gb);                        \
         load_a = load_a == (NST - 1) * OA::BYTES ? 0 : load_a + OA::BYTES;                       \
