@@ -28,6 +28,7 @@ struct SgemmArgs {
     const float *col_scale;                // multiplies column n after alpha (W8A32), or NULL
     const float *bias;
     int act;
+    int stream_b;                          // B is read once and is large: fetch it with non-temporal loads
 };
 
 // One operand's slab: R rows (M or N extent of the tile) x BK.
@@ -532,16 +533,19 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
             }                                                                                    \
             _Pragma("unroll") for (int j = 0; j < OB::IPW; j++) {                                \
                 const unsigned at = B_BASE + wave * OB::PITCH + (ST) * B_STAGE + j * NW * OB::PITCH; \
-                if (tb[j]) AXF_LOAD_LDS(lds0 + at, vb[j], gb);                                   \
-                else *reinterpret_cast<v4f *>(lds_raw + at + lane * 16) = v4f{0.f, 0.f, 0.f, 0.f}; \
+                if (!tb[j]) *reinterpret_cast<v4f *>(lds_raw + at + lane * 16) = v4f{0.f, 0.f, 0.f, 0.f}; \
+                else if (g.stream_b) AXF_LOAD_LDS_NT(lds0 + at, vb[j], gb);                      \
+                else AXF_LOAD_LDS(lds0 + at, vb[j], gb);                                         \
             }                                                                                    \
         } else {                                                                                 \
             _Pragma("unroll") for (int u = 0; u < SPS; u++) {                                    \
                 _Pragma("unroll") for (int j = 0; j < OA::IPW; j++)                              \
                     AXF_LOAD_LDS(dma_a + (ST) * A_STAGE + u * OA::BYTES + j * NW * OA::PITCH, va[j], ga + u * step_a); \
                 _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                              \
-                    if (!B_I8 || j * NW + wave < OB::NINSTR)                                     \
-                        AXF_LOAD_LDS(dma_b + B_BASE + (ST) * B_STAGE + u * OB::BYTES + j * NW * OB::PITCH, vb[j], gb + u * step_b); \
+                    if (!B_I8 || j * NW + wave < OB::NINSTR) {                                   \
+                        if (g.stream_b) AXF_LOAD_LDS_NT(dma_b + B_BASE + (ST) * B_STAGE + u * OB::BYTES + j * NW * OB::PITCH, vb[j], gb + u * step_b); \
+                        else AXF_LOAD_LDS(dma_b + B_BASE + (ST) * B_STAGE + u * OB::BYTES + j * NW * OB::PITCH, vb[j], gb + u * step_b); \
+                    }                                                                            \
             }                                                                                    \
         }                                                                                        \
         ga += SPS * step_a;                                                                      \
@@ -831,8 +835,16 @@ int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
         attr_set = true;
     }
     const int64_t tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+    // One row of tiles reads every byte of B once: large fp32 weights then arrive faster through non-temporal loads
+    // (the K ranges of a split and the entries of a batch count together).  Weights in rotation, plain -> non-temporal:
+    // 16 x 4096 x 4096 21.0 -> 19.3 us, 16 x 11008 x 4096 38.5 -> 36.3, 32 x 8192 x 8192 57.0 -> 53.2; the same matrix
+    // multiplied back to back out of the caches loses 3-12 %, which only a benchmark loop does.  Not for int8 weights: a
+    // slab takes 32 bytes of each of their 128-byte lines, and a line that is not kept is fetched four times
+    // (8 x 11008 x 4096: 25.0 -> 31.0 us).
+    SgemmArgs h = g;
+    h.stream_b = sizeof(BSRC) == 4 && g.M <= BM && g.N * g.K * 4 * batch >= (int64_t(32) << 20);
     note_kernel(name);
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)batch), dim3(NW * 64), smem, kStream, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)batch), dim3(NW * 64), smem, kStream, h);
     return check_launch(name);
 }
 
