@@ -226,6 +226,11 @@ int launch(const char *name, const int8_t *x, float x_scale, const int8_t *w,
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0val), \
                  "v"(voff), "s"(base)                                                        \
                  : "memory")
+// the same for an operand that is read once and is too large to be met again in the caches (non-temporal)
+#define AXI8_LOAD_LDS_NT(m0val, voff, base)                                                  \
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m0val), \
+                 "v"(voff), "s"(base)                                                        \
+                 : "memory")
 
 template <int ACT>
 __global__ void __launch_bounds__(512)
@@ -549,7 +554,7 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
                  int64_t K, float x_scale, const float *__restrict__ w_scales,
                  const float *__restrict__ bias, float *__restrict__ out,
                  int32_t *__restrict__ acc_out, int64_t ldc, int splits, int32_t *partials,
-                 int *__restrict__ counters, int phases) {
+                 int *__restrict__ counters, int phases, int stream_w) {
     constexpr int NWO = WAVES_M * WAVES_N, NW = NWO * WAVES_K, BKB = 128;      // waves that own outputs / all waves
     constexpr int KSTEPS = 4 / WAVES_K;                                        // k-steps of a slab per wave
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
@@ -654,14 +659,17 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
             }                                                                                    \
             _Pragma("unroll") for (int j = 0; j < IPW_W; j++) {                                  \
                 const unsigned at = wave * 1024 + W_BASE + (ST) * WS + j * NW * 1024;            \
-                if (tw[j]) AXI8_LOAD_LDS(lds0 + at, vw[j], gw);                                  \
-                else *reinterpret_cast<v4i *>(lds + at + lane * 16) = v4i{0, 0, 0, 0};           \
+                if (!tw[j]) *reinterpret_cast<v4i *>(lds + at + lane * 16) = v4i{0, 0, 0, 0};    \
+                else if (stream_w) AXI8_LOAD_LDS_NT(lds0 + at, vw[j], gw);                       \
+                else AXI8_LOAD_LDS(lds0 + at, vw[j], gw);                                        \
             }                                                                                    \
         } else {                                                                                 \
             _Pragma("unroll") for (int j = 0; j < IPW_X; j++)                                    \
                 AXI8_LOAD_LDS(lds_w + (ST) * XS + j * NW * 1024, vx[j], gx);                     \
-            _Pragma("unroll") for (int j = 0; j < IPW_W; j++)                                    \
-                AXI8_LOAD_LDS(lds_w + W_BASE + (ST) * WS + j * NW * 1024, vw[j], gw);            \
+            _Pragma("unroll") for (int j = 0; j < IPW_W; j++) {                                  \
+                if (stream_w) AXI8_LOAD_LDS_NT(lds_w + W_BASE + (ST) * WS + j * NW * 1024, vw[j], gw); \
+                else AXI8_LOAD_LDS(lds_w + W_BASE + (ST) * WS + j * NW * 1024, vw[j], gw);       \
+            }                                                                                    \
         }                                                                                        \
         gx += BKB;                                                                               \
         gw += BKB;                                                                               \
@@ -895,7 +903,7 @@ int launch_dma(const char *name, const char *split_name, const int8_t *x, float 
                int64_t K, int64_t ldc) {
     constexpr int smem = NST * SPB * (BM + BN) * 128 + 2 * BN * 4 + 16;      // stages, scale and bias rows, the split join's flag
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
-                           const float *, float *, int32_t *, int64_t, int, int32_t *, int *, int);
+                           const float *, float *, int32_t *, int64_t, int, int32_t *, int *, int, int);
     static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE, WAVES_K, SPB>,
                                     k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU, EDGE, WAVES_K, SPB>,
                                     k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE, WAVES_K, SPB>};
@@ -924,9 +932,13 @@ int launch_dma(const char *name, const char *split_name, const int8_t *x, float 
     // is fetched once per sharer (512 x 4096 x 11008: 31.6 -> 52.2 us): one round of tiles, all of X and an eighth
     // of W within 3 MiB (at 4 MiB, 512 x 4096 x 4096 on 128x64 tiles: 18.0 -> 16.6 us from HBM but 14.0 -> 15.1 cached).
     const int phases = (K % 128 == 0 && tiles <= cu_count() && (M + N / 8) * K <= (int64_t(3) << 20)) ? 4 : 0;
+    // one row of tiles reads every byte of W once: 40 MiB of weights and more then arrive faster through non-temporal
+    // loads (a slab here is a whole 128-byte line of every weight row, so nothing is fetched twice)
+    // (weights in rotation: 8 x 11008 x 4096 13.9 -> 13.2 us, 64 x 8192 x 8192 20.1 -> 18.8, 16 x 4096 x 11008 14.6 -> 13.5)
+    const int stream_w = (M <= BM && N * K >= (int64_t(40) << 20)) ? 1 : 0;
     note_kernel(splits > 1 ? split_name : name);
     hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles, (unsigned)splits), dim3(WAVES_M * WAVES_N * WAVES_K * 64), smem, kStream,
-                       x, w, M, N, K, x_scale, w_scales, bias, out, acc_out, ldc, splits, partials, counters, phases);
+                       x, w, M, N, K, x_scale, w_scales, bias, out, acc_out, ldc, splits, partials, counters, phases, stream_w);
     return check_launch(name);
 }
 

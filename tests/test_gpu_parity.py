@@ -82,6 +82,21 @@ def test_w8a8_accumulators_bit_exact(hip, oracle, M, N, K):
     assert np.array_equal(acc.numpy(), want_acc)
 
 
+@pytest.mark.parametrize("M,N,K", [(8, 11008, 4096), (64, 8192, 5120), (16, 4100, 11008)])
+def test_w8a8_streaming_weights_bit_exact(hip, M, N, K):
+    """One row of tiles against 40 MiB of weights and more: the weights are fetched with non-temporal loads.  The int32
+    accumulators stay exact (checked against an fp64 product, which is exact at these magnitudes)."""
+    say("w8a8 streaming", M, N, K)
+    rng = np.random.default_rng(M + N + K)
+    x = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    _, acc = hip.qgemm_w8a8(hip.array(x), 0.01, hip.array(w), None, None, 0, want_out=False)
+    say("  kernel", hip.last_kernel())
+    assert hip.last_kernel().startswith("qgemm_w8a8_64x64")
+    want = (x.astype(np.float64) @ w.astype(np.float64).T).astype(np.int64)
+    assert np.array_equal(acc.numpy().astype(np.int64), want)
+
+
 def test_w8a8_extreme_values_and_golden(hip, oracle, golden):
     x = np.full((128, 8192), -127, np.int8)
     w = np.full((128, 8192), -127, np.int8)
