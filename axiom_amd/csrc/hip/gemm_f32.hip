@@ -328,10 +328,12 @@ struct DmaOperand {
 
 // An int8 operand stored [rows, K] (K contiguous; the weights of the W8A32 product): a slab is 32 bytes
 // per row, one load instruction carries 32 rows (lane l -> row l >> 1, 16-byte half l & 1), and only the
-// first NINSTR waves have one to issue.  A fragment is one ds_read_b32 — a lane's four k values of a
-// k-block — converted to bf16 in registers right before use (bf16_of_i8 below), so LDS and the loads
-// carry a quarter of the bytes of an fp32 operand.  (Rows 32 bytes apart put the 32 lanes of a read on
-// 8 banks: a 4-way conflict on a read that is a quarter of the other operand's.)
+// first NINSTR waves have one to issue.  A fragment is one ds_read_b64 per pair of k-blocks — the lane's
+// eight consecutive k values, which is exactly one bf16 MFMA operand — converted to bf16 in registers right
+// before use (bf16_of_i8 below), so LDS and the loads carry a quarter of the bytes of an fp32 operand; the
+// fp32 operand is read to match (two 16-byte chunks side by side).  Reading the eight bytes at once instead
+// of four per k-block halves the LDS instructions of this operand: 4096^3 342 -> 331 us, 1024 x 4096 x 4096
+// 104.6 -> 96.8.  (Rows 32 bytes apart put the 32 lanes of a read on 8 banks: a 4-way conflict.)
 template <int R, int NW>
 struct DmaOperandI8 {
     static constexpr int PITCH = 1024;
@@ -344,15 +346,17 @@ struct DmaOperandI8 {
         const int row = q * 32 + (lane >> 1);
         return (unsigned)((row < valid ? row : valid - 1) * ld + (lane & 1) * 16);
     }
+    // a lane's 8 bytes of the pair of k-blocks kbi belongs to: k = 16 (kbi / 2) + 8 fhalf ..
     __device__ static unsigned frag_base(int first, int frow, int fhalf, int kbi) {
-        return (unsigned)((first + frow) * 32 + kbi * 8 + fhalf * 4);
+        return (unsigned)((first + frow) * 32 + (kbi >> 1) * 16 + fhalf * 8);
     }
     static constexpr int k_imm(int) { return 0; }
 };
 
 struct FragI8 {
-    int raw;       // k = 4 * (lane >> 5) + e of the k-block in byte e
-    __device__ __forceinline__ float get(int e) const { return (float)(signed char)(raw >> (8 * e)); }   // fp32 form, unused by the bf16 products
+    int2 raw;      // the lane's 8 consecutive k values of a pair of k-blocks (16 k): k = 8 * (lane >> 5) + byte index; held in
+                   // the even k-block's buffer, the odd one's stays unused
+    __device__ __forceinline__ float get(int e) const { return (float)(signed char)(raw.x >> (8 * e)); }   // fp32 form, unused by the bf16 products
 };
 
 // fp32 x int8 products on the bf16 matrix core, with fp32 accuracy.  Every int8 value is a bf16 exactly.  An fp32
@@ -412,6 +416,7 @@ template <> struct Frag<false> {
 
 #define AXF_DS128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 #define AXF_DS32(dst, addr, off) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
+#define AXF_DS64(dst, addr, off) asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 
 // EDGE: M and N need not be multiples of the tile (N a multiple of 4, and M too when A is stored
 // M-contiguous) nor K of the slab (K a multiple of 4).  Edge tiles fetch the last existing row /
@@ -439,6 +444,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
     constexpr int A_STAGE = SPS * OA::BYTES, B_STAGE = SPS * OB::BYTES;
     constexpr int B_BASE = NST * A_STAGE;
     constexpr int NREADS = TM * OA::READS + TN * OB::READS;
+    constexpr int NREADS_PAIR = 2 * TM * OA::READS + TN;      // int8 B: LDS reads of a pair of k-blocks (B once per pair)
     // loads a wave may leave in flight at the end of a slab: everything but the next slab's
     // int8 B with four stages: the fragments of slab s + 1 are read while slab s is converted and multiplied, so the
     // loop's barrier must already cover slab s + 2 and one stage less is in flight
@@ -504,7 +510,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         for (int kbi = 0; kbi < 4; kbi++) {
             // with a k split, entries 0 and 1 address this wave set's own two k-blocks
             const int kb = WAVES_K == 2 ? 2 * wk + (kbi & 1) : kbi;
-            ra[st][kbi] = lds0 + st * A_STAGE + OA::frag_base(wm * WTM, frow, fhalf, kb) +
+            // with int8 B a lane holds 8 consecutive k of a pair of k-blocks (as its 8 weight bytes lie): the fragment of
+            // k-block 2 P + j is the 16-byte chunk 4 P + 2 fhalf + j of the row
+            ra[st][kbi] = lds0 + st * A_STAGE + (B_I8 ? OA::frag_base(wm * WTM, frow, kb & 1, (kb & ~1) + fhalf)
+                                                      : OA::frag_base(wm * WTM, frow, fhalf, kb)) +
                           (WAVES_K == 2 && !A_KC ? wk * OA::k_imm(16) : 0);
             rb[st][kbi] = lds0 + B_BASE + st * B_STAGE + OB::frag_base(wn * WTN, frow, fhalf, kb) +
                           (WAVES_K == 2 && !B_KC ? wk * OB::k_imm(16) : 0);
@@ -567,7 +576,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         }                                                                                        \
         _Pragma("unroll") for (int t = 0; t < TN; t++) {                                         \
             if constexpr (B_I8) {                                                                \
-                AXF_DS32(fb[BUF][t].raw, rb[ST][KBI], t * 1024 + (U) * OB::BYTES);               \
+                if ((KBI) % 2 == 0) AXF_DS64(fb[BUF][t].raw, rb[ST][KBI], t * 1024 + (U) * OB::BYTES); \
             } else if constexpr (B_KC) {                                                         \
                 AXF_DS128(fb[BUF][t].q, rb[ST][KBI], t * 4096 + (U) * OB::BYTES);                \
             } else {                                                                             \
@@ -599,7 +608,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
         Bf16x3 ax[TM];                                                                           \
         v4i bx[TN];                                                                              \
         _Pragma("unroll") for (int i = 0; i < TM; i++) ax[i] = bf16x3_of(fa[B0][i].q, fa[B1][i].q); \
-        _Pragma("unroll") for (int j = 0; j < TN; j++) bx[j] = bf16_of_i8(fb[B0][j].raw, fb[B1][j].raw); \
+        _Pragma("unroll") for (int j = 0; j < TN; j++) bx[j] = bf16_of_i8(fb[B0][j].raw.x, fb[B0][j].raw.y); \
         __builtin_amdgcn_sched_barrier(0);                                                       \
         _Pragma("unroll") for (int t = 0; t < 3; t++)                                            \
             _Pragma("unroll") for (int i = 0; i < TM; i++)                                       \
@@ -624,7 +633,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
                     AXF_FRAGS(N0 + 2, NS, 2, 0);                                                 \
                     AXF_FRAGS(N0 + 3, NS, 3, 0);                                                 \
                 }                                                                                \
-                AXF_LGKM((WAVES_K == 1 ? 4 : 2) * NREADS);                                       \
+                AXF_LGKM((WAVES_K == 1 ? 2 : 1) * NREADS_PAIR);                                  \
             } else AXF_LGKM(0);                                                                  \
             AXF_PAIR(C0, C0 + 1);                                                                \
             if constexpr (WAVES_K == 1) AXF_PAIR(C0 + 2, C0 + 3);                                \
@@ -635,7 +644,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
                 if constexpr (WAVES_K == 1) {                                                    \
                     AXF_FRAGS(2, ST, 2, u);                                                      \
                     AXF_FRAGS(3, ST, 3, u);                                                      \
-                    AXF_LGKM(2 * NREADS);                                                        \
+                    AXF_LGKM(NREADS_PAIR);                                                       \
                     AXF_PAIR(0, 1);                                                              \
                     AXF_LGKM(0);                                                                 \
                     AXF_PAIR(2, 3);                                                              \
