@@ -28,7 +28,6 @@ struct SgemmArgs {
     const float *col_scale;                // multiplies column n after alpha (W8A32), or NULL
     const float *bias;
     int act;
-    int stream_b;                          // B is read once and is large: fetch it with non-temporal loads
 };
 
 // One operand's slab: R rows (M or N extent of the tile) x BK.
@@ -424,8 +423,10 @@ template <> struct Frag<false> {
 // and guard the write-back; in the last slab, lanes whose k values lie past K write zeros to
 // their LDS place instead of loading, in both operands, so the tail adds exact zeros.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_KC, int EPI, int WAVES_K,
-          bool EDGE = false, typename BSRC = float, int SPS = 1>
+          bool EDGE = false, typename BSRC = float, int SPS = 1, bool STREAM_B = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(SgemmArgs g) {
+    // STREAM_B: B is read once and is large, its loads are non-temporal (a template parameter: a run-time test in
+    // front of every load costs the tiles that do not stream 3-11 %)
     // SPS == 2: a stage holds two slabs (64 k) and the loop's barrier comes once per stage — for tiles whose slab is
     // only a few MFMAs per wave, where the barrier is a visible share of the slab (K a multiple of 64, no edge form)
     // WAVES_K == 2: a second set of waves shares each tile; set 0 multiplies k-blocks 0 and 1 of
@@ -543,7 +544,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
             _Pragma("unroll") for (int j = 0; j < OB::IPW; j++) {                                \
                 const unsigned at = B_BASE + wave * OB::PITCH + (ST) * B_STAGE + j * NW * OB::PITCH; \
                 if (!tb[j]) *reinterpret_cast<v4f *>(lds_raw + at + lane * 16) = v4f{0.f, 0.f, 0.f, 0.f}; \
-                else if (g.stream_b) AXF_LOAD_LDS_NT(lds0 + at, vb[j], gb);                      \
+                else if (STREAM_B) AXF_LOAD_LDS_NT(lds0 + at, vb[j], gb);                      \
                 else AXF_LOAD_LDS(lds0 + at, vb[j], gb);                                         \
             }                                                                                    \
         } else {                                                                                 \
@@ -552,7 +553,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64) k_sgemm_dma(Sg
                     AXF_LOAD_LDS(dma_a + (ST) * A_STAGE + u * OA::BYTES + j * NW * OA::PITCH, va[j], ga + u * step_a); \
                 _Pragma("unroll") for (int j = 0; j < OB::IPW; j++)                              \
                     if (!B_I8 || j * NW + wave < OB::NINSTR) {                                   \
-                        if (g.stream_b) AXF_LOAD_LDS_NT(dma_b + B_BASE + (ST) * B_STAGE + u * OB::BYTES + j * NW * OB::PITCH, vb[j], gb + u * step_b); \
+                        if (STREAM_B) AXF_LOAD_LDS_NT(dma_b + B_BASE + (ST) * B_STAGE + u * OB::BYTES + j * NW * OB::PITCH, vb[j], gb + u * step_b); \
                         else AXF_LOAD_LDS(dma_b + B_BASE + (ST) * B_STAGE + u * OB::BYTES + j * NW * OB::PITCH, vb[j], gb + u * step_b); \
                     }                                                                            \
             }                                                                                    \
@@ -829,31 +830,33 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool A_KC, bool B_K
           bool EDGE = false, typename BSRC = float, int SPS = 1>
 int launch_dma(const char *name, const SgemmArgs &g, int64_t batch) {
     static_assert(!EDGE || EPI == 1, "the edge form guards the turned write-back only");
-    auto kern = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K, EDGE, BSRC, SPS>;
     constexpr int NW = WAVES_M * WAVES_N * WAVES_K;
     using OB = typename std::conditional<sizeof(BSRC) == 1, DmaOperandI8<BN, NW>, DmaOperand<BN, B_KC, NW>>::type;
     constexpr int stage_bytes = NST * SPS * (DmaOperand<BM, A_KC, NW>::BYTES + OB::BYTES);
     // the write-back turns 4 KiB per output wave through the dead stages
     constexpr int after = WAVES_K == 2 ? BM * BN * 4 : WAVES_M * WAVES_N * 4096;   // the join of a k split needs the whole tile
     constexpr int smem = stage_bytes > after ? stage_bytes : after;
-    static bool attr_set = false;
-    if (!attr_set) {
-        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem),
-                      "hipFuncSetAttribute");
-        attr_set = true;
-    }
-    const int64_t tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     // One row of tiles reads every byte of B once: large fp32 weights then arrive faster through non-temporal loads
     // (the K ranges of a split and the entries of a batch count together).  Weights in rotation, plain -> non-temporal:
     // 16 x 4096 x 4096 21.0 -> 19.3 us, 16 x 11008 x 4096 38.5 -> 36.3, 32 x 8192 x 8192 57.0 -> 53.2; the same matrix
     // multiplied back to back out of the caches loses 3-12 %, which only a benchmark loop does.  Not for int8 weights: a
     // slab takes 32 bytes of each of their 128-byte lines, and a line that is not kept is fetched four times
-    // (8 x 11008 x 4096: 25.0 -> 31.0 us).
-    SgemmArgs h = g;
-    h.stream_b = sizeof(BSRC) == 4 && g.M <= BM && g.N * g.K * 4 * batch >= (int64_t(32) << 20);
+    // (8 x 11008 x 4096: 25.0 -> 31.0 us).  Built for the tiles of at most 64 rows, which are the ones few rows get.
+    constexpr bool CAN_STREAM = sizeof(BSRC) == 4 && BM <= 64;
+    const bool stream_b = CAN_STREAM && g.M <= BM && g.N * g.K * 4 * batch >= (int64_t(32) << 20);
+    auto plain = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K, EDGE, BSRC, SPS, false>;
+    auto streams = k_sgemm_dma<BM, BN, WAVES_M, WAVES_N, NST, A_KC, B_KC, EPI, WAVES_K, EDGE, BSRC, SPS, CAN_STREAM>;
+    auto kern = stream_b ? streams : plain;
+    static bool attr_set[2] = {false, false};
+    if (!attr_set[stream_b]) {
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem),
+                      "hipFuncSetAttribute");
+        attr_set[stream_b] = true;
+    }
+    const int64_t tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     note_kernel(name);
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)batch), dim3(NW * 64), smem, kStream, h);
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)batch), dim3(NW * 64), smem, kStream, g);
     return check_launch(name);
 }
 

@@ -548,13 +548,16 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 // waves on every SIMD with no more global traffic, so one wave's waits for LDS and for the slab
 // barrier are covered by the other's MFMAs: for a launch of at most one small tile per CU, whose
 // time is the chain of those waits rather than memory or matrix-core throughput.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int ACT, bool EDGE = false, int WAVES_K = 1, int SPB = 1>
+// STREAM_W: the weights are read once and are large, their loads are non-temporal (a template parameter: a run-time
+// test in front of every load costs the launches that do not stream 3-5 %).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int ACT, bool EDGE = false, int WAVES_K = 1, int SPB = 1,
+          bool STREAM_W = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N *WAVES_K * 64)
 k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
                  int64_t K, float x_scale, const float *__restrict__ w_scales,
                  const float *__restrict__ bias, float *__restrict__ out,
                  int32_t *__restrict__ acc_out, int64_t ldc, int splits, int32_t *partials,
-                 int *__restrict__ counters, int phases, int stream_w) {
+                 int *__restrict__ counters, int phases) {
     constexpr int NWO = WAVES_M * WAVES_N, NW = NWO * WAVES_K, BKB = 128;      // waves that own outputs / all waves
     constexpr int KSTEPS = 4 / WAVES_K;                                        // k-steps of a slab per wave
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
@@ -660,14 +663,14 @@ k_qgemm_w8a8_dma(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
             _Pragma("unroll") for (int j = 0; j < IPW_W; j++) {                                  \
                 const unsigned at = wave * 1024 + W_BASE + (ST) * WS + j * NW * 1024;            \
                 if (!tw[j]) *reinterpret_cast<v4i *>(lds + at + lane * 16) = v4i{0, 0, 0, 0};    \
-                else if (stream_w) AXI8_LOAD_LDS_NT(lds0 + at, vw[j], gw);                       \
+                else if (STREAM_W) AXI8_LOAD_LDS_NT(lds0 + at, vw[j], gw);                       \
                 else AXI8_LOAD_LDS(lds0 + at, vw[j], gw);                                        \
             }                                                                                    \
         } else {                                                                                 \
             _Pragma("unroll") for (int j = 0; j < IPW_X; j++)                                    \
                 AXI8_LOAD_LDS(lds_w + (ST) * XS + j * NW * 1024, vx[j], gx);                     \
             _Pragma("unroll") for (int j = 0; j < IPW_W; j++) {                                  \
-                if (stream_w) AXI8_LOAD_LDS_NT(lds_w + W_BASE + (ST) * WS + j * NW * 1024, vw[j], gw); \
+                if (STREAM_W) AXI8_LOAD_LDS_NT(lds_w + W_BASE + (ST) * WS + j * NW * 1024, vw[j], gw); \
                 else AXI8_LOAD_LDS(lds_w + W_BASE + (ST) * WS + j * NW * 1024, vw[j], gw);       \
             }                                                                                    \
         }                                                                                        \
@@ -903,10 +906,15 @@ int launch_dma(const char *name, const char *split_name, const int8_t *x, float 
                int64_t K, int64_t ldc) {
     constexpr int smem = NST * SPB * (BM + BN) * 128 + 2 * BN * 4 + 16;      // stages, scale and bias rows, the split join's flag
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
-                           const float *, float *, int32_t *, int64_t, int, int32_t *, int *, int, int);
-    static const kern_t kerns[3] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE, WAVES_K, SPB>,
+                           const float *, float *, int32_t *, int64_t, int, int32_t *, int *, int);
+    // the streaming forms are built for the tiles of at most 64 rows, which are the ones few rows get
+    constexpr bool CAN_STREAM = BM <= 64;
+    static const kern_t kerns[6] = {k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE, WAVES_K, SPB>,
                                     k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU, EDGE, WAVES_K, SPB>,
-                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE, WAVES_K, SPB>};
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE, WAVES_K, SPB>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_NONE, EDGE, WAVES_K, SPB, CAN_STREAM>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_RELU, EDGE, WAVES_K, SPB, CAN_STREAM>,
+                                    k_qgemm_w8a8_dma<BM, BN, WAVES_M, WAVES_N, NST, AXHIP_ACT_GELU, EDGE, WAVES_K, SPB, CAN_STREAM>};
     static bool attr_set = false;
     if (!attr_set) {
         for (kern_t kf : kerns)
@@ -935,10 +943,10 @@ int launch_dma(const char *name, const char *split_name, const int8_t *x, float 
     // one row of tiles reads every byte of W once: 40 MiB of weights and more then arrive faster through non-temporal
     // loads (a slab here is a whole 128-byte line of every weight row, so nothing is fetched twice)
     // (weights in rotation: 8 x 11008 x 4096 13.9 -> 13.2 us, 64 x 8192 x 8192 20.1 -> 18.8, 16 x 4096 x 11008 14.6 -> 13.5)
-    const int stream_w = (M <= BM && N * K >= (int64_t(40) << 20)) ? 1 : 0;
+    const int stream_w = (CAN_STREAM && M <= BM && N * K >= (int64_t(40) << 20)) ? 3 : 0;
     note_kernel(splits > 1 ? split_name : name);
-    hipLaunchKernelGGL(kerns[act], dim3((unsigned)tiles, (unsigned)splits), dim3(WAVES_M * WAVES_N * WAVES_K * 64), smem, kStream,
-                       x, w, M, N, K, x_scale, w_scales, bias, out, acc_out, ldc, splits, partials, counters, phases, stream_w);
+    hipLaunchKernelGGL(kerns[act + stream_w], dim3((unsigned)tiles, (unsigned)splits), dim3(WAVES_M * WAVES_N * WAVES_K * 64), smem, kStream,
+                       x, w, M, N, K, x_scale, w_scales, bias, out, acc_out, ldc, splits, partials, counters, phases);
     return check_launch(name);
 }
 
