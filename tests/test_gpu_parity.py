@@ -200,6 +200,18 @@ def test_sgemm_nn_nt_tn(hip, oracle, M, N, K):
     check_fp32(oracle, got, a, b, ref=ref)
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 2304), (64, 8192, 1056), (40, 4100, 2112), (12, 11008, 1024)])
+def test_sgemm_streaming_weight_tiles(hip, oracle, M, N, K):
+    """A single row of tiles against 32 MiB of fp32 weights and more: the tiles of at most 64 rows fetch B with
+    non-temporal loads (their own instantiation), whole and with clamped edges, alone and under the K split."""
+    say("sgemm streaming tiles", M, N, K)
+    oracle.seed(M + 31 * N + 977 * K)
+    a, b = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1)
+    got = hip.sgemm(hip.array(a), hip.array(b)).numpy()
+    say("  nn", hip.last_kernel())
+    check_fp32(oracle, got, a, b, ref=oracle.gemm_opt(a, b))
+
+
 @pytest.mark.parametrize("M,N,K,pad,off", [(256, 384, 128, 64, 32), (2048, 4096, 64, 128, 64),
                                            (256, 384, 128, 3, 1), (70, 50, 90, 5, 2)])
 def test_sgemm_submatrix_views(hip, oracle, M, N, K, pad, off):
