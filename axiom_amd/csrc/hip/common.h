@@ -23,6 +23,8 @@ void *workspace(size_t bytes);
 // `n` zero-initialised device ints owned by the runtime.  Kernels that use them as arrival counters
 // leave them at zero when they finish.
 int *strip_counters(size_t n);
+// Queues a fill that puts them back to zero (after a launch that was cut short).
+int strip_counters_reset();
 // The allocation pool behind axhip_malloc / axhip_free: the size class of a request, and the call
 // that hands every cached block back to the driver.
 size_t pool_class(size_t bytes);
@@ -32,6 +34,8 @@ float *ones_vector(size_t n);
 // Per-device set-up of the skinny-M kernels (LDS limits, address of the static scratch); the device
 // must be current.  Called by axhip_init.
 int skinny_setup();
+// Frees what skinny_setup allocated (axhip_shutdown).
+void skinny_teardown();
 
 // Tile-selection overrides from the environment (0 = choose by shape), read at axhip_init and by
 // axhip_tuning_reload; what each one forces is described next to axhip_tuning_reload in axhip.h.
@@ -41,6 +45,8 @@ struct Tuning {
     int f32_tile;        // AX_HIP_F32_TILE: 64 (64x64), 642 (64x64 with the k split over two wave sets), 128 (128x128, eight waves)
     int f32_splitk;      // AX_HIP_F32_SPLITK: 1 = never split K, 2.. = that many ranges where the route applies
     int skinny_blocks;   // AX_HIP_SKINNY_BLOCKS: workgroups the skinny-M route aims for
+    int skinny_form;     // AX_HIP_SKINNY_FORM: 1 (64 columns x 256 threads), 2 (the same, the lane groups of a wave added before LDS), 3 (64 columns x 512 threads)
+    int skinny_kps;      // AX_HIP_SKINNY_KPS: most rows of K one skinny-M workgroup takes (a multiple of 16)
     int w8a32_tile;      // AX_HIP_W8A32_TILE: 1 (128x256), 2 (128x128), 3 (64x128), 4 (32x128), 5 (32x64): W8A32 matrix-core tile for K > 128
 };
 const Tuning &tuning();

@@ -36,7 +36,7 @@ size_t g_pool_cached = 0;
 constexpr size_t kPoolMaxBlock = size_t(1) << 30;        // larger blocks go straight back to the driver
 constexpr size_t kPoolMaxCached = size_t(16) << 30;      // bytes the pool may hold back
 
-axhip::Tuning g_tuning = {0, 0, 0, 0, 0, 0};
+axhip::Tuning g_tuning = {0, 0, 0, 0, 0, 0, 0, 0};
 
 // "64x64" / "128x128" / "256x256" / "128x256" / "64x64k2" or the bare first number; 0 when absent or not one of `allowed`
 int parse_tile(const char *name, const int *allowed, int n_allowed) {
@@ -186,6 +186,12 @@ int *strip_counters(size_t n) {
     return g_ctr;
 }
 
+int strip_counters_reset() {
+    if (g_ctr && hipMemsetAsync(g_ctr, 0, g_ctr_n * sizeof(int), kStream) != hipSuccess)
+        return fail(AXHIP_ERR_BACKEND, "zero-fill of the arrival counters failed");
+    return AXHIP_OK;
+}
+
 }  // namespace axhip
 
 using axhip::fail;
@@ -207,10 +213,12 @@ int axhip_tuning_reload(void) {
     g_tuning.f32_tile = parse_tile("AX_HIP_F32_TILE", f32_tiles, 3);
     g_tuning.f32_splitk = parse_count("AX_HIP_F32_SPLITK", 1, 4096);
     g_tuning.skinny_blocks = parse_count("AX_HIP_SKINNY_BLOCKS", 1, 65535);
+    g_tuning.skinny_form = parse_count("AX_HIP_SKINNY_FORM", 1, 3);
+    g_tuning.skinny_kps = parse_count("AX_HIP_SKINNY_KPS", 16, 8192) / 16 * 16;
     static const char *const w8a32_tiles[] = {"128x256", "128x128", "64x128", "32x128", "32x64"};
     g_tuning.w8a32_tile = parse_choice("AX_HIP_W8A32_TILE", w8a32_tiles, 5);
     return (g_tuning.i8_tile != 0) + (g_tuning.i8_splitk != 0) + (g_tuning.f32_tile != 0) + (g_tuning.f32_splitk != 0) +
-           (g_tuning.skinny_blocks != 0) + (g_tuning.w8a32_tile != 0);
+           (g_tuning.skinny_blocks != 0) + (g_tuning.w8a32_tile != 0) + (g_tuning.skinny_form != 0) + (g_tuning.skinny_kps != 0);
 }
 
 int axhip_workspace_reserve(size_t bytes, size_t *have) {
@@ -227,6 +235,8 @@ int axhip_tuning_get(const char *name) {
     if (!strcmp(name, "AX_HIP_F32_TILE")) return g_tuning.f32_tile;
     if (!strcmp(name, "AX_HIP_F32_SPLITK")) return g_tuning.f32_splitk;
     if (!strcmp(name, "AX_HIP_SKINNY_BLOCKS")) return g_tuning.skinny_blocks;
+    if (!strcmp(name, "AX_HIP_SKINNY_FORM")) return g_tuning.skinny_form;
+    if (!strcmp(name, "AX_HIP_SKINNY_KPS")) return g_tuning.skinny_kps;
     if (!strcmp(name, "AX_HIP_W8A32_TILE")) return g_tuning.w8a32_tile;
     return -1;
 }
@@ -256,6 +266,7 @@ void axhip_shutdown(void) {
     if (!g_ready) return;
     (void)hipDeviceSynchronize();
     axhip::pool_release_all();
+    axhip::skinny_teardown();
     if (g_ws) (void)hipFree(g_ws);
     if (g_ctr) (void)hipFree(g_ctr);
     if (g_ones) (void)hipFree(g_ones);
@@ -363,6 +374,13 @@ void axhip_alloc_stats(int64_t *allocs, int64_t *frees, int64_t *bytes_alloc, in
     if (bytes_free) *bytes_free = g_stat_bytes_free;
     if (driver_allocs) *driver_allocs = g_stat_driver_allocs;
     if (bytes_cached) *bytes_cached = (int64_t)g_pool_cached;
+}
+
+int64_t axhip_device_free_bytes(void) {
+    if (axhip::ensure_ready()) return -1;
+    size_t free_bytes = 0, total = 0;
+    if (hipMemGetInfo(&free_bytes, &total) != hipSuccess) return -1;
+    return (int64_t)free_bytes;
 }
 
 void axhip_reset_alloc_stats(void) {

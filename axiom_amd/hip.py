@@ -28,6 +28,7 @@ SIGNATURES = {
     "axhip_free": (None, [vp]),
     "axhip_alloc_stats": (None, [C.POINTER(C.c_int64)] * 6),
     "axhip_reset_alloc_stats": (None, []),
+    "axhip_device_free_bytes": (C.c_int64, []),
     "axhip_memset": (C.c_int, [vp, C.c_int, C.c_size_t]),
     "axhip_memcpy_h2d": (C.c_int, [vp, vp, C.c_size_t]),
     "axhip_memcpy_d2h": (C.c_int, [vp, vp, C.c_size_t]),
@@ -39,6 +40,7 @@ SIGNATURES = {
     "axhip_sgemm_skinny": (C.c_int, [i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, C.c_int]),
     "axhip_sgemm_skinny_head": (C.c_int, [i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, C.c_int, i64, vp, vp, C.c_int, vp]),
     "axhip_sgemm_skinny_static": (C.c_int, [i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, C.c_int]),
+    "axhip_sgemm_skinny_reset": (C.c_int, []),
     "axhip_qgemm_w8a8": (C.c_int, [vp, C.c_float, vp, vp, vp, C.c_int, vp, vp, i64, i64, i64]),
     "axhip_qgemm_w8a32": (C.c_int, [vp, vp, vp, vp, i64, i64, i64]),
     "axhip_quantize_rows": (C.c_int, [vp, i64, i64, vp, vp]),

@@ -58,6 +58,9 @@ const char *axhip_device_name(void);          /* gcnArchName of device 0, "" wit
  *   AX_HIP_F32_TILE      64x64 | 64x64k2 | 128x128   fp32 tile on the aligned fast path (k2: two wave sets split each K slab)
  *   AX_HIP_F32_SPLITK    1..4096    K ranges of the fp32 few-tile route (1: never split)
  *   AX_HIP_SKINNY_BLOCKS 1..65535   workgroups the skinny-M route aims for
+ *   AX_HIP_SKINNY_KPS    16..8192   most rows of K one skinny-M workgroup takes (rounded down to a multiple of 16)
+ *   AX_HIP_SKINNY_FORM   1..3       form of the skinny-M kernel for M <= 8: 1, workgroups of 256 threads; 2, the same with the
+ *                        four lane groups of a wave added before LDS; 3, workgroups of 512 threads
  *   AX_HIP_W8A32_TILE    128x256 | 128x128 | 64x128 | 32x128 | 32x64   W8A32 matrix-core tile where K > 128 and a multiple of 32
  *                        (edge form off the tile grid)
  * axhip_tuning_get returns the value in effect (0: automatic; tiles as their first number, 64x64k2 as
@@ -88,6 +91,9 @@ void  axhip_free(void *device_ptr);             /* NULL, foreign and already-fre
 void  axhip_alloc_stats(int64_t *allocs, int64_t *frees, int64_t *bytes_alloc, int64_t *bytes_free,
                         int64_t *driver_allocs, int64_t *bytes_cached);
 void  axhip_reset_alloc_stats(void);
+/* Bytes of device memory the driver reports free on the current device (hipMemGetInfo), or -1 without
+ * a device.  The counterpart of what cudaMemGetInfo gives a caller of the reference's CUDA backend. */
+int64_t axhip_device_free_bytes(void);
 /* The shared device workspace (split-K partial sums, reduction partials, padded operand copies) is 64 MiB
  * from axhip_init on and grows when a call needs more; growing waits for the device, frees the old block and asks the
  * driver for a new one, which costs the first call at a larger shape some tens of microseconds that later
@@ -147,18 +153,30 @@ int axhip_sgemm_skinny_head(int64_t M, int64_t N, int64_t K, const float *A, int
                             int64_t ldb, float *C, int64_t ldc, const float *bias, int act, int64_t NH,
                             const float *W2, const float *bias2, int act2, float *out2);
 
-/* The same route for callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
- * Arguments, results and kernels are those of axhip_sgemm_skinny — outputs are bit-identical —
- * but the split-K partial sums and arrival counters live in an 8 MiB + 16 KiB array that is part of
- * the library's device code (one copy per GPU, held until the process ends), and the call makes no
- * hipMalloc / hipFree.  axhip_init must have run on the current device.  A shape whose partial sums
- * exceed 8 MiB or that spans more than 4096 strips of 64 columns (N > 262144) is refused with
- * AXHIP_ERR_SHAPE.  All calls on one GPU share the array: calls that overlap in time on one GPU
- * (two streams, two host threads) race; calls issued one after another do not. */
+/* The same route for callers that cannot allocate device memory (tight serving loops, harnesses that
+ * forbid hipMalloc).  It has no counterpart in the reference.  Arguments, results and kernels are those of
+ * axhip_sgemm_skinny — outputs are bit-identical — but what the K ranges of a launch are joined through
+ * (8 MiB of exchange slots, 8 MiB for partial tiles, 4096 strip counters) lives in a 16 MiB + 16 KiB
+ * array that is part of the library's device code (one copy per GPU, held until the process ends), and
+ * the call makes no hipMalloc / hipFree and grows no workspace.  Like every entry point here it launches
+ * on the HIP null stream, so it cannot itself be recorded into a HIP graph.  axhip_init must have run on
+ * the current device.  A plan that needs more than 8 MiB of either kind ((K ranges - 1) * M * N * 4 bytes
+ * of slots, or K ranges * M * N * 4 bytes of tiles for M >= 5 with more than four ranges) or more than
+ * 4096 strips of 64 columns with tiles is refused with AXHIP_ERR_SHAPE.  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (two streams, two host threads) race; calls issued one
+ * after another do not.  Slots must read "empty" and counters zero when a launch starts: axhip_init
+ * leaves them so and every launch that runs to its end does too; after a launch that did not (a device
+ * error reported by this or a later call), call axhip_sgemm_skinny_reset before the next one. */
 int axhip_sgemm_skinny_static(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                               const float *B, int64_t ldb, float *C, int64_t ldc,
                               const float *bias, int act);
+
+/* Empties the join slots and zeroes the arrival counters of the skinny-M route again (those of
+ * axhip_sgemm_skinny_static and those the allocating entry points own): fills queued on the null stream,
+ * no allocation.  Only needed after a skinny-M launch was cut short by a device error; without that, a
+ * later launch would take the stale sums or arrivals of the dead one for its own and leave outputs
+ * unwritten. */
+int axhip_sgemm_skinny_reset(void);
 
 /* ---- int8 -------------------------------------------------------------------------- */
 /* W8A8: acc[m,n] = sum_k (int32)x[m,k] * (int32)w[n,k]   (exact, int32 MFMA)
