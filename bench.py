@@ -14,6 +14,12 @@ reference's benchmark format (benchmarks/bench_common.h:25-42) go to stderr.
                                         # launches of a copy-shaped kernel of known size, no output line
     python bench.py --sustain 8 [--operands zeros]   # back-to-back headline launches, for clock sampling
     python bench.py --hbm-ceiling                    # read / write / copy rates of this GPU on 2 GiB arrays, one JSON line
+    python bench.py --dispatch-table                 # shape -> kernel -> us for a fixed list of shapes (fp32, W8A8, W8A32)
+
+`secondary.configs` holds one record per BASELINE configuration in the reference's record shape
+(benchmarks/bench_common.h:25-42 plus algorithmic work): workload, algorithmic_flops, algorithmic_bytes,
+time_s, achieved, unit, roofline {bound, peak, achieved = achieved / peak}, kernel, and cpu = the
+reference's own CPU path on the same shape, timed in this run on the host cores.
 """
 import argparse
 import ctypes as C
@@ -150,10 +156,133 @@ def headline(hip, steps, warmup):
             "algorithmic_bytes": M * K + N * K + 4 * M * N + 8 * N}
 
 
+def config_record(workload, flops, nbytes, time_s, bound, kernel, **extra):
+    """One BASELINE configuration in the reference's record shape.  `bound` picks the roofline the
+    configuration is priced against: "hbm" (GB/s of algorithmic bytes), "mfma_fp32" (TFLOP/s) or
+    "mfma_int8" (TOP/s); roofline.achieved is the fraction of that peak."""
+    if bound == "hbm":
+        achieved, unit, peak = nbytes / time_s / 1e9, "GB/s", PEAK_HBM_GBS
+    elif bound == "mfma_fp32":
+        achieved, unit, peak = flops / time_s / 1e12, "TFLOP/s", PEAK_FP32_TFLOPS
+    else:
+        achieved, unit, peak = flops / time_s / 1e12, "TOP/s", PEAK_INT8_TOPS
+    rec = {"workload": workload, "algorithmic_flops": float(flops), "algorithmic_bytes": float(nbytes),
+           "time_s": time_s, "achieved": achieved, "unit": unit,
+           "roofline": {"bound": "hbm" if bound == "hbm" else "mfma", "peak": peak, "achieved": achieved / peak},
+           "kernel": kernel, "cpu": None}
+    rec.update(extra)
+    return rec
+
+
+def cpu_config_legs(budget_s=4.0):
+    """The reference's own CPU path on each BASELINE configuration, on this box's host cores: a bounded
+    sample per configuration (a few warm-up runs, then timed runs until `budget_s` seconds or the run
+    count of the reference's own harness is reached).  Checker/baseline code only.  Returns
+    {config key: {value, unit, cores, kind, sample}}; empty when only the CPU restatement is present
+    (its legs are the two in cpu_baseline / cpu_baseline_fp32)."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_bind as ob
+    if not ob.ref_available():
+        return {}
+    lib = ob.RefLib()
+    L = lib.L
+    lib.backend(lib.CPU_SIMD)
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    rng = np.random.default_rng(4)
+    out = {}
+
+    def timed(fn, warm, most):
+        for _ in range(warm):
+            fn()
+        runs, t_end = [], time.perf_counter() + budget_s
+        while len(runs) < most and (len(runs) < 3 or time.perf_counter() < t_end):
+            t0 = time.perf_counter()
+            fn()
+            runs.append(time.perf_counter() - t0)
+        return float(np.median(runs)), len(runs)
+
+    # config 1: the 784-4096-4096-10 network through the reference's Sequential forward (src/core/layer.c:188-230)
+    L.ax_set_seed(1)
+    seq = L.ax_sequential_create()
+    for (i, o, relu) in ((784, 4096, True), (4096, 4096, True), (4096, 10, False)):
+        L.ax_sequential_add(seq, L.ax_dense_create(i, o, True))
+        if relu:
+            L.ax_sequential_add(seq, L.ax_relu_layer_create())
+    weight_bytes = 4 * (784 * 4096 + 4096 * 4096 + 4096 * 10)
+    for M in (1, 8):
+        tx = lib.tensor(rng.uniform(0, 1, (M, 784)).astype(np.float32))
+
+        def forward():
+            y = L.ax_layer_forward(seq, tx)
+            L.ax_tensor_destroy(y)
+        dt, n = timed(forward, 5, 40)
+        out[f"config1_M{M}"] = {"value": weight_bytes / dt / 1e9, "unit": "GB/s", "latency_us": dt * 1e6, "cores": cores,
+                                "kind": "reference",
+                                "sample": f"ax_layer_forward of Sequential(Dense 784-4096 + ReLU, Dense 4096-4096 + ReLU, Dense 4096-10) "
+                                          f"at M={M}, median of {n} runs after 5 warm-up runs; weights {weight_bytes / 1e6:.1f} MB per pass"}
+        lib.free(tx)
+    L.ax_layer_destroy(seq)
+
+    # config 2: the reference's quantized GEMM (W8A32: it has no int8 activations) at M=256, N=K=4096 (src/core/quantize.c:100)
+    M, N, K = 256, 4096, 4096
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    qw = L.ax_qweight_create_from_fp32(np.ascontiguousarray(rng.uniform(-1, 1, (N, K)).astype(np.float32)), N, K)
+    o = np.empty((M, N), np.float32)
+    dt, n = timed(lambda: L.ax_qgemm_w8a32(a, qw, o, M), 3, 10)
+    L.ax_qweight_destroy(qw)
+    out["config2"] = {"value": 2.0 * M * N * K / dt / 1e12, "unit": "TOP/s", "latency_us": dt * 1e6, "cores": cores, "kind": "reference",
+                      "sample": f"ax_qgemm_w8a32 (int8 weights x fp32 activations, fp32 accumulate) at M=256, N=K=4096, median of {n} runs "
+                                f"after 3 warm-up runs (benchmarks/bench_qgemm.c:46-57)"}
+
+    # config 3: the FFN block as the reference runs it: GEMM, GELU as its own pass, GEMM (benchmarks/bench_transformer.c:40-42)
+    x = lib.tensor(rng.normal(0, 1, (2048, 1024)).astype(np.float32))
+    w1 = lib.tensor(rng.normal(0, 0.02, (1024, 4096)).astype(np.float32))
+    w2 = lib.tensor(rng.normal(0, 0.02, (4096, 1024)).astype(np.float32))
+    h, y = lib.empty(2048, 4096), lib.empty(2048, 1024)
+
+    def ffn():
+        assert L.ax_compute_gemm(x, w1, h) == 0
+        g = L.ax_gelu(h)
+        assert L.ax_compute_gemm(g, w2, y) == 0
+        L.ax_tensor_destroy(g)
+    dt, n = timed(ffn, 3, 10)
+    lib.free(x, w1, w2, h, y)
+    out["config3"] = {"value": 2 * 2.0 * 2048 * 1024 * 4096 / dt / 1e12, "unit": "TFLOP/s", "latency_us": dt * 1e6, "cores": cores,
+                      "kind": "reference",
+                      "sample": f"ax_compute_gemm [2048,1024]x[1024,4096], ax_gelu, ax_compute_gemm [2048,4096]x[4096,1024] (cpu_opt), "
+                                f"median of {n} runs after 3 warm-up runs; biases left out (the reference drops them without ReLU)"}
+
+    # config 4b: 8 of the 512 heads, Q K^T through ax_compute_gemm_nt and P V through ax_compute_gemm
+    heads, S, D = 8, 512, 64
+    qs = [lib.tensor(rng.normal(0, 1, (S, D)).astype(np.float32)) for _ in range(heads)]
+    ks = [lib.tensor(rng.normal(0, 1, (S, D)).astype(np.float32)) for _ in range(heads)]
+    vs = [lib.tensor(rng.normal(0, 1, (S, D)).astype(np.float32)) for _ in range(heads)]
+    ss = [lib.empty(S, S) for _ in range(heads)]
+    os_ = [lib.empty(S, D) for _ in range(heads)]
+
+    def qkt():
+        for i in range(heads):
+            assert L.ax_compute_gemm_nt(qs[i], ks[i], ss[i]) == 0
+
+    def pv():
+        for i in range(heads):
+            assert L.ax_compute_gemm(ss[i], vs[i], os_[i]) == 0
+    for name, fn in (("config4b_qkt", qkt), ("config4b_pv", pv)):
+        dt, n = timed(fn, 3, 20)
+        out[name] = {"value": heads * 2.0 * S * S * D / dt / 1e12, "unit": "TFLOP/s", "latency_us_512_heads": dt * 1e6 * 512 / heads,
+                     "cores": cores, "kind": "reference",
+                     "sample": f"{heads} of the 512 heads of [512,64], one {'ax_compute_gemm_nt' if name.endswith('qkt') else 'ax_compute_gemm'} "
+                               f"per head (cpu_opt), median of {n} runs after 3 warm-up runs; time scaled by 512/{heads} for the whole batch"}
+    for t in qs + ks + vs + ss + os_:
+        lib.free(t)
+    return out
+
+
 def secondary(hip):
     """The metric's other configurations, each timed with HIP events on the kernels' stream."""
     rng = np.random.default_rng(1)
     res = {}
+    configs = []          # one record per BASELINE configuration (config_record)
 
     def f32(a_shape, b_shape):
         return (hip.array(rng.uniform(-1, 1, a_shape).astype(np.float32)),
@@ -168,6 +297,8 @@ def secondary(hip):
     res["fp32_gemm_1024"] = {"us": ms * 1e3, "TFLOP/s": tf, "frac_of_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS,
                              "kernel": hip.last_kernel()}
     result_line("axhip", "f32_nn_1024x1024x1024", "gflops", tf * 1e3)
+    configs.append(config_record("configs[0]: fp32 GEMM C = A B, M=N=K=1024, row-major", 2 * 1024 ** 3, 3 * 4 * 1024 * 1024,
+                                 ms * 1e-3, "mfma_fp32", hip.last_kernel(), key="config0"))
 
     # the same product at the sizes where the matrix cores, not the launch, set the time
     for n_ in (4096, 8192):
@@ -215,6 +346,9 @@ def secondary(hip):
     res["fp32_ffn_2048x1024x4096"] = {"us": ms * 1e3, "TFLOP/s": tf,
                                       "frac_of_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS}
     result_line("axhip", "f32_ffn_2048x1024x4096", "gflops", tf * 1e3)
+    configs.append(config_record("configs[3]: fp32 FFN block, tokens 2048, d_model 1024, d_ff 4096: GEMM + bias + GELU fused, GEMM + bias",
+                                 2 * 2 * 2048 * 1024 * 4096, 4 * (2048 * 1024 + 1024 * 4096 + 2 * 2048 * 4096 + 4096 * 1024 + 2048 * 1024),
+                                 ms * 1e-3, "mfma_fp32", "two launches of " + hip.last_kernel(), key="config3"))
 
     # dense backward of the FFN block's first layer (X [2048,1024], W [1024,4096], dY [2048,4096]):
     # dA = dY W^T (NT), dW = X^T dY (TN), dBias = sum(dY, 0)
@@ -259,6 +393,10 @@ def secondary(hip):
         hip.check(hip.L.axhip_qgemm_w8a8(xi.ptr, 0.01, wsets[turn[0]].ptr, ws.ptr, bi.ptr, 0, oi.ptr, None, 256, 4096, 4096))
     _, ms = time_calls(hip, config2_rotating)
     res["int8_qgemm_256x4096x4096"]["weights_from_hbm_us"] = ms * 1e3
+    configs.append(config_record("configs[2]: int8 W8A8 GEMM M=256, N=K=4096, dequantize + bias epilogue; weights read from HBM "
+                                 "(36 weight matrices in rotation)", 2 * 256 * 4096 * 4096, nbytes, ms * 1e-3, "hbm",
+                                 res["int8_qgemm_256x4096x4096"]["kernel"], key="config2",
+                                 time_s_weights_in_cache=res["int8_qgemm_256x4096x4096"]["us"] * 1e-6))
     del xi, wi, oi, wsets
 
     # one round of fp32 tiles over a long K (256 tiles, K = 4096), operands cached and in rotation (9 x 67 MB)
@@ -324,6 +462,13 @@ def secondary(hip):
                         "layer2_us": ms2 * 1e3, "layer2_GB/s": gbs2,
                         "layer2_frac_of_hbm_peak": gbs2 / PEAK_HBM_GBS}
         result_line("axhip", f"mlp3_bs{M}", "latency_us", ms * 1e3)
+        if M in (1, 8):
+            configs.append(config_record(f"configs[1]: fp32 MLP 784-4096-4096-10 at M={M} through the skinny-M route, weights read from "
+                                         f"HBM (8 weight sets in rotation); two launches, the 10-wide layer rides on the second",
+                                         2 * M * (784 * 4096 + 4096 * 4096 + 4096 * 10), weight_bytes + 4 * M * (784 + 2 * 4096 + 10),
+                                         ms * 1e-3, "hbm", "sgemm_skinny_vec4 + sgemm_skinny_with_head", key=f"config1_M{M}",
+                                         layer2_alone_time_s=ms2 * 1e-3,
+                                         layer2_alone_frac_of_hbm_peak=gbs2 / PEAK_HBM_GBS))
     res["skinny_mlp_784_4096_4096_10"] = mlp
     del sets
 
@@ -382,11 +527,20 @@ def secondary(hip):
         0, 1, S, S, D, 1.0, q.ptr, D, S * D, k.ptr, D, S * D, 0.0, s.ptr, S, S * S, Bn)))
     nbytes = 4 * (2 * Bn * S * D + Bn * S * S)
     res["fp32_batched_qkt"] = {"us": ms * 1e3, "TFLOP/s": 2 * Bn * S * S * D / ms / 1e9,
-                               "GB/s": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+                               "GB/s": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS,
+                               "kernel": hip.last_kernel()}
     _, ms = time_calls(hip, lambda: hip.check(hip.L.axhip_sgemm_strided_batched(
         0, 0, S, D, S, 1.0, s.ptr, S, S * S, v.ptr, D, S * D, 0.0, o.ptr, D, S * D, Bn)))
     res["fp32_batched_pv"] = {"us": ms * 1e3, "TFLOP/s": 2 * Bn * S * S * D / ms / 1e9,
                               "GB/s": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    res["fp32_batched_pv"]["kernel"] = hip.last_kernel()
+    # arithmetic intensity 25.6 flop/byte against a machine balance of 19.7: the roofline prices both at the matrix cores
+    # (109 us); the time the bytes alone take at 8 TB/s (84 us) is given beside it
+    for key, name, what in (("config4b_qkt", "fp32_batched_qkt", "S = Q K^T, [512,64] x [512,64]^T"),
+                            ("config4b_pv", "fp32_batched_pv", "O = S V, [512,512] x [512,64]")):
+        t = res[name]["us"] * 1e-6
+        configs.append(config_record(f"configs[4] (b): strided-batched fp32 GEMM over 512 heads, {what}", 2 * Bn * S * S * D, nbytes, t,
+                                     "mfma_fp32", res[name]["kernel"], key=key, frac_of_hbm_peak=nbytes / t / 1e9 / PEAK_HBM_GBS))
     # fused attention forward over the same heads (both products and the softmax in one kernel,
     # no [512,512] score matrix in memory); flops counted as the two GEMMs'
     l = hip.empty((Bn, S))
@@ -553,6 +707,7 @@ def secondary(hip):
         ax.free(tx)
         L.ax_layer_destroy(enc)
         L.ax_set_default_device(0)
+    res["configs"] = configs
     return res
 
 
@@ -652,6 +807,71 @@ def counter_probe(hip, case, repeat=1):
     print(f"counter probe: {what}, then 3 x ReLU (k_unary<0>) over {n} floats", file=sys.stderr, flush=True)
 
 
+DISPATCH_FP32 = [   # (M, N, K): the configurations, bench_qgemm.c:76-82, then one shape on each side of every tile / route rule
+    (1024, 1024, 1024), (2048, 4096, 1024), (2048, 1024, 4096), (1, 4096, 784), (1, 4096, 4096), (8, 4096, 4096), (1, 10, 4096),
+    (1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024), (64, 1024, 4096),
+    (8, 8192, 8192), (9, 4096, 4096), (16, 4096, 4096), (17, 4096, 4096), (32, 4096, 4096), (33, 4096, 4096),
+    (160, 11008, 4096), (224, 11008, 4096), (512, 1024, 1024), (576, 1024, 1024), (1280, 960, 2048), (1024, 256, 256),
+    (128, 4096, 2048), (768, 1024, 4096), (1024, 1024, 4096), (256, 4096, 4096), (2048, 2048, 2048), (1920, 2048, 2048),
+    (4096, 4096, 4096), (500, 4096, 4096), (256, 4096, 784), (4000, 4000, 4000)]
+DISPATCH_W8A8 = [
+    (256, 4096, 4096), (8192, 8192, 8192), (1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024),
+    (64, 1024, 4096), (1, 4096, 4096), (4, 4096, 4096), (5, 4096, 4096), (100, 4096, 4096), (128, 4096, 4096), (128, 16384, 4096),
+    (512, 4096, 4096), (1024, 4096, 4096), (1024, 4096, 1024), (2048, 2048, 4096), (2048, 2048, 8192), (2048, 4096, 4096),
+    (2304, 2304, 8192), (4096, 4096, 4096), (64, 64, 8192), (256, 2048, 8192), (8000, 8000, 8192), (2000, 2000, 2000)]
+DISPATCH_W8A32 = [
+    (1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024), (64, 1024, 4096), (1, 4096, 4096),
+    (4, 4096, 4096), (5, 4096, 4096), (6, 4096, 4096), (7, 4096, 4096), (8, 4096, 4096), (4, 11008, 4096), (6, 1024, 4096),
+    (32, 4096, 4096), (256, 4096, 4096), (512, 4096, 4096), (768, 11008, 4096), (1024, 4096, 4096), (4096, 4096, 4096),
+    (1000, 4096, 4096)]
+
+
+def dispatch_table(hip):
+    """Shape -> kernel -> microseconds for a fixed list of shapes, one line each: the five configurations, the seven shapes
+    of the reference's benchmarks/bench_qgemm.c:76-82 and one shape on each side of the rules that pick a tile, a split or
+    a route (the counterpart of benchmarks/bench_gemm_suite.c:44-63).  Operands stay the same from launch to launch (cached
+    where they fit the caches).  Re-run after any change to a rule: on one box, a line that moves by more than 5 % is a
+    finding."""
+    rng = np.random.default_rng(7)
+    L = hip.L
+    print(f"# device {L.axhip_device_name().decode()}; us per launch, sustained over >= 0.1 s of launches", flush=True)
+    print(f"# {'kind':6s} {'M':>5s} {'N':>6s} {'K':>6s}  {'us':>9s}  kernel", flush=True)
+
+    def line(kind, M, N, K, fn):
+        fn()
+        kern = hip.last_kernel()
+        _, ms = time_calls(hip, fn, seconds=0.1)
+        print(f"  {kind:6s} {M:5d} {N:6d} {K:6d}  {ms * 1e3:9.2f}  {kern}", flush=True)
+
+    for (M, N, K) in DISPATCH_FP32:
+        a = hip.array(rng.uniform(-1, 1, (M, K)).astype(np.float32))
+        b = hip.array(rng.uniform(-1, 1, (K, N)).astype(np.float32))
+        c = hip.empty((M, N))
+        line("fp32", M, N, K, lambda: hip.check(L.axhip_sgemm(0, 0, M, N, K, 1.0, a.ptr, K, b.ptr, N, 0.0, c.ptr, N, None, 0)))
+        del a, b, c
+    Bn, S, D = 512, 512, 64
+    q, k, v = (hip.array(rng.normal(0, 1, (Bn, S, D)).astype(np.float32)) for _ in range(3))
+    sc, o = hip.empty((Bn, S, S)), hip.empty((Bn, S, D))
+    line("fp32nt", S, S, D, lambda: hip.check(L.axhip_sgemm_strided_batched(0, 1, S, S, D, 1.0, q.ptr, D, S * D, k.ptr, D, S * D, 0.0,
+                                                                         sc.ptr, S, S * S, Bn)))
+    line("fp32b", S, D, S, lambda: hip.check(L.axhip_sgemm_strided_batched(0, 0, S, D, S, 1.0, sc.ptr, S, S * S, v.ptr, D, S * D, 0.0,
+                                                                        o.ptr, D, S * D, Bn)))
+    del q, k, v, sc, o
+    for (M, N, K) in DISPATCH_W8A8:
+        x, w = hip.array(rand_i8(rng, (M, K))), hip.array(rand_i8(rng, (N, K)))
+        ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+        out = hip.empty((M, N))
+        line("w8a8", M, N, K, lambda: hip.check(L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, None, 0, out.ptr, None, M, N, K)))
+        del x, w, ws, out
+    for (M, N, K) in DISPATCH_W8A32:
+        a = hip.array(rng.uniform(-1, 1, (M, K)).astype(np.float32))
+        w = hip.array(rand_i8(rng, (N, K)))
+        ws = hip.array(rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+        out = hip.empty((M, N))
+        line("w8a32", M, N, K, lambda: hip.check(L.axhip_qgemm_w8a32(a.ptr, w.ptr, ws.ptr, out.ptr, M, N, K)))
+        del a, w, ws, out
+
+
 def hbm_ceiling(hip):
     """What this GPU's memory delivers to the library's plainest streaming kernels, on arrays far larger than the 256 MB
     Infinity Cache (2 GiB each): a read-only pass (sum of all elements), a write-only pass (fill), a copy (ReLU: one read,
@@ -661,7 +881,12 @@ def hbm_ceiling(hip):
     src, dst, one = hip.empty((n,)), hip.empty((n,)), hip.empty((1,))
     hip.check(hip.L.axhip_fill_f32(src.ptr, 0.25, n))
     res = {}
+    # the same 2 GiB read as a [65536, 8192] matrix by the skinny-M route at M = 1, whose weight loads are non-temporal
+    # 16-byte loads: the rate the bandwidth-bound GEMM kernels themselves can reach
+    xk, yk = hip.empty((1, 65536)), hip.empty((1, 8192))
     for name, fn, nbytes in (("read_sum_all", lambda: hip.check(hip.L.axhip_sum_all(src.ptr, n, one.ptr)), 4 * n),
+                             ("read_nontemporal_skinny_m1", lambda: hip.check(hip.L.axhip_sgemm(
+                                 0, 0, 1, 8192, 65536, 1.0, xk.ptr, 65536, src.ptr, 8192, 0.0, yk.ptr, 8192, None, 0)), 4 * n),
                              ("write_fill", lambda: hip.check(hip.L.axhip_fill_f32(dst.ptr, 1.0, n)), 4 * n),
                              ("copy_relu", lambda: hip.check(hip.L.axhip_relu(src.ptr, dst.ptr, n)), 8 * n)):
         fn()
@@ -810,10 +1035,16 @@ def main():
     ap.add_argument("--probe-repeat", type=int, default=1, help="multiplies the launch counts of --counter-probe")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of back-to-back headline launches")
     ap.add_argument("--hbm-ceiling", action="store_true", help="read / write / copy rates of this GPU on 2 GiB arrays")
+    ap.add_argument("--dispatch-table", action="store_true", help="shape -> kernel -> us for a fixed list of shapes")
+    ap.add_argument("--cpu-legs", action="store_true", help="only the reference's CPU path on the configurations (no GPU), one JSON line")
     ap.add_argument("--operands", choices=["random", "zeros", "fp32", "fp32zeros", "qkt", "qktzeros", "pv", "pvzeros"], default="random")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.cpu_legs:
+        print(json.dumps({"cpu_baseline": cpu_baseline(), "cpu_baseline_fp32": cpu_baseline_fp32(),
+                          "legs": {} if args.no_secondary else cpu_config_legs()}), flush=True)
+        return
 
     from axiom_amd import AxHip
     hip = AxHip()
@@ -826,6 +1057,9 @@ def main():
         return
     if args.hbm_ceiling:
         hbm_ceiling(hip)
+        return
+    if args.dispatch_table:
+        dispatch_table(hip)
         return
 
     h = headline(hip, args.steps, args.warmup)
@@ -852,10 +1086,31 @@ def main():
     }
     if not args.no_secondary:
         line["secondary"] = secondary(hip)
+        line["secondary"]["configs"].append(config_record(
+            "configs[4] (a): int8 W8A8 GEMM M=N=K=8192, dequantize + bias epilogue (the headline)", h["ops"], h["algorithmic_bytes"],
+            h["event_ms"] * 1e-3, "mfma_int8", h["kernel"], key="config4a"))
     hip.sync()
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline()
-        line["cpu_baseline_fp32"] = cpu_baseline_fp32()
+        # The CPU legs run in a process of their own that never touches the GPU: this process has the HIP host library
+        # loaded, which exports the reference's own function names (it mirrors its API), and the reference library's
+        # internal calls would bind to those.
+        import subprocess
+        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--cpu-legs"] + (["--no-secondary"] if args.no_secondary else []),
+                               capture_output=True, text=True, timeout=600)
+        sys.stderr.write(child.stderr)
+        if child.returncode != 0:
+            sys.exit(f"cpu legs failed with status {child.returncode}")
+        cpu = json.loads(child.stdout.strip().splitlines()[-1])
+        line["cpu_baseline"] = cpu["cpu_baseline"]
+        line["cpu_baseline_fp32"] = cpu["cpu_baseline_fp32"]
+        if not args.no_secondary:
+            legs = cpu["legs"]
+            legs["config4a"] = line["cpu_baseline"]
+            legs["config0"] = line["cpu_baseline_fp32"]
+            for rec in line["secondary"]["configs"]:
+                rec["cpu"] = legs.get(rec["key"])
+    if not args.no_secondary:
+        line["secondary"]["configs"].sort(key=lambda r: r["key"])
     print(json.dumps(line), flush=True)
 
 
