@@ -42,6 +42,7 @@ void skinny_teardown();
 struct Tuning {
     int i8_tile;         // AX_HIP_I8_TILE: 64 (64x64), 642 (64x64 with the k-steps split over two wave sets), 1264 (128x64), 128 or 256
     int i8_splitk;       // AX_HIP_I8_SPLITK: 1..16
+    int i8_mfma;         // AX_HIP_I8_MFMA: 32 (v_mfma_i32_32x32x32_i8) or 16 (v_mfma_i32_16x16x64_i8) in the persistent 256x256 kernel
     int f32_tile;        // AX_HIP_F32_TILE: 64 (64x64), 642 (64x64 with the k split over two wave sets), 128 (128x128, eight waves)
     int f32_splitk;      // AX_HIP_F32_SPLITK: 1 = never split K, 2.. = that many ranges where the route applies
     int skinny_blocks;   // AX_HIP_SKINNY_BLOCKS: workgroups the skinny-M route aims for

@@ -534,6 +534,293 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
 #undef AXI8_SLAB
 
 // ---------------------------------------------------------------------------------------
+// The same kernel on v_mfma_i32_16x16x64_i8.  The instruction does half the multiply-adds of
+// the 32x32x32 one with a quarter of its accumulator registers, so every accumulator is read
+// and written half as often per multiply-add.  On operands that change from instruction to
+// instruction the matrix cores run into the GPU's power limit; with that traffic halved the same
+// multiply-adds and LDS fragment reads take 13 % less time at a clock 13 % higher (measured with
+// axhip_probe_int8_matrix_core: 352.7 us at 1646 MHz against 305.7 us at 1858 MHz).  Everything
+// outside the inner loop is as above: tile, waves, stages, direct-to-LDS loads, loader and storer
+// waves, persistent walk over the tiles, write-back through LDS.
+//
+// A slab of 128 bytes is two k-steps of 64.  Per k-step a wave multiplies its 128x64 tile as 8 x 4
+// tiles of 16x16: lane (r = l & 15, q = l >> 4) of a fragment holds row r, bytes 16 q .. of the
+// k-step, i.e. logical chunk 4 ks + q of the LDS row, kept at chunk ^ ((row >> 1) & 7) like above
+// (16 lanes read 16 rows at one logical chunk: 8 physical chunks on even and odd rows, every
+// bank once).  With W as the first operand lane l then holds, for tile (i, j), the outputs m =
+// 16 i + (l & 15), n = 16 j + 4 (l >> 4) + v: four consecutive n, as above.
+#define AXK_LOAD_X(stage, j) AXI8_LOAD_LDS(lds_w + (stage) * OPER + (j) * 4096, voff[j], gx)
+#define AXK_LOAD_W(stage, j) AXI8_LOAD_LDS(lds_w + 2 * OPER + (stage) * OPER + (j) * 4096, voff[j], gw)
+#define AXK_ISSUE(stage)                                                                          \
+    do {                                                                                          \
+        AXK_LOAD_X(stage, 0); AXK_LOAD_X(stage, 1); AXK_LOAD_X(stage, 2); AXK_LOAD_X(stage, 3);   \
+        AXK_LOAD_X(stage, 4); AXK_LOAD_X(stage, 5); AXK_LOAD_X(stage, 6); AXK_LOAD_X(stage, 7);   \
+        AXK_LOAD_W(stage, 0); AXK_LOAD_W(stage, 1); AXK_LOAD_W(stage, 2); AXK_LOAD_W(stage, 3);   \
+        AXK_LOAD_W(stage, 4); AXK_LOAD_W(stage, 5); AXK_LOAD_W(stage, 6); AXK_LOAD_W(stage, 7);   \
+        gx += BKB;                                                                                \
+        gw += BKB;                                                                                \
+    } while (0)
+// fragment reads of k-step ks of a stage: X tile i at rows 16 i .. (2 KiB apart), W tile j likewise
+#define AXK_RX(buf, stage, ks, i) AXI8_DS_READ(fx[buf][i], rx[ks], (stage) * OPER + (i) * 2048)
+#define AXK_RW(buf, stage, ks, j) AXI8_DS_READ(fw[buf][j], rw[ks], (stage) * OPER + (j) * 2048)
+#define AXK_FRAGS(buf, stage, ks)                                                                 \
+    do {                                                                                          \
+        AXK_RW(buf, stage, ks, 0); AXK_RX(buf, stage, ks, 0); AXK_RW(buf, stage, ks, 1);          \
+        AXK_RW(buf, stage, ks, 2); AXK_RW(buf, stage, ks, 3); AXK_RX(buf, stage, ks, 1);          \
+        AXK_RX(buf, stage, ks, 2); AXK_RX(buf, stage, ks, 3); AXK_RX(buf, stage, ks, 4);          \
+        AXK_RX(buf, stage, ks, 5); AXK_RX(buf, stage, ks, 6); AXK_RX(buf, stage, ks, 7);          \
+    } while (0)
+#define AXK_M(buf, i, j)                                                                          \
+    do {                                                                                          \
+        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[buf][j], fx[buf][i], acc[i][j], 0, 0, 0); \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+    } while (0)
+// The 32 MFMAs of the k-step held in fragment buffer `buf`, tile row by tile row.  Behind the even ones
+// of the first 24: (RD) the 12 fragment reads of k-step rks of stage rstage into the other buffer, in
+// the order the next block consumes them; behind the odd ones: (LD, loader waves only) the 16 loads of
+// the next unfetched slab into stage lstage.
+#define AXK_ROW(buf, i, RD, r0, r1, LD, l0, l1, l2, l3)                                           \
+    do {                                                                                          \
+        AXK_M(buf, i, 0);                                                                         \
+        if (RD) { r0; }                                                                           \
+        AXK_M(buf, i, 1);                                                                         \
+        if (LD) { l0; l1; }                                                                       \
+        AXK_M(buf, i, 2);                                                                         \
+        if (RD) { r1; }                                                                           \
+        AXK_M(buf, i, 3);                                                                         \
+        if (LD) { l2; l3; }                                                                       \
+    } while (0)
+#define AXK_BLOCK(buf, RD, rstage, rks, LD, lstage)                                                                      \
+    do {                                                                                                                 \
+        AXK_ROW(buf, 0, RD, AXK_RW(1 - (buf), rstage, rks, 0), AXK_RX(1 - (buf), rstage, rks, 0), LD,                    \
+                AXK_LOAD_X(lstage, 0), AXK_LOAD_W(lstage, 0), (void)0, (void)0);                                         \
+        AXK_ROW(buf, 1, RD, AXK_RW(1 - (buf), rstage, rks, 1), AXK_RW(1 - (buf), rstage, rks, 2), LD,                    \
+                AXK_LOAD_X(lstage, 1), AXK_LOAD_W(lstage, 1), (void)0, (void)0);                                         \
+        AXK_ROW(buf, 2, RD, AXK_RW(1 - (buf), rstage, rks, 3), AXK_RX(1 - (buf), rstage, rks, 1), LD,                    \
+                AXK_LOAD_X(lstage, 2), AXK_LOAD_W(lstage, 2), (void)0, (void)0);                                         \
+        AXK_ROW(buf, 3, RD, AXK_RX(1 - (buf), rstage, rks, 2), AXK_RX(1 - (buf), rstage, rks, 3), LD,                    \
+                AXK_LOAD_X(lstage, 3), AXK_LOAD_W(lstage, 3), (void)0, (void)0);                                         \
+        AXK_ROW(buf, 4, RD, AXK_RX(1 - (buf), rstage, rks, 4), AXK_RX(1 - (buf), rstage, rks, 5), LD,                    \
+                AXK_LOAD_X(lstage, 4), AXK_LOAD_W(lstage, 4), (void)0, (void)0);                                         \
+        AXK_ROW(buf, 5, RD, AXK_RX(1 - (buf), rstage, rks, 6), AXK_RX(1 - (buf), rstage, rks, 7), LD,                    \
+                AXK_LOAD_X(lstage, 5), AXK_LOAD_W(lstage, 5), (void)0, (void)0);                                         \
+        AXK_ROW(buf, 6, 0, (void)0, (void)0, LD, AXK_LOAD_X(lstage, 6), AXK_LOAD_W(lstage, 6), (void)0, (void)0);        \
+        AXK_ROW(buf, 7, 0, (void)0, (void)0, LD, AXK_LOAD_X(lstage, 7), AXK_LOAD_W(lstage, 7), gx += BKB, gw += BKB);    \
+        __builtin_amdgcn_sched_barrier(0);                                                                               \
+    } while (0)
+#define AXK_WAIT_FRAGS() do { AXI8_LGKM(0); __builtin_amdgcn_sched_barrier(0); } while (0)
+// One slab resident in `stage`, its k-step 0 already (being) read into buffer 0.  After the first
+// k-step every wave has read all it needs of this stage and waits for its own loads of the next
+// slab; past the barrier the stage is free, so the second k-step's MFMAs cover the first fragment
+// reads of the next slab (after the last slab they fetch stale bytes nobody uses) and, when more2,
+// the loads of the slab after.
+#define AXK_SLAB(stage, more2)                                               \
+    do {                                                                     \
+        AXK_WAIT_FRAGS();                                                    \
+        AXK_BLOCK(0, 1, stage, 1, 0, 0);                                     \
+        AXK_WAIT_FRAGS();                                                    \
+        if (loader) AXI8_VM0();                                              \
+        __builtin_amdgcn_s_barrier();                                        \
+        __builtin_amdgcn_sched_barrier(0);                                   \
+        AXK_BLOCK(1, 1, 1 - (stage), 0, (more2) && loader, stage);           \
+    } while (0)
+
+template <int ACT>
+__global__ void __launch_bounds__(512)
+k_qgemm_w8a8_256_k64(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int64_t M, int64_t N,
+                     int64_t K, float x_scale, const float *__restrict__ w_scales,
+                     const float *__restrict__ bias, float *__restrict__ out,
+                     int32_t *__restrict__ acc_out, int64_t ldc) {
+    constexpr int BM = 256, BN = 256, BKB = 128, WAVES_N = 4, WTM = 128, WTN = 64, TM = 8, TN = 4;
+    constexpr int OPER = BM * BKB;   // bytes of one operand in one stage
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int tiles_m = (int)(M / BM), tiles_n = (int)(N / BN), total = tiles_m * tiles_n;
+    const int slabs = (int)(K / BKB);
+    const bool loader = wave < 4;         // waves 0-3 load and never store, waves 4-7 store and never load
+    // load instruction j (0..7) of loader wave w fills rows (j*4+w)*8 .. +8 of an operand stage
+    unsigned voff[8];
+    {
+        const int sw = (wave & 1) * 4 + (lane >> 4);      // (row >> 1) & 7 of this lane's row
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            voff[j] = (unsigned)(((j * 4 + (wave & 3)) * 8 + (lane >> 3)) * K + (((lane & 7) ^ sw) << 4));
+    }
+    const int8_t *gx = X, *gw = W;
+    const unsigned lds_w = (unsigned)(uintptr_t)lds + (wave & 3) * 1024;
+
+    // fragment reads: lane (frow, fq) of tile i takes row i*16 + frow, logical chunk ks*4 + fq
+    const int frow = lane & 15, fq = lane >> 4;
+    unsigned rx[2], rw[2];
+    {
+        const int sw = (frow >> 1) & 7;
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            const unsigned inrow = (unsigned)(frow * BKB + (((ks * 4 + fq) ^ sw) << 4));
+            rx[ks] = (unsigned)(uintptr_t)lds + wm * WTM * BKB + inrow;
+            rw[ks] = (unsigned)(uintptr_t)lds + 2 * OPER + wn * WTN * BKB + inrow;
+        }
+    }
+
+    typedef float v4f_t __attribute__((ext_vector_type(4)));
+    float *lds_scale = reinterpret_cast<float *>(lds + 4 * OPER);     // [2 slots][scale 256 | bias 256]
+    v4i acc[TM][TN];
+
+    const bool carry = (slabs & 1) == 0;
+    bool fetched = false;
+    v4f_t col_s = {0.f, 0.f, 0.f, 0.f}, col_b = {0.f, 0.f, 0.f, 0.f};
+    auto load_cols = [&](int64_t n0) {            // issued a whole tile ahead of store_cols
+        if (out && wave == 0) {
+            col_s = *reinterpret_cast<const v4f_t *>(w_scales + n0 + lane * 4);
+            if (bias) col_b = *reinterpret_cast<const v4f_t *>(bias + n0 + lane * 4);
+        }
+    };
+    auto store_cols = [&](int slot) {
+        if (out && wave == 0) {
+            v4f_t v = col_s;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = x_scale * v[e];
+            float *dst = lds_scale + slot * 2 * BN + lane * 4;
+            *reinterpret_cast<v4f_t *>(dst) = v;
+            *reinterpret_cast<v4f_t *>(dst + BN) = col_b;
+        }
+    };
+    int slot = 0;
+    v4i fx[2][TM], fw[2][TN];
+
+    // Write-back of one 32x32 sub-tile (2 x 2 tiles of 16x16) per wave and round.  r[2a + b] is tile (a, b)
+    // of the sub-tile: lane l holds its row 16 a + (l & 15) and the four columns of 16-byte chunk
+    // 4 b + (l >> 4).  Every wave writes its sub-tile (chunk c of row r at chunk c ^ ((r>>1)&7), conflict-free
+    // both ways) into its 4 KiB of a turn buffer; after the barrier storer wave 4+s reads the sub-tiles of
+    // waves 2s and 2s+1 back row-major and stores whole 128-byte rows, as in the kernel above.
+    int round = 0;
+    auto emit = [&](const auto (&r)[4], auto *base, int64_t m0, int64_t n0, int i, int j) {
+        typedef typename std::remove_const<typename std::remove_reference<decltype(r[0])>::type>::type V4;
+        unsigned char *buf = lds + ((round & 1) ? 3 * OPER : OPER);
+        round++;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const int row = (g >> 1) * 16 + frow, chunk = 4 * (g & 1) + fq;
+            *reinterpret_cast<V4 *>(buf + wave * 4096 + row * 128 + ((chunk ^ ((frow >> 1) & 7)) << 4)) = r[g];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+        if (!loader) {
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const int src = 2 * (wave - 4) + q;                     // wave whose sub-tile this is
+                auto *dst = base + (m0 + (src / WAVES_N) * WTM + i * 32) * ldc + n0 + (src % WAVES_N) * WTN + j * 32;
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    const int row = p * 8 + (lane >> 3);
+                    const V4 v = *reinterpret_cast<const V4 *>(buf + src * 4096 + row * 128 +
+                                                               (((lane & 7) ^ ((row >> 1) & 7)) << 4));
+                    __builtin_nontemporal_store(v, reinterpret_cast<V4 *>(dst + (int64_t)row * ldc + (lane & 7) * 4));
+                }
+            }
+        }
+    };
+
+    for (int t = blockIdx.x; t < total; t += gridDim.x) {
+        int tm, tn;
+        tile_of_block(t, tiles_m, tiles_n, tm, tn);
+        const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+        if (!fetched) {
+            gx = X + m0 * K;
+            gw = W + n0 * K;
+            if (loader) AXK_ISSUE(0);
+            load_cols(n0);
+            store_cols(slot);
+        }
+        const int t_next = t + (int)gridDim.x;
+        const bool will_fetch = carry && t_next < total;
+        int tm2 = 0, tn2 = 0;
+        if (will_fetch) {
+            tile_of_block(t_next, tiles_m, tiles_n, tm2, tn2);
+            load_cols((int64_t)tn2 * BN);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) acc[i][j] = v4i{0, 0, 0, 0};
+
+        if (loader) AXI8_VM0();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        if (slabs > 1 && loader) AXK_ISSUE(1);
+        AXK_FRAGS(0, 0, 0);
+
+        for (int s = 0; s < slabs; s += 2) {       // the flags are wave-uniform: scalar branches only
+            AXK_SLAB(0, s + 2 < slabs);
+            if (s + 1 < slabs) AXK_SLAB(1, s + 3 < slabs);
+        }
+        AXK_WAIT_FRAGS();      // the stale reads must land before their registers are reused
+
+        fetched = will_fetch;
+        if (fetched) {
+            store_cols(slot ^ 1);
+            gx = X + (int64_t)tm2 * BM * K;
+            gw = W + (int64_t)tn2 * BN * K;
+            if (loader) AXK_ISSUE(0);
+        }
+
+        if (acc_out) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const v4i r[4] = {acc[2 * i][2 * j], acc[2 * i][2 * j + 1], acc[2 * i + 1][2 * j], acc[2 * i + 1][2 * j + 1]};
+                    emit(r, acc_out, m0, n0, i, j);
+                }
+        }
+        if (out) {
+            const float *sp = lds_scale + slot * 2 * BN + wn * WTN + 4 * fq, *bp = sp + BN;
+            const bool has_bias = bias != nullptr;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                v4f_t sc[2], bv[2];
+#pragma unroll
+                for (int b = 0; b < 2; b++) {
+                    sc[b] = *reinterpret_cast<const v4f_t *>(sp + j * 32 + 16 * b);
+                    bv[b] = *reinterpret_cast<const v4f_t *>(bp + j * 32 + 16 * b);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    v4f_t r[4];
+#pragma unroll
+                    for (int g = 0; g < 4; g++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float f = (float)acc[2 * i + (g >> 1)][2 * j + (g & 1)][e];
+                            // a fused multiply-add with bias = 0 would round differently from the plain product
+                            r[g][e] = apply_act(has_bias ? __builtin_fmaf(f, sc[g & 1][e], bv[g & 1][e]) : f * sc[g & 1][e], ACT);
+                        }
+                    emit(r, out, m0, n0, i, j);
+                }
+            }
+        }
+        slot ^= 1;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    }
+}
+#undef AXK_LOAD_X
+#undef AXK_LOAD_W
+#undef AXK_ISSUE
+#undef AXK_RX
+#undef AXK_RW
+#undef AXK_FRAGS
+#undef AXK_M
+#undef AXK_ROW
+#undef AXK_BLOCK
+#undef AXK_WAIT_FRAGS
+#undef AXK_SLAB
+
+// ---------------------------------------------------------------------------------------
 // Mid-size aligned shapes (M, N multiples of the tile, K a multiple of 128) that cannot fill
 // the chip with 256x256 tiles: the same direct-to-LDS, VALU-free loop over smaller tiles with
 // NST LDS stages, so NST-1 slabs of loads are in flight per workgroup (a 64x64 tile has only
@@ -956,8 +1243,9 @@ int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_s
     constexpr int smem = 4 * 256 * 128 + 2 * 2 * 256 * 4;   // two stages of both operands + two slots of scale and bias
     typedef void (*kern_t)(const int8_t *, const int8_t *, int64_t, int64_t, int64_t, float, const float *,
                            const float *, float *, int32_t *, int64_t);
-    static const kern_t kerns[3] = {k_qgemm_w8a8_256<AXHIP_ACT_NONE>, k_qgemm_w8a8_256<AXHIP_ACT_RELU>,
-                                    k_qgemm_w8a8_256<AXHIP_ACT_GELU>};
+    static const kern_t kerns[6] = {k_qgemm_w8a8_256<AXHIP_ACT_NONE>, k_qgemm_w8a8_256<AXHIP_ACT_RELU>,
+                                    k_qgemm_w8a8_256<AXHIP_ACT_GELU>, k_qgemm_w8a8_256_k64<AXHIP_ACT_NONE>,
+                                    k_qgemm_w8a8_256_k64<AXHIP_ACT_RELU>, k_qgemm_w8a8_256_k64<AXHIP_ACT_GELU>};
     static bool attr_set = false;
     if (!attr_set) {
         for (kern_t kf : kerns)
@@ -968,9 +1256,11 @@ int launch_256(const int8_t *x, float x_scale, const int8_t *w, const float *w_s
     }
     const int64_t tiles = (M / 256) * (N / 256);
     if (tiles > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a8: too many tiles");
-    note_kernel("qgemm_w8a8_256x256_dma");
+    // AX_HIP_I8_MFMA: 32 = v_mfma_i32_32x32x32_i8, 16 (and by default) = v_mfma_i32_16x16x64_i8
+    const bool k64 = tuning().i8_mfma != 32;
+    note_kernel(k64 ? "qgemm_w8a8_256x256_dma" : "qgemm_w8a8_256x256_dma_mfma32x32x32");
     const int64_t grid = tiles < cu_count() ? tiles : cu_count();     // one persistent workgroup per CU
-    hipLaunchKernelGGL(kerns[act], dim3((unsigned)grid), dim3(512), smem, kStream, x, w, M, N, K,
+    hipLaunchKernelGGL(kerns[act + (k64 ? 3 : 0)], dim3((unsigned)grid), dim3(512), smem, kStream, x, w, M, N, K,
                        x_scale, w_scales, bias, out, acc_out, ldc);
     return check_launch("qgemm_w8a8_256x256_dma");
 }

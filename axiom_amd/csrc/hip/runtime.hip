@@ -36,7 +36,7 @@ size_t g_pool_cached = 0;
 constexpr size_t kPoolMaxBlock = size_t(1) << 30;        // larger blocks go straight back to the driver
 constexpr size_t kPoolMaxCached = size_t(16) << 30;      // bytes the pool may hold back
 
-axhip::Tuning g_tuning = {0, 0, 0, 0, 0, 0, 0, 0};
+axhip::Tuning g_tuning = {};
 
 // "64x64" / "128x128" / "256x256" / "128x256" / "64x64k2" or the bare first number; 0 when absent or not one of `allowed`
 int parse_tile(const char *name, const int *allowed, int n_allowed) {
@@ -210,6 +210,8 @@ int axhip_tuning_reload(void) {
     static const int i8_tiles[] = {64, 642, 128, 1264, 256}, f32_tiles[] = {64, 642, 128};
     g_tuning.i8_tile = parse_tile("AX_HIP_I8_TILE", i8_tiles, 5);
     g_tuning.i8_splitk = parse_count("AX_HIP_I8_SPLITK", 1, 16);
+    g_tuning.i8_mfma = parse_count("AX_HIP_I8_MFMA", 16, 32);
+    if (g_tuning.i8_mfma != 16 && g_tuning.i8_mfma != 32) g_tuning.i8_mfma = 0;
     g_tuning.f32_tile = parse_tile("AX_HIP_F32_TILE", f32_tiles, 3);
     g_tuning.f32_splitk = parse_count("AX_HIP_F32_SPLITK", 1, 4096);
     g_tuning.skinny_blocks = parse_count("AX_HIP_SKINNY_BLOCKS", 1, 65535);
@@ -218,7 +220,7 @@ int axhip_tuning_reload(void) {
     static const char *const w8a32_tiles[] = {"128x256", "128x128", "64x128", "32x128", "32x64"};
     g_tuning.w8a32_tile = parse_choice("AX_HIP_W8A32_TILE", w8a32_tiles, 5);
     return (g_tuning.i8_tile != 0) + (g_tuning.i8_splitk != 0) + (g_tuning.f32_tile != 0) + (g_tuning.f32_splitk != 0) +
-           (g_tuning.skinny_blocks != 0) + (g_tuning.w8a32_tile != 0) + (g_tuning.skinny_form != 0) + (g_tuning.skinny_kps != 0);
+           (g_tuning.skinny_blocks != 0) + (g_tuning.w8a32_tile != 0) + (g_tuning.skinny_form != 0) + (g_tuning.skinny_kps != 0) + (g_tuning.i8_mfma != 0);
 }
 
 int axhip_workspace_reserve(size_t bytes, size_t *have) {
@@ -232,6 +234,7 @@ int axhip_tuning_get(const char *name) {
     if (!name) return -1;
     if (!strcmp(name, "AX_HIP_I8_TILE")) return g_tuning.i8_tile;
     if (!strcmp(name, "AX_HIP_I8_SPLITK")) return g_tuning.i8_splitk;
+    if (!strcmp(name, "AX_HIP_I8_MFMA")) return g_tuning.i8_mfma;
     if (!strcmp(name, "AX_HIP_F32_TILE")) return g_tuning.f32_tile;
     if (!strcmp(name, "AX_HIP_F32_SPLITK")) return g_tuning.f32_splitk;
     if (!strcmp(name, "AX_HIP_SKINNY_BLOCKS")) return g_tuning.skinny_blocks;

@@ -895,15 +895,50 @@ def hbm_ceiling(hip):
     print(json.dumps({"hbm_ceiling_2GiB_arrays": res, "device": hip.L.axhip_device_name().decode()}), flush=True)
 
 
-def sustain(hip, seconds, operands):
-    """One GEMM launched back to back for `seconds`, so that clock and power can be sampled from outside
-    (rocm-smi) while it runs: the headline over random int8 operands or all-zero ones (same instruction
-    stream, no switching activity in the matrix core), the fp32 8192^3 product over random / zero
-    operands ("fp32", "fp32zeros"), or the batched attention products ("qkt", "pv", each also with "zeros").
+def sample_sclk(stop, out, first_after_s=2.5, every_s=0.6):
+    """Shader clock as rocm-smi reports it, sampled beside a running loop (a child process per sample, which
+    only reads the driver's counters); appends MHz figures to `out` until `stop` is set."""
+    import re
+    import subprocess
+    time.sleep(first_after_s)
+    while not stop.is_set():
+        try:
+            txt = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
+            m = re.search(r"sclk clock level[^(]*\((\d+)Mhz\)", txt)
+            if m:
+                out.append(int(m.group(1)))
+        except Exception as e:                      # no rocm-smi on the box: the times are still printed
+            out.append(f"rocm-smi: {e}")
+            return
+        time.sleep(every_s)
+
+
+def sustain(hip, seconds, operands, clocks=False):
+    """One kernel launched back to back for `seconds`, so that clock and power can be sampled while it runs
+    (--sample-clocks does it from a thread of this process with rocm-smi): the headline over random int8
+    operands or all-zero ones (same instruction stream, no switching activity in the matrix core), the
+    fp32 8192^3 product over random / zero operands ("fp32", "fp32zeros"), the batched attention products
+    ("qkt", "pv", each also with "zeros"), or the int8 matrix-core probe ("probe<shape>r<reads>[zeros]",
+    e.g. probe32r6: the headline's MFMAs and LDS fragment reads with nothing else, axhip_probe_int8_matrix_core).
     Prints the average time per launch about once a second."""
     M = N = K = 8192
     rng = np.random.default_rng(0)
-    if operands.startswith("qkt") or operands.startswith("pv"):
+    import threading
+    stop, mhz = threading.Event(), []
+    sampler = threading.Thread(target=sample_sclk, args=(stop, mhz), daemon=True) if clocks else None
+    if operands.startswith("probe"):
+        import re
+        m = re.fullmatch(r"probe(16|32)r([0-6])(zeros)?", operands)
+        if not m:
+            sys.exit("probe operands are probe<16|32>r<0..6>[zeros]")
+        shape, reads = int(m.group(1)), int(m.group(2))
+        src = hip.empty((128 * 1024,), np.int8) if m.group(3) else hip.array(rand_i8(rng, (128 * 1024,)))
+        sink = hip.empty((512 * 1024,), np.int32)
+        per_print = 2000
+
+        def launch():
+            hip.check(hip.L.axhip_probe_int8_matrix_core(shape, reads, src.ptr, sink.ptr))
+    elif operands.startswith("qkt") or operands.startswith("pv"):
         # the attention-shaped products of 512 heads of [512, 64]: Q K^T (writes 537 MB) or P V (reads it)
         Bn, S, D = 512, 512, 64
         zeros = operands.endswith("zeros")
@@ -932,7 +967,7 @@ def sustain(hip, seconds, operands):
 
         def launch():
             hip.check(hip.L.axhip_sgemm(0, 0, M, N, K, 1.0, a.ptr, K, b.ptr, N, 0.0, out.ptr, N, None, 0))
-    else:
+    elif operands in ("random", "zeros"):
         if operands == "zeros":
             x, w = hip.empty((M, K), np.int8), hip.empty((N, K), np.int8)
         else:
@@ -944,6 +979,8 @@ def sustain(hip, seconds, operands):
 
         def launch():
             hip.check(hip.L.axhip_qgemm_w8a8(x.ptr, 0.01, w.ptr, ws.ptr, bias.ptr, 0, out.ptr, None, M, N, K))
+    if sampler:
+        sampler.start()
     t_end = time.perf_counter() + seconds
     while time.perf_counter() < t_end:
         t0 = time.perf_counter()
@@ -952,6 +989,10 @@ def sustain(hip, seconds, operands):
         hip.sync()
         print(f"sustain {operands}: {(time.perf_counter() - t0) / per_print * 1e6:.1f} us per launch "
               f"({hip.last_kernel()})", flush=True)
+    if sampler:
+        stop.set()
+        sampler.join(timeout=15)
+        print(f"sustain {operands}: sclk MHz while the loop ran: {' '.join(str(x) for x in mhz)}", flush=True)
 
 
 def cpu_baseline():
@@ -1037,7 +1078,9 @@ def main():
     ap.add_argument("--hbm-ceiling", action="store_true", help="read / write / copy rates of this GPU on 2 GiB arrays")
     ap.add_argument("--dispatch-table", action="store_true", help="shape -> kernel -> us for a fixed list of shapes")
     ap.add_argument("--cpu-legs", action="store_true", help="only the reference's CPU path on the configurations (no GPU), one JSON line")
-    ap.add_argument("--operands", choices=["random", "zeros", "fp32", "fp32zeros", "qkt", "qktzeros", "pv", "pvzeros"], default="random")
+    ap.add_argument("--operands", default="random",
+                    help="random | zeros | fp32 | fp32zeros | qkt | qktzeros | pv | pvzeros | probe<16|32>r<0..6>[zeros]")
+    ap.add_argument("--sample-clocks", action="store_true", help="with --sustain: sample the shader clock with rocm-smi while the loop runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -1053,7 +1096,7 @@ def main():
         counter_probe(hip, args.counter_probe, args.probe_repeat)
         return
     if args.sustain > 0:
-        sustain(hip, args.sustain, args.operands)
+        sustain(hip, args.sustain, args.operands, args.sample_clocks)
         return
     if args.hbm_ceiling:
         hbm_ceiling(hip)

@@ -55,6 +55,8 @@ const char *axhip_device_name(void);          /* gcnArchName of device 0, "" wit
  *   AX_HIP_I8_TILE       64x64 | 64x64k2 | 128x64 | 128x128 | 256x256   W8A8 tile (256x256: M, N multiples of 256;
  *                        k2: two wave sets split each K slab)
  *   AX_HIP_I8_SPLITK     1..16      workgroups over K per W8A8 tile of 64x64 / 128x128 (1: never split)
+ *   AX_HIP_I8_MFMA       16 | 32    matrix-core instruction of the persistent 256x256 W8A8 kernel: v_mfma_i32_16x16x64_i8 (what
+ *                        runs by default) or v_mfma_i32_32x32x32_i8; the results are the same bits
  *   AX_HIP_F32_TILE      64x64 | 64x64k2 | 128x128   fp32 tile on the aligned fast path (k2: two wave sets split each K slab)
  *   AX_HIP_F32_SPLITK    1..4096    K ranges of the fp32 few-tile route (1: never split)
  *   AX_HIP_SKINNY_BLOCKS 1..65535   workgroups the skinny-M route aims for
@@ -177,6 +179,19 @@ int axhip_sgemm_skinny_static(int64_t M, int64_t N, int64_t K, const float *A, i
  * later launch would take the stale sums or arrivals of the dead one for its own and leave outputs
  * unwritten. */
 int axhip_sgemm_skinny_reset(void);
+
+/* ---- measurement probe --------------------------------------------------------------- */
+/* Not a compute path: one launch does the int8 matrix-core work of axhip_qgemm_w8a8 at M = N = K = 8192 on
+ * a 256-CU device (8192 blocks of 262144 multiply-adds per CU-resident wave) with nothing around it but LDS
+ * fragment reads, so that a committed command (bench.py --sustain S --operands probe...) can show what the
+ * matrix cores of the GPU at hand sustain, and at what clock, on operands that change from instruction to
+ * instruction.  mfma_shape: 32 (v_mfma_i32_32x32x32_i8) or 16 (v_mfma_i32_16x16x64_i8, twice as many
+ * instructions for the same multiply-adds); lds_reads: 16-byte fragment reads per block, 0..6 (6 = the
+ * 128x64 wave tile of the GEMM kernel, 4 = what a 128x128 wave tile would need, 0 = operands that never
+ * change); operand_bytes: 128 KiB of device memory that every workgroup copies into LDS (random bytes, or
+ * zeros for a loop without switching activity); sink: 512 ints per CU, receives checksums.  It has no
+ * counterpart in the reference. */
+int axhip_probe_int8_matrix_core(int mfma_shape, int lds_reads, const int8_t *operand_bytes, int32_t *sink);
 
 /* ---- int8 -------------------------------------------------------------------------- */
 /* W8A8: acc[m,n] = sum_k (int32)x[m,k] * (int32)w[n,k]   (exact, int32 MFMA)

@@ -381,7 +381,8 @@ def test_w8a8_dispatch_sweep(hip, oracle):
 def test_forced_tiles_and_splits_keep_parity(hip, oracle):
     """The environment overrides change which kernel runs, never the result: W8A8 accumulators and outputs stay
     bit-exact and fp32 / skinny products stay inside their gates under every forced tile, split and block count."""
-    names = ("AX_HIP_I8_TILE", "AX_HIP_I8_SPLITK", "AX_HIP_F32_TILE", "AX_HIP_F32_SPLITK", "AX_HIP_SKINNY_BLOCKS")
+    names = ("AX_HIP_I8_TILE", "AX_HIP_I8_SPLITK", "AX_HIP_F32_TILE", "AX_HIP_F32_SPLITK", "AX_HIP_SKINNY_BLOCKS", "AX_HIP_I8_MFMA",
+             "AX_HIP_SKINNY_FORM", "AX_HIP_SKINNY_KPS")
     saved = {n: os.environ.get(n) for n in names}
     rng = np.random.default_rng(77)
     M, N, K = 256, 512, 2048
@@ -405,9 +406,17 @@ def test_forced_tiles_and_splits_keep_parity(hip, oracle):
             seen.add(hip.last_kernel())
             assert np.array_equal(acc.numpy(), want_acc), (tile, split, hip.last_kernel())
             assert np.array_equal(out.numpy(), want_out), (tile, split, hip.last_kernel())
+        # the persistent 256x256 kernel on the other MFMA shape
+        os.environ["AX_HIP_I8_TILE"], os.environ["AX_HIP_I8_SPLITK"], os.environ["AX_HIP_I8_MFMA"] = "256x256", "1", "32"
+        hip.L.axhip_tuning_reload()
+        say("forced i8 256x256 on 32x32x32")
+        out, acc = hip.qgemm_w8a8(dx, 0.02, dw, dws, db, 1)
+        seen.add(hip.last_kernel())
+        assert np.array_equal(acc.numpy(), want_acc) and np.array_equal(out.numpy(), want_out)
+        del os.environ["AX_HIP_I8_MFMA"]
         assert {"qgemm_w8a8_64x64_dma", "qgemm_w8a8_64x64_dma_splitk", "qgemm_w8a8_64x64k2_dma", "qgemm_w8a8_64x64k2_dma_splitk",
                 "qgemm_w8a8_128x128_dma_splitk", "qgemm_w8a8_128x64_dma", "qgemm_w8a8_128x64_dma_splitk",
-                "qgemm_w8a8_256x256_dma"} <= seen, seen
+                "qgemm_w8a8_256x256_dma", "qgemm_w8a8_256x256_dma_mfma32x32x32"} <= seen, seen
         seen = set()
         for tile, split in (("64x64", "1"), ("64x64k2", "1"), ("128x128", "1"), ("", "4"), ("64x64", "8")):
             os.environ["AX_HIP_F32_TILE"], os.environ["AX_HIP_F32_SPLITK"] = tile, split
@@ -421,6 +430,11 @@ def test_forced_tiles_and_splits_keep_parity(hip, oracle):
             os.environ["AX_HIP_SKINNY_BLOCKS"] = blocks
             hip.L.axhip_tuning_reload()
             say("forced skinny blocks", blocks)
+            check_fp32(oracle, hip.sgemm_skinny(dsa, dbm).numpy(), sa, b, ref=sref)
+        for form, kps in (("1", "64"), ("2", "1024"), ("3", "256"), ("3", "8192")):
+            os.environ["AX_HIP_SKINNY_BLOCKS"], os.environ["AX_HIP_SKINNY_FORM"], os.environ["AX_HIP_SKINNY_KPS"] = "64", form, kps
+            hip.L.axhip_tuning_reload()
+            say("forced skinny form", form, kps)
             check_fp32(oracle, hip.sgemm_skinny(dsa, dbm).numpy(), sa, b, ref=sref)
     finally:
         for n, v in saved.items():
