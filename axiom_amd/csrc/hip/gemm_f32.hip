@@ -379,6 +379,8 @@ __device__ __forceinline__ Bf16x3 bf16x3_of(const v4f &p, const v4f &q) {
     for (int e = 0; e < 8; e++) {
         const float a = e < 4 ? p[e] : q[e - 4];
         h[e] = __float_as_uint(a);
+        // a NaN whose payload sits in the low 16 bits only would be cut to an infinity: give it a quiet bit the cut keeps
+        if ((h[e] & 0x7fffffffu) > 0x7f800000u) h[e] |= 0x00400000u;
         float r = a - __uint_as_float(h[e] & 0xffff0000u);
         r = __builtin_amdgcn_fmed3f(r, r, 0.0f);     // NaN (a infinite or NaN) -> 0, anything else unchanged
         m[e] = __float_as_uint(r);

@@ -590,22 +590,34 @@ k_qgemm_w8a8_256(const int8_t *__restrict__ X, const int8_t *__restrict__ W, int
         AXK_M(buf, i, 3);                                                                         \
         if (LD) { l2; l3; }                                                                       \
     } while (0)
+// the same with the tile columns walked backwards: between one row of tiles and the next only the X fragment changes
+#define AXK_ROW_REV(buf, i, RD, r0, r1, LD, l0, l1, l2, l3)                                       \
+    do {                                                                                          \
+        AXK_M(buf, i, 3);                                                                         \
+        if (RD) { r0; }                                                                           \
+        AXK_M(buf, i, 2);                                                                         \
+        if (LD) { l0; l1; }                                                                       \
+        AXK_M(buf, i, 1);                                                                         \
+        if (RD) { r1; }                                                                           \
+        AXK_M(buf, i, 0);                                                                         \
+        if (LD) { l2; l3; }                                                                       \
+    } while (0)
 #define AXK_BLOCK(buf, RD, rstage, rks, LD, lstage)                                                                      \
     do {                                                                                                                 \
         AXK_ROW(buf, 0, RD, AXK_RW(1 - (buf), rstage, rks, 0), AXK_RX(1 - (buf), rstage, rks, 0), LD,                    \
                 AXK_LOAD_X(lstage, 0), AXK_LOAD_W(lstage, 0), (void)0, (void)0);                                         \
-        AXK_ROW(buf, 1, RD, AXK_RW(1 - (buf), rstage, rks, 1), AXK_RW(1 - (buf), rstage, rks, 2), LD,                    \
+        AXK_ROW_REV(buf, 1, RD, AXK_RW(1 - (buf), rstage, rks, 1), AXK_RW(1 - (buf), rstage, rks, 2), LD,                    \
                 AXK_LOAD_X(lstage, 1), AXK_LOAD_W(lstage, 1), (void)0, (void)0);                                         \
         AXK_ROW(buf, 2, RD, AXK_RW(1 - (buf), rstage, rks, 3), AXK_RX(1 - (buf), rstage, rks, 1), LD,                    \
                 AXK_LOAD_X(lstage, 2), AXK_LOAD_W(lstage, 2), (void)0, (void)0);                                         \
-        AXK_ROW(buf, 3, RD, AXK_RX(1 - (buf), rstage, rks, 2), AXK_RX(1 - (buf), rstage, rks, 3), LD,                    \
+        AXK_ROW_REV(buf, 3, RD, AXK_RX(1 - (buf), rstage, rks, 2), AXK_RX(1 - (buf), rstage, rks, 3), LD,                    \
                 AXK_LOAD_X(lstage, 3), AXK_LOAD_W(lstage, 3), (void)0, (void)0);                                         \
         AXK_ROW(buf, 4, RD, AXK_RX(1 - (buf), rstage, rks, 4), AXK_RX(1 - (buf), rstage, rks, 5), LD,                    \
                 AXK_LOAD_X(lstage, 4), AXK_LOAD_W(lstage, 4), (void)0, (void)0);                                         \
-        AXK_ROW(buf, 5, RD, AXK_RX(1 - (buf), rstage, rks, 6), AXK_RX(1 - (buf), rstage, rks, 7), LD,                    \
+        AXK_ROW_REV(buf, 5, RD, AXK_RX(1 - (buf), rstage, rks, 6), AXK_RX(1 - (buf), rstage, rks, 7), LD,                    \
                 AXK_LOAD_X(lstage, 5), AXK_LOAD_W(lstage, 5), (void)0, (void)0);                                         \
         AXK_ROW(buf, 6, 0, (void)0, (void)0, LD, AXK_LOAD_X(lstage, 6), AXK_LOAD_W(lstage, 6), (void)0, (void)0);        \
-        AXK_ROW(buf, 7, 0, (void)0, (void)0, LD, AXK_LOAD_X(lstage, 7), AXK_LOAD_W(lstage, 7), gx += BKB, gw += BKB);    \
+        AXK_ROW_REV(buf, 7, 0, (void)0, (void)0, LD, AXK_LOAD_X(lstage, 7), AXK_LOAD_W(lstage, 7), gx += BKB, gw += BKB);    \
         __builtin_amdgcn_sched_barrier(0);                                                                               \
     } while (0)
 #define AXK_WAIT_FRAGS() do { AXI8_LGKM(0); __builtin_amdgcn_sched_barrier(0); } while (0)
@@ -816,6 +828,7 @@ k_qgemm_w8a8_256_k64(const int8_t *__restrict__ X, const int8_t *__restrict__ W,
 #undef AXK_FRAGS
 #undef AXK_M
 #undef AXK_ROW
+#undef AXK_ROW_REV
 #undef AXK_BLOCK
 #undef AXK_WAIT_FRAGS
 #undef AXK_SLAB

@@ -1,5 +1,6 @@
 /* Dense / ReLU / GELU / LayerNorm / Sequential, forward only (Axiom's src/core/layer.c:48-103,
  * 181-300; src/core/norm.c:1278-1455). */
+#include <stdio.h>
 #include <stdlib.h>
 
 #include "axiom/compute.h"
@@ -195,10 +196,25 @@ static ax_tensor_t *try_dense_head(ax_sequential_t *seq, int i, ax_tensor_t *x, 
     if (j >= seq->n_layers || seq->layers[j]->type != AX_LAYER_DENSE || seq->layers[j]->output_features > 16) return NULL;
     ax_dense_t *d1 = (ax_dense_t *)seq->layers[i], *d2 = (ax_dense_t *)seq->layers[j++];
     if (j < seq->n_layers && fused_act_of(seq->layers[j]->type) >= 0) act2 = fused_act_of(seq->layers[j++]->type);
+    /* What the backend would decline is declined here, before an output tensor is allocated for nothing: no such
+     * operation, or a head whose weight rows are not packed one after the other. */
+    const ax_tensor_t *w2 = d2->weight;
+    if (!ax_compute_has_gemm_act_head() || !w2 || w2->ndim != 2 || w2->strides[1] != 1 || w2->strides[0] != w2->shape[1])
+        return NULL;
+    /* a decline must leave the caller's error state as it was */
+    const ax_status_t held = ax_err_last_status();
+    char held_msg[256];
+    snprintf(held_msg, sizeof held_msg, "%s", ax_err_last_message());
     ax_tensor_t *y = ax_matmul_bias_act_head(x, d1->weight, dense_bias(d1), act, d2->weight, dense_bias(d2), act2);
-    if (y) *consumed = j - i;
-    else if (ax_err_last_status() != AX_ERR_NOT_IMPLEMENTED) *consumed = -1;
-    else ax_err_clear();                       /* not an error: the layers run one by one */
+    if (y) {
+        *consumed = j - i;
+    } else if (ax_err_last_status() != AX_ERR_NOT_IMPLEMENTED) {
+        *consumed = -1;
+    } else if (held != AX_OK) {                /* not an error: the layers run one by one */
+        ax_err_set(held, "%s", held_msg);
+    } else {
+        ax_err_clear();
+    }
     return y;
 }
 

@@ -887,6 +887,7 @@ def test_w8a32_non_finite_activations(hip, oracle):
     a[3, 200] = np.nan
     a[4, 7] = -np.inf
     a[5, 300] = np.float32(3.0e38)                                    # finite, overflows in the product
+    a[6, 50] = np.array([0x7f800001], np.uint32).view(np.float32)[0]  # a NaN whose payload lies in the low 16 bits only
     s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
     for rows in (M, 6):                                               # matrix-core form, weight-streaming form
         x = a[1:1 + rows] if rows == 6 else a
