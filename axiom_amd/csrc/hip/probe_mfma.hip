@@ -133,6 +133,112 @@ int launch_probe(int reads, const int8_t *src, int *sink) {
     hipLaunchKernelGGL(kerns[reads], dim3((unsigned)cu_count()), dim3(512), kLdsBytes, kStream, src, kBlocksPerLaunch, sink);
     return check_launch("probe_int8_matrix_core");
 }
+
+// The fp32 counterpart: the MFMAs of a 64x32 wave tile (the batched attention products' kernels) per block of 16384
+// multiply-adds, as 8 x v_mfma_f32_32x32x2_f32 (fragments fa[2], fb[1], four k each) or 16 x v_mfma_f32_16x16x4_f32
+// (half of fa[4], fb[2]), with READS (0..3) 16-byte fragment reads per block.
+template <int SHAPE, int READS>
+__global__ void __launch_bounds__(512)
+k_probe_f32(const float *__restrict__ src, int blocks, float *__restrict__ sink) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    for (int i = tid; i < kLdsBytes / 16; i += 512)
+        reinterpret_cast<v4f *>(lds)[i] = reinterpret_cast<const v4f *>(src)[i];
+    __syncthreads();
+    const unsigned base = (unsigned)(uintptr_t)lds + ((tid >> 6) & 7) * 8192 + lane * 16;
+    v4f f[2][3];
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+        for (int r = 0; r < 3; r++) f[b][r] = *reinterpret_cast<const v4f *>(lds + ((tid >> 6) & 7) * 8192 + lane * 16 + r * 1024);
+    float sum = 0.0f;
+    if constexpr (SHAPE == 32) {
+        v16f acc[2];
+#pragma unroll
+        for (int m = 0; m < 2; m++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[m][v] = 0.0f;
+#define AXP_FBLOCK32(cur, off)                                                                                   \
+    do {                                                                                                         \
+        AXP_LGKM0();                                                                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                                       \
+        _Pragma("unroll") for (int m = 0; m < 8; m++) {                                                          \
+            acc[m & 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[cur][2][m >> 1], f[cur][m & 1][m >> 1], acc[m & 1], 0, 0, 0); \
+            __builtin_amdgcn_sched_barrier(0);                                                                   \
+            if (m == 0 && READS > 0) AXP_DS_READ(f[1 - (cur)][0], base, (off) + 0 * 1024);                       \
+            if (m == 2 && READS > 1) AXP_DS_READ(f[1 - (cur)][1], base, (off) + 1 * 1024);                       \
+            if (m == 4 && READS > 2) AXP_DS_READ(f[1 - (cur)][2], base, (off) + 2 * 1024);                       \
+            __builtin_amdgcn_sched_barrier(0);                                                                   \
+        }                                                                                                        \
+    } while (0)
+        for (int s = 0; s < blocks; s += 8) {
+            AXP_FBLOCK32(0, 0 * 3072 + 16);
+            AXP_FBLOCK32(1, 1 * 3072 + 32);
+            AXP_FBLOCK32(0, 2 * 3072 + 48);
+            AXP_FBLOCK32(1, 3 * 3072 + 64);
+            AXP_FBLOCK32(0, 4 * 3072 + 80);
+            AXP_FBLOCK32(1, 5 * 3072 + 96);
+            AXP_FBLOCK32(0, 6 * 3072 + 112);
+            AXP_FBLOCK32(1, 7 * 3072 + 0);
+        }
+#undef AXP_FBLOCK32
+        AXP_LGKM0();
+#pragma unroll
+        for (int m = 0; m < 2; m++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) sum += acc[m][v];
+    } else {
+        v4f acc[4];
+#pragma unroll
+        for (int m = 0; m < 4; m++) acc[m] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#define AXP_FBLOCK16(cur, off)                                                                                   \
+    do {                                                                                                         \
+        AXP_LGKM0();                                                                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                                       \
+        _Pragma("unroll") for (int m = 0; m < 16; m++) {                                                         \
+            acc[m & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(f[cur][2][m >> 2], f[cur][m & 1][m >> 2], acc[m & 3], 0, 0, 0); \
+            __builtin_amdgcn_sched_barrier(0);                                                                   \
+            if (m == 0 && READS > 0) AXP_DS_READ(f[1 - (cur)][0], base, (off) + 0 * 1024);                       \
+            if (m == 4 && READS > 1) AXP_DS_READ(f[1 - (cur)][1], base, (off) + 1 * 1024);                       \
+            if (m == 8 && READS > 2) AXP_DS_READ(f[1 - (cur)][2], base, (off) + 2 * 1024);                       \
+            __builtin_amdgcn_sched_barrier(0);                                                                   \
+        }                                                                                                        \
+    } while (0)
+        for (int s = 0; s < blocks; s += 8) {
+            AXP_FBLOCK16(0, 0 * 3072 + 16);
+            AXP_FBLOCK16(1, 1 * 3072 + 32);
+            AXP_FBLOCK16(0, 2 * 3072 + 48);
+            AXP_FBLOCK16(1, 3 * 3072 + 64);
+            AXP_FBLOCK16(0, 4 * 3072 + 80);
+            AXP_FBLOCK16(1, 5 * 3072 + 96);
+            AXP_FBLOCK16(0, 6 * 3072 + 112);
+            AXP_FBLOCK16(1, 7 * 3072 + 0);
+        }
+#undef AXP_FBLOCK16
+        AXP_LGKM0();
+#pragma unroll
+        for (int m = 0; m < 4; m++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) sum += acc[m][v];
+    }
+    sink[(int64_t)blockIdx.x * 512 + tid] = sum;
+}
+
+constexpr int kF32BlocksPerLaunch = 1024;   // blocks of 16384 multiply-adds per wave: 70 GFLOP per launch on 256 CUs
+
+template <int SHAPE>
+int launch_probe_f32(int reads, const float *src, float *sink) {
+    typedef void (*kern_t)(const float *, int, float *);
+    static const kern_t kerns[4] = {k_probe_f32<SHAPE, 0>, k_probe_f32<SHAPE, 1>, k_probe_f32<SHAPE, 2>, k_probe_f32<SHAPE, 3>};
+    static bool raised[4] = {};
+    if (!raised[reads]) {
+        AXHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kerns[reads]), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes),
+                      "hipFuncSetAttribute");
+        raised[reads] = true;
+    }
+    hipLaunchKernelGGL(kerns[reads], dim3((unsigned)cu_count()), dim3(512), kLdsBytes, kStream, src, kF32BlocksPerLaunch, sink);
+    return check_launch("probe_fp32_matrix_core");
+}
 }  // namespace
 
 extern "C" int axhip_probe_int8_matrix_core(int mfma_shape, int lds_reads, const int8_t *operand_bytes, int32_t *sink) {
@@ -142,4 +248,13 @@ extern "C" int axhip_probe_int8_matrix_core(int mfma_shape, int lds_reads, const
         return axhip::fail(AXHIP_ERR_SHAPE, "probe_int8_matrix_core: shape %d (32 or 16), reads %d (0..6)", mfma_shape, lds_reads);
     axhip::note_kernel(mfma_shape == 32 ? "probe_i8_mfma_32x32x32" : "probe_i8_mfma_16x16x64");
     return mfma_shape == 32 ? launch_probe<32>(lds_reads, operand_bytes, sink) : launch_probe<16>(lds_reads, operand_bytes, sink);
+}
+
+extern "C" int axhip_probe_fp32_matrix_core(int mfma_shape, int lds_reads, const float *operand_floats, float *sink) {
+    if (int rc = axhip::ensure_ready()) return rc;
+    if (!operand_floats || !sink) return axhip::fail(AXHIP_ERR_NULL_ARG, "probe_fp32_matrix_core: NULL buffer");
+    if ((mfma_shape != 32 && mfma_shape != 16) || lds_reads < 0 || lds_reads > 3)
+        return axhip::fail(AXHIP_ERR_SHAPE, "probe_fp32_matrix_core: shape %d (32 or 16), reads %d (0..3)", mfma_shape, lds_reads);
+    axhip::note_kernel(mfma_shape == 32 ? "probe_f32_mfma_32x32x2" : "probe_f32_mfma_16x16x4");
+    return mfma_shape == 32 ? launch_probe_f32<32>(lds_reads, operand_floats, sink) : launch_probe_f32<16>(lds_reads, operand_floats, sink);
 }

@@ -42,6 +42,7 @@ SIGNATURES = {
     "axhip_sgemm_skinny_static": (C.c_int, [i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, C.c_int]),
     "axhip_sgemm_skinny_reset": (C.c_int, []),
     "axhip_probe_int8_matrix_core": (C.c_int, [C.c_int, C.c_int, vp, vp]),
+    "axhip_probe_fp32_matrix_core": (C.c_int, [C.c_int, C.c_int, vp, vp]),
     "axhip_qgemm_w8a8": (C.c_int, [vp, C.c_float, vp, vp, vp, C.c_int, vp, vp, i64, i64, i64]),
     "axhip_qgemm_w8a32": (C.c_int, [vp, vp, vp, vp, i64, i64, i64]),
     "axhip_quantize_rows": (C.c_int, [vp, i64, i64, vp, vp]),

@@ -919,18 +919,31 @@ def sustain(hip, seconds, operands, clocks=False):
     operands or all-zero ones (same instruction stream, no switching activity in the matrix core), the
     fp32 8192^3 product over random / zero operands ("fp32", "fp32zeros"), the batched attention products
     ("qkt", "pv", each also with "zeros"), or the int8 matrix-core probe ("probe<shape>r<reads>[zeros]",
-    e.g. probe32r6: the headline's MFMAs and LDS fragment reads with nothing else, axhip_probe_int8_matrix_core).
+    e.g. probe32r6: the headline's MFMAs and LDS fragment reads with nothing else, axhip_probe_int8_matrix_core;
+    "fprobe<shape>r<reads>[zeros]": the fp32 counterpart, axhip_probe_fp32_matrix_core).
     Prints the average time per launch about once a second."""
     M = N = K = 8192
     rng = np.random.default_rng(0)
     import threading
     stop, mhz = threading.Event(), []
     sampler = threading.Thread(target=sample_sclk, args=(stop, mhz), daemon=True) if clocks else None
-    if operands.startswith("probe"):
+    if operands.startswith("fprobe"):
+        import re
+        m = re.fullmatch(r"fprobe(16|32)r([0-3])(zeros)?", operands)
+        if not m:
+            sys.exit("fp32 probe operands are fprobe<16|32>r<0..3>[zeros]")
+        shape, reads = int(m.group(1)), int(m.group(2))
+        src = hip.empty((32 * 1024,)) if m.group(3) else hip.array(rng.normal(0, 1, (32 * 1024,)).astype(np.float32))
+        sink = hip.empty((512 * 1024,))
+        per_print = 500
+
+        def launch():
+            hip.check(hip.L.axhip_probe_fp32_matrix_core(shape, reads, src.ptr, sink.ptr))
+    elif operands.startswith("probe"):
         import re
         m = re.fullmatch(r"probe(16|32)r([0-6])(zeros)?", operands)
         if not m:
-            sys.exit("probe operands are probe<16|32>r<0..6>[zeros]")
+            sys.exit("probe operands are probe<16|32>r<0..6>[zeros] | fprobe<16|32>r<0..3>[zeros]")
         shape, reads = int(m.group(1)), int(m.group(2))
         src = hip.empty((128 * 1024,), np.int8) if m.group(3) else hip.array(rand_i8(rng, (128 * 1024,)))
         sink = hip.empty((512 * 1024,), np.int32)

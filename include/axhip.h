@@ -192,6 +192,11 @@ int axhip_sgemm_skinny_reset(void);
  * zeros for a loop without switching activity); sink: 512 ints per CU, receives checksums.  It has no
  * counterpart in the reference. */
 int axhip_probe_int8_matrix_core(int mfma_shape, int lds_reads, const int8_t *operand_bytes, int32_t *sink);
+/* The fp32 counterpart (bench.py --sustain S --operands fprobe...): per launch 1024 blocks of 16384 multiply-adds per
+ * wave, eight waves per CU, as v_mfma_f32_32x32x2_f32 (mfma_shape 32) or v_mfma_f32_16x16x4_f32 (16), with lds_reads
+ * (0..3) 16-byte fragment reads per block (3 = the 64x32 wave tile of the batched attention kernels); operand_floats:
+ * 128 KiB of device memory, sink: 512 floats per CU. */
+int axhip_probe_fp32_matrix_core(int mfma_shape, int lds_reads, const float *operand_floats, float *sink);
 
 /* ---- int8 -------------------------------------------------------------------------- */
 /* W8A8: acc[m,n] = sum_k (int32)x[m,k] * (int32)w[n,k]   (exact, int32 MFMA)
