@@ -1195,6 +1195,35 @@ def test_error_paths(hip):
     hip.sync()
 
 
+def test_matrix_core_probes_run_and_check_arguments(hip):
+    """The measurement probes are no compute path, but they are exported: each shape launches, all-zero
+    operands give all-zero checksums (the sink is written by every lane), and bad arguments are refused."""
+    L = hip.L
+    zeros8, sink32 = hip.empty((128 * 1024,), np.int8), hip.empty((512 * 1024,), np.int32)
+    zerosf, sinkf = hip.empty((32 * 1024,)), hip.empty((512 * 1024,))
+    cus = 256
+    for shape in (32, 16):
+        for reads in (0, 6):
+            say("probe int8", shape, reads)
+            hip.check(L.axhip_memset(sink32.ptr, 0xFF, sink32.nbytes))
+            hip.check(L.axhip_probe_int8_matrix_core(shape, reads, zeros8.ptr, sink32.ptr))
+            assert hip.last_kernel().startswith("probe_i8_mfma")
+            assert not sink32.numpy()[: cus * 512].any()
+        for reads in (0, 3):
+            say("probe fp32", shape, reads)
+            hip.check(L.axhip_memset(sinkf.ptr, 0xFF, sinkf.nbytes))
+            hip.check(L.axhip_probe_fp32_matrix_core(shape, reads, zerosf.ptr, sinkf.ptr))
+            assert hip.last_kernel().startswith("probe_f32_mfma")
+            assert not sinkf.numpy()[: cus * 512].any()
+    assert L.axhip_probe_int8_matrix_core(8, 0, zeros8.ptr, sink32.ptr) == 3
+    assert L.axhip_probe_int8_matrix_core(32, 7, zeros8.ptr, sink32.ptr) == 3
+    assert L.axhip_probe_int8_matrix_core(32, 0, None, sink32.ptr) == 1
+    assert L.axhip_probe_fp32_matrix_core(16, 4, zerosf.ptr, sinkf.ptr) == 3
+    assert L.axhip_probe_fp32_matrix_core(16, 0, zerosf.ptr, None) == 1
+    assert L.axhip_device_free_bytes() > 0
+    hip.sync()
+
+
 # ---------------------------------------------------------------- elementwise / reduction / optimizer slots
 import ctypes as C  # noqa: E402
 
