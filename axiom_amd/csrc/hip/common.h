@@ -48,6 +48,7 @@ struct Tuning {
     int skinny_blocks;   // AX_HIP_SKINNY_BLOCKS: workgroups the skinny-M route aims for
     int skinny_form;     // AX_HIP_SKINNY_FORM: 1 (64 columns x 256 threads), 2 (the same, the lane groups of a wave added before LDS), 3 (64 columns x 512 threads)
     int skinny_kps;      // AX_HIP_SKINNY_KPS: most rows of K one skinny-M workgroup takes (a multiple of 16)
+    int nt_walk;         // AX_HIP_NT_WALK: short-K batched A B^T: 1 = a block of A rows resident, blocks of B walked; 2 = 256 rows of B resident, blocks of A walked
     int w8a32_tile;      // AX_HIP_W8A32_TILE: 1 (128x256), 2 (128x128), 3 (64x128), 4 (32x128), 5 (32x64): W8A32 matrix-core tile for K > 128
 };
 const Tuning &tuning();

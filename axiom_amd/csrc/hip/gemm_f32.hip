@@ -1060,6 +1060,210 @@ int try_nt_rows(const SgemmArgs &g, int64_t batch) {
 }
 
 // =====================================================================================
+// The same product walked the other way: a workgroup keeps 256 rows of B (= 256 columns of C) for its whole
+// life — in registers: each of its four waves holds the fragments of its own 64 columns, 8 K / 32 vectors —
+// and walks the rows of A in blocks of 32 through two LDS buffers.  Every step therefore finishes 32 rows of
+// C over the workgroup's whole width: a wave's store instruction writes four pieces of 256 contiguous bytes,
+// the four waves' pieces of a row are neighbours (1 KiB per row and step), and a row of C is complete after
+// one step of the N / 256 workgroups that share it instead of being visited N / 64 times over the life of
+// one.  The stream of stores that reaches memory is then made of long runs instead of 256-byte fragments
+// spread over 128 rows.  Only the A fragments are read from LDS (one ds_read_b128 per 8 MFMAs); loads of the
+// next block are issued before the stores of the previous tile, as above.  LDS: two A blocks of K / 32 x 4
+// KiB, 8 KiB per wave to turn the write-back into rows of 256 bytes.
+template <int KS>
+__global__ void __launch_bounds__(256) k_sgemm_nt_cols(SgemmArgs g) {
+    constexpr int BMS = 32, BN = 256, NW = 4, TN = 2;                    // rows per step, columns per workgroup
+    using OA = DmaOperand<BMS, true, NW>;
+    constexpr int A_BYTES = KS * OA::BYTES;                               // one A buffer
+    constexpr int TURN_BASE = 2 * A_BYTES;
+    constexpr int NSTORES = 8;                                            // store instructions of a wave per step
+    static_assert(OA::IPW == 1, "one load instruction per wave and slab");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int tm = 0, tn = (int)blockIdx.x;
+    int64_t batch = 0;
+    if (gridDim.y > 1) tile_of_batched_block(1, (int)(g.N / BN), tm, tn, batch);
+    const int64_t n0 = (int64_t)tn * BN + wave * 64;                      // this wave's first column
+    const float *A = static_cast<const float *>(g.A) + batch * g.stride_a;
+    const float *B = static_cast<const float *>(g.B) + batch * g.stride_b + n0 * g.ldb;
+    float *C = g.C + batch * g.stride_c + n0;
+    const int nblk = (int)(g.M / BMS);
+
+    const unsigned va = OA::lane_offset(wave, lane, g.lda);
+    const char *ga = reinterpret_cast<const char *>(A);
+    const int64_t step_a = (int64_t)BMS * g.lda * 4;                      // bytes from one block of A to the next
+    const unsigned lds0 = (unsigned)(uintptr_t)lds_raw;
+    const unsigned dma_a = lds0 + wave * OA::PITCH;
+
+    const int frow = lane & 31, fhalf = lane >> 5;
+    unsigned ra[4];
+#pragma unroll
+    for (int kbi = 0; kbi < 4; kbi++) ra[kbi] = lds0 + OA::frag_base(0, frow, fhalf, kbi);
+
+    // This wave's B fragments, kept for the workgroup's life: tile j, k-block kk -> row n0 + 32 j + frow of B,
+    // k = 8 kk + 4 fhalf .. + 3 (the pairing of k values over the two lane halves is that of the A fragments).
+    // Fetched as whole 128-byte lines (a load instruction takes one slab of 8 rows: lane l -> row l >> 3, 16-byte
+    // chunk l & 7; all of them in flight at once) and brought into fragment order through the wave's own turn
+    // area, one 32-row slab at a time, rows 144 bytes apart so that neither side meets a bank twice: loading the
+    // fragments straight from memory touches every line with four instructions, 32 bytes at a time.
+#define AXC_ISSUE_A(BUFK)                                                                        \
+    do {                                                                                         \
+        _Pragma("unroll") for (int s = 0; s < KS; s++)                                           \
+            AXF_LOAD_LDS(dma_a + (BUFK) * A_BYTES + s * OA::BYTES, va, ga + s * 128);            \
+        ga += step_a;                                                                            \
+    } while (0)
+    unsigned char *turn = lds_raw + TURN_BASE + wave * 8192;
+    v4f fb[TN][4 * KS];
+    {
+        v4f raw[TN][KS][4];
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int sl = 0; sl < KS; sl++)
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    raw[j][sl][q] = *reinterpret_cast<const v4f *>(B + (int64_t)(j * 32 + q * 8 + (lane >> 3)) * g.ldb + sl * 32 + (lane & 7) * 4);
+        AXC_ISSUE_A(0);                             // the first block of A, behind the loads of B
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int sl = 0; sl < KS; sl++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    *reinterpret_cast<v4f *>(turn + (q * 8 + (lane >> 3)) * 144 + (lane & 7) * 16) = raw[j][sl][q];
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int kbi = 0; kbi < 4; kbi++)
+                    fb[j][sl * 4 + kbi] = *reinterpret_cast<const v4f *>(turn + frow * 144 + (2 * kbi + fhalf) * 16);
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            }
+    }
+    const int rrow = lane >> 4, rchunk = lane & 15;
+    float *cdst = C + (int64_t)rrow * g.ldc + rchunk * 4;                 // this lane's 16 bytes of a write-back row
+    v16f acc[TN];
+    Frag<true> fa[2];
+    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+#define AXC_FRAG(BUF, BUFK, KK) AXF_DS128(fa[BUF].q, ra[(KK) & 3], (BUFK) * A_BYTES + ((KK) >> 2) * OA::BYTES)
+// one step out of A buffer BUFK: 4 * KS k-blocks of 8 MFMAs, the fragment of the next one requested first
+#define AXC_TILE(BUFK)                                                                           \
+    do {                                                                                         \
+        AXC_FRAG(0, BUFK, 0);                                                                    \
+        _Pragma("unroll") for (int kk = 0; kk < 4 * KS; kk++) {                                  \
+            if (kk + 1 < 4 * KS) {                                                               \
+                AXC_FRAG((kk + 1) & 1, BUFK, kk + 1);                                            \
+                AXF_LGKM(1);                                                                     \
+            } else {                                                                             \
+                AXF_LGKM(0);                                                                     \
+            }                                                                                    \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+            _Pragma("unroll") for (int e = 0; e < 4; e++)                                        \
+                _Pragma("unroll") for (int j = 0; j < TN; j++)                                   \
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][kk][e], fa[kk & 1].get(e), \
+                                                                  (kk == 0 && e == 0) ? zero : acc[j], 0, 0, 0); \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+        }                                                                                        \
+    } while (0)
+
+    // Write-back of the 32 x 64 tile in `acc` (rows m0 ..): register v of lane l is row l & 31, column
+    // 32 j + 8 (v >> 2) + 4 (l >> 5) + (v & 3).  The tile is turned through the wave's 8 KiB of LDS as rows of
+    // 256 bytes (16-byte chunk c of row r kept at chunk c ^ (r & 15): 16 rows of one chunk column, or the 16
+    // chunks of one row, touch every bank once), so that a store instruction writes 4 rows of 256 bytes.
+    auto write_back = [&](int64_t m0) {
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int gq = 0; gq < 4; gq++)
+                *reinterpret_cast<v4f *>(turn + frow * 256 + (((j * 8 + 2 * gq + fhalf) ^ (frow & 15)) << 4)) =
+                    v4f{acc[j][4 * gq], acc[j][4 * gq + 1], acc[j][4 * gq + 2], acc[j][4 * gq + 3]};
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            v4f r[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const int row = (half * 4 + p) * 4 + rrow;
+                r[p] = *reinterpret_cast<const v4f *>(turn + row * 256 + ((rchunk ^ (row & 15)) << 4));
+            }
+            if (half == 1) {
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            }
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                v4f o = r[p];
+                if (g.alpha != 1.0f) o *= g.alpha;
+                    __builtin_nontemporal_store(o, reinterpret_cast<v4f *>(cdst + (m0 + (half * 4 + p) * 4) * g.ldc));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+#define AXC_STEP(BUFK, i)                                                                        \
+    do {                                                                                         \
+        const bool more = (i) + 1 < nblk;                                                        \
+        if (more) AXC_ISSUE_A(1 - (BUFK));                                                       \
+        if ((i) > 0) write_back((int64_t)((i) - 1) * BMS);                                       \
+        AXC_TILE(BUFK);                                                                          \
+        if (more) {                                                                              \
+            if ((i) > 0) AXF_VM(NSTORES); else AXF_VM(0);                                        \
+            __builtin_amdgcn_s_barrier();                                                        \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+        }                                                                                        \
+    } while (0)
+
+    AXF_VM(0);                                    // the first block of A
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    for (int i = 0; i < nblk; i += 2) {
+        AXC_STEP(0, i);
+        if (i + 1 >= nblk) break;
+        AXC_STEP(1, i + 1);
+    }
+    write_back((int64_t)(nblk - 1) * BMS);
+#undef AXC_ISSUE_A
+#undef AXC_FRAG
+#undef AXC_TILE
+#undef AXC_STEP
+}
+
+template <int KS>
+int launch_nt_cols(const SgemmArgs &g, int64_t batch) {
+    constexpr int smem = 2 * KS * 4096 + 4 * 8192;                        // 64 KiB at most
+    note_kernel("sgemm_nt_cols256_dma");
+    // One workgroup walks all the rows of A: cutting them into two or four runs (shorter workgroups, more of them) costs
+    // more in loads of B fragments than it evens out at the end of the launch (512 heads of 512 x 512, K = 64, zeros:
+    // 151.6 us whole, 154.0 in halves, 161.6 in quarters).
+    hipLaunchKernelGGL((k_sgemm_nt_cols<KS>), dim3((unsigned)(g.N / 256), (unsigned)batch), dim3(256), smem, kStream, g);
+    return check_launch("sgemm_nt_cols256_dma");
+}
+
+// Taken ahead of the row-block walk when the columns come in blocks of 256 and the rows in blocks of 32, from eight
+// steps per workgroup on (same box, row-block walk -> this one; 512 heads of 512 x 512, K = 64: 171 -> 163 us on
+// random operands, 155 -> 149 on zeros; K = 128: 305 -> 276; K = 32: 113 -> 108; 256 heads of 1024 x 1024: 337 ->
+// 319; with M = 128, four steps, the row-block walk stays ahead, 92 against 94).  A forced AX_HIP_NT_WALK=2 takes
+// it from four steps on.  -1: not taken.
+int try_nt_cols(const SgemmArgs &g, int64_t batch) {
+    if (tuning().f32_tile != 0 || tuning().nt_walk == 1) return -1;
+    if (g.K % 32 != 0 || g.K < 32 || g.K > 128 || g.M % 32 != 0 || g.M < (tuning().nt_walk == 2 ? 128 : 256) || g.N % 256 != 0) return -1;
+    if (g.beta != 0.0f || g.bias || g.col_scale || g.act != AXHIP_ACT_NONE) return -1;
+    if ((g.N / 256) * batch < 2 * cu_count() || batch > 65535 || g.N / 256 > 0x7fffffff) return -1;
+    if ((((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.C) & 15) != 0 || g.lda % 4 != 0 || g.ldb % 4 != 0 || g.ldc % 4 != 0 ||
+        g.stride_a % 4 != 0 || g.stride_b % 4 != 0 || g.stride_c % 4 != 0 || g.lda >= (1 << 20) || g.ldb >= (1 << 20))
+        return -1;
+    switch (g.K / 32) {
+        case 1: return launch_nt_cols<1>(g, batch);
+        case 2: return launch_nt_cols<2>(g, batch);
+        case 3: return launch_nt_cols<3>(g, batch);
+        default: return launch_nt_cols<4>(g, batch);
+    }
+}
+
+// =====================================================================================
 // C = alpha * A * B for batched products with many output tiles and a K of a few hundred (P V of
 // attention heads: K = 512, N = 64).  With a workgroup per tile, a third of each workgroup's life is its
 // first load latency and its write-back, and the workgroups that share a CU go through both together.
@@ -1617,7 +1821,8 @@ int dispatch_f32(const SgemmArgs &g, int transa, int transb, int64_t batch) {
     static const char *const nt_d[3] = {"sgemm_nt_128x128_dma", "sgemm_nt_64x64_dma", "sgemm_nt_64x64k2_dma"};
     static const char *const tn_d[3] = {"sgemm_tn_128x128_dma", "sgemm_tn_64x64_dma", "sgemm_tn_64x64k2_dma"};
     int rc = -1;
-    if (!transa && transb) rc = try_nt_rows(g, batch);
+    if (!transa && transb) rc = try_nt_cols(g, batch);
+    if (rc < 0 && !transa && transb) rc = try_nt_rows(g, batch);
     if (!transa && !transb) rc = try_nn_stream(g, batch);
     if (rc >= 0) return rc;
     if (!transa && !transb) rc = try_dma<true, false>(nn_d, g, batch);

@@ -217,10 +217,11 @@ int axhip_tuning_reload(void) {
     g_tuning.skinny_blocks = parse_count("AX_HIP_SKINNY_BLOCKS", 1, 65535);
     g_tuning.skinny_form = parse_count("AX_HIP_SKINNY_FORM", 1, 3);
     g_tuning.skinny_kps = parse_count("AX_HIP_SKINNY_KPS", 16, 8192) / 16 * 16;
+    g_tuning.nt_walk = parse_count("AX_HIP_NT_WALK", 1, 2);
     static const char *const w8a32_tiles[] = {"128x256", "128x128", "64x128", "32x128", "32x64"};
     g_tuning.w8a32_tile = parse_choice("AX_HIP_W8A32_TILE", w8a32_tiles, 5);
     return (g_tuning.i8_tile != 0) + (g_tuning.i8_splitk != 0) + (g_tuning.f32_tile != 0) + (g_tuning.f32_splitk != 0) +
-           (g_tuning.skinny_blocks != 0) + (g_tuning.w8a32_tile != 0) + (g_tuning.skinny_form != 0) + (g_tuning.skinny_kps != 0) + (g_tuning.i8_mfma != 0);
+           (g_tuning.skinny_blocks != 0) + (g_tuning.w8a32_tile != 0) + (g_tuning.skinny_form != 0) + (g_tuning.skinny_kps != 0) + (g_tuning.i8_mfma != 0) + (g_tuning.nt_walk != 0);
 }
 
 int axhip_workspace_reserve(size_t bytes, size_t *have) {
@@ -240,6 +241,7 @@ int axhip_tuning_get(const char *name) {
     if (!strcmp(name, "AX_HIP_SKINNY_BLOCKS")) return g_tuning.skinny_blocks;
     if (!strcmp(name, "AX_HIP_SKINNY_FORM")) return g_tuning.skinny_form;
     if (!strcmp(name, "AX_HIP_SKINNY_KPS")) return g_tuning.skinny_kps;
+    if (!strcmp(name, "AX_HIP_NT_WALK")) return g_tuning.nt_walk;
     if (!strcmp(name, "AX_HIP_W8A32_TILE")) return g_tuning.w8a32_tile;
     return -1;
 }

@@ -59,6 +59,8 @@ const char *axhip_device_name(void);          /* gcnArchName of device 0, "" wit
  *                        runs by default) or v_mfma_i32_32x32x32_i8; the results are the same bits
  *   AX_HIP_F32_TILE      64x64 | 64x64k2 | 128x128   fp32 tile on the aligned fast path (k2: two wave sets split each K slab)
  *   AX_HIP_F32_SPLITK    1..4096    K ranges of the fp32 few-tile route (1: never split)
+ *   AX_HIP_NT_WALK       1 | 2      batched A B^T with K <= 128: 1, a 128-row block of A stays in LDS and the column blocks of B^T
+ *                        are walked; 2, 256 rows of B stay in registers and A is walked in blocks of 32 rows (N a multiple of 256)
  *   AX_HIP_SKINNY_BLOCKS 1..65535   workgroups the skinny-M route aims for
  *   AX_HIP_SKINNY_KPS    16..8192   most rows of K one skinny-M workgroup takes (rounded down to a multiple of 16)
  *   AX_HIP_SKINNY_FORM   1..3       form of the skinny-M kernel for M <= 8: 1, workgroups of 256 threads; 2, the same with the

@@ -43,7 +43,7 @@ def test_tuning_variables_parse(monkeypatch):
     from axiom_amd import AxHip
     h = AxHip()
     names = ("AX_HIP_I8_TILE", "AX_HIP_I8_SPLITK", "AX_HIP_F32_TILE", "AX_HIP_F32_SPLITK", "AX_HIP_SKINNY_BLOCKS", "AX_HIP_W8A32_TILE",
-             "AX_HIP_SKINNY_FORM", "AX_HIP_SKINNY_KPS", "AX_HIP_I8_MFMA")
+             "AX_HIP_SKINNY_FORM", "AX_HIP_SKINNY_KPS", "AX_HIP_I8_MFMA", "AX_HIP_NT_WALK")
     for n in names:
         monkeypatch.delenv(n, raising=False)
     assert h.L.axhip_tuning_reload() == 0
@@ -56,6 +56,7 @@ def test_tuning_variables_parse(monkeypatch):
              "AX_HIP_SKINNY_BLOCKS": [("512", 512), ("65535", 65535), ("65536", 0), ("many", 0)],
              "AX_HIP_I8_MFMA": [("16", 16), ("32", 32), ("24", 0), ("64", 0), ("x", 0)],
              "AX_HIP_SKINNY_FORM": [("1", 1), ("3", 3), ("4", 0), ("0", 0), ("pre", 0)],
+             "AX_HIP_NT_WALK": [("1", 1), ("2", 2), ("3", 0), ("0", 0), ("cols", 0)],
              "AX_HIP_SKINNY_KPS": [("512", 512), ("1000", 992), ("16", 16), ("15", 0), ("8193", 0)],
              "AX_HIP_W8A32_TILE": [("128x256", 1), ("128x128", 2), ("64x128", 3), ("32x128", 4), ("32x64", 5), ("64x64", 0), ("128", 0)]}
     for name, pairs in cases.items():

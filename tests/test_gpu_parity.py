@@ -674,20 +674,37 @@ def test_config4b_attention_shapes_full_size(hip, oracle):
     assert (np.abs(got - want) <= 1e-5 * scale).all()
 
 
+@pytest.mark.parametrize("walk", [0, 1, 2])
 @pytest.mark.parametrize("Bn,M,N,K,alpha", [(600, 128, 256, 64, 1.0), (300, 256, 320, 32, 0.5), (130, 512, 512, 96, 0.125),
-                                             (520, 128, 448, 128, 1.0), (1, 65536, 256, 64, 2.0), (513, 128, 256, 64, 1.0)])
-def test_short_k_nt_row_blocks(hip, oracle, Bn, M, N, K, alpha):
-    """A B^T with K of 32..128 and many row blocks: the kernel that keeps a 128-row block of A in LDS and
-    walks the column blocks; against the fp64 bound and, on sampled batch entries, the CPU path."""
-    say("short-k nt", Bn, M, N, K, alpha)
+                                             (520, 128, 448, 128, 1.0), (1, 65536, 256, 64, 2.0), (513, 128, 256, 64, 1.0),
+                                             (260, 160, 512, 128, 0.5), (300, 224, 512, 32, 1.0), (70, 1024, 2048, 96, 1.0), (512, 96 + 64, 512, 64, 1.0), (130, 256, 2048, 64, 0.25)])
+def test_short_k_nt_row_blocks(hip, oracle, monkeypatch, Bn, M, N, K, alpha, walk):
+    """A B^T with K of 32..128 and many output rows.  Walk 1: the kernel that keeps a 128-row block of A in
+    LDS and walks the column blocks of B^T; walk 2: the one that keeps 256 rows of B in registers and walks
+    A in blocks of 32 rows (taken when N is a multiple of 256, M of 32, and the workgroups fill the chip);
+    walk 0: the library's own choice.
+    Against the fp64 bound and, on sampled batch entries, the CPU path."""
+    say("short-k nt", Bn, M, N, K, alpha, "walk", walk)
     oracle.seed(Bn + M + N + K)
     a, b = oracle.normal((Bn, M, K)), oracle.normal((Bn, N, K))
     da, db = hip.array(a), hip.array(b)
     c = hip.empty((Bn, M, N))
     hip.check(hip.L.axhip_memset(c.ptr, 0xFF, c.nbytes))                 # every output must be written
-    hip.check(hip.L.axhip_sgemm_strided_batched(0, 1, M, N, K, alpha, da.ptr, K, M * K, db.ptr, K, N * K, 0.0,
-                                                c.ptr, N, M * N, Bn))
-    assert hip.last_kernel() == "sgemm_nt_rows128_dma"
+    if walk:
+        monkeypatch.setenv("AX_HIP_NT_WALK", str(walk))
+    assert hip.L.axhip_tuning_reload() == (1 if walk else 0)
+    try:
+        hip.check(hip.L.axhip_sgemm_strided_batched(0, 1, M, N, K, alpha, da.ptr, K, M * K, db.ptr, K, N * K, 0.0,
+                                                    c.ptr, N, M * N, Bn))
+        cols_route = walk != 1 and N % 256 == 0 and M % 32 == 0 and M >= (128 if walk == 2 else 256) and (N // 256) * Bn >= 512
+        rows_route = M % 128 == 0 and N % 64 == 0 and N >= 256 and (M // 128) * Bn >= 512
+        if cols_route:
+            assert hip.last_kernel() == "sgemm_nt_cols256_dma"
+        elif rows_route:
+            assert hip.last_kernel() == "sgemm_nt_rows128_dma"
+    finally:
+        monkeypatch.delenv("AX_HIP_NT_WALK", raising=False)
+        assert hip.L.axhip_tuning_reload() == 0
     got = c.numpy()
     assert not np.isnan(got).any()
     for h in sorted({0, Bn // 2, Bn - 1}):
