@@ -718,6 +718,42 @@ def test_short_k_nt_row_blocks(hip, oracle, monkeypatch, Bn, M, N, K, alpha, wal
     assert (np.abs(got.astype(np.float64).sum(axis=2) - want) <= 1e-5 * scale).all()
 
 
+@pytest.mark.parametrize("walk", [1, 2])
+@pytest.mark.parametrize("Bn,M,N,K,alpha,pad", [(520, 256, 256, 64, 0.5, 4), (260, 384, 512, 96, 1.0, 8), (600, 128, 256, 32, 2.0, 12)])
+def test_short_k_nt_padded_leading_dimensions(hip, oracle, monkeypatch, Bn, M, N, K, alpha, pad, walk):
+    """The two short-K A B^T walks on operands and a result whose rows are `pad` floats longer than the
+    matrices: pad columns are neither read into the sums nor written."""
+    say("short-k nt padded", Bn, M, N, K, alpha, pad, "walk", walk)
+    oracle.seed(3 * Bn + M + N + K)
+    lda, ldb, ldc = K + pad, K + pad, N + pad
+    a_full, b_full = oracle.normal((Bn, M, lda)), oracle.normal((Bn, N, ldb))
+    a_full[:, :, K:] = np.float32(1e30)           # would wreck every sum it got into
+    b_full[:, :, K:] = np.float32(-1e30)
+    a, b = a_full[:, :, :K], b_full[:, :, :K]
+    da, db = hip.array(a_full), hip.array(b_full)
+    c = hip.empty((Bn, M, ldc))
+    hip.check(hip.L.axhip_memset(c.ptr, 0xFF, c.nbytes))
+    monkeypatch.setenv("AX_HIP_NT_WALK", str(walk))
+    assert hip.L.axhip_tuning_reload() == 1
+    try:
+        hip.check(hip.L.axhip_sgemm_strided_batched(0, 1, M, N, K, alpha, da.ptr, lda, M * lda, db.ptr, ldb, N * ldb, 0.0,
+                                                    c.ptr, ldc, M * ldc, Bn))
+        assert hip.last_kernel() == ("sgemm_nt_cols256_dma" if walk == 2 else "sgemm_nt_rows128_dma")
+    finally:
+        monkeypatch.delenv("AX_HIP_NT_WALK", raising=False)
+        assert hip.L.axhip_tuning_reload() == 0
+    full = c.numpy()
+    got = full[:, :, :N]
+    assert not np.isnan(got).any() and np.isnan(full[:, :, N:]).all()
+    for h in sorted({0, Bn // 2, Bn - 1}):
+        want = oracle.gemm_opt_nt(np.ascontiguousarray(a[h]), np.ascontiguousarray(b[h])) * np.float32(alpha)
+        assert np.abs(got[h] - want).max() <= REL_FP32 * np.abs(want).max()
+    bsum = b.astype(np.float64).sum(axis=1)
+    want = alpha * np.einsum("hmk,hk->hm", a.astype(np.float64), bsum)
+    scale = abs(alpha) * np.einsum("hmk,hk->hm", np.abs(a).astype(np.float64), np.abs(b).astype(np.float64).sum(axis=1))
+    assert (np.abs(got.astype(np.float64).sum(axis=2) - want) <= 1e-5 * scale).all()
+
+
 @pytest.mark.parametrize("Bn,M,N,K,alpha,pad", [(200, 512, 64, 128, 1.0, 0), (67, 256, 384, 160, 0.5, 0), (280, 384, 64, 512, 1.0, 0),
                                                  (72, 512, 128, 1024, 0.25, 0), (264, 256, 64, 224, 2.0, 8), (9, 4096, 256, 192, 1.0, 4)])
 def test_streamed_nn_tiles(hip, oracle, Bn, M, N, K, alpha, pad):
