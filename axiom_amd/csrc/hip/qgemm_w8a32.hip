@@ -390,7 +390,9 @@ int launch_gemv(const float *a, const int8_t *w, const float *s, float *out, int
         }
     }
     if (N >= 64 * cus) return launch_rows<MR, 4>(a, w, s, out, N, K);
-    if (N >= 16 * cus) return launch_rows<MR, 2>(a, w, s, out, N, K);
+    // eight rows of activations leave room for two workgroups per CU only: two weight rows per wave from 2560 on, so that one
+    // round of workgroups covers N (M = 8, 3072 x 768: 9.7 -> 6.7 us; 2048 x 2048 stays on one, 7.2 against 8.0)
+    if (N >= 16 * cus || (MR >= 8 && N >= 10 * cus)) return launch_rows<MR, 2>(a, w, s, out, N, K);
     return launch_rows<MR, 1>(a, w, s, out, N, K);
 }
 
@@ -403,12 +405,19 @@ extern "C" int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w
     if (M < 0 || N < 0 || K < 0) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a32: negative dimension");
     if (M == 0 || N == 0) return AXHIP_OK;
     // The weight-streaming form pays M multiply-adds per weight byte on the vector ALU (4096 x 4096: 4.6 us at
-    // M = 1, +1.4 us per further row); from M = 7 on the matrix-core tiles are level or ahead everywhere, and with a
+    // M = 1, +1.4 us per further row); from M = 7 on the matrix-core tiles are level or ahead wherever K is long, and with a
     // long K already at M = 6, at M = 5 for large weights (us, streaming against tiles — M = 6: 4096 x 4096 11.7 / 11.5,
     // 1024 x 4096 10.0 / 8.2, 768 x 3072 10.0 / 8.5, 11008 x 4096 35.0 / 21.9; M = 5: 11008 x 4096 31.2 / 21.9 but
     // 4096 x 4096 10.5 / 11.5; with K = 768 or 1024 the streaming form stays ahead up to M = 6, 4.9-5.7 against 7.8-8.2).
     const bool tiles_for_rows = K >= 2048 && K % 32 == 0 && (M == 6 || (M == 5 && N * K > (int64_t(1) << 24)));
-    if (M > 6 || tiles_for_rows) return axhip::sgemm_i8w(M, N, K, a, w, w_scales, out);
+    // M = 7, 8 against a short K: the tiles' two launches (products, then the join of the K ranges) cost more than the
+    // vector ALU's extra rows (us, weights cached / from HBM, streaming against tiles — 768 x 768: M = 7 5.3 / 5.3 against
+    // 6.6 / 6.8, M = 8 5.5 / 5.6 against 6.6 / 7.4; 1024 x 1024, M = 8: 4.9 against 7.8; 4096 x 1024: 5.9 against 8.1 / 8.5;
+    // 8192 x 1024: 7.5 / 8.7 against 10.1 / 11.2; 2048 x 2048: 7.2 / 7.7 against 8.0 / 8.5; but 16384 x 768: 12.5 / 16.0
+    // against 11.5 / 13.7, 768 x 3072: 12.2 / 12.6 against 8.7 / 9.0, 4096 x 4096: 14.5 / 19.4 against 13.0 / 15.1).
+    const bool small_rows = (M == 7 || M == 8) && tuning().w8a32_tile == 0 &&
+                            ((K <= 1024 && N * K <= (int64_t(8) << 20)) || (K <= 2048 && N <= 2048));
+    if ((M > 6 && !small_rows) || tiles_for_rows) return axhip::sgemm_i8w(M, N, K, a, w, w_scales, out);
     if ((N + 3) / 4 > 0x7fffffff) return fail(AXHIP_ERR_SHAPE, "qgemm_w8a32: N too large");
     note_kernel("qgemm_w8a32_gemv");
     switch (M) {
@@ -417,6 +426,8 @@ extern "C" int axhip_qgemm_w8a32(const float *a, const int8_t *w, const float *w
         case 3: return launch_gemv<3>(a, w, w_scales, out, N, K);
         case 4: return launch_gemv<4>(a, w, w_scales, out, N, K);
         case 5: return launch_gemv<5>(a, w, w_scales, out, N, K);
-        default: return launch_gemv<6>(a, w, w_scales, out, N, K);
+        case 6: return launch_gemv<6>(a, w, w_scales, out, N, K);
+        case 7: return launch_gemv<7>(a, w, w_scales, out, N, K);
+        default: return launch_gemv<8>(a, w, w_scales, out, N, K);
     }
 }

@@ -813,7 +813,10 @@ W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 
                 (6, 33, 10000), (1, 70, 20000),
                 (6, 4100, 8192), (5, 8192, 2048), (6, 64, 2048),   # five or six rows with a long K: the tiles
                 (128, 4096, 192), (96, 2048, 320), (128, 3072, 160),   # 32x64 tiles: two slabs per stage (three and five stages), one
-                (32, 128, 517), (70, 260, 1031), (3, 64, 1037)]   # rows at odd byte offsets
+                (32, 128, 517), (70, 260, 1031), (3, 64, 1037),   # rows at odd byte offsets
+                # seven and eight rows against a short K: the weight-streaming form again (one and two weight rows per wave)
+                (7, 1024, 1024), (8, 3072, 768), (7, 2048, 2048), (8, 8192, 1024), (8, 2050, 1000), (7, 100, 517), (8, 40, 1024),
+                (8, 16384, 768), (7, 768, 3072)]   # ... and past its limits: the tiles
 
 
 @pytest.mark.parametrize("M,N,K", W8A32_SHAPES)
@@ -828,6 +831,9 @@ def test_w8a32_against_oracle(hip, oracle, golden, M, N, K):
     q, s = oracle.quantize_rows(w)
     got = hip.qgemm_w8a32(hip.array(a), hip.array(q), hip.array(s)).numpy()
     say("  ", hip.last_kernel())
+    if M in (7, 8):
+        streams = (K <= 1024 and N * K <= 8 << 20) or (K <= 2048 and N <= 2048)
+        assert (hip.last_kernel() == "qgemm_w8a32_gemv") == streams
     ref = oracle.qgemm_w8a32(a, q, s)
     key = f"w8a32_{M}x{N}x{K}_out"
     if key in golden.files:
