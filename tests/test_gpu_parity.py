@@ -800,6 +800,43 @@ def test_streamed_nn_tiles(hip, oracle, Bn, M, N, K, alpha, pad):
     assert np.abs(got - other).max() <= REL_FP32 * np.abs(other).max()
 
 
+@pytest.mark.parametrize("M,N,K,splits", [(128, 4096, 2048, 0), (64, 2048, 2048, 0), (256, 1024, 2048, 4), (96, 1024, 4096, 16), (100, 1000, 2048, 2)])
+def test_split_k_with_epilogue(hip, oracle, monkeypatch, M, N, K, splits):
+    """A product whose K is split over workgroups (by the library's own rule, or a forced count), with alpha, beta, bias
+    and an activation applied where the ranges meet, for fp32 operands (NN, NT, TN) and int8 weights: inside the fp64 bound."""
+    say("split-k with epilogue", M, N, K, splits)
+    oracle.seed(M + N + K)
+    a, b = oracle.uniform((M, K), -1, 1), oracle.uniform((K, N), -1, 1)
+    c0, bias = oracle.uniform((M, N), -1, 1), oracle.normal((N,), 0.0, 0.5)
+    da, db, dat, dbt, dbias = hip.array(a), hip.array(b), hip.array(np.ascontiguousarray(a.T)), hip.array(np.ascontiguousarray(b.T)), hip.array(bias)
+    w8 = np.random.default_rng(K).integers(-127, 128, (N, K), dtype=np.int8)
+    ws = np.random.default_rng(N).uniform(1e-3, 1e-2, N).astype(np.float32)
+    dw8, dws = hip.array(w8), hip.array(ws)
+    alpha, beta = np.float32(0.5), np.float32(1.0)
+    exact = alpha * (a.astype(np.float64) @ b.astype(np.float64)) + beta * c0 + bias
+    want = np.maximum(exact, 0.0)
+    bound = BOUND_FP32 * (abs(alpha) * (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)) + np.abs(c0) + np.abs(bias)) + 1e-30
+    want8 = (a.astype(np.float64) @ w8.astype(np.float64).T) * ws
+    bound8 = BOUND_FP32 * (np.abs(a).astype(np.float64) @ np.abs(w8).astype(np.float64).T) * ws + 1e-30
+    try:
+        if splits:
+            monkeypatch.setenv("AX_HIP_F32_SPLITK", str(splits))
+        hip.L.axhip_tuning_reload()
+        for name, (ta, tb, pa, lda, pb, ldb) in {"nn": (0, 0, da, K, db, N), "nt": (0, 1, da, K, dbt, K), "tn": (1, 0, dat, M, db, N)}.items():
+            c = hip.array(c0)
+            hip.check(hip.L.axhip_sgemm(ta, tb, M, N, K, alpha, pa.ptr, lda, pb.ptr, ldb, beta, c.ptr, N, dbias.ptr, 1))
+            say("  ", name, hip.last_kernel())
+            assert hip.last_kernel() == "sgemm_splitk"
+            got = c.numpy()
+            assert (np.abs(got - want) <= bound).all(), (name, float((np.abs(got - want) / bound).max()))
+        got8 = hip.qgemm_w8a32(da, dw8, dws).numpy()
+        say("  ", "w8a32", hip.last_kernel())
+        assert (np.abs(got8 - want8) <= bound8).all(), float((np.abs(got8 - want8) / bound8).max())
+    finally:
+        monkeypatch.delenv("AX_HIP_F32_SPLITK", raising=False)
+        assert hip.L.axhip_tuning_reload() == 0
+
+
 # ------------------------------------------------------------------ W8A32
 W8A32_SHAPES = [(1, 8, 8), (4, 16, 32), (8, 64, 128), (32, 128, 512), (16, 256, 1024), (3, 17, 45),
                 (1, 768, 3072), (1, 3072, 768), (8, 768, 768), (32, 768, 768), (128, 4096, 1024),
